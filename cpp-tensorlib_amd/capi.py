@@ -1,0 +1,290 @@
+"""ctypes binding of libtensorlib_hip.so (include/tensorlib_hip.h).
+
+This is the Python-side view of the C ABI used by the tests, bench.py and
+__graft_entry__.py. It adds nothing to the library: every method is one C call
+plus error translation. There is no CPU fallback here or anywhere below it — a
+missing library or a missing GPU raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libtensorlib_hip.so")
+
+i64, f32, cint, u32, u64, sz = C.c_int64, C.c_float, C.c_int, C.c_uint32, C.c_uint64, C.c_size_t
+P = C.c_void_p
+
+OK, ENODEVICE, EINVAL, EUNSUPPORTED, ENOMEM, ERUNTIME = 0, -1, -2, -3, -4, -5
+
+OPS = dict(add=0, sub=1, mul=2, div=3, pow=4, exp=5, log=6, sqrt=7, sigmoid=8, relu=9, affine=10,
+           badd=11, bsub=12, bmul=13, bdiv=14, bpow=15, softmax=26, row_sum=27, row_max=28,
+           recip=64)
+
+CENSUS = ["binary", "bcast", "unary", "row_op", "gemm", "gemv_f32", "gemv_bf16", "gemv_bf16_row",
+          "gemv_q4", "attn_decode", "rope", "rmsnorm", "rmsnorm_res", "swiglu", "argmax",
+          "kv_append", "kv_fill", "split_heads", "merge_heads", "gemm_bf16_nt", "attn_prefill"]
+
+# name -> (restype, argtypes): exactly the declarations of include/tensorlib_hip.h
+SIGNATURES = {
+    "tlhip_init": (cint, [cint]),
+    "tlhip_abi_version": (cint, []),
+    "tlhip_arch": (C.c_char_p, []),
+    "tlhip_last_error": (C.c_char_p, []),
+    "tlhip_device_info": (cint, [C.POINTER(cint), C.POINTER(i64), C.POINTER(cint)]),
+    "tlhip_malloc": (cint, [C.POINTER(P), sz]),
+    "tlhip_free": (cint, [P]),
+    "tlhip_host_alloc": (cint, [C.POINTER(P), sz]),
+    "tlhip_host_free": (cint, [P]),
+    "tlhip_memcpy_h2d": (cint, [P, P, sz]),
+    "tlhip_memcpy_d2h": (cint, [P, P, sz]),
+    "tlhip_memcpy_h2d_async": (cint, [P, P, sz]),
+    "tlhip_memcpy_d2d_async": (cint, [P, P, sz]),
+    "tlhip_fill_u32": (cint, [P, u32, sz]),
+    "tlhip_sync": (cint, []),
+    "tlhip_graph_begin": (cint, []),
+    "tlhip_graph_end": (cint, [C.POINTER(P)]),
+    "tlhip_graph_launch": (cint, [P]),
+    "tlhip_graph_destroy": (cint, [P]),
+    "tlhip_event_create": (cint, [C.POINTER(P)]),
+    "tlhip_event_record": (cint, [P]),
+    "tlhip_event_elapsed_ms": (cint, [P, P, C.POINTER(f32)]),
+    "tlhip_event_destroy": (cint, [P]),
+    "tlhip_census": (cint, [C.POINTER(u64), cint]),
+    "tlhip_census_reset": (cint, []),
+    "tlhip_binary": (cint, [cint, P, i64, P, i64, P, i64, i64, f32, f32]),
+    "tlhip_binary_bcast": (cint, [cint, P, i64, i64, i64, P, i64, i64, i64, P, i64, i64, i64, f32, f32]),
+    "tlhip_unary": (cint, [cint, P, i64, P, i64, i64, f32, f32]),
+    "tlhip_row_op": (cint, [cint, P, i64, P, i64, i64, i64, f32, f32]),
+    "tlhip_gemm": (cint, [P, i64, i64, cint, P, i64, i64, cint, P, i64, i64, i64, i64, f32, f32]),
+    "tlhip_gemv_f32": (cint, [P, P, P, i64, i64]),
+    "tlhip_gemv_bf16": (cint, [P, P, P, i64, i64]),
+    "tlhip_gemv_bf16_row": (cint, [P, P, P, i64, i64]),
+    "tlhip_gemv_q4": (cint, [P, P, P, P, i64, i64, i64]),
+    "tlhip_attn_decode": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
+    "tlhip_attn_prefill": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint, i64]),
+    "tlhip_kv_append": (cint, [P, P, P, P, i64, i64, i64, i64, cint]),
+    "tlhip_kv_fill": (cint, [P, P, P, P, i64, i64, i64, i64, cint, i64]),
+    "tlhip_rope": (cint, [P, P, i64, i64, i64, i64, f32, P]),
+    "tlhip_rmsnorm": (cint, [P, P, P, i64, f32, i64]),
+    "tlhip_rmsnorm_res": (cint, [P, P, P, P, P, i64, f32, i64]),
+    "tlhip_swiglu": (cint, [P, P, i64, i64]),
+    "tlhip_argmax": (cint, [P, i64, C.POINTER(i64)]),
+    "tlhip_argmax_async": (cint, [P, i64, P]),
+    "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
+    "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
+    "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
+    "tlhip_tune_gemv_q4": (cint, [cint, cint, cint]),
+}
+
+
+class TlHipError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("tlhip error %d: %s" % (code, msg))
+        self.code = code
+
+
+class DevBuf:
+    """A device allocation with its logical numpy dtype/shape."""
+
+    def __init__(self, lib, nbytes, dtype=np.float32, shape=None):
+        self.lib, self.nbytes = lib, int(nbytes)
+        self.dtype = np.dtype(dtype)
+        self.shape = tuple(shape) if shape is not None else (self.nbytes // self.dtype.itemsize,)
+        p = P()
+        lib._chk(lib.c.tlhip_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value
+
+    def at(self, byte_off):
+        return C.c_void_p(self.ptr + int(byte_off))
+
+    def upload(self, arr):
+        a = np.ascontiguousarray(arr)
+        assert a.nbytes <= self.nbytes, (a.nbytes, self.nbytes)
+        self.lib._chk(self.lib.c.tlhip_memcpy_h2d(self.ptr, a.ctypes.data_as(P), a.nbytes))
+        return self
+
+    def numpy(self, dtype=None, shape=None):
+        dtype = np.dtype(dtype or self.dtype)
+        out = np.empty(self.nbytes // dtype.itemsize, dtype)
+        self.lib._chk(self.lib.c.tlhip_memcpy_d2h(out.ctypes.data_as(P), self.ptr, out.nbytes))
+        shape = shape or (self.shape if dtype == self.dtype else None)
+        return out.reshape(shape) if shape is not None else out
+
+    def free(self):
+        if self.ptr:
+            self.lib.c.tlhip_free(self.ptr)
+            self.ptr = None
+
+
+class TlHip:
+    def __init__(self, path=LIB_PATH, init=True):
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                "%s is missing: build it with `python cpp-tensorlib_amd/build.py`" % path)
+        self.path = path
+        self.c = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(self.c, name)
+            fn.restype, fn.argtypes = res, args
+        if init:
+            self._chk(self.c.tlhip_init(0))
+
+    # ---- plumbing -----------------------------------------------------------
+    def _chk(self, rc):
+        if rc != 0:
+            raise TlHipError(rc, self.c.tlhip_last_error().decode())
+        return rc
+
+    def last_error(self):
+        return self.c.tlhip_last_error().decode()
+
+    def device_info(self):
+        cu, hbm, lds = cint(), i64(), cint()
+        self._chk(self.c.tlhip_device_info(C.byref(cu), C.byref(hbm), C.byref(lds)))
+        return dict(compute_units=cu.value, hbm_bytes=hbm.value, lds_bytes_per_cu=lds.value,
+                    arch=self.c.tlhip_arch().decode())
+
+    def empty(self, shape, dtype=np.float32):
+        shape = (shape,) if isinstance(shape, int) else tuple(shape)
+        n = int(np.prod(shape)) if shape else 1
+        return DevBuf(self, max(n, 1) * np.dtype(dtype).itemsize, dtype, shape)
+
+    def empty_bytes(self, nbytes):
+        return DevBuf(self, nbytes, np.uint8, (int(nbytes),))
+
+    def to_device(self, arr):
+        a = np.ascontiguousarray(arr)
+        return DevBuf(self, max(a.nbytes, 4), a.dtype, a.shape).upload(a)
+
+    def sync(self):
+        self._chk(self.c.tlhip_sync())
+
+    def census(self):
+        buf = (u64 * len(CENSUS))()
+        self._chk(self.c.tlhip_census(buf, len(CENSUS)))
+        return dict(zip(CENSUS, [int(v) for v in buf]))
+
+    def census_reset(self):
+        self.c.tlhip_census_reset()
+
+    # events
+    def event(self):
+        e = P()
+        self._chk(self.c.tlhip_event_create(C.byref(e)))
+        return e
+
+    def record(self, ev):
+        self._chk(self.c.tlhip_event_record(ev))
+
+    def elapsed_ms(self, a, b):
+        ms = f32()
+        self._chk(self.c.tlhip_event_elapsed_ms(a, b, C.byref(ms)))
+        return ms.value
+
+    # graphs
+    def graph_begin(self):
+        self._chk(self.c.tlhip_graph_begin())
+
+    def graph_end(self):
+        g = P()
+        self._chk(self.c.tlhip_graph_end(C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        self._chk(self.c.tlhip_graph_launch(g))
+
+    def graph_destroy(self, g):
+        self._chk(self.c.tlhip_graph_destroy(g))
+
+    # ---- ops (thin; raise on any non-zero status) -----------------------------
+    def binary(self, op, a, b, out, n, scale=1.0, offset=0.0, ao=0, bo=0, oo=0):
+        self._chk(self.c.tlhip_binary(OPS[op], a.ptr, ao, b.ptr, bo, out.ptr, oo, n, scale, offset))
+
+    def binary_bcast(self, op, a, astr, b, bstr, out, m, n, scale=1.0, offset=0.0):
+        self._chk(self.c.tlhip_binary_bcast(OPS[op], a.ptr, 0, astr[0], astr[1], b.ptr, 0, bstr[0],
+                                            bstr[1], out.ptr, 0, m, n, scale, offset))
+
+    def unary(self, op, a, out, n, scale=1.0, offset=0.0, ao=0, oo=0):
+        self._chk(self.c.tlhip_unary(OPS[op], a.ptr, ao, out.ptr, oo, n, scale, offset))
+
+    def row_op(self, op, a, out, rows, cols, scale=1.0, offset=0.0):
+        self._chk(self.c.tlhip_row_op(OPS[op], a.ptr, 0, out.ptr, 0, rows, cols, scale, offset))
+
+    def gemm(self, a, lda, ta, b, ldb, tb, out, m, n, k, scale=1.0, offset=0.0):
+        self._chk(self.c.tlhip_gemm(a.ptr, 0, lda, int(ta), b.ptr, 0, ldb, int(tb), out.ptr, 0, m, n,
+                                    k, scale, offset))
+
+    def gemv_f32(self, a, B, y, n, k):
+        self._chk(self.c.tlhip_gemv_f32(a.ptr, B.ptr, y.ptr, n, k))
+
+    def gemv_bf16(self, a, B, y, n, k):
+        self._chk(self.c.tlhip_gemv_bf16(a.ptr, B.ptr, y.ptr, n, k))
+
+    def gemv_bf16_row(self, a, W, y, n, k):
+        self._chk(self.c.tlhip_gemv_bf16_row(a.ptr, W.ptr, y.ptr, n, k))
+
+    def gemv_q4(self, a, wq, y, N, K, group=32, wq_off=0):
+        """wq: one buffer [packed N*K/2 bytes | scales], as the reference stores it."""
+        qp = wq.ptr + wq_off
+        self._chk(self.c.tlhip_gemv_q4(a.ptr, qp, qp + N * K // 2, y.ptr, N, K, group))
+
+    def attn_decode(self, q, K, V, out, Hq, Hkv, ctx, kv_max, D, scale, kv_bf16=False):
+        self._chk(self.c.tlhip_attn_decode(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, ctx, kv_max, D,
+                                           scale, int(kv_bf16)))
+
+    def attn_prefill(self, q, K, V, out, Hq, Hkv, T, kv_max, D, scale, kv_bf16=False, pos0=0):
+        self._chk(self.c.tlhip_attn_prefill(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, T, kv_max, D,
+                                            scale, int(kv_bf16), pos0))
+
+    def kv_append(self, Kc, Vc, k, v, pos, kv_max, Hkv, D, kv_bf16=False):
+        self._chk(self.c.tlhip_kv_append(Kc.ptr, Vc.ptr, k.ptr, v.ptr, pos, kv_max, Hkv, D,
+                                         int(kv_bf16)))
+
+    def kv_fill(self, Kc, Vc, K, V, T, kv_max, Hkv, D, kv_bf16=False, pos0=0):
+        self._chk(self.c.tlhip_kv_fill(Kc.ptr, Vc.ptr, K.ptr, V.ptr, T, kv_max, Hkv, D,
+                                       int(kv_bf16), pos0))
+
+    def rope(self, x, out, rows, T, D, pos, base, bias=None):
+        self._chk(self.c.tlhip_rope(x.ptr, out.ptr, rows, T, D, pos, base,
+                                    bias.ptr if bias is not None else None))
+
+    def rmsnorm(self, x, w, out, n, eps, rows=1):
+        self._chk(self.c.tlhip_rmsnorm(x.ptr, w.ptr, out.ptr, n, eps, rows))
+
+    def rmsnorm_res(self, x, delta, w, xout, hout, n, eps, rows=1):
+        self._chk(self.c.tlhip_rmsnorm_res(x.ptr, delta.ptr, w.ptr, xout.ptr, hout.ptr, n, eps, rows))
+
+    def swiglu(self, gu, out, ff, rows=1):
+        self._chk(self.c.tlhip_swiglu(gu.ptr, out.ptr, ff, rows))
+
+    def argmax(self, x, n):
+        idx = i64()
+        self._chk(self.c.tlhip_argmax(x.ptr, n, C.byref(idx)))
+        return idx.value
+
+    def gemm_bf16_nt(self, A, W, out, M, N, K):
+        self._chk(self.c.tlhip_gemm_bf16_nt(A.ptr, W.ptr, out.ptr, M, N, K))
+
+    def split_heads(self, src, bias, dst, T, ld, off, H, D):
+        self._chk(self.c.tlhip_split_heads(src.ptr, bias.ptr if bias is not None else None, dst.ptr,
+                                           T, ld, off, H, D))
+
+    def merge_heads(self, src, dst, T, H, D):
+        self._chk(self.c.tlhip_merge_heads(src.ptr, dst.ptr, T, H, D))
+
+    def tune_gemv_q4(self, rows=0, kw=0, bpc=0):
+        self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc))
+
+
+_lib = None
+
+
+def load():
+    """The process-wide library handle (initialises device 0). Raises when the
+    library has not been built or no gfx950 GPU is present."""
+    global _lib
+    if _lib is None:
+        _lib = TlHip()
+    return _lib

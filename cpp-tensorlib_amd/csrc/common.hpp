@@ -1,0 +1,107 @@
+// Shared host/device helpers for the gfx950 kernels behind the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/tensorlib_hip.h"
+
+namespace tlhip {
+
+constexpr int kWave = 64;  // CDNA wavefront width; every tiling below assumes it
+
+// ---- library state (one device, one stream) -------------------------------
+struct Context {
+  bool ready = false;
+  int device = -1;
+  int cus = 0;
+  int lds_per_cu = 0;
+  int64_t hbm_bytes = 0;
+  hipStream_t stream = nullptr;   // every launch and async copy goes here
+  bool capturing = false;
+  // grow-only device scratch (split-K / split-KV partials, argmax partials)
+  void* scratch = nullptr;
+  size_t scratch_bytes = 0;
+  int* argmax_dev = nullptr;      // one int32 result slot
+  int* argmax_host = nullptr;     // pinned landing slot for the 4-byte result
+  uint64_t census[TLHIP_C_COUNT] = {};
+  // int4 GEMV launch-shape override (tlhip_tune_gemv_q4)
+  int tune_q4_rows = 0, tune_q4_kw = 0, tune_q4_bpc = 0;
+};
+
+Context& ctx();
+int fail(int code, const char* fmt, ...);   // records the message, returns code
+int hip_fail(hipError_t e, const char* what);
+void* scratch(size_t bytes);                // nullptr on allocation failure
+
+inline const char* at(const void* base, int64_t byte_off) {
+  return static_cast<const char*>(base) + byte_off;
+}
+inline char* at(void* base, int64_t byte_off) { return static_cast<char*>(base) + byte_off; }
+
+#define TLHIP_REQUIRE_READY()                                                   \
+  do {                                                                          \
+    if (!::tlhip::ctx().ready) {                                                \
+      int rc_ = tlhip_init(0);                                                  \
+      if (rc_ != 0) return rc_;                                                 \
+    }                                                                           \
+  } while (0)
+
+#define TLHIP_CHECK_LAUNCH(id)                                                  \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) return ::tlhip::hip_fail(e_, "kernel launch");        \
+    ::tlhip::ctx().census[id]++;                                                \
+    return TLHIP_OK;                                                            \
+  } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device helpers ----------------------------------------------------------
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+  return v;
+}
+
+// Block-wide sum for blocks of NW wavefronts; `red` is NW floats of LDS.
+// Every thread gets the result. Summation order is fixed (wave 0..NW-1).
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; i++) t += red[i];
+  __syncthreads();
+  return t;
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t packed) {  // element 0 of a pair
+  return __uint_as_float(packed << 16);
+}
+__device__ __forceinline__ float bf16_hi(uint32_t packed) {  // element 1 of a pair
+  return __uint_as_float(packed & 0xffff0000u);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t x = __float_as_uint(f);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return static_cast<uint16_t>(x >> 16);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace tlhip

@@ -1,0 +1,494 @@
+// Decode GEMV kernels (batch 1, weight-stationary, HBM-bound).
+//
+// Row layouts (int4 [N][K/2] + scales, bf16 [N][K]): gemv_rows_kernel.
+//   * persistent blocks: the activation vector x is staged ONCE per block into
+//     LDS in a lane-interleaved layout, then the block walks row tiles;
+//   * every lane streams 16-byte units of a weight row (32 int4 weights = one
+//     scale group, or 8 bf16 weights) with global_load_dwordx4, fully
+//     coalesced along K, R rows in flight per wavefront so that one x fragment
+//     (held in VGPRs) is reused R times;
+//   * nibbles are unpacked and scaled in registers, fp32 accumulate;
+//   * K is split over the lanes of a wavefront and, for short-N shapes, over
+//     KW wavefronts of the block; partial sums are combined with wave
+//     shuffles and a fixed-order LDS pass: no atomics, deterministic.
+//
+// Column layouts (f32/bf16 [K][N], the array seam's layout): gemv_cols_kernel.
+//   * a lane owns 16 bytes of consecutive columns, a wavefront 64 of those,
+//     K is split over the 4 wavefronts of a block and over gridDim.y; split
+//     partials go to scratch and are summed in a fixed order by a second
+//     kernel.
+#include "common.hpp"
+
+namespace tlhip {
+
+// ---------------------------------------------------------------------------
+// weight formats for the row kernel
+// ---------------------------------------------------------------------------
+
+// 16-byte streaming load: weights are read exactly once per GEMV, so they are
+// marked non-temporal and do not displace x and the scales in the caches.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream16(const uint4* p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// int4: a byte of a packed row holds k even in its low nibble and k+1 in its
+// high nibble. Instead of isolating the high nibble, the kernel converts the
+// WHOLE byte (lo + 16*hi) and the masked low nibble, and folds the difference
+// into the activations when they are staged:
+//     lo*x_e + hi*x_o  =  lo*(x_e - x_o/16) + (lo + 16*hi)*(x_o/16)
+// so a 32-bit word of 8 weights costs one v_and, eight v_cvt_f32_ubyteN and
+// eight FMAs. The "-8" of the offset-binary nibbles becomes -8*sum(x) per
+// group, also formed once at staging.
+__device__ __forceinline__ uint32_t low_nibbles(uint32_t v) {
+  uint32_t r;  // opaque to the optimiser so the byte converts below stay byte converts
+  asm("v_and_b32 %0, 0x0f0f0f0f, %1" : "=v"(r) : "v"(v));
+  return r;
+}
+__device__ __forceinline__ float byte0(uint32_t v) { return (float)(v & 0xffu); }
+__device__ __forceinline__ float byte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
+__device__ __forceinline__ float byte2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
+__device__ __forceinline__ float byte3(uint32_t v) { return (float)(v >> 24); }
+
+struct FmtQ4 {
+  static constexpr int E = 32;  // weights per 16-byte unit == one scale group
+  static constexpr bool kScaled = true;
+  // staged form of (x_even, x_odd, x_even, x_odd)
+  static __device__ __forceinline__ float4 stage(const float4 v) {
+    const float o0 = v.y * 0.0625f, o1 = v.w * 0.0625f;
+    return make_float4(v.x - o0, o0, v.z - o1, o1);
+  }
+  // sum_k nib_k * x_k over the unit, x in staged form
+  static __device__ __forceinline__ float dot(const uint4 w, const float4 (&x)[8]) {
+    const uint32_t d[4] = {w.x, w.y, w.z, w.w};
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t full = d[i], lo = low_nibbles(full);
+      const float4 xa = x[2 * i], xb = x[2 * i + 1];
+      a0 = fmaf(byte0(lo), xa.x, a0);
+      a1 = fmaf(byte0(full), xa.y, a1);
+      a0 = fmaf(byte1(lo), xa.z, a0);
+      a1 = fmaf(byte1(full), xa.w, a1);
+      a0 = fmaf(byte2(lo), xb.x, a0);
+      a1 = fmaf(byte2(full), xb.y, a1);
+      a0 = fmaf(byte3(lo), xb.z, a0);
+      a1 = fmaf(byte3(full), xb.w, a1);
+    }
+    return a0 + a1;
+  }
+};
+
+struct FmtBf16 {
+  static constexpr int E = 8;
+  static constexpr bool kScaled = false;
+  static __device__ __forceinline__ float4 stage(const float4 v) { return v; }
+  static __device__ __forceinline__ float dot(const uint4 w, const float4 (&x)[2]) {
+    float a0 = 0.f, a1 = 0.f;
+    a0 = fmaf(bf16_lo(w.x), x[0].x, a0);
+    a1 = fmaf(bf16_hi(w.x), x[0].y, a1);
+    a0 = fmaf(bf16_lo(w.y), x[0].z, a0);
+    a1 = fmaf(bf16_hi(w.y), x[0].w, a1);
+    a0 = fmaf(bf16_lo(w.z), x[1].x, a0);
+    a1 = fmaf(bf16_hi(w.z), x[1].y, a1);
+    a0 = fmaf(bf16_lo(w.w), x[1].z, a0);
+    a1 = fmaf(bf16_hi(w.w), x[1].w, a1);
+    return a0 + a1;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// row kernel
+// ---------------------------------------------------------------------------
+// W: [N][upr] 16-byte units. scales: [N][upr] f32 (int4 only).
+// Block = nw wavefronts arranged as (nw/KW row groups) x (KW K-splits).
+// LDS: x as float4 xs[(chunk*J + j)*64 + lane], J = E/4, so that lane l's j-th
+// fragment of chunk c is one conflict-free ds_read_b128; then KW*rows floats.
+template <typename Fmt, int R>
+__global__ __launch_bounds__(1024) void gemv_rows_kernel(
+    const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
+    float* __restrict__ y, int N, int upr, int KW, int ntiles) {
+  constexpr int J = Fmt::E / 4;
+  extern __shared__ float4 smem4[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nw = blockDim.x >> 6;
+  const int chunks = (upr + 63) >> 6;
+  float4* xs = smem4;
+  float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * 64);  // [chunks*64], int4 only
+  float* red = xsum + (Fmt::kScaled ? chunks * 64 : 0);
+
+  {  // stage x (K = upr*E floats) into the interleaved layout
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int n4 = upr * J;
+    for (int i = tid; i < n4; i += blockDim.x) {
+      const int u = i / J, j = i - u * J;
+      xs[((u >> 6) * J + j) * 64 + (u & 63)] = Fmt::stage(x4[i]);
+    }
+    if (Fmt::kScaled) {
+      for (int u = tid; u < upr; u += blockDim.x) {
+        float sx = 0.f;
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+          const float4 v = x4[u * J + j];
+          sx += (v.x + v.y) + (v.z + v.w);
+        }
+        xsum[u] = -8.0f * sx;  // sum_k (nib_k - 8) x_k = sum nib_k x_k - 8 sum x_k
+      }
+    }
+  }
+  __syncthreads();
+
+  const int kw = wave % KW;          // which K split this wavefront takes
+  const int wn = wave / KW;          // which row group of the block tile
+  const int groups = nw / KW;        // row groups per block tile
+  const int rows_per_tile = groups * R;
+
+  for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int row0 = t * rows_per_tile + wn * R;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+    for (int c = kw; c < chunks; c += KW) {
+      const int u = (c << 6) + lane;
+      if (u < upr) {
+        uint4 w[R];
+        float sc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const int row = min(row0 + r, N - 1);
+          const size_t idx = (size_t)row * upr + u;
+          w[r] = load_stream16(&W[idx]);
+          if (Fmt::kScaled) sc[r] = __builtin_nontemporal_load(&scales[idx]);
+        }
+        float4 xv[J];
+#pragma unroll
+        for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * 64 + lane];
+        if (Fmt::kScaled) {
+          const float bias = xsum[u];
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r] = fmaf(sc[r], Fmt::dot(w[r], xv) + bias, acc[r]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r] += Fmt::dot(w[r], xv);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+
+    if (KW == 1) {
+      float v = acc[0];
+#pragma unroll
+      for (int r = 1; r < R; r++) v = (lane == r) ? acc[r] : v;
+      if (lane < R && row0 + lane < N) y[row0 + lane] = v;
+    } else {
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) red[(wn * KW + kw) * R + r] = acc[r];
+      }
+      __syncthreads();
+      if (kw == 0 && lane < R && row0 + lane < N) {
+        float v = 0.f;
+        for (int s = 0; s < KW; s++) v += red[(wn * KW + s) * R + lane];
+        y[row0 + lane] = v;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// Generic int4 kernel for group sizes other than 32 (group % 8 == 0): one
+// wavefront per row, a lane eats one 32-bit word (8 nibbles, all in one group).
+__global__ __launch_bounds__(256) void gemv_q4_generic_kernel(
+    const float* __restrict__ x, const uint32_t* __restrict__ qw,
+    const float* __restrict__ scales, float* __restrict__ y, int N, int K, int group) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= N) return;
+  const int words = K >> 3, gpr = K / group;
+  const uint32_t* wr = qw + (size_t)row * words;
+  const float* sr = scales + (size_t)row * gpr;
+  float acc = 0.f;
+  for (int wi = lane; wi < words; wi += 64) {
+    const uint32_t v = wr[wi];
+    const float s = sr[(wi << 3) / group];
+    const float* xp = x + (wi << 3);
+    float d = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) d = fmaf((float)((int)((v >> (4 * j)) & 0xf) - 8), xp[j], d);
+    acc = fmaf(s, d, acc);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) y[row] = acc;
+}
+
+// ---------------------------------------------------------------------------
+// column kernel: B is [K][N], N contiguous
+// ---------------------------------------------------------------------------
+template <typename T> struct ColVec;
+template <> struct ColVec<float> {
+  static constexpr int V = 4;
+  using Raw = float4;
+  static __device__ __forceinline__ void fma(float (&acc)[4], float a, const Raw b) {
+    acc[0] = fmaf(a, b.x, acc[0]); acc[1] = fmaf(a, b.y, acc[1]);
+    acc[2] = fmaf(a, b.z, acc[2]); acc[3] = fmaf(a, b.w, acc[3]);
+  }
+};
+template <> struct ColVec<uint16_t> {
+  static constexpr int V = 8;
+  using Raw = uint4;
+  static __device__ __forceinline__ void fma(float (&acc)[8], float a, const Raw b) {
+    acc[0] = fmaf(a, bf16_lo(b.x), acc[0]); acc[1] = fmaf(a, bf16_hi(b.x), acc[1]);
+    acc[2] = fmaf(a, bf16_lo(b.y), acc[2]); acc[3] = fmaf(a, bf16_hi(b.y), acc[3]);
+    acc[4] = fmaf(a, bf16_lo(b.z), acc[4]); acc[5] = fmaf(a, bf16_hi(b.z), acc[5]);
+    acc[6] = fmaf(a, bf16_lo(b.w), acc[6]); acc[7] = fmaf(a, bf16_hi(b.w), acc[7]);
+  }
+};
+
+// grid = (ceil(N/(64*V)), S). Block = 4 wavefronts on the same 64*V columns,
+// wavefront w takes rows k0+w, k0+w+4, ... of this block's K range.
+// out = y when S == 1, else partials [S][N].
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_cols_kernel(const float* __restrict__ a,
+                                                        const T* __restrict__ B,
+                                                        float* __restrict__ out, int N, int K,
+                                                        int kchunk) {
+  constexpr int V = ColVec<T>::V;
+  using Raw = typename ColVec<T>::Raw;
+  __shared__ float red[3][64][V + 1];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col = (blockIdx.x * 64 + lane) * V;
+  const int k0 = blockIdx.y * kchunk;
+  const int k1 = min(K, k0 + kchunk);
+  float acc[V];
+#pragma unroll
+  for (int v = 0; v < V; v++) acc[v] = 0.f;
+  if (col < N) {  // N % V == 0 is guaranteed by the launcher
+    const T* bp = B + col;
+    int k = k0 + w;
+    for (; k + 12 < k1; k += 16) {  // 4 rows in flight per lane
+      const Raw b0 = *reinterpret_cast<const Raw*>(bp + (size_t)k * N);
+      const Raw b1 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 4) * N);
+      const Raw b2 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 8) * N);
+      const Raw b3 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 12) * N);
+      ColVec<T>::fma(acc, a[k], b0);
+      ColVec<T>::fma(acc, a[k + 4], b1);
+      ColVec<T>::fma(acc, a[k + 8], b2);
+      ColVec<T>::fma(acc, a[k + 12], b3);
+    }
+    for (; k < k1; k += 4) {
+      const Raw b0 = *reinterpret_cast<const Raw*>(bp + (size_t)k * N);
+      ColVec<T>::fma(acc, a[k], b0);
+    }
+  }
+  if (w > 0) {
+#pragma unroll
+    for (int v = 0; v < V; v++) red[w - 1][lane][v] = acc[v];
+  }
+  __syncthreads();
+  if (w == 0 && col < N) {
+    float* o = out + (size_t)blockIdx.y * N + col;
+#pragma unroll
+    for (int v = 0; v < V; v++) o[v] = ((acc[v] + red[0][lane][v]) + red[1][lane][v]) + red[2][lane][v];
+  }
+}
+
+// scalar-column fallback (N not a multiple of the vector width): one lane per column
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_cols_scalar_kernel(const float* __restrict__ a,
+                                                               const T* __restrict__ B,
+                                                               float* __restrict__ out, int N,
+                                                               int K, int kchunk) {
+  const int col = blockIdx.x * blockDim.x + threadIdx.x;
+  if (col >= N) return;
+  const int k0 = blockIdx.y * kchunk, k1 = min(K, k0 + kchunk);
+  float acc = 0.f;
+  for (int k = k0; k < k1; k++) {
+    float b;
+    if constexpr (sizeof(T) == 2) b = __uint_as_float((uint32_t)B[(size_t)k * N + col] << 16);
+    else b = B[(size_t)k * N + col];
+    acc = fmaf(a[k], b, acc);
+  }
+  out[(size_t)blockIdx.y * N + col] = acc;
+}
+
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part,
+                                                              float* __restrict__ y, int N,
+                                                              int S) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+  float v = part[i];
+  for (int s = 1; s < S; s++) v += part[(size_t)s * N + i];
+  y[i] = v;
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+struct RowCfg { int R, KW, nw, blocks; size_t lds; };
+
+// Launch shape for the row kernel. Goal: every CU holds >= ~16 wavefronts of
+// independent 16-byte loads, x is staged as few times as possible, and the
+// tile count divides evenly over the persistent blocks.
+static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, int tR, int tKW,
+                            int tBPC) {
+  const int chunks = (upr + 63) / 64;
+  const size_t xbytes = (size_t)chunks * 64 * E * 4;
+  RowCfg c{};
+  // wavefronts per block: enough that one or two blocks fill a CU even when x is big
+  c.nw = xbytes > 40 * 1024 ? 16 : 8;
+  int bpc = (int)((size_t)lds_per_cu / (xbytes + (size_t)chunks * 256 + 1024));
+  const int max_by_waves = 32 / c.nw;  // 8 wavefronts per SIMD, 4 SIMDs
+  if (bpc > max_by_waves) bpc = max_by_waves;
+  if (bpc < 1) bpc = 1;
+  if (tBPC > 0) bpc = tBPC;
+  const int64_t slots = (int64_t)cus * bpc * c.nw;  // resident wavefronts on the chip
+  // rows per wavefront: large when rows are plentiful (x fragment reuse), small otherwise
+  int R = 1;
+  for (int cand : {8, 4, 2}) {
+    if (N / cand >= slots * 2) { R = cand; break; }
+  }
+  if (R == 1 && N >= slots) R = 1;
+  // wavefronts sharing a row's K range: only when rows alone cannot fill the chip
+  int KW = 1;
+  while (KW < c.nw && KW * 2 <= chunks && (N / R) * KW < slots) KW *= 2;
+  if (tR > 0) R = tR;
+  if (tKW > 0) KW = tKW;
+  if (KW > c.nw) KW = c.nw;
+  c.R = R;
+  c.KW = KW;
+  const int rows_per_tile = (c.nw / KW) * R;
+  const int64_t ntiles = (N + rows_per_tile - 1) / rows_per_tile;
+  int64_t maxb = (int64_t)cus * bpc;
+  int64_t passes = (ntiles + maxb - 1) / maxb;
+  c.blocks = (int)((ntiles + passes - 1) / passes);
+  c.lds = xbytes + (size_t)chunks * 64 * 4 + (size_t)c.nw * 8 * 4 + 64;
+  return c;
+}
+
+template <typename Fmt>
+static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
+                       int64_t K, int census_id, int tR, int tKW, int tBPC) {
+  Context& c = ctx();
+  const int upr = (int)(K / Fmt::E);
+  RowCfg cfg = pick_rows_cfg(N, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC);
+  const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
+  const int ntiles = (int)((N + rows_per_tile - 1) / rows_per_tile);
+  using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int);
+  K_t fn = nullptr;
+  switch (cfg.R) {
+    case 1: fn = gemv_rows_kernel<Fmt, 1>; break;
+    case 2: fn = gemv_rows_kernel<Fmt, 2>; break;
+    case 4: fn = gemv_rows_kernel<Fmt, 4>; break;
+    case 8: fn = gemv_rows_kernel<Fmt, 8>; break;
+    default: return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
+  }
+  if (cfg.lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)cfg.lds);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
+  }
+  hipLaunchKernelGGL(fn, dim3(cfg.blocks), dim3(cfg.nw * 64), cfg.lds, c.stream, x,
+                     static_cast<const uint4*>(W), scales, y, (int)N, upr, cfg.KW, ntiles);
+  TLHIP_CHECK_LAUNCH(census_id);
+}
+
+template <typename T>
+static int launch_cols(const float* a, const T* B, float* y, int64_t N, int64_t K, int census_id) {
+  Context& c = ctx();
+  constexpr int V = ColVec<T>::V;
+  const bool vec = (N % V) == 0 && aligned16(B);
+  const int64_t ctiles = vec ? (N + 64 * V - 1) / (64 * V) : (N + 255) / 256;
+  // K splits: fill ~8 blocks per CU, keep >= 64 rows per split
+  int64_t S = ((int64_t)c.cus * 8 + ctiles - 1) / ctiles;
+  if (S > K / 64) S = K / 64;
+  if (S < 1) S = 1;
+  int kchunk = (int)((K + S - 1) / S);
+  kchunk = (kchunk + 3) & ~3;
+  S = (K + kchunk - 1) / kchunk;
+  float* out = y;
+  if (S > 1) {
+    out = static_cast<float*>(scratch((size_t)S * N * sizeof(float)));
+    if (!out) return fail(TLHIP_ENOMEM, "gemv: no scratch for %lld K-splits", (long long)S);
+  }
+  if (vec)
+    hipLaunchKernelGGL(gemv_cols_kernel<T>, dim3((unsigned)ctiles, (unsigned)S), dim3(256), 0,
+                       c.stream, a, B, out, (int)N, (int)K, kchunk);
+  else
+    hipLaunchKernelGGL(gemv_cols_scalar_kernel<T>, dim3((unsigned)ctiles, (unsigned)S), dim3(256),
+                       0, c.stream, a, B, out, (int)N, (int)K, kchunk);
+  if (S > 1)
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0,
+                       c.stream, out, y, (int)N, (int)S);
+  TLHIP_CHECK_LAUNCH(census_id);
+}
+
+static int check_gemv_args(const void* a, const void* B, const void* y, int64_t n, int64_t k,
+                           const char* who) {
+  if (!a || !B || !y) return fail(TLHIP_EINVAL, "%s: null pointer", who);
+  if (n <= 0 || k <= 0) return fail(TLHIP_EINVAL, "%s: n and k must be positive", who);
+  if (n > (int64_t)1 << 30 || k > (int64_t)1 << 30)
+    return fail(TLHIP_EUNSUPPORTED, "%s: dimension beyond 2^30", who);
+  if (!aligned16(a)) return fail(TLHIP_EINVAL, "%s: activation pointer not 16-byte aligned", who);
+  return 0;
+}
+
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" {
+
+int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, int64_t N,
+                  int64_t K, int64_t group) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(a, qw, y, N, K, "tlhip_gemv_q4")) return rc;
+  if (!scales) return fail(TLHIP_EINVAL, "tlhip_gemv_q4: null scales");
+  // the reference's gate (cuda.h:889-890)
+  if (group <= 0 || (K % group) != 0 || (group % 8) != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_q4: need group>0, K%%group==0, group%%8==0");
+  Context& c = ctx();
+  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
+  if (group == 32 && aligned16(qw) && xbytes + 2048 <= (size_t)c.lds_per_cu)
+    return launch_rows<FmtQ4>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
+                              static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
+                              c.tune_q4_kw, c.tune_q4_bpc);
+  hipLaunchKernelGGL(gemv_q4_generic_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, c.stream,
+                     static_cast<const float*>(a), static_cast<const uint32_t*>(qw),
+                     static_cast<const float*>(scales), static_cast<float*>(y), (int)N, (int)K,
+                     (int)group);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_GEMV_Q4);
+}
+
+int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_t k) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(a, W, y, n, k, "tlhip_gemv_bf16_row")) return rc;
+  if ((k % 8) != 0) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K %% 8 != 0");  // cuda.h:772
+  if (!aligned16(W)) return fail(TLHIP_EINVAL, "tlhip_gemv_bf16_row: weight pointer not 16-byte aligned");
+  const size_t xbytes = (size_t)((k / 8 + 63) / 64) * 64 * 8 * 4;
+  if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K too large for the LDS-staged kernel");
+  return launch_rows<FmtBf16>(static_cast<const float*>(a), W, nullptr, static_cast<float*>(y), n, k,
+                              TLHIP_C_GEMV_BF16_ROW, 0, 0, 0);
+}
+
+int tlhip_gemv_f32(const void* a, const void* B, void* y, int64_t n, int64_t k) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(a, B, y, n, k, "tlhip_gemv_f32")) return rc;
+  return launch_cols<float>(static_cast<const float*>(a), static_cast<const float*>(B),
+                            static_cast<float*>(y), n, k, TLHIP_C_GEMV_F32);
+}
+
+int tlhip_gemv_bf16(const void* a, const void* B, void* y, int64_t n, int64_t k) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(a, B, y, n, k, "tlhip_gemv_bf16")) return rc;
+  return launch_cols<uint16_t>(static_cast<const float*>(a), static_cast<const uint16_t*>(B),
+                               static_cast<float*>(y), n, k, TLHIP_C_GEMV_BF16);
+}
+
+}  // extern "C"

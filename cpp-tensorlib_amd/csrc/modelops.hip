@@ -1,0 +1,332 @@
+// Model ops of the decode step: rope, rmsnorm (+fused residual), swiglu,
+// argmax, KV-cache writes and the token-major/head-major moves of prefill.
+// All are launch- or latency-bound at decode sizes; rows are processed with
+// 128-bit accesses where the layout allows.
+#include "common.hpp"
+
+namespace tlhip {
+
+// ---- rope ---------------------------------------------------------------------
+// The angle is formed in fp64 exactly as the CPU path does (array.h:1719-1727):
+// theta = pow((double)base, -2j/D), ang = position*theta, then cos/sin are
+// rounded to f32 and the rotation runs in f32. Fast f32 intrinsics lose 1e-4
+// at positions in the thousands with base 1e6.
+__global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x,
+                                                   const float* __restrict__ bias,
+                                                   float* __restrict__ out, int64_t rows, int T,
+                                                   int D, int64_t pos, float base) {
+  const int half = D >> 1;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * half) return;
+  const int64_t r = i / half;
+  const int j = (int)(i - r * half);
+  const int64_t t = T ? r % T : 0;
+  const double position = (double)(pos + t);
+  const double theta = pow((double)base, -2.0 * (double)j / (double)D);
+  const double ang = position * theta;
+  const float c = (float)cos(ang), s = (float)sin(ang);
+  const size_t bi = (size_t)r * D;
+  float x0 = x[bi + j], x1 = x[bi + j + half];
+  if (bias) {
+    x0 += bias[bi + j];
+    x1 += bias[bi + j + half];
+  }
+  out[bi + j] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+  out[bi + j + half] = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+}
+
+// ---- rmsnorm --------------------------------------------------------------------
+// One block per row. Follows the array composition (array.h:2429-2433):
+// ms = sum(x*x) * (1/n); inv = 1/sqrt(ms + eps); out = (x*inv)*w.
+template <bool RES>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x,
+                                                      const float* __restrict__ delta,
+                                                      const float* __restrict__ w,
+                                                      float* __restrict__ xout,
+                                                      float* __restrict__ hout, int n, float eps) {
+  __shared__ float red[4];
+  const size_t base = (size_t)blockIdx.x * n;
+  float acc = 0.f;
+  if ((n & 3) == 0) {
+    const float4* x4 = reinterpret_cast<const float4*>(x + base);
+    const float4* d4 = RES ? reinterpret_cast<const float4*>(delta + base) : nullptr;
+    float4* xo4 = RES ? reinterpret_cast<float4*>(xout + base) : nullptr;
+    for (int i = threadIdx.x; i < (n >> 2); i += 256) {
+      float4 v = x4[i];
+      if (RES) {
+        const float4 d = d4[i];
+        v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        xo4[i] = v;
+      }
+      acc += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      float v = x[base + i];
+      if (RES) {
+        v += delta[base + i];
+        xout[base + i] = v;
+      }
+      acc += v * v;
+    }
+  }
+  if (RES) __threadfence_block();
+  const float sum = block_sum<4>(acc, red);  // also orders the xout stores before the re-read
+  const float inv = 1.0f / sqrtf(sum * (1.0f / (float)n) + eps);
+  const float* src = RES ? xout : x;
+  for (int i = threadIdx.x; i < n; i += 256) hout[base + i] = (src[base + i] * inv) * w[i];
+}
+
+// ---- swiglu -----------------------------------------------------------------------
+// out = (g * sigmoid(g)) * u, the order of array.h:2435-2439.
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gu,
+                                                     float* __restrict__ out, int64_t ff) {
+  const int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (f >= ff) return;
+  const size_t src = (size_t)blockIdx.y * 2 * ff + f;
+  const float g = gu[src];
+  const float sg = 1.0f / (1.0f + expf(-g));
+  out[(size_t)blockIdx.y * ff + f] = (g * sg) * gu[src + ff];
+}
+
+// ---- argmax ---------------------------------------------------------------------------
+// Stage 1: each block scans a slice and keeps (max, smallest index attaining it).
+// Stage 2: one block merges the slices. Ties always go to the smallest index
+// (array.h:2481-2494 uses a strict '>').
+__device__ __forceinline__ void argmax_merge(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+__device__ __forceinline__ void argmax_block(float& v, int& i, float* sv, int* si) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float ov = __shfl_xor(v, m, kWave);
+    const int oi = __shfl_xor(i, m, kWave);
+    argmax_merge(v, i, ov, oi);
+  }
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { sv[w] = v; si[w] = i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; k++) argmax_merge(v, i, sv[k], si[k]);
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_stage1(const float* __restrict__ in, int64_t n,
+                                                     float* __restrict__ pv, int* __restrict__ pi) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  float v = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float x = in[i];
+    if (x > v || idx == 0x7fffffff) { v = x; idx = (int)i; }
+  }
+  argmax_block(v, idx, sv, si);
+  if (threadIdx.x == 0) { pv[blockIdx.x] = v; pi[blockIdx.x] = idx; }
+}
+
+__global__ __launch_bounds__(256) void argmax_stage2(const float* __restrict__ pv,
+                                                     const int* __restrict__ pi, int nparts,
+                                                     int* __restrict__ out) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  float v = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < nparts; i += 256) argmax_merge(v, idx, pv[i], pi[i]);
+  argmax_block(v, idx, sv, si);
+  if (threadIdx.x == 0) out[0] = idx == 0x7fffffff ? 0 : idx;
+}
+
+// ---- cache writes and head moves -----------------------------------------------------------
+template <typename KT>
+__device__ __forceinline__ KT kv_narrow(float v);
+template <> __device__ __forceinline__ float kv_narrow<float>(float v) { return v; }
+template <> __device__ __forceinline__ uint16_t kv_narrow<uint16_t>(float v) { return f32_to_bf16_rne(v); }
+
+// k,v [Hkv,T,D] -> cache [Hkv,kv_max,D] rows pos0..pos0+T (T == 1: append)
+template <typename KT>
+__global__ __launch_bounds__(256) void kv_write_kernel(KT* __restrict__ Kc, KT* __restrict__ Vc,
+                                                       const float* __restrict__ k,
+                                                       const float* __restrict__ v, int64_t T,
+                                                       int64_t kv_max, int D, int64_t pos0,
+                                                       int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int d = (int)(i % D);
+  const int64_t hp = i / D;
+  const int64_t p = hp % T, h = hp / T;
+  const size_t dst = ((size_t)h * kv_max + pos0 + p) * D + d;
+  Kc[dst] = kv_narrow<KT>(k[i]);
+  Vc[dst] = kv_narrow<KT>(v[i]);
+}
+
+__global__ __launch_bounds__(256) void split_heads_kernel(const float* __restrict__ src,
+                                                          const float* __restrict__ bias,
+                                                          float* __restrict__ dst, int64_t T,
+                                                          int64_t ld, int64_t off, int D,
+                                                          int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;  // i indexes dst [H,T,D]
+  const int d = (int)(i % D);
+  const int64_t ht = i / D;
+  const int64_t t = ht % T, h = ht / T;
+  float v = src[(size_t)t * ld + off + h * D + d];
+  if (bias) v += bias[h * D + d];
+  dst[i] = v;
+}
+
+__global__ __launch_bounds__(256) void merge_heads_kernel(const float* __restrict__ src,
+                                                          float* __restrict__ dst, int64_t T,
+                                                          int64_t H, int D, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;  // i indexes dst [T,H*D]
+  const int d = (int)(i % D);
+  const int64_t th = i / D;
+  const int64_t h = th % H, t = th / H;
+  dst[i] = src[((size_t)h * T + t) * D + d];
+}
+
+static unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" {
+
+int tlhip_rope(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos,
+               float base, const void* bias) {
+  TLHIP_REQUIRE_READY();
+  if (!x || !out || rows < 0 || T < 0) return fail(TLHIP_EINVAL, "tlhip_rope: bad arguments");
+  if (D <= 0 || (D & 1)) return fail(TLHIP_EUNSUPPORTED, "tlhip_rope: head_dim must be even");  // cuda.h:1208
+  if (rows == 0) return TLHIP_OK;
+  const int64_t n = rows * (D / 2);
+  if (n > (int64_t)0x7fffffff * 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_rope: too large");
+  rope_kernel<<<dim3(blocks_for(n)), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(x), static_cast<const float*>(bias), static_cast<float*>(out), rows,
+      (int)T, (int)D, pos, base);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_ROPE);
+}
+
+int tlhip_rmsnorm(const void* x, const void* w, void* out, int64_t n, float eps, int64_t rows) {
+  TLHIP_REQUIRE_READY();
+  if (!x || !w || !out) return fail(TLHIP_EINVAL, "tlhip_rmsnorm: null pointer");
+  if (n <= 0 || rows <= 0 || n > 0x7fffffff || rows > 0x7fffffff)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_rmsnorm: n and rows must be positive");  // cuda.h:1290
+  if (!aligned16(x) || !aligned16(out)) return fail(TLHIP_EINVAL, "tlhip_rmsnorm: misaligned");
+  rmsnorm_kernel<false><<<dim3((unsigned)rows), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(x), nullptr, static_cast<const float*>(w), nullptr,
+      static_cast<float*>(out), (int)n, eps);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_RMSNORM);
+}
+
+int tlhip_rmsnorm_res(const void* x, const void* delta, const void* w, void* xout, void* hout,
+                      int64_t n, float eps, int64_t rows) {
+  TLHIP_REQUIRE_READY();
+  if (!x || !delta || !w || !xout || !hout) return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res: null pointer");
+  if (n <= 0 || rows <= 0 || n > 0x7fffffff || rows > 0x7fffffff)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_rmsnorm_res: n and rows must be positive");
+  if (!aligned16(x) || !aligned16(delta) || !aligned16(xout))
+    return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res: misaligned");
+  rmsnorm_kernel<true><<<dim3((unsigned)rows), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(x), static_cast<const float*>(delta), static_cast<const float*>(w),
+      static_cast<float*>(xout), static_cast<float*>(hout), (int)n, eps);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_RMSNORM_RES);
+}
+
+int tlhip_swiglu(const void* gu, void* out, int64_t ff, int64_t rows) {
+  TLHIP_REQUIRE_READY();
+  if (!gu || !out) return fail(TLHIP_EINVAL, "tlhip_swiglu: null pointer");
+  if (ff <= 0 || rows <= 0 || rows > 65535)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_swiglu: ff>0 and 0<rows<=65535 required");
+  swiglu_kernel<<<dim3(blocks_for(ff), (unsigned)rows), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(gu), static_cast<float*>(out), ff);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_SWIGLU);
+}
+
+int tlhip_argmax_async(const void* in, int64_t n, void* out_idx_dev) {
+  TLHIP_REQUIRE_READY();
+  if (!in || !out_idx_dev || n <= 0 || n > 0x7fffffff)
+    return fail(TLHIP_EINVAL, "tlhip_argmax: bad arguments");  // cuda.h:1263
+  int parts = (int)((n + 2047) / 2048);
+  if (parts > 1024) parts = 1024;
+  char* s = static_cast<char*>(scratch(2 * 1024 * sizeof(float)));
+  if (!s) return fail(TLHIP_ENOMEM, "tlhip_argmax: no scratch");
+  float* pv = reinterpret_cast<float*>(s);
+  int* pi = reinterpret_cast<int*>(s + 1024 * sizeof(float));
+  argmax_stage1<<<dim3(parts), dim3(256), 0, ctx().stream>>>(static_cast<const float*>(in), n, pv, pi);
+  argmax_stage2<<<dim3(1), dim3(256), 0, ctx().stream>>>(pv, pi, parts, static_cast<int*>(out_idx_dev));
+  TLHIP_CHECK_LAUNCH(TLHIP_C_ARGMAX);
+}
+
+int tlhip_argmax(const void* in, int64_t n, int64_t* out_idx) {
+  TLHIP_REQUIRE_READY();
+  if (!out_idx) return fail(TLHIP_EINVAL, "tlhip_argmax: null out pointer");
+  Context& c = ctx();
+  if (int rc = tlhip_argmax_async(in, n, c.argmax_dev)) return rc;
+  hipError_t e = hipMemcpyAsync(c.argmax_host, c.argmax_dev, sizeof(int), hipMemcpyDeviceToHost, c.stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+  if (e != hipSuccess) return hip_fail(e, "argmax result copy");
+  *out_idx = *c.argmax_host;
+  return TLHIP_OK;
+}
+
+static int kv_write(void* Kc, void* Vc, const void* k, const void* v, int64_t T, int64_t kv_max,
+                    int64_t n_kv_heads, int64_t D, int kv_bf16, int64_t pos0, int census_id,
+                    const char* who) {
+  if (!Kc || !Vc || !k || !v) return fail(TLHIP_EINVAL, "%s: null pointer", who);
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "%s: head_dim must be 64 or 128", who);  // cuda.h:1122
+  if (T <= 0 || n_kv_heads <= 0 || pos0 < 0 || pos0 + T > kv_max)
+    return fail(TLHIP_EINVAL, "%s: rows [%lld,%lld) outside the cache of %lld", who, (long long)pos0,
+                (long long)(pos0 + T), (long long)kv_max);
+  const int64_t total = n_kv_heads * T * D;
+  if (kv_bf16)
+    kv_write_kernel<uint16_t><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+        static_cast<uint16_t*>(Kc), static_cast<uint16_t*>(Vc), static_cast<const float*>(k),
+        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total);
+  else
+    kv_write_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+        static_cast<float*>(Kc), static_cast<float*>(Vc), static_cast<const float*>(k),
+        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total);
+  TLHIP_CHECK_LAUNCH(census_id);
+}
+
+int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, int64_t pos,
+                    int64_t kv_max, int64_t n_kv_heads, int64_t D, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  return kv_write(Kc, Vc, k_new, v_new, 1, kv_max, n_kv_heads, D, kv_bf16, pos, TLHIP_C_KV_APPEND,
+                  "tlhip_kv_append");
+}
+
+int tlhip_kv_fill(void* Kc, void* Vc, const void* K, const void* V, int64_t T, int64_t kv_max,
+                  int64_t n_kv_heads, int64_t D, int kv_bf16, int64_t pos0) {
+  TLHIP_REQUIRE_READY();
+  return kv_write(Kc, Vc, K, V, T, kv_max, n_kv_heads, D, kv_bf16, pos0, TLHIP_C_KV_FILL,
+                  "tlhip_kv_fill");
+}
+
+int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, int64_t ld,
+                      int64_t off, int64_t H, int64_t D) {
+  TLHIP_REQUIRE_READY();
+  if (!src || !dst) return fail(TLHIP_EINVAL, "tlhip_split_heads: null pointer");
+  if (T <= 0 || H <= 0 || D <= 0) return fail(TLHIP_EUNSUPPORTED, "tlhip_split_heads: empty");  // cuda.h:851
+  if (off < 0 || off + H * D > ld) return fail(TLHIP_EINVAL, "tlhip_split_heads: column block outside ld");
+  const int64_t total = H * T * D;
+  split_heads_kernel<<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(src), static_cast<const float*>(bias), static_cast<float*>(dst), T, ld,
+      off, (int)D, total);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_SPLIT_HEADS);
+}
+
+int tlhip_merge_heads(const void* src, void* dst, int64_t T, int64_t H, int64_t D) {
+  TLHIP_REQUIRE_READY();
+  if (!src || !dst) return fail(TLHIP_EINVAL, "tlhip_merge_heads: null pointer");
+  if (T <= 0 || H <= 0 || D <= 0) return fail(TLHIP_EUNSUPPORTED, "tlhip_merge_heads: empty");
+  const int64_t total = H * T * D;
+  merge_heads_kernel<<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+      static_cast<const float*>(src), static_cast<float*>(dst), T, H, (int)D, total);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_MERGE_HEADS);
+}
+
+}  // extern "C"

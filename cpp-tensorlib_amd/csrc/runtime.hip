@@ -1,0 +1,289 @@
+// Library state, memory, stream, graph capture, events and the dispatch census.
+#include "common.hpp"
+
+#include <cstring>
+#include <string>
+
+namespace tlhip {
+
+static thread_local char g_err[512] = "";
+
+Context& ctx() {
+  static Context* c = new Context();  // leaked on purpose: outlives late frees
+  return *c;
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(e == hipErrorOutOfMemory ? TLHIP_ENOMEM : TLHIP_ERUNTIME, "%s: %s", what,
+              hipGetErrorString(e));
+}
+
+void* scratch(size_t bytes) {
+  Context& c = ctx();
+  if (bytes <= c.scratch_bytes) return c.scratch;
+  if (c.capturing) return nullptr;  // growing would synchronise mid-capture
+  if (c.scratch) {
+    (void)hipStreamSynchronize(c.stream);
+    (void)hipFree(c.scratch);
+    c.scratch = nullptr;
+    c.scratch_bytes = 0;
+  }
+  size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+  if (hipMalloc(&c.scratch, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  c.scratch_bytes = want;
+  return c.scratch;
+}
+
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t v, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) dst[i] = v;
+}
+
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" {
+
+int tlhip_abi_version(void) { return TLHIP_ABI_VERSION; }
+
+const char* tlhip_last_error(void) { return g_err; }
+
+const char* tlhip_arch(void) { return ctx().ready ? "gfx950" : ""; }
+
+int tlhip_init(int device) {
+  Context& c = ctx();
+  if (c.ready) {
+    if (device != c.device) return fail(TLHIP_EINVAL, "already initialised on device %d", c.device);
+    return TLHIP_OK;
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count < 1) {
+    (void)hipGetLastError();
+    return fail(TLHIP_ENODEVICE, "no HIP device (%s)", e == hipSuccess ? "count 0" : hipGetErrorString(e));
+  }
+  if (device < 0 || device >= count) return fail(TLHIP_EINVAL, "device %d out of range", device);
+  hipDeviceProp_t prop;
+  if ((e = hipGetDeviceProperties(&prop, device)) != hipSuccess) return hip_fail(e, "hipGetDeviceProperties");
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(TLHIP_ENODEVICE, "device %d is %s; this library holds gfx950 code only", device,
+                prop.gcnArchName);
+  if ((e = hipSetDevice(device)) != hipSuccess) return hip_fail(e, "hipSetDevice");
+  if ((e = hipStreamCreate(&c.stream)) != hipSuccess) return hip_fail(e, "hipStreamCreate");
+  if ((e = hipMalloc((void**)&c.argmax_dev, 256)) != hipSuccess) return hip_fail(e, "hipMalloc");
+  if ((e = hipHostMalloc((void**)&c.argmax_host, 256, hipHostMallocDefault)) != hipSuccess)
+    return hip_fail(e, "hipHostMalloc");
+  c.device = device;
+  c.cus = prop.multiProcessorCount;
+  c.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+  c.hbm_bytes = (int64_t)prop.totalGlobalMem;
+  c.ready = true;
+  return TLHIP_OK;
+}
+
+int tlhip_device_info(int* compute_units, int64_t* hbm_bytes, int* lds_bytes_per_cu) {
+  TLHIP_REQUIRE_READY();
+  if (compute_units) *compute_units = ctx().cus;
+  if (hbm_bytes) *hbm_bytes = ctx().hbm_bytes;
+  if (lds_bytes_per_cu) *lds_bytes_per_cu = ctx().lds_per_cu;
+  return TLHIP_OK;
+}
+
+int tlhip_malloc(void** dptr, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!dptr) return fail(TLHIP_EINVAL, "tlhip_malloc: null out pointer");
+  *dptr = nullptr;
+  hipError_t e = hipMalloc(dptr, bytes ? bytes : 4);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return hip_fail(e, "hipMalloc");
+  }
+  return TLHIP_OK;
+}
+
+int tlhip_free(void* dptr) {
+  if (!dptr) return TLHIP_OK;
+  TLHIP_REQUIRE_READY();
+  hipError_t e = hipFree(dptr);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipFree");
+}
+
+int tlhip_host_alloc(void** hptr, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!hptr) return fail(TLHIP_EINVAL, "tlhip_host_alloc: null out pointer");
+  *hptr = nullptr;
+  hipError_t e = hipHostMalloc(hptr, bytes ? bytes : 4, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return hip_fail(e, "hipHostMalloc");
+  }
+  return TLHIP_OK;
+}
+
+int tlhip_host_free(void* hptr) {
+  if (!hptr) return TLHIP_OK;
+  TLHIP_REQUIRE_READY();
+  hipError_t e = hipHostFree(hptr);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipHostFree");
+}
+
+int tlhip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!bytes) return TLHIP_OK;
+  if (!dst || !src) return fail(TLHIP_EINVAL, "tlhip_memcpy_h2d: null pointer");
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "h2d copy");
+}
+
+int tlhip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!bytes) return TLHIP_OK;
+  if (!dst || !src) return fail(TLHIP_EINVAL, "tlhip_memcpy_d2h: null pointer");
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "d2h copy");
+}
+
+int tlhip_memcpy_h2d_async(void* dst, const void* src, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!bytes) return TLHIP_OK;
+  if (!dst || !src) return fail(TLHIP_EINVAL, "tlhip_memcpy_h2d_async: null pointer");
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "h2d async copy");
+}
+
+int tlhip_memcpy_d2d_async(void* dst, const void* src, size_t bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!bytes) return TLHIP_OK;
+  if (!dst || !src) return fail(TLHIP_EINVAL, "tlhip_memcpy_d2d_async: null pointer");
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "d2d async copy");
+}
+
+int tlhip_fill_u32(void* dst, uint32_t value, size_t count) {
+  TLHIP_REQUIRE_READY();
+  if (!count) return TLHIP_OK;
+  if (!dst || (reinterpret_cast<uintptr_t>(dst) & 3u)) return fail(TLHIP_EINVAL, "tlhip_fill_u32: bad pointer");
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  fill_u32_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx().stream>>>(
+      static_cast<uint32_t*>(dst), value, count);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "fill kernel");
+}
+
+int tlhip_sync(void) {
+  TLHIP_REQUIRE_READY();
+  hipError_t e = hipStreamSynchronize(ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipStreamSynchronize");
+}
+
+int tlhip_graph_begin(void) {
+  TLHIP_REQUIRE_READY();
+  Context& c = ctx();
+  if (c.capturing) return fail(TLHIP_EINVAL, "capture already open");
+  hipError_t e = hipStreamSynchronize(c.stream);
+  if (e == hipSuccess) e = hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal);
+  if (e != hipSuccess) return hip_fail(e, "hipStreamBeginCapture");
+  c.capturing = true;
+  return TLHIP_OK;
+}
+
+int tlhip_graph_end(void** graph_exec) {
+  TLHIP_REQUIRE_READY();
+  Context& c = ctx();
+  if (!c.capturing) return fail(TLHIP_EINVAL, "no capture open");
+  if (!graph_exec) return fail(TLHIP_EINVAL, "tlhip_graph_end: null out pointer");
+  *graph_exec = nullptr;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(c.stream, &g);
+  c.capturing = false;
+  if (e != hipSuccess || !g) return hip_fail(e, "hipStreamEndCapture");
+  hipGraphExec_t ex = nullptr;
+  e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+  *graph_exec = ex;
+  return TLHIP_OK;
+}
+
+int tlhip_graph_launch(void* graph_exec) {
+  TLHIP_REQUIRE_READY();
+  if (!graph_exec) return fail(TLHIP_EINVAL, "tlhip_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipGraphLaunch");
+}
+
+int tlhip_graph_destroy(void* graph_exec) {
+  if (!graph_exec) return TLHIP_OK;
+  hipError_t e = hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec));
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipGraphExecDestroy");
+}
+
+int tlhip_event_create(void** ev) {
+  TLHIP_REQUIRE_READY();
+  if (!ev) return fail(TLHIP_EINVAL, "tlhip_event_create: null out pointer");
+  hipEvent_t e_ = nullptr;
+  hipError_t e = hipEventCreate(&e_);
+  if (e != hipSuccess) return hip_fail(e, "hipEventCreate");
+  *ev = e_;
+  return TLHIP_OK;
+}
+
+int tlhip_event_record(void* ev) {
+  TLHIP_REQUIRE_READY();
+  if (!ev) return fail(TLHIP_EINVAL, "tlhip_event_record: null event");
+  hipError_t e = hipEventRecord(static_cast<hipEvent_t>(ev), ctx().stream);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipEventRecord");
+}
+
+int tlhip_event_elapsed_ms(void* start, void* stop, float* ms) {
+  TLHIP_REQUIRE_READY();
+  if (!start || !stop || !ms) return fail(TLHIP_EINVAL, "tlhip_event_elapsed_ms: null argument");
+  hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(stop));
+  if (e == hipSuccess)
+    e = hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop));
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipEventElapsedTime");
+}
+
+int tlhip_event_destroy(void* ev) {
+  if (!ev) return TLHIP_OK;
+  hipError_t e = hipEventDestroy(static_cast<hipEvent_t>(ev));
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipEventDestroy");
+}
+
+int tlhip_census(uint64_t* counts, int n) {
+  if (!counts || n < 0) return fail(TLHIP_EINVAL, "tlhip_census: bad arguments");
+  int m = n < TLHIP_C_COUNT ? n : (int)TLHIP_C_COUNT;
+  for (int i = 0; i < m; i++) counts[i] = ctx().census[i];
+  return TLHIP_OK;
+}
+
+int tlhip_census_reset(void) {
+  for (int i = 0; i < TLHIP_C_COUNT; i++) ctx().census[i] = 0;
+  return TLHIP_OK;
+}
+
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu) {
+  Context& c = ctx();
+  c.tune_q4_rows = rows_per_wave;
+  c.tune_q4_kw = k_waves;
+  c.tune_q4_bpc = blocks_per_cu;
+  return TLHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,199 @@
+/*
+ * libtensorlib_hip.so — C ABI of the MI355X (gfx950) backend for the
+ * cpp-tensorlib LLM decode path.
+ *
+ * This is the boundary a cpp-tensorlib backend header binds with
+ * dlopen()/dlsym(), the way the reference's cuda.h binds libcuda
+ * (include/cuda.h:240-321) — except that the kernels live behind this ABI too,
+ * so the header above it is a thin launch/coherence layer. Plain C types only.
+ *
+ * Conventions
+ *  - Every function returns 0 on success and a negative tlhip_status on
+ *    failure; tlhip_last_error() describes the last failure of the calling
+ *    thread. Nothing throws, nothing aborts.
+ *  - All tensor pointers are DEVICE pointers obtained from tlhip_malloc.
+ *    `*_off` arguments are byte offsets added to the base (the reference passes
+ *    element offsets * 4, array.h:1480).
+ *  - Launchers enqueue on the library's stream and return immediately;
+ *    tlhip_sync() is the only blocking call besides the synchronous copies and
+ *    tlhip_argmax. While a capture is open (tlhip_graph_begin) launches are
+ *    recorded instead of run.
+ *  - Shapes a kernel does not support are refused with TLHIP_EUNSUPPORTED
+ *    before anything is launched; the caller (the backend header) turns that
+ *    into the reference's "declined" (`false`).
+ *  - One device, one stream, single-threaded use, as the reference's evaluator
+ *    (README.md:182).
+ */
+#ifndef TENSORLIB_HIP_H
+#define TENSORLIB_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLHIP_ABI_VERSION 1
+
+typedef enum {
+  TLHIP_OK = 0,
+  TLHIP_ENODEVICE = -1,    /* no usable gfx950 device / HIP runtime failure at init */
+  TLHIP_EINVAL = -2,       /* null pointer, negative size, misaligned operand */
+  TLHIP_EUNSUPPORTED = -3, /* shape/dtype outside what the kernels cover: caller falls back */
+  TLHIP_ENOMEM = -4,
+  TLHIP_ERUNTIME = -5      /* a HIP call failed; see tlhip_last_error() */
+} tlhip_status;
+
+/* Elementwise / row op codes. Values are those of the reference's shared
+ * tl::metal::kop enum (include/metal.h:41-47) so a backend header can pass
+ * static_cast<int>(op) straight through. */
+typedef enum {
+  TLHIP_ADD = 0, TLHIP_SUB = 1, TLHIP_MUL = 2, TLHIP_DIV = 3, TLHIP_POW = 4,
+  TLHIP_EXP = 5, TLHIP_LOG = 6, TLHIP_SQRT = 7, TLHIP_SIGMOID = 8, TLHIP_RELU = 9,
+  TLHIP_AFFINE = 10,
+  TLHIP_BADD = 11, TLHIP_BSUB = 12, TLHIP_BMUL = 13, TLHIP_BDIV = 14, TLHIP_BPOW = 15,
+  TLHIP_SOFTMAX = 26, TLHIP_ROW_SUM = 27, TLHIP_ROW_MAX = 28,
+  TLHIP_RECIP = 64 /* extension: 1/x, so array::rmsnorm's `1.0f / sqrt` stays on device
+                      (the reference evaluates recip on the CPU, array.h:2064-2066) */
+} tlhip_op;
+
+/* ---- lifecycle ------------------------------------------------------------
+ * replaces cuda.h:240-321 (context ctor: driver load, device 0, module load) */
+int tlhip_init(int device);               /* idempotent; device must be gfx950 */
+int tlhip_abi_version(void);
+const char* tlhip_arch(void);             /* "gfx950" once initialised, else "" */
+const char* tlhip_last_error(void);
+int tlhip_device_info(int* compute_units, int64_t* hbm_bytes, int* lds_bytes_per_cu);
+
+/* ---- memory -----------------------------------------------------------------
+ * replaces cuMemAlloc/cuMemFree/cuMemcpy* as used by cuda.h:553-637 */
+int tlhip_malloc(void** dptr, size_t bytes);
+int tlhip_free(void* dptr);
+int tlhip_host_alloc(void** hptr, size_t bytes);    /* pinned, for the mirror's host side */
+int tlhip_host_free(void* hptr);
+int tlhip_memcpy_h2d(void* dst, const void* src, size_t bytes);       /* blocking */
+int tlhip_memcpy_d2h(void* dst, const void* src, size_t bytes);       /* blocking, drains stream */
+int tlhip_memcpy_h2d_async(void* dst, const void* src, size_t bytes); /* src must stay valid */
+int tlhip_memcpy_d2d_async(void* dst, const void* src, size_t bytes);
+int tlhip_fill_u32(void* dst, uint32_t value, size_t count);          /* fill kernel, capturable */
+int tlhip_sync(void);                     /* cuda.h:501-506 flush() */
+
+/* ---- graph capture (cuda.h:508-551) and timing events ----------------------- */
+int tlhip_graph_begin(void);
+int tlhip_graph_end(void** graph_exec);
+int tlhip_graph_launch(void* graph_exec);
+int tlhip_graph_destroy(void* graph_exec);
+int tlhip_event_create(void** ev);
+int tlhip_event_record(void* ev);         /* on the library's stream */
+int tlhip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
+int tlhip_event_destroy(void* ev);
+
+/* ---- dispatch census ----------------------------------------------------------
+ * Per-entry-point launch counters, so a test can assert that kernels ran
+ * (the reference's WebGPU backend keeps the same census, webgpu.h:197-202). */
+typedef enum {
+  TLHIP_C_BINARY = 0, TLHIP_C_BCAST, TLHIP_C_UNARY, TLHIP_C_ROW_OP, TLHIP_C_GEMM,
+  TLHIP_C_GEMV_F32, TLHIP_C_GEMV_BF16, TLHIP_C_GEMV_BF16_ROW, TLHIP_C_GEMV_Q4,
+  TLHIP_C_ATTN_DECODE, TLHIP_C_ROPE, TLHIP_C_RMSNORM, TLHIP_C_RMSNORM_RES, TLHIP_C_SWIGLU,
+  TLHIP_C_ARGMAX, TLHIP_C_KV_APPEND, TLHIP_C_KV_FILL, TLHIP_C_SPLIT_HEADS,
+  TLHIP_C_MERGE_HEADS, TLHIP_C_GEMM_BF16_NT, TLHIP_C_ATTN_PREFILL, TLHIP_C_COUNT
+} tlhip_census_id;
+int tlhip_census(uint64_t* counts, int n);  /* copies min(n, TLHIP_C_COUNT) counters */
+int tlhip_census_reset(void);
+
+/* ---- elementwise / rows (the gpu:: seam of array.h:1470-1507, 1738-1773) ------ */
+/* out = (a OP b)*scale + offset, n contiguous f32.  cuda.h:640-654 */
+int tlhip_binary(int op, const void* a, int64_t a_off, const void* b, int64_t b_off,
+                 void* out, int64_t out_off, int64_t n, float scale, float offset);
+/* rank-2 broadcast, op in TLHIP_BADD..TLHIP_BPOW; element (i,j) reads
+ * a[i*ars+j*acs], b[i*brs+j*bcs] (strides in elements, 0 = broadcast).
+ * cuda.h:656-662 declines this; metal.h has it — implemented here. */
+int tlhip_binary_bcast(int op, const void* a, int64_t a_off, int64_t ars, int64_t acs,
+                       const void* b, int64_t b_off, int64_t brs, int64_t bcs, void* out,
+                       int64_t out_off, int64_t m, int64_t n, float scale, float offset);
+/* out = f(a)*scale + offset.  cuda.h:664-675 */
+int tlhip_unary(int op, const void* a, int64_t a_off, void* out, int64_t out_off, int64_t n,
+                float scale, float offset);
+/* last-axis softmax (rows x cols out) or row_sum/row_max (rows out, affine epilogue).
+ * cuda.h:1487-1503 */
+int tlhip_row_op(int op, const void* in, int64_t in_off, void* out, int64_t out_off,
+                 int64_t rows, int64_t cols, float scale, float offset);
+/* C[m,n] = (A.B)*scale + offset, f32; lda/ldb row strides, ta/tb read a transposed
+ * view in place.  cuda.h:1409-1483 */
+int tlhip_gemm(const void* a, int64_t a_off, int64_t lda, int ta, const void* b, int64_t b_off,
+               int64_t ldb, int tb, void* out, int64_t out_off, int64_t m, int64_t n,
+               int64_t k, float scale, float offset);
+
+/* ---- decode GEMV -------------------------------------------------------------- */
+/* y[n] = sum_k a[k]*B[k,n], B f32 [K,N] row-major.  cuda.h:719-728 */
+int tlhip_gemv_f32(const void* a, const void* B, void* y, int64_t n, int64_t k);
+/* same, B bf16 [K,N].  cuda.h:729-742 */
+int tlhip_gemv_bf16(const void* a, const void* B, void* y, int64_t n, int64_t k);
+/* y[n] = sum_k a[k]*W[n,k], W bf16 [N,K] row-major; K % 8 == 0.  cuda.h:770-785 */
+int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_t k);
+/* y[n] = sum_k a[k] * scales[n][k/group] * (nibble(n,k) - 8).
+ * qw: packed int4 [N][K/2] bytes, even k in the low nibble (array.h:735-737);
+ * scales: f32 [N][K/group]. group > 0, K % group == 0, group % 8 == 0.
+ * cuda.h:886-905 */
+int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, int64_t N,
+                  int64_t K, int64_t group);
+
+/* ---- attention ---------------------------------------------------------------- */
+/* out[h,:] = softmax(scale * q[h,:].K[kv(h)]^T) . V[kv(h)],  kv(h) = h/(Hq/Hkv);
+ * q,out [Hq,D] f32; K,V [Hkv,kv_max,D] read over rows [0,ctx); D in {64,128};
+ * kv_bf16 != 0: K,V hold bf16.  cuda.h:962-1009 */
+int tlhip_attn_decode(const void* q, const void* K, const void* V, void* out,
+                      int64_t n_q_heads, int64_t n_kv_heads, int64_t ctx, int64_t kv_max,
+                      int64_t D, float scale, int kv_bf16);
+/* causal prefill: q,out [Hq,T,D]; query p is at position pos0+p and sees keys
+ * [0,pos0+p].  cuda.h:1166-1201 */
+int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out,
+                       int64_t n_q_heads, int64_t n_kv_heads, int64_t T, int64_t kv_max,
+                       int64_t D, float scale, int kv_bf16, int64_t pos0);
+/* scatter one token's k,v [Hkv,D] into the cache row pos.  cuda.h:1116-1138 */
+int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, int64_t pos,
+                    int64_t kv_max, int64_t n_kv_heads, int64_t D, int kv_bf16);
+/* bulk copy k,v [Hkv,T,D] into cache rows [pos0,pos0+T).  cuda.h:1140-1164 */
+int tlhip_kv_fill(void* Kc, void* Vc, const void* K, const void* V, int64_t T, int64_t kv_max,
+                  int64_t n_kv_heads, int64_t D, int kv_bf16, int64_t pos0);
+
+/* ---- model ops ---------------------------------------------------------------- */
+/* half-split rotary on [rows,D]; row r sits at position pos + r%T; bias (may be
+ * NULL, [rows,D]) is added before rotating. Angles are computed in fp64 like the
+ * reference CPU path (array.h:1709-1734).  cuda.h:1203-1222 */
+int tlhip_rope(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos,
+               float base, const void* bias);
+/* out = x * 1/sqrt(mean(x^2)+eps) * w per row of n.  cuda.h:1284-1302 */
+int tlhip_rmsnorm(const void* x, const void* w, void* out, int64_t n, float eps, int64_t rows);
+/* xout = x + delta; hout = rmsnorm(xout)*w.  xout may alias x.  cuda.h:1229-1252 */
+int tlhip_rmsnorm_res(const void* x, const void* delta, const void* w, void* xout, void* hout,
+                      int64_t n, float eps, int64_t rows);
+/* out[rows,ff] = silu(gu[:, :ff]) * gu[:, ff:], gu [rows,2*ff].  cuda.h:1304-1319 */
+int tlhip_swiglu(const void* gu, void* out, int64_t ff, int64_t rows);
+/* index of the maximum of in[0..n), ties to the smallest index; blocks until the
+ * result is on the host.  cuda.h:1254-1282 */
+int tlhip_argmax(const void* in, int64_t n, int64_t* out_idx);
+/* same reduction, result left in a device int32 (no sync; capturable) */
+int tlhip_argmax_async(const void* in, int64_t n, void* out_idx_dev);
+
+/* ---- prefill ------------------------------------------------------------------ */
+/* C[M,N] = A[M,K] f32 . W[N,K]^T bf16, fp32 accumulate; K % 8 == 0.  cuda.h:787-841 */
+int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K);
+/* [T,ld] token-major (+ optional bias [H*D]) -> [H,T,D]; `off` selects a column
+ * block of a fused projection.  cuda.h:846-864 */
+int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, int64_t ld,
+                      int64_t off, int64_t H, int64_t D);
+/* [H,T,D] -> [T,H*D].  cuda.h:866-879 */
+int tlhip_merge_heads(const void* src, void* dst, int64_t T, int64_t H, int64_t D);
+
+/* ---- tuning hook (benchmarks only) --------------------------------------------
+ * Overrides the int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts
+ * sharing one row's K range (1,2,4) and resident blocks per CU; 0 restores the
+ * built-in choice. Results do not depend on it beyond fp32 summation order. */
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENSORLIB_HIP_H */

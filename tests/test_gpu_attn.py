@@ -1,0 +1,97 @@
+"""GPU parity: decode attention through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+from oraclelib import allclose, maxrel
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _run(lib, q, K, V, ctx, scale, kv_bf16=False):
+    Hq, D = q.shape
+    Hkv, kv_max, _ = K.shape
+    dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, D))
+    lib.attn_decode(dq, dk, dv, do, Hq, Hkv, ctx, kv_max, D, scale, kv_bf16)
+    out = do.numpy()
+    for b in (dq, dk, dv, do):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("ctx", [512, 2048, 8192])
+def test_attn_config3(lib, orc, ctx):
+    """BASELINE config 3: q[28,128], K/V[28,ctx,128] ~ N(0,1), scale 1/sqrt(128)."""
+    H, D = 28, 128
+    print("case attn config3", ctx, flush=True)
+    q = orc.normal(H * D, 1).reshape(H, D)
+    K = orc.normal(H * ctx * D, 2).reshape(H, ctx, D)
+    V = orc.normal(H * ctx * D, 3).reshape(H, ctx, D)
+    scale = 1.0 / np.sqrt(128.0)
+    got = _run(lib, q, K, V, ctx, scale)
+    want = orc.attn_decode(q, K, V, scale)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(64, 14, 2), (128, 28, 4), (128, 4, 2), (64, 6, 2),
+                                      (128, 3, 1), (64, 16, 1), (128, 5, 5)])
+@pytest.mark.parametrize("ctx", [1, 2, 63, 64, 65, 255, 256, 257, 1000, 2047])
+def test_attn_gqa_and_split_boundaries(lib, orc, D, Hq, Hkv, ctx):
+    """GQA head map h/group and the split/tile boundaries (check_attn64.cpp:65-66),
+    reading a cache prefix: kv_max > ctx, rows past ctx hold garbage that must not leak."""
+    print("case attn gqa", D, Hq, Hkv, ctx, flush=True)
+    kv_max = ctx + 37
+    q = orc.normal(Hq * D, 4 + ctx).reshape(Hq, D)
+    K = orc.normal(Hkv * kv_max * D, 5 + ctx).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 6 + ctx).reshape(Hkv, kv_max, D)
+    K[:, ctx:, :] = 1e30
+    V[:, ctx:, :] = np.nan
+    scale = 1.0 / np.sqrt(float(D))
+    got = _run(lib, q, K, V, ctx, scale)
+    want = orc.attn_decode(q, K, V, scale, ctx=ctx)
+    assert np.all(np.isfinite(got))
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_attn_closed_forms(lib, orc):
+    H, D, ctx = 4, 128, 300
+    q = orc.normal(H * D, 1).reshape(H, D)
+    K = orc.normal(H * ctx * D, 2).reshape(H, ctx, D)
+    V = orc.normal(H * ctx * D, 3).reshape(H, ctx, D)
+    # ctx == 1 => out == V[:,0]
+    got = _run(lib, q, K, V, 1, 0.3)
+    assert allclose(got, V[:, 0, :], 1e-6, 1e-6)
+    # scale == 0 => uniform weights => mean of V
+    got = _run(lib, q, K, V, ctx, 0.0)
+    assert allclose(got, V.astype(np.float64).mean(axis=1), 1e-5, 1e-5)
+    # identical keys => mean of V as well
+    K2 = np.repeat(K[:, :1, :], ctx, axis=1).copy()
+    got = _run(lib, q, K2, V, ctx, 0.7)
+    assert allclose(got, V.astype(np.float64).mean(axis=1), 1e-5, 1e-5)
+    # large scores stay finite ({1000,1001} stability, test_array.cpp:273-274)
+    q3 = np.zeros((1, 128), np.float32); q3[0, 0] = 1.0
+    K3 = np.zeros((1, 2, 128), np.float32); K3[0, 0, 0] = 1000.0; K3[0, 1, 0] = 1001.0
+    V3 = np.zeros((1, 2, 128), np.float32); V3[0, 0, :] = 1.0; V3[0, 1, :] = 3.0
+    got = _run(lib, q3, K3, V3, 2, 1.0)
+    e = np.exp(-1.0)
+    assert allclose(got, np.full((1, 128), (1 * e + 3) / (1 + e)), 1e-5, 1e-5)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_attn_bf16_cache(lib, orc, D):
+    Hq, Hkv, ctx = 8, 2, 700
+    q = orc.normal(Hq * D, 1).reshape(Hq, D)
+    Kb = orc.to_bf16(orc.normal(Hkv * ctx * D, 2).reshape(Hkv, ctx, D))
+    Vb = orc.to_bf16(orc.normal(Hkv * ctx * D, 3).reshape(Hkv, ctx, D))
+    scale = 1.0 / np.sqrt(float(D))
+    got = _run(lib, q, Kb, Vb, ctx, scale, kv_bf16=True)
+    want = orc.attn_decode(q, orc.bf16_widen(Kb), orc.bf16_widen(Vb), scale)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_attn_declines(lib, pkg):
+    b = lib.empty(4096)
+    for args in [(4, 4, 8, 8, 96), (5, 2, 8, 8, 128), (4, 0, 8, 8, 128)]:
+        with pytest.raises(pkg.TlHipError) as e:
+            lib.attn_decode(b, b, b, b, *args, 1.0)
+        assert e.value.code == -3

@@ -1,0 +1,167 @@
+"""GPU parity: decode GEMVs through the C ABI vs the CPU oracle.
+
+Bar (BASELINE.json): allclose(rtol=1e-4, atol=1e-5) against the reference CPU
+path with fp32 accumulation — |gpu - ref| <= 1e-5 + 1e-4*|ref|, the reference's
+own allclose (array.h:2538-2547).
+"""
+import numpy as np
+import pytest
+
+from oraclelib import allclose, maxrel
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _q4_case(lib, orc, N, K, seed, from_weights):
+    x = orc.normal(K, seed + 1)
+    if from_weights:   # config 2: N(0,0.02) weights quantised with group-32 scales
+        w = orc.normal(K * N, seed, 0.0, 0.02).reshape(K, N)
+        buf = orc.to_q4(w)
+    else:              # config 1: uniform nibbles, scales ~ U(0.005, 0.02)
+        buf = orc.fill_q4(N, K, seed)
+    want = orc.gemv_q4(x, buf, N, K)
+    dx, dw, dy = lib.to_device(x), lib.to_device(buf), lib.empty(N)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    got = dy.numpy()
+    for b in (dx, dw, dy):
+        b.free()
+    return got, want
+
+
+@pytest.mark.parametrize("N,K", [(4864, 896), (3584, 3584), (512, 3584), (1024, 18944)])
+def test_gemv_q4_baseline_shapes(lib, orc, N, K):
+    print("case gemv_q4", N, K, flush=True)
+    got, want = _q4_case(lib, orc, N, K, 100 + N % 97, from_weights=(K != 896))
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+@pytest.mark.parametrize("N,K", [(1, 32), (3, 64), (7, 96), (48, 256), (130, 2048 + 32),
+                                 (257, 4096), (33, 160), (5, 32768 - 32)])
+def test_gemv_q4_ragged(lib, orc, N, K):
+    print("case gemv_q4 ragged", N, K, flush=True)
+    got, want = _q4_case(lib, orc, N, K, 7 + N + K, from_weights=True)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+@pytest.mark.parametrize("rows,kw", [(1, 1), (2, 1), (4, 1), (8, 1), (1, 2), (2, 4), (1, 8), (4, 2)])
+def test_gemv_q4_every_launch_shape(lib, orc, rows, kw):
+    """All (rows per wavefront, K-split) variants compute the same product."""
+    N, K = 777, 3584
+    print("case gemv_q4 tuned", rows, kw, flush=True)
+    lib.tune_gemv_q4(rows, kw, 0)
+    try:
+        got, want = _q4_case(lib, orc, N, K, 31, from_weights=True)
+    finally:
+        lib.tune_gemv_q4(0, 0, 0)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_gemv_q4_closed_forms(lib, orc):
+    """One-hot weight => y = scale*q*x_k exactly; all q == 1 => y = s*sum(x)."""
+    N, K = 8, 256
+    buf = np.zeros(orc.q4_bytes(N, K), np.uint8)
+    buf[:N * K // 2] = 0x88                      # every nibble 8 => q = 0
+    sc = buf[N * K // 2:].view(np.float32)
+    sc[:] = 0.5
+    # row 2: k=37 (odd => high nibble of byte 18) gets q=+3 ; row 5: k=200 (even) gets q=-8
+    buf[2 * (K // 2) + 18] = (8 + 3) << 4 | 8
+    buf[5 * (K // 2) + 100] = 0x80 | 0
+    x = orc.normal(K, 5)
+    dx, dw, dy = lib.to_device(x), lib.to_device(buf), lib.empty(N)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    y = dy.numpy()
+    want = np.zeros(N, np.float32)
+    want[2] = np.float32(0.5) * np.float32(3.0) * x[37]
+    want[5] = np.float32(0.5) * np.float32(-8.0) * x[200]
+    assert allclose(y, want, 1e-6, 1e-6), (y, want)
+    buf[:N * K // 2] = 0x99                      # every q = 1
+    sc[:] = 0.25
+    dw.upload(buf)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    y = dy.numpy()
+    s = np.float32(0.25 * float(np.sum(x.astype(np.float64))))
+    assert allclose(y, np.full(N, s), 1e-5, 1e-5), (y, s)
+
+
+@pytest.mark.parametrize("group", [8, 16, 64, 128])
+def test_gemv_q4_other_groups(lib, orc, group):
+    """group != 32 is legal at the C ABI (cuda.h:889-890); checked against an fp64
+    dequant-dot like bench_q4_gemv.cpp:98-104."""
+    N, K = 19, 512
+    rng = np.random.default_rng(group)
+    packed = rng.integers(0, 256, N * K // 2, dtype=np.uint8)
+    scales = rng.uniform(0.005, 0.02, (N, K // group)).astype(np.float32)
+    x = orc.normal(K, 3)
+    nib = np.empty((N, K), np.int32)
+    pk = packed.reshape(N, K // 2)
+    nib[:, 0::2] = pk & 0xF
+    nib[:, 1::2] = pk >> 4
+    deq = (nib - 8).astype(np.float64) * np.repeat(scales.astype(np.float64), group, axis=1)
+    want = deq @ x.astype(np.float64)
+    buf = np.concatenate([packed, scales.view(np.uint8).ravel()])
+    dx, dw, dy = lib.to_device(x), lib.to_device(buf), lib.empty(N)
+    lib.gemv_q4(dx, dw, dy, N, K, group=group)
+    assert allclose(dy.numpy(), want, RTOL, ATOL)
+
+
+def test_gemv_q4_declines(lib, pkg):
+    a, w, y = lib.empty(64), lib.empty_bytes(4096), lib.empty(8)
+    for N, K, g in [(8, 48, 32), (8, 64, 12), (8, 64, 0)]:
+        with pytest.raises(pkg.TlHipError) as e:
+            lib.gemv_q4(a, w, y, N, K, group=g)
+        assert e.value.code == -3   # TLHIP_EUNSUPPORTED => the backend header declines
+
+
+@pytest.mark.parametrize("N,K", [(3584, 3584), (512, 3584), (4864, 896), (40, 64), (1000, 520),
+                                 (9, 8), (151936 // 8, 896)])
+def test_gemv_bf16_row(lib, orc, N, K):
+    print("case gemv_bf16_row", N, K, flush=True)
+    w = orc.to_bf16(orc.normal(N * K, 11 + N, 0.0, 0.02).reshape(N, K))
+    x = orc.normal(K, 12)
+    want = orc.gemv_bf16_row(x, w)
+    dx, dw, dy = lib.to_device(x), lib.to_device(w), lib.empty(N)
+    lib.gemv_bf16_row(dx, dw, dy, N, K)
+    got = dy.numpy()
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+@pytest.mark.parametrize("N,K", [(3584, 3584), (512, 3584), (4864, 896), (48, 256), (1001, 300),
+                                 (8, 5), (18944, 1024)])
+def test_gemv_bf16_and_f32_kn(lib, orc, N, K):
+    print("case gemv [K,N]", N, K, flush=True)
+    wf = orc.normal(K * N, 21 + N, 0.0, 0.02).reshape(K, N)
+    wb = orc.to_bf16(wf)
+    x = orc.normal(K, 22)
+    dx, dy = lib.to_device(x), lib.empty(N)
+    dwb = lib.to_device(wb)
+    lib.gemv_bf16(dx, dwb, dy, N, K)
+    got = dy.numpy()
+    want = orc.gemv_bf16(x, wb)
+    assert allclose(got, want, RTOL, ATOL), ("bf16", maxrel(got, want))
+    dwf = lib.to_device(wf)
+    lib.gemv_f32(dx, dwf, dy, N, K)
+    got = dy.numpy()
+    want = orc.dot(x.reshape(1, K), wf).ravel()
+    assert allclose(got, want, RTOL, ATOL), ("f32", maxrel(got, want))
+
+
+def test_gemv_is_deterministic(lib, orc):
+    N, K = 3584, 3584
+    buf = orc.fill_q4(N, K, 9)
+    x = orc.normal(K, 10)
+    dx, dw, dy = lib.to_device(x), lib.to_device(buf), lib.empty(N)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    first = dy.numpy().copy()
+    for _ in range(3):
+        lib.gemv_q4(dx, dw, dy, N, K)
+        assert np.array_equal(dy.numpy(), first)
+
+
+def test_census_counts_launches(lib, orc):
+    lib.census_reset()
+    N, K = 64, 64
+    dx, dw, dy = lib.to_device(orc.normal(K, 1)), lib.to_device(orc.fill_q4(N, K, 2)), lib.empty(N)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    lib.gemv_q4(dx, dw, dy, N, K)
+    assert lib.census()["gemv_q4"] == 2

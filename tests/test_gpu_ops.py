@@ -1,0 +1,186 @@
+"""GPU parity: rope, rmsnorm, swiglu, argmax, cache writes, elementwise and row
+ops through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+from oraclelib import allclose, maxrel
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+
+
+@pytest.mark.parametrize("rows,T,D,pos,base", [(16, 1, 64, 0, 1e6), (16, 1, 64, 4095, 1e6),
+                                               (32, 1, 128, 4096, 1e6), (6, 3, 64, 77, 1e4),
+                                               (28 * 16, 16, 128, 32000, 1e6), (2, 1, 2, 5, 1e4)])
+def test_rope(lib, orc, rows, T, D, pos, base):
+    x = orc.normal(rows * D, 1 + rows).reshape(rows, D)
+    dx, do = lib.to_device(x), lib.empty((rows, D))
+    lib.rope(dx, do, rows, T, D, pos, base)
+    got = do.numpy()
+    want = orc.rope(x, pos, base, T=T)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    if pos == 0 and T == 1:
+        assert np.array_equal(got, x)          # pos 0 is the identity
+    half = D // 2                              # rotations preserve each pair's norm
+    n_in = x[:, :half] ** 2 + x[:, half:] ** 2
+    n_out = got[:, :half] ** 2 + got[:, half:] ** 2
+    assert allclose(n_out, n_in, 1e-5, 1e-6)
+
+
+def test_rope_bias_and_inplace(lib, orc):
+    rows, D, pos = 14, 64, 1234
+    x = orc.normal(rows * D, 3).reshape(rows, D)
+    b = orc.normal(rows * D, 4, 0, 0.02).reshape(rows, D)
+    dx, db = lib.to_device(x), lib.to_device(b)
+    lib.rope(dx, dx, rows, 1, D, pos, 1e6, bias=db)
+    want = orc.rope(x, pos, 1e6, bias=b)
+    assert allclose(dx.numpy(), want, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 896), (1, 3584), (5, 3584), (3, 1000), (2, 7), (512, 896)])
+def test_rmsnorm(lib, orc, rows, n):
+    x = orc.normal(rows * n, 5 + n).reshape(rows, n)
+    w = orc.normal(n, 6, 1.0, 0.02)
+    dx, dw, do = lib.to_device(x), lib.to_device(w), lib.empty((rows, n))
+    lib.rmsnorm(dx, dw, do, n, 1e-6, rows)
+    got, want = do.numpy(), orc.rmsnorm(x, w, 1e-6)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    # constant row c => c/sqrt(c^2+eps) * w
+    xc = np.full((1, n), 3.0, np.float32)
+    dxc = lib.to_device(xc)
+    lib.rmsnorm(dxc, dw, do, n, 1e-6, 1)
+    assert allclose(do.numpy()[0], 3.0 / np.sqrt(9.0 + 1e-6) * w.astype(np.float64), 1e-6, 1e-6)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 896), (1, 3584), (4, 1001)])
+def test_rmsnorm_res(lib, orc, rows, n):
+    x = orc.normal(rows * n, 7).reshape(rows, n)
+    d = orc.normal(rows * n, 8).reshape(rows, n)
+    w = orc.normal(n, 9, 1.0, 0.02)
+    dx, dd, dw, dh = lib.to_device(x), lib.to_device(d), lib.to_device(w), lib.empty((rows, n))
+    lib.rmsnorm_res(dx, dd, dw, dx, dh, n, 1e-6, rows)      # xout aliases x
+    xo, ho = orc.rmsnorm_res(x, d, w, 1e-6)
+    assert np.array_equal(dx.numpy(), xo)
+    assert allclose(dh.numpy(), ho, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("rows,ff", [(1, 4864), (1, 18944), (3, 1000), (2, 1)])
+def test_swiglu(lib, orc, rows, ff):
+    gu = orc.normal(rows * 2 * ff, 10, 0, 3.0).reshape(rows, 2 * ff)
+    dg, do = lib.to_device(gu), lib.empty((rows, ff))
+    lib.swiglu(dg, do, ff, rows)
+    got, want = do.numpy(), orc.swiglu_fused(gu, ff)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    z = np.zeros((1, 2 * ff), np.float32); z[0, ff:] = 5.0
+    dz = lib.to_device(z)
+    lib.swiglu(dz, do, ff, 1)
+    assert np.all(do.numpy()[0] == 0.0)                      # g = 0 => 0
+
+
+@pytest.mark.parametrize("n", [1, 5, 256, 4097, 151936, 152064])
+def test_argmax(lib, orc, n):
+    v = orc.normal(n, 11 + n)
+    dv = lib.to_device(v)
+    assert lib.argmax(dv, n) == orc.argmax(v)
+    v[:] = -3.0                                             # all ties => index 0
+    dv.upload(v)
+    assert lib.argmax(dv, n) == 0
+    if n > 300:
+        v[n - 7] = 2.0; v[123] = 2.0; v[299] = 2.0          # ties => smallest index
+        dv.upload(v)
+        assert lib.argmax(dv, n) == 123 == orc.argmax(v)
+
+
+def test_kv_append_fill(lib, orc):
+    Hkv, D, kv_max = 4, 128, 50
+    Kc = np.zeros((Hkv, kv_max, D), np.float32); Vc = Kc.copy()
+    dK, dV = lib.to_device(Kc), lib.to_device(Vc)
+    for pos in (0, 1, 49):
+        k = orc.normal(Hkv * D, 20 + pos).reshape(Hkv, D); v = orc.normal(Hkv * D, 30 + pos).reshape(Hkv, D)
+        lib.kv_append(dK, dV, lib.to_device(k), lib.to_device(v), pos, kv_max, Hkv, D)
+        Kc[:, pos] = k; Vc[:, pos] = v
+    T = 9
+    k = orc.normal(Hkv * T * D, 40).reshape(Hkv, T, D); v = orc.normal(Hkv * T * D, 41).reshape(Hkv, T, D)
+    lib.kv_fill(dK, dV, lib.to_device(k), lib.to_device(v), T, kv_max, Hkv, D, pos0=10)
+    Kc[:, 10:19] = k; Vc[:, 10:19] = v
+    assert np.array_equal(dK.numpy(), Kc) and np.array_equal(dV.numpy(), Vc)
+    with pytest.raises(RuntimeError):                        # full cache => refused
+        lib.kv_append(dK, dV, lib.to_device(k), lib.to_device(v), kv_max, kv_max, Hkv, D)
+
+
+def test_split_merge_heads(lib, orc):
+    T, H, D, ld, off = 7, 6, 64, 6 * 64 + 128, 128
+    src = orc.normal(T * ld, 50).reshape(T, ld)
+    bias = orc.normal(H * D, 51)
+    ds, db, dd = lib.to_device(src), lib.to_device(bias), lib.empty((H, T, D))
+    lib.split_heads(ds, db, dd, T, ld, off, H, D)
+    want = (src[:, off:off + H * D].reshape(T, H, D) + bias.reshape(1, H, D)).transpose(1, 0, 2)
+    assert np.array_equal(dd.numpy(), want)
+    dm = lib.empty((T, H * D))
+    lib.merge_heads(dd, dm, T, H, D)
+    assert np.array_equal(dm.numpy(), want.transpose(1, 0, 2).reshape(T, H * D))
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("epi", [(1.0, 0.0), (2.0, 1.0)])
+def test_binary(lib, orc, op, epi):
+    n = 70001
+    a = orc.normal(n, 60); b = orc.normal(n, 61) + np.float32(3.0)
+    da, db, do = lib.to_device(a), lib.to_device(b), lib.empty(n)
+    lib.binary(op, da, db, do, n, *epi)
+    want = orc.binary(op, a, b, *epi)
+    assert allclose(do.numpy(), want, 1e-6, 1e-7)
+    lib.binary(op, da, db, do, n - 5, *epi, ao=8, bo=12, oo=4)     # byte offsets
+    assert allclose(do.numpy()[1:n - 4], orc.binary(op, a[2:n - 3], b[3:n - 2], *epi), 1e-6, 1e-7)
+
+
+@pytest.mark.parametrize("op", ["exp", "log", "sqrt", "sigmoid", "relu", "affine", "recip"])
+def test_unary(lib, orc, op):
+    n = 5000
+    a = np.abs(orc.normal(n, 62)) + np.float32(0.1)
+    if op == "relu":
+        a = orc.normal(n, 63)
+    da, do = lib.to_device(a), lib.empty(n)
+    for epi in [(1.0, 0.0), (1.5, -0.25)]:
+        lib.unary(op, da, do, n, *epi)
+        assert allclose(do.numpy(), orc.unary(op, a, *epi), 2e-6, 1e-6), op
+
+
+def test_binary_bcast(lib, orc):
+    m, n = 5, 896
+    x = orc.normal(m * n, 64).reshape(m, n)
+    col = orc.normal(m, 65).reshape(m, 1) + np.float32(2.0)
+    row = orc.normal(n, 66).reshape(1, n)
+    dx, dc, dr, do = lib.to_device(x), lib.to_device(col), lib.to_device(row), lib.empty((m, n))
+    lib.binary_bcast("bmul", dx, (n, 1), dc, (1, 0), do, m, n)          # x * inv  (rmsnorm)
+    assert np.array_equal(do.numpy(), x * col)
+    lib.binary_bcast("badd", dx, (n, 1), dr, (0, 1), do, m, n, 2.0, 1.0)  # + bias row, epilogue
+    assert allclose(do.numpy(), orc.binary_bcast("add", x, (n, 1), row, (0, 1), m, n, 2.0, 1.0), 1e-6, 1e-7)
+    lib.binary_bcast("bdiv", dx, (n, 1), dc, (1, 0), do, m, n)
+    assert allclose(do.numpy(), x / col, 1e-6, 1e-7)
+
+
+def test_row_ops(lib, orc):
+    rows, cols = 9, 1500
+    x = orc.normal(rows * cols, 67).reshape(rows, cols)
+    dx, dr, ds = lib.to_device(x), lib.empty(rows), lib.empty((rows, cols))
+    lib.row_op("row_sum", dx, dr, rows, cols, 1.0 / cols, 1e-6)      # mean + eps, as rmsnorm lowers it
+    assert allclose(dr.numpy(), orc.row_sum(x, 1.0 / cols, 1e-6), 1e-5, 1e-6)
+    lib.row_op("row_max", dx, dr, rows, cols)
+    assert np.array_equal(dr.numpy(), orc.row_max(x))
+    lib.row_op("softmax", dx, ds, rows, cols)
+    got = ds.numpy()
+    assert allclose(got, orc.softmax(x), RTOL, 1e-7)
+    assert allclose(got.sum(axis=1), np.ones(rows), 1e-5, 1e-5)
+
+
+@pytest.mark.parametrize("m,n,k,ta,tb", [(3, 40, 100, 0, 0), (2, 300, 700, 0, 1), (65, 64, 1030, 1, 0),
+                                         (1, 17, 33, 1, 1)])
+def test_gemm_seam(lib, orc, m, n, k, ta, tb):
+    A = orc.normal(m * k, 70).reshape(m, k); B = orc.normal(k * n, 71).reshape(k, n)
+    As = np.ascontiguousarray(A.T) if ta else A
+    Bs = np.ascontiguousarray(B.T) if tb else B
+    da, db, do = lib.to_device(As), lib.to_device(Bs), lib.empty((m, n))
+    lib.gemm(da, As.shape[1], ta, db, Bs.shape[1], tb, do, m, n, k, 2.0, 1.0)
+    want = orc.dot(A, B, 2.0, 1.0)
+    assert allclose(do.numpy(), want, RTOL, 1e-4), maxrel(do.numpy(), want)
