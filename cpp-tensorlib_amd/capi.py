@@ -75,7 +75,9 @@ SIGNATURES = {
     "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
-    "tlhip_tune_gemv_q4": (cint, [cint, cint, cint]),
+    "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint]),
+    "tlhip_bench_copy": (cint, [P, P, sz, cint]),
+    "tlhip_bench_read": (cint, [P, sz, P, cint]),
 }
 
 
@@ -274,8 +276,14 @@ class TlHip:
     def merge_heads(self, src, dst, T, H, D):
         self._chk(self.c.tlhip_merge_heads(src.ptr, dst.ptr, T, H, D))
 
-    def tune_gemv_q4(self, rows=0, kw=0, bpc=0):
-        self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc))
+    def bench_copy(self, dst, src, nbytes, blocks=0):
+        self._chk(self.c.tlhip_bench_copy(dst.ptr, src.ptr, nbytes, blocks))
+
+    def bench_read(self, src, nbytes, sink, blocks=0, off=0):
+        self._chk(self.c.tlhip_bench_read(src.ptr + off, nbytes, sink.ptr, blocks))
+
+    def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0):
+        self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw))
 
 
 _lib = None

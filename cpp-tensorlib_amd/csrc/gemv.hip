@@ -106,7 +106,28 @@ struct FmtBf16 {
 // LDS: x as float4 xs[(chunk*J + j)*64 + lane], J = E/4, so that lane l's j-th
 // fragment of chunk c is one conflict-free ds_read_b128; then KW*rows floats.
 template <typename Fmt, int R>
-__global__ __launch_bounds__(1024) void gemv_rows_kernel(
+struct RowFrag {          // one (row tile, chunk) work item of a lane: R weight units in flight
+  uint4 w[R];
+  float sc[R];
+};
+
+template <typename Fmt, int R>
+__device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __restrict__ W,
+                                          const float* __restrict__ scales, int N, int upr,
+                                          int row0, int u) {
+  if (u < upr) {
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const int row = min(row0 + r, N - 1);
+      const size_t idx = (size_t)row * upr + u;
+      f.w[r] = load_stream16(&W[idx]);
+      if (Fmt::kScaled) f.sc[r] = __builtin_nontemporal_load(&scales[idx]);
+    }
+  }
+}
+
+template <typename Fmt, int R>
+__global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
     float* __restrict__ y, int N, int upr, int KW, int ntiles) {
   constexpr int J = Fmt::E / 4;
@@ -118,85 +139,94 @@ __global__ __launch_bounds__(1024) void gemv_rows_kernel(
   float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * 64);  // [chunks*64], int4 only
   float* red = xsum + (Fmt::kScaled ? chunks * 64 : 0);
 
-  {  // stage x (K = upr*E floats) into the interleaved layout
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    const int n4 = upr * J;
-    for (int i = tid; i < n4; i += blockDim.x) {
-      const int u = i / J, j = i - u * J;
-      xs[((u >> 6) * J + j) * 64 + (u & 63)] = Fmt::stage(x4[i]);
-    }
-    if (Fmt::kScaled) {
-      for (int u = tid; u < upr; u += blockDim.x) {
-        float sx = 0.f;
-#pragma unroll
-        for (int j = 0; j < J; j++) {
-          const float4 v = x4[u * J + j];
-          sx += (v.x + v.y) + (v.z + v.w);
-        }
-        xsum[u] = -8.0f * sx;  // sum_k (nib_k - 8) x_k = sum nib_k x_k - 8 sum x_k
-      }
-    }
-  }
-  __syncthreads();
-
   const int kw = wave % KW;          // which K split this wavefront takes
   const int wn = wave / KW;          // which row group of the block tile
   const int groups = nw / KW;        // row groups per block tile
   const int rows_per_tile = groups * R;
 
-  for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const int row0 = t * rows_per_tile + wn * R;
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
+  // The first work item's weights are requested before x is staged, so that the
+  // HBM latency of the weights and the L2 latency of x overlap.
+  int t = blockIdx.x, c = kw;
+  RowFrag<Fmt, R> cur, nxt;
+  if (t < ntiles) load_frag<Fmt, R>(cur, W, scales, N, upr, t * rows_per_tile + wn * R, (c << 6) + lane);
 
-    for (int c = kw; c < chunks; c += KW) {
-      const int u = (c << 6) + lane;
-      if (u < upr) {
-        uint4 w[R];
-        float sc[R];
+  {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
+     // thread i owns float4 i; the J threads of a unit are adjacent lanes, so the
+     // unit's sum(x) is a J-lane shuffle reduction (J is 8 or 2, both divide 64).
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int n4 = upr * J;
+    const int n4_padded = (n4 + 63) & ~63;   // whole wavefronts take part in the shuffles
+    for (int i = tid; i < n4_padded; i += blockDim.x) {
+      const bool live = i < n4;
+      const float4 v = live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      const int u = i / J, j = i - u * J;
+      if (live) xs[((u >> 6) * J + j) * 64 + (u & 63)] = Fmt::stage(v);
+      if (Fmt::kScaled) {
+        float sx = (v.x + v.y) + (v.z + v.w);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-          const int row = min(row0 + r, N - 1);
-          const size_t idx = (size_t)row * upr + u;
-          w[r] = load_stream16(&W[idx]);
-          if (Fmt::kScaled) sc[r] = __builtin_nontemporal_load(&scales[idx]);
-        }
-        float4 xv[J];
+        for (int msk = J / 2; msk >= 1; msk >>= 1) sx += __shfl_xor(sx, msk, kWave);
+        if (live && j == 0) xsum[u] = -8.0f * sx;  // sum_k (nib_k-8) x_k = sum nib_k x_k - 8 sum x_k
+      }
+    }
+  }
+  __syncthreads();
+
+  float acc[R];
 #pragma unroll
-        for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * 64 + lane];
-        if (Fmt::kScaled) {
-          const float bias = xsum[u];
+  for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+  // Software pipeline over this wavefront's (tile, chunk) items: the next item's
+  // loads are in flight while the current one is unpacked and accumulated.
+  while (t < ntiles) {
+    int nc = c + KW, nt = t;
+    if (nc >= chunks) { nc = kw; nt = t + gridDim.x; }
+    if (nt < ntiles)
+      load_frag<Fmt, R>(nxt, W, scales, N, upr, nt * rows_per_tile + wn * R, (nc << 6) + lane);
+
+    const int u = (c << 6) + lane;
+    if (u < upr) {
+      float4 xv[J];
 #pragma unroll
-          for (int r = 0; r < R; r++) acc[r] = fmaf(sc[r], Fmt::dot(w[r], xv) + bias, acc[r]);
-        } else {
+      for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * 64 + lane];
+      if (Fmt::kScaled) {
+        const float bias = xsum[u];
 #pragma unroll
-          for (int r = 0; r < R; r++) acc[r] += Fmt::dot(w[r], xv);
-        }
+        for (int r = 0; r < R; r++) acc[r] = fmaf(cur.sc[r], Fmt::dot(cur.w[r], xv) + bias, acc[r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] += Fmt::dot(cur.w[r], xv);
       }
     }
 
+    if (nt != t) {  // last chunk of tile t for this wavefront: reduce and store
+      const int row0 = t * rows_per_tile + wn * R;
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
-
-    if (KW == 1) {
-      float v = acc[0];
+      for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+      if (KW == 1) {
+        float v = acc[0];
 #pragma unroll
-      for (int r = 1; r < R; r++) v = (lane == r) ? acc[r] : v;
-      if (lane < R && row0 + lane < N) y[row0 + lane] = v;
-    } else {
-      if (lane == 0) {
+        for (int r = 1; r < R; r++) v = (lane == r) ? acc[r] : v;
+        if (lane < R && row0 + lane < N) y[row0 + lane] = v;
+      } else {
+        // every wavefront of the block passes these two barriers once per tile
+        if (lane == 0) {
 #pragma unroll
-        for (int r = 0; r < R; r++) red[(wn * KW + kw) * R + r] = acc[r];
+          for (int r = 0; r < R; r++) red[(wn * KW + kw) * R + r] = acc[r];
+        }
+        __syncthreads();
+        if (kw == 0 && lane < R && row0 + lane < N) {
+          float v = 0.f;
+          for (int s = 0; s < KW; s++) v += red[(wn * KW + s) * R + lane];
+          y[row0 + lane] = v;
+        }
+        __syncthreads();
       }
-      __syncthreads();
-      if (kw == 0 && lane < R && row0 + lane < N) {
-        float v = 0.f;
-        for (int s = 0; s < KW; s++) v += red[(wn * KW + s) * R + lane];
-        y[row0 + lane] = v;
-      }
-      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < R; r++) acc[r] = 0.f;
     }
+    cur = nxt;
+    t = nt;
+    c = nc;
   }
 }
 
@@ -332,51 +362,57 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
 
 struct RowCfg { int R, KW, nw, blocks; size_t lds; };
 
-// Launch shape for the row kernel. Goal: every CU holds >= ~16 wavefronts of
-// independent 16-byte loads, x is staged as few times as possible, and the
-// tile count divides evenly over the persistent blocks.
+// Launch shape for the row kernel, from sweeps on MI355X:
+//  * one fat block per CU (16 wavefronts) so x is staged once per CU; 8-wave
+//    blocks only when a row tile must be smaller than KW allows;
+//  * rows per block tile grow with the rows a CU owns, up to 64 (4 rows per
+//    wavefront: the x fragment held in VGPRs is reused 4 times);
+//  * K is split over KW wavefronts of a block only when rows alone cannot give
+//    every CU a tile.
 static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, int tR, int tKW,
-                            int tBPC) {
+                            int tBPC, int tNW) {
   const int chunks = (upr + 63) / 64;
-  const size_t xbytes = (size_t)chunks * 64 * E * 4;
+  const size_t xbytes = (size_t)chunks * 64 * E * 4 + (size_t)chunks * 256;
   RowCfg c{};
-  // wavefronts per block: enough that one or two blocks fill a CU even when x is big
-  c.nw = xbytes > 40 * 1024 ? 16 : 8;
-  int bpc = (int)((size_t)lds_per_cu / (xbytes + (size_t)chunks * 256 + 1024));
-  const int max_by_waves = 32 / c.nw;  // 8 wavefronts per SIMD, 4 SIMDs
-  if (bpc > max_by_waves) bpc = max_by_waves;
-  if (bpc < 1) bpc = 1;
-  if (tBPC > 0) bpc = tBPC;
-  const int64_t slots = (int64_t)cus * bpc * c.nw;  // resident wavefronts on the chip
-  // rows per wavefront: large when rows are plentiful (x fragment reuse), small otherwise
-  int R = 1;
-  for (int cand : {8, 4, 2}) {
-    if (N / cand >= slots * 2) { R = cand; break; }
+  const int64_t rows_per_cu = N / cus;
+  int nw = 16, R, KW;
+  if (rows_per_cu >= 128) { R = 4; KW = 1; }        // 64 rows per block tile
+  else if (rows_per_cu >= 32) { R = 2; KW = 1; }    // 32
+  else if (rows_per_cu >= 8) { R = 2; KW = 2; }     // 16
+  else { nw = 8; R = 1; KW = 2; }                   // 4
+  while (KW > chunks) {  // not enough K to split that far: more row groups instead
+    KW /= 2;
+    if (R > 1) R /= 2; else if (nw > 4) nw /= 2;
   }
-  if (R == 1 && N >= slots) R = 1;
-  // wavefronts sharing a row's K range: only when rows alone cannot fill the chip
-  int KW = 1;
-  while (KW < c.nw && KW * 2 <= chunks && (N / R) * KW < slots) KW *= 2;
+  if (tNW > 0) nw = tNW;
   if (tR > 0) R = tR;
   if (tKW > 0) KW = tKW;
-  if (KW > c.nw) KW = c.nw;
+  if (R >= 8 && nw > 8) nw = 8;  // the 8-row variant is built for <= 512 threads
+  if (KW > nw) KW = nw;
+  int bpc = (int)((size_t)lds_per_cu / (xbytes + 1024));
+  const int max_by_waves = 32 / nw > 0 ? 32 / nw : 1;
+  const int want_bpc = nw >= 16 ? 1 : nw == 8 ? 2 : 4;
+  if (bpc > max_by_waves) bpc = max_by_waves;
+  if (bpc > want_bpc) bpc = want_bpc;
+  if (bpc < 1) bpc = 1;
+  if (tBPC > 0) bpc = tBPC;
   c.R = R;
   c.KW = KW;
-  const int rows_per_tile = (c.nw / KW) * R;
+  c.nw = nw;
+  const int rows_per_tile = (nw / KW) * R;
   const int64_t ntiles = (N + rows_per_tile - 1) / rows_per_tile;
-  int64_t maxb = (int64_t)cus * bpc;
-  int64_t passes = (ntiles + maxb - 1) / maxb;
-  c.blocks = (int)((ntiles + passes - 1) / passes);
-  c.lds = xbytes + (size_t)chunks * 64 * 4 + (size_t)c.nw * 8 * 4 + 64;
+  const int64_t maxb = (int64_t)cus * bpc;
+  c.blocks = (int)(ntiles < maxb ? ntiles : maxb);
+  c.lds = xbytes + (size_t)nw * 8 * 4 + 64;
   return c;
 }
 
 template <typename Fmt>
 static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
-                       int64_t K, int census_id, int tR, int tKW, int tBPC) {
+                       int64_t K, int census_id, int tR, int tKW, int tBPC, int tNW) {
   Context& c = ctx();
   const int upr = (int)(K / Fmt::E);
-  RowCfg cfg = pick_rows_cfg(N, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC);
+  RowCfg cfg = pick_rows_cfg(N, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC, tNW);
   const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
   const int ntiles = (int)((N + rows_per_tile - 1) / rows_per_tile);
   using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int);
@@ -457,7 +493,7 @@ int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, in
   if (group == 32 && aligned16(qw) && xbytes + 2048 <= (size_t)c.lds_per_cu)
     return launch_rows<FmtQ4>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
                               static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
-                              c.tune_q4_kw, c.tune_q4_bpc);
+                              c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw);
   hipLaunchKernelGGL(gemv_q4_generic_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, c.stream,
                      static_cast<const float*>(a), static_cast<const uint32_t*>(qw),
                      static_cast<const float*>(scales), static_cast<float*>(y), (int)N, (int)K,
@@ -474,7 +510,7 @@ int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_
   if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K too large for the LDS-staged kernel");
   return launch_rows<FmtBf16>(static_cast<const float*>(a), W, nullptr, static_cast<float*>(y), n, k,
-                              TLHIP_C_GEMV_BF16_ROW, 0, 0, 0);
+                              TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0);
 }
 
 int tlhip_gemv_f32(const void* a, const void* B, void* y, int64_t n, int64_t k) {

@@ -51,6 +51,34 @@ __global__ void fill_u32_kernel(uint32_t* dst, uint32_t v, size_t n) {
   for (; i < n; i += stride) dst[i] = v;
 }
 
+// Plain streaming kernels of known size: the yardstick the GEMV numbers and the
+// HBM traffic counters are scaled against.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void copy16_kernel(u32x4* __restrict__ dst,
+                                                     const u32x4* __restrict__ src, size_t n16) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
+}
+__global__ __launch_bounds__(256) void read16_kernel(const u32x4* __restrict__ src, size_t n16,
+                                                     uint32_t* __restrict__ sink) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  uint32_t acc = 0;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const u32x4 a = __builtin_nontemporal_load(&src[i]);
+    const u32x4 b = __builtin_nontemporal_load(&src[i + stride]);
+    const u32x4 c = __builtin_nontemporal_load(&src[i + 2 * stride]);
+    const u32x4 d = __builtin_nontemporal_load(&src[i + 3 * stride]);
+    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  }
+  for (; i < n16; i += stride) {
+    const u32x4 a = __builtin_nontemporal_load(&src[i]);
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;  // practically never: keeps the loads alive
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;
@@ -278,11 +306,34 @@ int tlhip_census_reset(void) {
   return TLHIP_OK;
 }
 
-int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu) {
+int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks) {
+  TLHIP_REQUIRE_READY();
+  if (!dst || !src || (bytes & 15) || !aligned16(dst) || !aligned16(src))
+    return fail(TLHIP_EINVAL, "tlhip_bench_copy: need 16-byte aligned pointers and size");
+  if (blocks <= 0) blocks = ctx().cus * 8;
+  copy16_kernel<<<dim3(blocks), dim3(256), 0, ctx().stream>>>(
+      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "copy kernel");
+}
+
+int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks) {
+  TLHIP_REQUIRE_READY();
+  if (!src || !sink4 || (bytes & 15) || !aligned16(src))
+    return fail(TLHIP_EINVAL, "tlhip_bench_read: need a 16-byte aligned pointer and size");
+  if (blocks <= 0) blocks = ctx().cus * 8;
+  read16_kernel<<<dim3(blocks), dim3(256), 0, ctx().stream>>>(static_cast<const u32x4*>(src),
+                                                              bytes / 16, static_cast<uint32_t*>(sink4));
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "read kernel");
+}
+
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block) {
   Context& c = ctx();
   c.tune_q4_rows = rows_per_wave;
   c.tune_q4_kw = k_waves;
   c.tune_q4_bpc = blocks_per_cu;
+  c.tune_q4_nw = waves_per_block;
   return TLHIP_OK;
 }
 

@@ -187,11 +187,19 @@ int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, i
 /* [H,T,D] -> [T,H*D].  cuda.h:866-879 */
 int tlhip_merge_heads(const void* src, void* dst, int64_t T, int64_t H, int64_t D);
 
+/* ---- measurement yardsticks (benchmarks only; no reference counterpart) --------
+ * A plain 16-byte-per-lane streaming copy / read of `bytes` bytes, used to find
+ * the HBM rate this GPU really sustains and to scale the profiler's traffic
+ * counters. blocks <= 0 picks 8 blocks per CU. */
+int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks);
+int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
+
 /* ---- tuning hook (benchmarks only) --------------------------------------------
  * Overrides the int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts
- * sharing one row's K range (1,2,4) and resident blocks per CU; 0 restores the
- * built-in choice. Results do not depend on it beyond fp32 summation order. */
-int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu);
+ * sharing one row's K range (a power of two), resident blocks per CU and
+ * wavefronts per block (<= 16); 0 restores the built-in choice for that field.
+ * Results do not depend on it beyond fp32 summation order. */
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block);
 
 #ifdef __cplusplus
 }

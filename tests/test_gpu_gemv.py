@@ -58,7 +58,11 @@ def test_gemv_q4_every_launch_shape(lib, orc, rows, kw):
 
 
 def test_gemv_q4_closed_forms(lib, orc):
-    """One-hot weight => y = scale*q*x_k exactly; all q == 1 => y = s*sum(x)."""
+    """One-hot weight => y = scale*q*x_k; all q == 1 => y = s*sum(x).
+
+    The kernel evaluates sum((nib-8)*x) as sum(nib*x) - 8*sum(x), so a row of
+    q == 0 carries fp32 rounding noise of the size of eps*8*sum|x| instead of an
+    exact zero; the bound is BASELINE's atol."""
     N, K = 8, 256
     buf = np.zeros(orc.q4_bytes(N, K), np.uint8)
     buf[:N * K // 2] = 0x88                      # every nibble 8 => q = 0
@@ -74,7 +78,7 @@ def test_gemv_q4_closed_forms(lib, orc):
     want = np.zeros(N, np.float32)
     want[2] = np.float32(0.5) * np.float32(3.0) * x[37]
     want[5] = np.float32(0.5) * np.float32(-8.0) * x[200]
-    assert allclose(y, want, 1e-6, 1e-6), (y, want)
+    assert allclose(y, want, 1e-5, 1e-5), (y, want)
     buf[:N * K // 2] = 0x99                      # every q = 1
     sc[:] = 0.25
     dw.upload(buf)
