@@ -68,7 +68,26 @@ def build(force=False, verbose=True):
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
+    build_host(force, verbose)
     return LIB
+
+
+QWEN_LIB = os.path.join(LIBDIR, "libtl_qwen.so")
+
+
+def build_host(force=False, verbose=True):
+    """libtl_qwen.so: the header-only C++ host layer (include/tl/) behind a C entry
+    layer, compiled with plain g++; it reaches the HIP library through dlopen."""
+    src = os.path.join(CSRC, "qwen_capi.cpp")
+    inc = os.path.join(HERE, "include")
+    deps = [src] + [os.path.join(inc, "tl", f) for f in os.listdir(os.path.join(inc, "tl"))]
+    if force or _stale(QWEN_LIB, deps):
+        cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra", "-I", inc, src,
+               "-o", QWEN_LIB, "-ldl"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    return QWEN_LIB
 
 
 if __name__ == "__main__":

@@ -1,0 +1,664 @@
+#pragma once
+
+// tl::hip — the MI355X (gfx950) backend header for cpp-tensorlib's tl::gpu seam.
+//
+// It exposes the free-function set every backend of the reference exposes
+// (reference include/gpu.h:1-12; signatures as include/cuda.h:494-506, 586-675,
+// 719-742, 886-905, 962-1009, 1203-1222, 1487-1503 and the stubs of
+// include/metal.h:434-484), plus the harness-level calls of include/cuda.h
+// (gemv_bf16_row, gemm_bf16_nt, rmsnorm, rmsnorm_res, swiglu, argmax,
+// split/merge_heads, kv_append, kv_fill, attn_prefill, kv_cache, upload,
+// graph capture). array.h / storage.h call it as tl::gpu::X after
+// `namespace gpu = hip;`.
+//
+// Unlike cuda.h, which dlopens the driver and loads an embedded PTX blob, this
+// header dlopens ONE shared object, libtensorlib_hip.so, that holds the gfx950
+// code objects and a plain C ABI (include/tensorlib_hip.h). What stays here is
+// the host policy the reference keeps in its backend header: the host/device
+// mirror with HOST/DEVICE/BOTH dirty state, the size-keyed buffer pool, the
+// `pending` flag, and turning every refusal of the library into the seam's
+// "declined" (`false` / nullptr) so the evaluator takes its CPU path. No
+// exception and no error code crosses the seam.
+//
+// Header-only C++17, single-threaded use like the rest of the evaluator.
+
+#include <dlfcn.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+#include "types.h"
+
+namespace tl {
+
+// The op enum all backends share. The reference declares it in metal.h:41-47
+// as tl::metal::kop; a build that includes that header picks it up, a
+// standalone build of this host layer gets the identical enumerator order.
+#ifndef TL_HIP_USE_METAL_KOP
+namespace metal {
+enum class kop {
+  add, sub, mul, div, pow_, exp_, log_, sqrt_, sigmoid, relu, affine,
+  badd, bsub, bmul, bdiv, bpow,
+  sgemm32, sgemm32x64, sgemm64x32, sgemm64,
+  steel, steel32x64, steel_ta, steel_tb, steel32x64_ta, steel32x64_tb,
+  softmax, row_sum, row_max
+};
+}  // namespace metal
+#endif
+
+namespace hip {
+
+using kop = tl::metal::kop;
+
+// ---- the C ABI, bound by name ------------------------------------------------
+struct api {
+  int (*init)(int) = nullptr;
+  int (*abi_version)() = nullptr;
+  const char* (*last_error)() = nullptr;
+  int (*malloc_)(void**, size_t) = nullptr;
+  int (*free_)(void*) = nullptr;
+  int (*host_alloc)(void**, size_t) = nullptr;
+  int (*host_free)(void*) = nullptr;
+  int (*memcpy_h2d)(void*, const void*, size_t) = nullptr;
+  int (*memcpy_d2h)(void*, const void*, size_t) = nullptr;
+  int (*memcpy_h2d_async)(void*, const void*, size_t) = nullptr;
+  int (*memcpy_d2d_async)(void*, const void*, size_t) = nullptr;
+  int (*fill_u32)(void*, uint32_t, size_t) = nullptr;
+  int (*sync)() = nullptr;
+  int (*graph_begin)() = nullptr;
+  int (*graph_end)(void**) = nullptr;
+  int (*graph_launch)(void*) = nullptr;
+  int (*graph_destroy)(void*) = nullptr;
+  int (*census)(uint64_t*, int) = nullptr;
+  int (*binary)(int, const void*, int64_t, const void*, int64_t, void*, int64_t, int64_t, float,
+                float) = nullptr;
+  int (*binary_bcast)(int, const void*, int64_t, int64_t, int64_t, const void*, int64_t, int64_t,
+                      int64_t, void*, int64_t, int64_t, int64_t, float, float) = nullptr;
+  int (*unary)(int, const void*, int64_t, void*, int64_t, int64_t, float, float) = nullptr;
+  int (*row_op)(int, const void*, int64_t, void*, int64_t, int64_t, int64_t, float, float) = nullptr;
+  int (*gemm)(const void*, int64_t, int64_t, int, const void*, int64_t, int64_t, int, void*, int64_t,
+              int64_t, int64_t, int64_t, float, float) = nullptr;
+  int (*gemv_f32)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
+  int (*gemv_bf16)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
+  int (*gemv_bf16_row)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
+  int (*gemv_q4)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*attn_decode)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
+                     int64_t, float, int) = nullptr;
+  int (*attn_prefill)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
+                      int64_t, int64_t, float, int, int64_t) = nullptr;
+  int (*kv_append)(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t,
+                   int) = nullptr;
+  int (*kv_fill)(void*, void*, const void*, const void*, int64_t, int64_t, int64_t, int64_t, int,
+                 int64_t) = nullptr;
+  int (*rope)(const void*, void*, int64_t, int64_t, int64_t, int64_t, float, const void*) = nullptr;
+  int (*rmsnorm)(const void*, const void*, void*, int64_t, float, int64_t) = nullptr;
+  int (*rmsnorm_res)(const void*, const void*, const void*, void*, void*, int64_t, float,
+                     int64_t) = nullptr;
+  int (*swiglu)(const void*, void*, int64_t, int64_t) = nullptr;
+  int (*argmax)(const void*, int64_t, int64_t*) = nullptr;
+  int (*argmax_async)(const void*, int64_t, void*) = nullptr;
+  int (*gemm_bf16_nt)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*split_heads)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
+                     int64_t) = nullptr;
+  int (*merge_heads)(const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+};
+
+struct context {
+  void* lib = nullptr;
+  api f;
+  bool ready = false;
+  bool pending = false;
+  bool capturing = false;
+  std::string why;  // why the backend is unavailable (diagnostics only)
+
+  // Host/device mirror per allocation, keyed by the device pointer (== the
+  // `native` handle storage keeps). Ordered, so that a pointer INTO an
+  // allocation (q4 scales at native + N*K/2, a slice of a fused projection)
+  // finds its owner too.
+  enum loc { HOST, DEVICE, BOTH };
+  struct mirror {
+    float* host = nullptr;
+    char* dev = nullptr;
+    size_t bytes = 0;
+    loc where = HOST;
+  };
+  std::map<uintptr_t, mirror> mirrors;
+  // size-keyed free list; buffers are recycled, never freed (cuda.h:211-216)
+  std::unordered_map<size_t, std::vector<std::pair<char*, float*>>> pool;
+
+  static context& get() {
+    static auto* c = new context();  // leaked: outlives every storage deleter
+    return *c;
+  }
+
+  template <typename T>
+  bool bind(T& slot, const char* name) {
+    slot = reinterpret_cast<T>(dlsym(lib, name));
+    if (!slot) why = std::string("missing symbol ") + name;
+    return slot != nullptr;
+  }
+
+  context() {
+    // TENSORLIB_HIP_LIB names the library explicitly; otherwise the usual
+    // dynamic-loader search applies.
+    std::vector<std::string> paths;
+    if (const char* e = std::getenv("TENSORLIB_HIP_LIB")) paths.emplace_back(e);
+    paths.emplace_back("libtensorlib_hip.so");
+    for (const auto& p : paths) {
+      lib = dlopen(p.c_str(), RTLD_NOW | RTLD_LOCAL);
+      if (lib) break;
+    }
+    if (!lib) {
+      const char* e = dlerror();
+      why = e ? e : "libtensorlib_hip.so not found";
+      return;  // available() == false: every op declines, the CPU path runs
+    }
+    bool ok = bind(f.init, "tlhip_init") && bind(f.abi_version, "tlhip_abi_version") &&
+              bind(f.last_error, "tlhip_last_error") && bind(f.malloc_, "tlhip_malloc") &&
+              bind(f.free_, "tlhip_free") && bind(f.host_alloc, "tlhip_host_alloc") &&
+              bind(f.host_free, "tlhip_host_free") && bind(f.memcpy_h2d, "tlhip_memcpy_h2d") &&
+              bind(f.memcpy_d2h, "tlhip_memcpy_d2h") &&
+              bind(f.memcpy_h2d_async, "tlhip_memcpy_h2d_async") &&
+              bind(f.memcpy_d2d_async, "tlhip_memcpy_d2d_async") &&
+              bind(f.fill_u32, "tlhip_fill_u32") && bind(f.sync, "tlhip_sync") &&
+              bind(f.graph_begin, "tlhip_graph_begin") && bind(f.graph_end, "tlhip_graph_end") &&
+              bind(f.graph_launch, "tlhip_graph_launch") &&
+              bind(f.graph_destroy, "tlhip_graph_destroy") && bind(f.census, "tlhip_census") &&
+              bind(f.binary, "tlhip_binary") && bind(f.binary_bcast, "tlhip_binary_bcast") &&
+              bind(f.unary, "tlhip_unary") && bind(f.row_op, "tlhip_row_op") &&
+              bind(f.gemm, "tlhip_gemm") && bind(f.gemv_f32, "tlhip_gemv_f32") &&
+              bind(f.gemv_bf16, "tlhip_gemv_bf16") && bind(f.gemv_bf16_row, "tlhip_gemv_bf16_row") &&
+              bind(f.gemv_q4, "tlhip_gemv_q4") && bind(f.attn_decode, "tlhip_attn_decode") &&
+              bind(f.attn_prefill, "tlhip_attn_prefill") && bind(f.kv_append, "tlhip_kv_append") &&
+              bind(f.kv_fill, "tlhip_kv_fill") && bind(f.rope, "tlhip_rope") &&
+              bind(f.rmsnorm, "tlhip_rmsnorm") && bind(f.rmsnorm_res, "tlhip_rmsnorm_res") &&
+              bind(f.swiglu, "tlhip_swiglu") && bind(f.argmax, "tlhip_argmax") &&
+              bind(f.argmax_async, "tlhip_argmax_async") &&
+              bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
+              bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads");
+    if (!ok) return;
+    if (f.abi_version() != 1) {
+      why = "libtensorlib_hip.so has a different ABI version";
+      return;
+    }
+    if (f.init(0) != 0) {
+      why = f.last_error();
+      return;  // no gfx950 device: stay unavailable
+    }
+    ready = true;
+  }
+
+  // the allocation containing p, or nullptr
+  mirror* mirror_(const void* p) {
+    if (!p || mirrors.empty()) return nullptr;
+    auto it = mirrors.upper_bound(reinterpret_cast<uintptr_t>(p));
+    if (it == mirrors.begin()) return nullptr;
+    --it;
+    mirror& m = it->second;
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    return (a >= it->first && a < it->first + m.bytes) ? &m : nullptr;
+  }
+  // A kernel is about to READ this buffer: make the device copy current.
+  void device_read_(const void* native) {
+    mirror* m = mirror_(native);
+    if (m && m->where == HOST) {
+      f.memcpy_h2d(m->dev, m->host, m->bytes);  // blocking, stream-ordered
+      m->where = BOTH;
+    }
+  }
+  // A kernel is about to WRITE this buffer: it becomes the live copy. A write
+  // into part of a buffer whose live copy is on the host uploads first, so the
+  // untouched part is not lost.
+  void device_write_(void* native) {
+    mirror* m = mirror_(native);
+    if (!m) return;
+    if (m->where == HOST && reinterpret_cast<char*>(native) != m->dev) {
+      f.memcpy_h2d(m->dev, m->host, m->bytes);
+    }
+    m->where = DEVICE;
+  }
+};
+
+inline bool available() { return context::get().ready; }
+inline const char* unavailable_reason() { return context::get().why.c_str(); }
+inline bool pending() { return context::get().pending; }
+
+// End the batch: block until the GPU has drained (cuda.h:501-506).
+inline void flush() {
+  auto& c = context::get();
+  if (!c.ready || !c.pending) return;
+  c.f.sync();
+  c.pending = false;
+}
+
+inline void cpu_barrier() {
+  if (pending()) flush();
+}
+
+// Dispatch census of the library (launches per entry point), so a caller can
+// assert that a green result was computed on the GPU (webgpu.h:197-202).
+inline std::vector<uint64_t> census() {
+  auto& c = context::get();
+  std::vector<uint64_t> v(32, 0);
+  if (c.ready) c.f.census(v.data(), (int)v.size());
+  return v;
+}
+
+// ---- memory (cuda.h:553-637) ---------------------------------------------------
+inline void* alloc(int64_t bytes, float** contents) {
+  auto& c = context::get();
+  if (!c.ready) return nullptr;
+  const size_t nb = bytes > 0 ? (size_t)bytes : 4;
+  char* dev = nullptr;
+  float* host = nullptr;
+  auto it = c.pool.find(nb);
+  if (it != c.pool.end() && !it->second.empty()) {
+    dev = it->second.back().first;
+    host = it->second.back().second;
+    it->second.pop_back();
+  } else {
+    void* d = nullptr;
+    if (c.f.malloc_(&d, nb) != 0) return nullptr;
+    void* h = nullptr;
+    if (c.f.host_alloc(&h, nb) != 0) {  // pinned: H2D/D2H run at full PCIe rate
+      c.f.free_(d);
+      return nullptr;
+    }
+    dev = static_cast<char*>(d);
+    host = static_cast<float*>(h);
+  }
+  c.mirrors[reinterpret_cast<uintptr_t>(dev)] = context::mirror{host, dev, nb, context::HOST};
+  if (contents) *contents = host;
+  return dev;
+}
+
+// A buffer that only ever lives on the device (weights written by device
+// copies, KV caches): no host half, so nothing is pinned for it and
+// sync_to_host has nothing to bring back.
+inline void* alloc_device(int64_t bytes) {
+  auto& c = context::get();
+  if (!c.ready) return nullptr;
+  const size_t nb = bytes > 0 ? (size_t)bytes : 4;
+  void* d = nullptr;
+  if (c.f.malloc_(&d, nb) != 0) return nullptr;
+  c.mirrors[reinterpret_cast<uintptr_t>(d)] =
+      context::mirror{nullptr, static_cast<char*>(d), nb, context::DEVICE};
+  return d;
+}
+
+// Stream-ordered device-to-device copy between two managed buffers.
+inline bool copy_d2d(void* dst, const void* src, int64_t bytes) {
+  auto& c = context::get();
+  if (!c.ready || !dst || !src || bytes < 0) return false;
+  c.device_read_(src);
+  c.device_write_(dst);
+  if (c.f.memcpy_d2d_async(dst, src, (size_t)bytes) != 0) return false;
+  c.pending = true;
+  return true;
+}
+
+inline void release(void* buf, int64_t, float*) {
+  auto& c = context::get();
+  if (!c.ready || !buf) return;
+  auto it = c.mirrors.find(reinterpret_cast<uintptr_t>(buf));
+  if (it == c.mirrors.end()) return;
+  // a kernel still in flight may be using the buffer; recycle only after the drain
+  if (c.pending && !c.capturing) flush();
+  if (it->second.host) c.pool[it->second.bytes].push_back({it->second.dev, it->second.host});
+  else c.f.free_(it->second.dev);  // device-only buffers are not pooled
+  c.mirrors.erase(it);
+}
+
+inline void sync_to_host(void* native, bool for_write) {
+  auto& c = context::get();
+  if (!c.ready || !native) return;
+  context::mirror* m = c.mirror_(native);
+  if (!m) return;
+  if (c.pending) flush();
+  if (!m->host) return;  // device-only buffer
+  if (m->where == context::DEVICE) {
+    c.f.memcpy_d2h(m->host, m->dev, m->bytes);
+    m->where = context::BOTH;
+  }
+  if (for_write) m->where = context::HOST;
+}
+
+// Blocking H2D of the buffer's first n floats (cuda.h:553-568).
+inline void upload(void* native, const float* src, int64_t n) {
+  auto& c = context::get();
+  if (!c.ready || !native) return;
+  context::mirror* m = c.mirror_(native);
+  if (!m || !m->host) return;
+  size_t bytes = (size_t)n * sizeof(float);
+  if (bytes > m->bytes) bytes = m->bytes;
+  if (src != m->host) std::memcpy(m->host, src, bytes);
+  c.f.memcpy_h2d(m->dev, m->host, bytes);
+  m->where = context::BOTH;
+}
+
+inline void upload_u32(void* native, unsigned val) {
+  auto& c = context::get();
+  if (!c.ready || !native) return;
+  context::mirror* m = c.mirror_(native);
+  if (!m || !m->host || m->bytes < 4) return;
+  std::memcpy(m->host, &val, 4);
+  c.f.memcpy_h2d(m->dev, m->host, 4);
+  m->where = context::BOTH;
+}
+
+namespace detail {
+inline bool done_(context& c, int rc) {
+  if (rc != 0) return false;  // declined or failed: the caller falls back
+  c.pending = true;
+  return true;
+}
+}  // namespace detail
+
+// ---- the seam ------------------------------------------------------------------
+inline bool binary(kop op, void* a, int64_t ao, void* b, int64_t bo, void* out, int64_t oo,
+                   int64_t n, float scale, float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_read_(b);
+  c.device_write_(out);
+  return detail::done_(c, c.f.binary(static_cast<int>(op), a, ao, b, bo, out, oo, n, scale, offset));
+}
+
+inline bool binary_bcast(kop op, void* a, int64_t ao, int64_t ars, int64_t acs, void* b, int64_t bo,
+                         int64_t brs, int64_t bcs, void* out, int64_t oo, int64_t m, int64_t n,
+                         float scale, float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_read_(b);
+  c.device_write_(out);
+  return detail::done_(c, c.f.binary_bcast(static_cast<int>(op), a, ao, ars, acs, b, bo, brs, bcs,
+                                           out, oo, m, n, scale, offset));
+}
+
+inline bool unary(kop op, void* a, int64_t ao, void* out, int64_t oo, int64_t n, float scale,
+                  float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_write_(out);
+  return detail::done_(c, c.f.unary(static_cast<int>(op), a, ao, out, oo, n, scale, offset));
+}
+
+// 1/x with an affine epilogue: an op the reference's seam lacks (its `recip`
+// node always runs on the CPU, array.h:2064-2066); offered so a host layer that
+// knows about it can keep array::rmsnorm on the device.
+inline bool recip(void* a, int64_t ao, void* out, int64_t oo, int64_t n, float scale, float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_write_(out);
+  return detail::done_(c, c.f.unary(64 /* TLHIP_RECIP */, a, ao, out, oo, n, scale, offset));
+}
+
+inline bool gemm(void* a, int64_t ao, int64_t lda, bool ta, void* b, int64_t bo, int64_t ldb, bool tb,
+                 void* out, int64_t oo, int64_t m, int64_t n, int64_t k, float scale, float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_read_(b);
+  c.device_write_(out);
+  return detail::done_(c, c.f.gemm(a, ao, lda, ta ? 1 : 0, b, bo, ldb, tb ? 1 : 0, out, oo, m, n, k,
+                                   scale, offset));
+}
+
+inline bool row_op(kop op, void* in, int64_t io, void* out, int64_t oo, int64_t rows, int64_t cols,
+                   float scale, float offset) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(in);
+  c.device_write_(out);
+  return detail::done_(c, c.f.row_op(static_cast<int>(op), in, io, out, oo, rows, cols, scale, offset));
+}
+
+inline bool gemv_f32(void* a, void* B, void* y, int64_t n, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_f32(a, B, y, n, k));
+}
+
+inline bool gemv_bf16(void* a, void* B, void* y, int64_t n, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_bf16(a, B, y, n, k));
+}
+
+inline bool gemv_bf16_row(void* a, void* B, void* y, int64_t n, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_bf16_row(a, B, y, n, k));
+}
+
+inline bool gemv_q4(void* a, void* qw, void* scales, void* y, int64_t N, int64_t K, int64_t group) {
+  auto& c = context::get();
+  if (!c.ready || group <= 0 || (K % group) != 0 || (group % 8) != 0) return false;
+  c.device_read_(a);
+  c.device_read_(qw);
+  c.device_read_(scales);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_q4(a, qw, scales, y, N, K, group));
+}
+
+inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0 || m <= 0 || n <= 0) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(out);
+  return detail::done_(c, c.f.gemm_bf16_nt(a, B, out, m, n, k));
+}
+
+inline bool attn_decode(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
+                        int64_t ctx, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64)) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  c.device_read_(q);
+  c.device_read_(K);
+  c.device_read_(V);
+  c.device_write_(out);
+  return detail::done_(c, c.f.attn_decode(q, K, V, out, n_q_heads, n_kv_heads, ctx, kv_max, D, scale,
+                                          kv_bf16 ? 1 : 0));
+}
+
+inline bool attn_prefill(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
+                         int64_t T, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false,
+                         int64_t pos0 = 0) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64)) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  if (T <= 0 || T > 65535) return false;
+  c.device_read_(q);
+  c.device_read_(K);
+  c.device_read_(V);
+  c.device_write_(out);
+  return detail::done_(c, c.f.attn_prefill(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
+                                           kv_bf16 ? 1 : 0, pos0));
+}
+
+inline bool kv_append(void* Kc, void* Vc, void* k_new, void* v_new, int64_t pos, int64_t kv_max,
+                      int64_t n_kv_heads, int64_t D, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64)) return false;
+  c.device_read_(k_new);
+  c.device_read_(v_new);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.kv_append(Kc, Vc, k_new, v_new, pos, kv_max, n_kv_heads, D,
+                                        kv_bf16 ? 1 : 0));
+}
+
+inline bool kv_fill(void* Kc, void* Vc, void* K, void* V, int64_t T, int64_t kv_max,
+                    int64_t n_kv_heads, int64_t D, bool kv_bf16 = false, int64_t pos0 = 0) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64)) return false;
+  c.device_read_(K);
+  c.device_read_(V);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.kv_fill(Kc, Vc, K, V, T, kv_max, n_kv_heads, D, kv_bf16 ? 1 : 0, pos0));
+}
+
+inline bool rope(void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos, float base,
+                 void* bias = nullptr) {
+  auto& c = context::get();
+  if (!c.ready || D <= 0 || (D & 1)) return false;
+  c.device_read_(x);
+  if (bias) c.device_read_(bias);
+  c.device_write_(out);
+  return detail::done_(c, c.f.rope(x, out, rows, T, D, pos, base, bias));
+}
+
+inline bool rmsnorm(void* x, void* w, void* out, int64_t n, float eps, int64_t rows = 1) {
+  auto& c = context::get();
+  if (!c.ready || n <= 0 || rows <= 0) return false;
+  c.device_read_(x);
+  c.device_read_(w);
+  c.device_write_(out);
+  return detail::done_(c, c.f.rmsnorm(x, w, out, n, eps, rows));
+}
+
+inline bool rmsnorm_res(void* x, void* delta, void* w, void* xout, void* hout, int64_t n, float eps,
+                        int64_t rows = 1) {
+  auto& c = context::get();
+  if (!c.ready || n <= 0 || rows <= 0) return false;
+  c.device_read_(x);
+  c.device_read_(delta);
+  c.device_read_(w);
+  c.device_write_(xout);
+  c.device_write_(hout);
+  return detail::done_(c, c.f.rmsnorm_res(x, delta, w, xout, hout, n, eps, rows));
+}
+
+inline bool swiglu(void* gu, void* out, int64_t ff, int64_t rows = 1) {
+  auto& c = context::get();
+  if (!c.ready || ff <= 0 || rows <= 0) return false;
+  c.device_read_(gu);
+  c.device_write_(out);
+  return detail::done_(c, c.f.swiglu(gu, out, ff, rows));
+}
+
+// Greedy token: reduces on the device, copies 4 bytes back; the one blocking
+// call of a decode step (cuda.h:1254-1282).
+inline bool argmax(void* in, int64_t n, int64_t* out_idx) {
+  auto& c = context::get();
+  if (!c.ready || !in || n <= 0 || !out_idx) return false;
+  c.device_read_(in);
+  if (c.f.argmax(in, n, out_idx) != 0) return false;
+  c.pending = false;  // the library drained the stream to deliver the index
+  return true;
+}
+
+inline bool split_heads(void* src, void* bias, void* dst, int64_t T, int64_t ld, int64_t off,
+                        int64_t H, int64_t D) {
+  auto& c = context::get();
+  if (!c.ready || T <= 0 || H <= 0 || D <= 0) return false;
+  c.device_read_(src);
+  if (bias) c.device_read_(bias);
+  c.device_write_(dst);
+  return detail::done_(c, c.f.split_heads(src, bias, dst, T, ld, off, H, D));
+}
+
+inline bool merge_heads(void* src, void* dst, int64_t T, int64_t H, int64_t D) {
+  auto& c = context::get();
+  if (!c.ready || T <= 0 || H <= 0 || D <= 0) return false;
+  c.device_read_(src);
+  c.device_write_(dst);
+  return detail::done_(c, c.f.merge_heads(src, dst, T, H, D));
+}
+
+// ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------
+inline bool graph_available() { return context::get().ready; }
+inline bool capture_begin() {
+  auto& c = context::get();
+  if (!c.ready || c.capturing) return false;
+  if (c.pending) flush();
+  if (c.f.graph_begin() != 0) return false;
+  c.capturing = true;
+  return true;
+}
+inline void* capture_end() {
+  auto& c = context::get();
+  if (!c.capturing) return nullptr;
+  void* g = nullptr;
+  int rc = c.f.graph_end(&g);
+  c.capturing = false;
+  c.pending = false;  // recorded launches did not run
+  return rc == 0 ? g : nullptr;
+}
+inline bool graph_launch(void* g) {
+  auto& c = context::get();
+  if (!c.ready || !g) return false;
+  return detail::done_(c, c.f.graph_launch(g));
+}
+inline void graph_destroy(void* g) {
+  auto& c = context::get();
+  if (c.ready && g) c.f.graph_destroy(g);
+}
+
+// ---- persistent KV cache (cuda.h:1321-1405) --------------------------------------
+struct kv_cache {
+  void* K = nullptr;
+  void* V = nullptr;
+  int64_t n_kv_heads = 0, max_ctx = 0, D = 0, pos = 0;
+  bool kv_bf16 = false;
+
+  bool init(int64_t kv_heads, int64_t maxctx, int64_t d, dtype kv_dt = dtype::f32) {
+    n_kv_heads = kv_heads;
+    max_ctx = maxctx;
+    D = d;
+    pos = 0;
+    kv_bf16 = (kv_dt == dtype::bf16);
+    const int64_t w = kv_bf16 ? 2 : 4;
+    K = alloc_device(n_kv_heads * max_ctx * D * w);  // the cache never visits the host
+    V = alloc_device(n_kv_heads * max_ctx * D * w);
+    return K && V;
+  }
+  bool append(void* k_new, void* v_new) {
+    if (pos >= max_ctx) return false;
+    if (!kv_append(K, V, k_new, v_new, pos, max_ctx, n_kv_heads, D, kv_bf16)) return false;
+    pos++;
+    return true;
+  }
+  bool attn(void* q, void* out, int64_t n_q_heads, float scale) {
+    return attn_decode(q, K, V, out, n_q_heads, n_kv_heads, pos, max_ctx, D, scale, kv_bf16);
+  }
+  bool prefill(void* q, void* k_src, void* v_src, void* out, int64_t T, int64_t n_q_heads,
+               float scale) {
+    if (T <= 0 || pos + T > max_ctx) return false;
+    if (!kv_fill(K, V, k_src, v_src, T, max_ctx, n_kv_heads, D, kv_bf16, pos)) return false;
+    const int64_t p0 = pos;
+    pos += T;
+    return attn_prefill(q, K, V, out, n_q_heads, n_kv_heads, T, max_ctx, D, scale, kv_bf16, p0);
+  }
+  void destroy() {
+    if (K) release(K, 0, nullptr);
+    if (V) release(V, 0, nullptr);
+    K = V = nullptr;
+  }
+};
+
+}  // namespace hip
+}  // namespace tl

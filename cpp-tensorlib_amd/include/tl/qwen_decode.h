@@ -1,0 +1,353 @@
+#pragma once
+
+// A Qwen2.5-architecture decoder driven imperatively through the tl::hip
+// backend: the counterpart of the reference's bench/cuda/qwen_model.h
+// (Layer/Scratch/Model: 175-308; run_layers_: 673-740; step_imperative:
+// 747-752; captured_decoder: 791-905), with two differences that the task
+// asks for: the dimensions are parameters (0.5B and 7B shapes), and weights
+// come from memory blobs instead of a GGUF file.
+//
+// Per token and layer the step issues, in stream order and with no host sync:
+//   fused QKV GEMV -> rope(q,+bias) , rope(k,+bias) , v += bias -> cache append
+//   -> decode attention over the cache prefix -> o-proj GEMV
+//   -> rmsnorm_res (x1 = x + attn ; h2 = norm(x1)) -> fused gate|up GEMV
+//   -> swiglu -> down GEMV -> rmsnorm_res (x2 = x1 + mlp ; next layer's input norm)
+// then the lm_head GEMV and a device argmax whose 4-byte copy is the single
+// blocking call of the step.
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "hip.h"
+#include "types.h"
+
+namespace tl {
+namespace qwen {
+
+struct dims {
+  int64_t n_layers, hidden, n_q_heads, n_kv_heads, head_dim, ff, vocab, max_ctx;
+  float eps, rope_base;
+  int64_t q_dim() const { return n_q_heads * head_dim; }
+  int64_t kv_dim() const { return n_kv_heads * head_dim; }
+  int64_t qkv_dim() const { return q_dim() + 2 * kv_dim(); }
+};
+
+inline dims qwen25_05b(int64_t max_ctx = 4096) {
+  return dims{24, 896, 14, 2, 64, 4864, 151936, max_ctx, 1e-6f, 1e6f};
+}
+inline dims qwen25_7b(int64_t max_ctx = 4352) {
+  return dims{28, 3584, 28, 4, 128, 18944, 152064, max_ctx, 1e-6f, 1e6f};
+}
+
+// A linear weight resident on the device. q4: the reference's one-buffer layout
+// [packed [N][K/2] | scales [N][K/32]] (types.h:25-31). bf16_row: [N][K] bf16,
+// the layout gemv_bf16_row and gemm_bf16_nt share (cuda.h:765-841).
+enum class wfmt { q4, bf16_row };
+struct linear {
+  void* w = nullptr;
+  int64_t N = 0, K = 0;
+  wfmt fmt = wfmt::q4;
+  int64_t bytes() const { return fmt == wfmt::q4 ? q4_bytes(N, K) : N * K * 2; }
+};
+
+// y[N] = a[K] . W
+inline bool gemv(const linear& L, void* a, void* y) {
+  if (L.fmt == wfmt::q4) {
+    void* scales = static_cast<char*>(L.w) + L.N * L.K / 2;
+    return hip::gemv_q4(a, L.w, scales, y, L.N, L.K, kQ4Group);
+  }
+  return hip::gemv_bf16_row(a, L.w, y, L.N, L.K);
+}
+
+struct layer {
+  linear wqkv, wo, wgu, wd;          // fused [wq|wk|wv] and [wg|wu] (qm:188-199)
+  void *bq = nullptr, *bk = nullptr, *bv = nullptr;  // [q_dim], [kv_dim], [kv_dim]
+  void *an = nullptr, *fn = nullptr;                 // attention / ffn norm weights [hidden]
+  hip::kv_cache cache;
+};
+
+// Every per-step intermediate, allocated once (qm:208-246).
+struct scratch {
+  void* res[2] = {nullptr, nullptr};
+  void *hb = nullptr, *h2b = nullptr, *qkvb = nullptr, *ab = nullptr, *mb = nullptr, *gub = nullptr,
+       *mdb = nullptr, *logitsb = nullptr, *embedb = nullptr;
+  float* embed_host = nullptr;
+  float* logits_host = nullptr;
+};
+
+struct model {
+  dims d{};
+  std::vector<uint16_t> embed;  // bf16 [vocab, hidden], gathered on the host (qm:530-535)
+  void* onorm = nullptr;
+  linear lm_head;
+  std::vector<layer> layers;
+  scratch s;
+  bool ready = false;
+};
+
+namespace detail {
+
+inline void* dev_from_host(const void* src, int64_t bytes) {
+  float* host = nullptr;
+  void* n = hip::alloc(bytes, &host);
+  if (!n) return nullptr;
+  std::memcpy(host, src, (size_t)bytes);
+  hip::upload(n, host, (bytes + 3) / 4);  // device copy current from now on
+  return n;
+}
+
+// Rows of several q4 matrices with the same K, stacked: packed parts first,
+// then the scale parts, which is again a valid q4 buffer of N = sum(N_i).
+inline std::vector<uint8_t> fuse_q4(const std::vector<const uint8_t*>& parts,
+                                    const std::vector<int64_t>& Ns, int64_t K) {
+  int64_t N = 0;
+  for (auto n : Ns) N += n;
+  std::vector<uint8_t> out((size_t)q4_bytes(N, K));
+  uint8_t* pk = out.data();
+  uint8_t* sc = out.data() + N * K / 2;
+  for (size_t i = 0; i < parts.size(); i++) {
+    const int64_t pb = Ns[i] * K / 2, sb = Ns[i] * (K / kQ4Group) * 4;
+    std::memcpy(pk, parts[i], (size_t)pb);
+    std::memcpy(sc, parts[i] + pb, (size_t)sb);
+    pk += pb;
+    sc += sb;
+  }
+  return out;
+}
+
+}  // namespace detail
+
+// Host-side description of one layer's weights in the reference's storage
+// forms: q4 buffers of logical [K,N] weights (array.h:703-742) and f32 vectors.
+struct layer_blobs {
+  const uint8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
+  const float *bq, *bk, *bv, *an, *fn;
+};
+
+inline bool init(model& M, const dims& d) {
+  if (!hip::available()) return false;
+  M.d = d;
+  M.layers.assign((size_t)d.n_layers, layer{});
+  auto A = [](int64_t n) { return hip::alloc(n * 4, nullptr); };
+  scratch& S = M.s;
+  S.embedb = hip::alloc(d.hidden * 4, &S.embed_host);
+  S.res[0] = A(d.hidden);
+  S.res[1] = A(d.hidden);
+  S.hb = A(d.hidden);
+  S.h2b = A(d.hidden);
+  S.qkvb = A(d.qkv_dim());
+  S.ab = A(d.q_dim());
+  S.mb = A(d.ff);
+  S.gub = A(2 * d.ff);
+  S.mdb = A(d.hidden);
+  S.logitsb = hip::alloc(d.vocab * 4, &S.logits_host);
+  for (auto& L : M.layers)
+    if (!L.cache.init(d.n_kv_heads, d.max_ctx, d.head_dim)) return false;
+  return S.logitsb != nullptr && S.embedb != nullptr;
+}
+
+inline bool set_layer_q4(model& M, int64_t li, const layer_blobs& b) {
+  const dims& d = M.d;
+  layer& L = M.layers[(size_t)li];
+  const int64_t E = d.hidden;
+  auto fused_qkv = detail::fuse_q4({b.wq, b.wk, b.wv}, {d.q_dim(), d.kv_dim(), d.kv_dim()}, E);
+  auto fused_gu = detail::fuse_q4({b.wg, b.wu}, {d.ff, d.ff}, E);
+  L.wqkv = linear{detail::dev_from_host(fused_qkv.data(), (int64_t)fused_qkv.size()), d.qkv_dim(), E,
+                  wfmt::q4};
+  L.wgu = linear{detail::dev_from_host(fused_gu.data(), (int64_t)fused_gu.size()), 2 * d.ff, E,
+                 wfmt::q4};
+  L.wo = linear{detail::dev_from_host(b.wo, q4_bytes(E, d.q_dim())), E, d.q_dim(), wfmt::q4};
+  L.wd = linear{detail::dev_from_host(b.wd, q4_bytes(E, d.ff)), E, d.ff, wfmt::q4};
+  L.bq = detail::dev_from_host(b.bq, d.q_dim() * 4);
+  L.bk = detail::dev_from_host(b.bk, d.kv_dim() * 4);
+  L.bv = detail::dev_from_host(b.bv, d.kv_dim() * 4);
+  L.an = detail::dev_from_host(b.an, E * 4);
+  L.fn = detail::dev_from_host(b.fn, E * 4);
+  return L.wqkv.w && L.wgu.w && L.wo.w && L.wd.w && L.bq && L.bk && L.bv && L.an && L.fn;
+}
+
+inline bool set_head_q4(model& M, const uint16_t* embed_bf16, const float* onorm,
+                        const uint8_t* outw_q4) {
+  const dims& d = M.d;
+  M.embed.assign(embed_bf16, embed_bf16 + d.vocab * d.hidden);
+  M.onorm = detail::dev_from_host(onorm, d.hidden * 4);
+  M.lm_head = linear{detail::dev_from_host(outw_q4, q4_bytes(d.vocab, d.hidden)), d.vocab, d.hidden,
+                     wfmt::q4};
+  M.ready = M.onorm && M.lm_head.w;
+  return M.ready;
+}
+
+// Synthetic weights for throughput runs (a 7B-shape model is 4.4 GB of int4):
+// one 32 MB block of seeded random nibbles and one of scales ~U(0.002,0.006) are
+// uploaded once and tiled into device-only weight buffers with device copies.
+// Values do not affect kernel time; they keep activations finite.
+inline bool set_random_q4(model& M, uint32_t seed) {
+  const dims& d = M.d;
+  const int64_t blk = int64_t(32) << 20;
+  std::vector<uint32_t> nib((size_t)blk / 4);
+  std::vector<float> scl((size_t)blk / 4);
+  uint32_t s = seed * 2654435761u + 1u;
+  auto next = [&s] { s ^= s << 13; s ^= s >> 17; s ^= s << 5; return s; };
+  for (auto& v : nib) v = next();
+  for (auto& v : scl) v = 0.002f + 0.004f * (float)(next() >> 8) * (1.0f / 16777216.0f);
+  void* dn = detail::dev_from_host(nib.data(), blk);
+  void* ds = detail::dev_from_host(scl.data(), blk);
+  if (!dn || !ds) return false;
+  bool ok = true;
+  auto make = [&](int64_t N, int64_t K) {
+    linear L{hip::alloc_device(q4_bytes(N, K)), N, K, wfmt::q4};
+    if (!L.w) { ok = false; return L; }
+    const int64_t pb = N * K / 2, sb = N * (K / kQ4Group) * 4;
+    for (int64_t o = 0; o < pb; o += blk)
+      ok &= hip::copy_d2d(static_cast<char*>(L.w) + o, dn, std::min(blk, pb - o));
+    for (int64_t o = 0; o < sb; o += blk)
+      ok &= hip::copy_d2d(static_cast<char*>(L.w) + pb + o, ds, std::min(blk, sb - o));
+    return L;
+  };
+  auto vec = [&](int64_t n, float mean, float std_) {
+    std::vector<float> v((size_t)n);
+    for (auto& e : v) e = mean + std_ * ((float)(int32_t)next() * (1.0f / 2147483648.0f));
+    return detail::dev_from_host(v.data(), n * 4);
+  };
+  for (auto& L : M.layers) {
+    L.wqkv = make(d.qkv_dim(), d.hidden);
+    L.wo = make(d.hidden, d.q_dim());
+    L.wgu = make(2 * d.ff, d.hidden);
+    L.wd = make(d.hidden, d.ff);
+    L.bq = vec(d.q_dim(), 0.f, 0.02f);
+    L.bk = vec(d.kv_dim(), 0.f, 0.02f);
+    L.bv = vec(d.kv_dim(), 0.f, 0.02f);
+    L.an = vec(d.hidden, 1.f, 0.02f);
+    L.fn = vec(d.hidden, 1.f, 0.02f);
+    ok = ok && L.bq && L.bk && L.bv && L.an && L.fn;
+  }
+  M.lm_head = make(d.vocab, d.hidden);
+  M.onorm = vec(d.hidden, 1.f, 0.02f);
+  M.embed.resize((size_t)(d.vocab * d.hidden));
+  for (size_t i = 0; i < M.embed.size(); i++)
+    M.embed[i] = f32_to_bf16(0.02f * ((float)(int32_t)next() * (1.0f / 2147483648.0f)));
+  hip::flush();
+  M.ready = ok && M.onorm;
+  return M.ready;
+}
+
+// Fill every layer's cache rows [0, upto) with seeded N(0,1)-like values so a
+// decode step at a deep position reads a realistic cache.
+inline bool fill_cache_random(model& M, int64_t upto, uint32_t seed) {
+  const dims& d = M.d;
+  const int64_t per = d.n_kv_heads * d.max_ctx * d.head_dim;
+  std::vector<float> blkv((size_t)per);
+  uint32_t s = seed * 2654435761u + 7u;
+  auto next = [&s] { s ^= s << 13; s ^= s >> 17; s ^= s << 5; return s; };
+  for (auto& e : blkv) {  // sum of 4 uniforms: variance 1, near-normal
+    float a = 0.f;
+    for (int i = 0; i < 4; i++) a += (float)(int32_t)next() * (1.0f / 2147483648.0f);
+    e = a * 0.8660254f;
+  }
+  void* stage = detail::dev_from_host(blkv.data(), per * 4);
+  if (!stage) return false;
+  bool ok = true;
+  for (auto& L : M.layers) {
+    ok &= hip::copy_d2d(L.cache.K, stage, per * 4);
+    ok &= hip::copy_d2d(L.cache.V, stage, per * 4);
+    L.cache.pos = upto;
+  }
+  hip::flush();
+  hip::release(stage, 0, nullptr);
+  return ok;
+}
+
+inline void reset_cache(model& M) {
+  for (auto& L : M.layers) L.cache.pos = 0;
+}
+inline void set_cache_pos(model& M, int64_t p) {
+  for (auto& L : M.layers) L.cache.pos = p;
+}
+
+// Widen one embedding row into the staged input (host gather, one small H2D).
+inline void stage_embed(model& M, int64_t token) {
+  const dims& d = M.d;
+  const uint16_t* r = M.embed.data() + (size_t)token * d.hidden;
+  for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = bf16_to_f32(r[j]);
+  hip::upload(M.s.embedb, M.s.embed_host, d.hidden);
+}
+
+// All layers + final norm + lm_head on the scratch buffers, no allocation, no
+// sync: capturable as one graph. Reads the layer-0 residual from x0, writes
+// logits to S.logitsb (or logits_out).
+inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullptr) {
+  const dims& d = M.d;
+  scratch& S = M.s;
+  const float scale = 1.0f / std::sqrt((float)d.head_dim);
+  const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim();
+  bool ok = true;
+  void* x = x0;
+  ok &= hip::rmsnorm(x, M.layers[0].an, S.hb, E, d.eps);
+  for (int64_t l = 0; l < d.n_layers; l++) {
+    layer& L = M.layers[(size_t)l];
+    void* ro = S.res[l & 1];
+    ok &= gemv(L.wqkv, S.hb, S.qkvb);
+    void* qp = S.qkvb;
+    void* kp = static_cast<char*>(S.qkvb) + QD * 4;
+    void* vp = static_cast<char*>(S.qkvb) + (QD + KD) * 4;
+    ok &= hip::rope(qp, qp, d.n_q_heads, 1, d.head_dim, pos, d.rope_base, L.bq);
+    ok &= hip::rope(kp, kp, d.n_kv_heads, 1, d.head_dim, pos, d.rope_base, L.bk);
+    ok &= hip::binary(hip::kop::add, vp, 0, L.bv, 0, vp, 0, KD, 1.0f, 0.0f);
+    L.cache.pos = pos;
+    ok &= L.cache.append(kp, vp);
+    ok &= L.cache.attn(qp, S.ab, d.n_q_heads, scale);
+    ok &= gemv(L.wo, S.ab, ro);
+    ok &= hip::rmsnorm_res(ro, x, L.fn, ro, S.h2b, E, d.eps);
+    ok &= gemv(L.wgu, S.h2b, S.gub);
+    ok &= hip::swiglu(S.gub, S.mb, d.ff);
+    ok &= gemv(L.wd, S.mb, S.mdb);
+    void* nextw = (l + 1 < d.n_layers) ? M.layers[(size_t)l + 1].an : M.onorm;
+    ok &= hip::rmsnorm_res(ro, S.mdb, nextw, ro, S.hb, E, d.eps);
+    x = ro;
+  }
+  ok &= gemv(M.lm_head, S.hb, logits_out ? logits_out : S.logitsb);
+  return ok;
+}
+
+// embed -> layers -> device argmax. Returns the greedy token, or -1 when any
+// launch was declined.
+inline int64_t step_greedy(model& M, int64_t token, int64_t pos) {
+  stage_embed(M, token);
+  if (!run_layers(M, M.s.embedb, pos)) return -1;
+  int64_t idx = -1;
+  if (!hip::argmax(M.s.logitsb, M.d.vocab, &idx)) return -1;
+  return idx;
+}
+
+// Host view of the logits the last step left on the device.
+inline const float* logits(model& M) {
+  hip::sync_to_host(M.s.logitsb, false);
+  return M.s.logits_host;
+}
+
+// One decode step recorded as a hipGraph at a FIXED position (the throughput
+// measurement replays the same step; replaying re-writes the same cache row).
+struct captured_step {
+  void* graph = nullptr;
+  bool capture(model& M, int64_t pos) {
+    // warm: lets the library size its scratch before the capture opens
+    if (!run_layers(M, M.s.embedb, pos)) return false;
+    hip::flush();
+    if (!hip::capture_begin()) return false;
+    const bool ok = run_layers(M, M.s.embedb, pos);
+    graph = hip::capture_end();
+    return ok && graph != nullptr;
+  }
+  bool replay() { return hip::graph_launch(graph); }
+  void destroy() {
+    hip::graph_destroy(graph);
+    graph = nullptr;
+  }
+};
+
+}  // namespace qwen
+}  // namespace tl

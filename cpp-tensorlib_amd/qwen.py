@@ -1,0 +1,141 @@
+"""ctypes binding of libtl_qwen.so: the C++ decode harness (include/tl/qwen_decode.h)
+as seen from Python tests and benchmarks. The harness finds the HIP library through
+tl::hip's dlopen, so TENSORLIB_HIP_LIB is pointed at the in-tree build first."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+QWEN_LIB_PATH = os.path.join(HERE, "lib", "libtl_qwen.so")
+HIP_LIB_PATH = os.path.join(HERE, "lib", "libtensorlib_hip.so")
+
+i64, f32, u32, cint = C.c_int64, C.c_float, C.c_uint32, C.c_int
+P = C.c_void_p
+
+
+class Dims(C.Structure):
+    _fields_ = [("n_layers", i64), ("hidden", i64), ("n_q_heads", i64), ("n_kv_heads", i64),
+                ("head_dim", i64), ("ff", i64), ("vocab", i64), ("max_ctx", i64),
+                ("eps", f32), ("rope_base", f32)]
+
+
+QWEN_05B = dict(n_layers=24, hidden=896, n_q_heads=14, n_kv_heads=2, head_dim=64, ff=4864,
+                vocab=151936, max_ctx=512, eps=1e-6, rope_base=1e6)
+QWEN_7B = dict(n_layers=28, hidden=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ff=18944,
+               vocab=152064, max_ctx=4352, eps=1e-6, rope_base=1e6)
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(QWEN_LIB_PATH):
+            raise FileNotFoundError("%s is missing: run `python cpp-tensorlib_amd/build.py`" % QWEN_LIB_PATH)
+        os.environ.setdefault("TENSORLIB_HIP_LIB", HIP_LIB_PATH)
+        L = C.CDLL(QWEN_LIB_PATH)
+        sig = {
+            "tlq_available": (cint, []),
+            "tlq_unavailable_reason": (C.c_char_p, []),
+            "tlq_create": (P, [C.POINTER(Dims)]),
+            "tlq_destroy": (None, [P]),
+            "tlq_set_layer_q4": (cint, [P, i64] + [P] * 12),
+            "tlq_set_head_q4": (cint, [P, P, P, P]),
+            "tlq_set_random_q4": (cint, [P, u32]),
+            "tlq_fill_cache_random": (cint, [P, i64, u32]),
+            "tlq_step": (i64, [P, i64, i64, P]),
+            "tlq_run_layers": (cint, [P, i64, i64]),
+            "tlq_argmax": (i64, [P]),
+            "tlq_capture": (cint, [P, i64, i64]),
+            "tlq_replay": (cint, [P]),
+            "tlq_flush": (None, []),
+            "tlq_census": (cint, [C.POINTER(C.c_uint64), cint]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(P)
+
+
+class QwenGPU:
+    """A decoder on the GPU. No CPU fallback: construction raises when the HIP
+    backend is unavailable."""
+
+    def __init__(self, dims):
+        self.L = _load()
+        if not self.L.tlq_available():
+            raise RuntimeError("tl::hip backend unavailable: %s" % self.L.tlq_unavailable_reason().decode())
+        self.d = Dims(**dims) if isinstance(dims, dict) else dims
+        self.h = self.L.tlq_create(C.byref(self.d))
+        if not self.h:
+            raise RuntimeError("tlq_create failed")
+        self._keep = []
+
+    @classmethod
+    def from_oracle(cls, om):
+        """Upload the very weight bytes an oracle model (tests/oraclelib.OracleQwen) holds."""
+        d = om.d
+        g = cls(dict((f, getattr(d, f)) for f, _ in Dims._fields_))
+        for li in range(d.n_layers):
+            w = [np.ascontiguousarray(om.weight(li, n)) for n in ("wq", "wk", "wv", "wo", "wg", "wu", "wd")]
+            v = [np.ascontiguousarray(om.weight(li, n)) for n in ("bq", "bk", "bv", "an", "fn")]
+            rc = g.L.tlq_set_layer_q4(g.h, li, *[_p(a) for a in w + v])
+            if rc != 0:
+                raise RuntimeError("tlq_set_layer_q4(%d) failed" % li)
+        emb = np.ascontiguousarray(om.weight(-1, "embed"))
+        onorm = np.ascontiguousarray(om.weight(-1, "onorm"))
+        outw = np.ascontiguousarray(om.weight(-1, "outw"))
+        if g.L.tlq_set_head_q4(g.h, _p(emb), _p(onorm), _p(outw)) != 0:
+            raise RuntimeError("tlq_set_head_q4 failed")
+        return g
+
+    def set_random(self, seed=1):
+        if self.L.tlq_set_random_q4(self.h, seed) != 0:
+            raise RuntimeError("tlq_set_random_q4 failed")
+
+    def fill_cache_random(self, upto, seed=2):
+        if self.L.tlq_fill_cache_random(self.h, upto, seed) != 0:
+            raise RuntimeError("tlq_fill_cache_random failed")
+
+    def step(self, token, pos, want_logits=False):
+        logits = np.empty(self.d.vocab, np.float32) if want_logits else None
+        tok = self.L.tlq_step(self.h, token, pos, _p(logits) if want_logits else None)
+        if tok < 0:
+            raise RuntimeError("decode step declined by the backend")
+        return (int(tok), logits) if want_logits else int(tok)
+
+    def run_layers(self, token, pos):
+        if self.L.tlq_run_layers(self.h, token, pos) != 0:
+            raise RuntimeError("run_layers declined by the backend")
+
+    def argmax(self):
+        return int(self.L.tlq_argmax(self.h))
+
+    def capture(self, token, pos):
+        if self.L.tlq_capture(self.h, token, pos) != 0:
+            raise RuntimeError("graph capture failed")
+
+    def replay(self):
+        if self.L.tlq_replay(self.h) != 0:
+            raise RuntimeError("graph replay failed")
+
+    def flush(self):
+        self.L.tlq_flush()
+
+    def census(self):
+        from .capi import CENSUS
+        buf = (C.c_uint64 * len(CENSUS))()
+        self.L.tlq_census(buf, len(CENSUS))
+        return dict(zip(CENSUS, [int(v) for v in buf]))
+
+    def close(self):
+        if self.h:
+            self.L.tlq_destroy(self.h)
+            self.h = None
