@@ -75,6 +75,7 @@ SIGNATURES = {
     "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
+    "tlhip_qkv_rope_append": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
@@ -281,6 +282,10 @@ class TlHip:
 
     def bench_read(self, src, nbytes, sink, blocks=0, off=0):
         self._chk(self.c.tlhip_bench_read(src.ptr + off, nbytes, sink.ptr, blocks))
+
+    def qkv_rope_append(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, D, pos, kv_max, base, kv_bf16=False):
+        self._chk(self.c.tlhip_qkv_rope_append(qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None,
+                                               Kc.ptr, Vc.ptr, Hq, Hkv, D, pos, kv_max, base, int(kv_bf16)))
 
     def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0):
         self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw))

@@ -3,11 +3,11 @@
 // One block serves ONE kv head and up to G of its query heads, so with GQA the
 // K/V rows are fetched from HBM once per group instead of once per query head.
 // Keys are split over gridDim.y (split-KV) and over the wavefronts of a block
-// in tiles of 64 keys. Inside a wavefront a key row is spread over LPK = D/4
-// lanes (one 128-bit load per lane, 64/LPK keys per load instruction, fully
-// coalesced); scores are reduced over those lanes, parked one-key-per-lane so
-// that the softmax exponentials cost one instruction per 64 keys, and fed back
-// to the P.V pass through a per-wave LDS line. Running (max, sum, acc) states
+// in tiles of 16-64 keys. Inside a wavefront a key row is spread over the 16
+// lanes of a DPP row (one or two 128-bit loads per lane, 4 keys per load step,
+// fully coalesced); scores are reduced inside the row with DPP adds, parked
+// one-key-per-lane so that the softmax exponentials cost one instruction per
+// tile, and fed back to the P.V pass through a per-wave LDS line. Running (max, sum, acc) states
 // are merged wave -> block -> split in a fixed order: no atomics.
 #include "common.hpp"
 
@@ -31,71 +31,100 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// ---- 16-lane reductions on DPP (no LDS round trips) ------------------------------
+// A key row is spread over the 16 lanes of one DPP row, so a score is finished
+// with four v_add_f32 carrying DPP modifiers: xor-1 and xor-2 inside a quad,
+// then mirroring the half row and the row. Every lane of the row ends up with
+// the full sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+  return v + __int_as_float(t);
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  return v;
+}
+
 // grid = (Hkv, S, ceil(group/G)); block = nw*64 threads (nw in 1,2,4).
+// A wavefront works on tiles of TK keys (16, 32 or 64): 4 keys per load step
+// (one per DPP row), each lane holding EPL = D/16 consecutive floats of its key.
 // part_m/part_l: [Hq*S], part_acc: [Hq*S*D]; used when S > 1, else `out` is final.
 template <int D, int G, typename KT>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
     float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
-    float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, float scale,
-    int S) {
-  constexpr int LPK = D / 4;        // lanes per key row
-  constexpr int KPS = 64 / LPK;     // keys per load step
-  constexpr int UNR = 8;            // loads in flight per lane
-  __shared__ float pbuf[4][G][64];              // per-wave probabilities of the current tile
-  __shared__ float st_m[4][G], st_l[4][G];      // per-wave softmax state for the block merge
+    float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, int TK,
+    float scale, int S) {
+  constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
+  constexpr int NV = EPL / 4;        // float4 loads per lane per key
+  constexpr int UNR = 4;             // key steps in flight per lane
+  __shared__ float pbuf[4][G][64];               // per-wave probabilities of the current tile
+  __shared__ float st_m[4][G], st_l[4][G];       // per-wave softmax state for the block merge
   __shared__ float st_acc[4][G][D];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  const int slot = lane / LPK, c = lane % LPK;
+  const int slot = lane >> 4, c = lane & 15;     // DPP row = key slot, c = position in the row
   const int kvh = blockIdx.x, split = blockIdx.y;
-  const int g0 = blockIdx.z * G;                // first query head (within the group) of this block
+  const int g0 = blockIdx.z * G;
   const int ng = min(G, group - g0);
-  const int h0 = kvh * group + g0;              // absolute query head of g == 0
+  const int h0 = kvh * group + g0;
   const KT* Kh = K + (size_t)kvh * kv_stride;
   const KT* Vh = V + (size_t)kvh * kv_stride;
   const int k_begin = split * chunk, k_end = min(ctx, k_begin + chunk);
+  const int steps = TK >> 2;                     // load steps per tile
 
-  float4 qv[G];
+  float4 qv[G][NV];
 #pragma unroll
-  for (int g = 0; g < G; g++) {
-    qv[g] = g < ng ? *reinterpret_cast<const float4*>(q + (size_t)(h0 + g) * D + c * 4)
-                   : make_float4(0.f, 0.f, 0.f, 0.f);
-  }
+  for (int g = 0; g < G; g++)
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+      qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (size_t)(h0 + g) * D + c * EPL + v * 4)
+                        : make_float4(0.f, 0.f, 0.f, 0.f);
   float m[G], l[G];
-  float4 acc[G];
+  float4 acc[G][NV];
 #pragma unroll
   for (int g = 0; g < G; g++) {
     m[g] = -INFINITY;
     l[g] = 0.f;
-    acc[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int v = 0; v < NV; v++) acc[g][v] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
 
-  for (int kb = k_begin + wave * 64; kb < k_end; kb += nw * 64) {
-    // ---- scores: lane (slot,c) ends up holding key kb + c*KPS + slot ----------
+  for (int kb = k_begin + wave * TK; kb < k_end; kb += nw * TK) {
+    // ---- scores: lane (slot,c) ends up holding key kb + c*4 + slot (c < steps) ----
     float sreg[G];
 #pragma unroll
     for (int g = 0; g < G; g++) sreg[g] = -INFINITY;
-#pragma unroll
-    for (int i0 = 0; i0 < LPK; i0 += UNR) {
-      float4 kv[UNR];
+    for (int i0 = 0; i0 < steps; i0 += UNR) {
+      float4 kv[UNR][NV];
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
-        const int key = kb + (i0 + u) * KPS + slot;
-        kv[u] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * 4)
-                            : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int key = kb + (i0 + u) * 4 + slot;
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+          kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * EPL + v * 4)
+                                 : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
-        const int key = kb + (i0 + u) * KPS + slot;
+        const int key = kb + (i0 + u) * 4 + slot;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-          float p = qv[g].x * kv[u].x;
-          p = fmaf(qv[g].y, kv[u].y, p);
-          p = fmaf(qv[g].z, kv[u].z, p);
-          p = fmaf(qv[g].w, kv[u].w, p);
-#pragma unroll
-          for (int msk = LPK / 2; msk >= 1; msk >>= 1) p += __shfl_xor(p, msk, kWave);
+          float p = qv[g][0].x * kv[u][0].x;
+          p = fmaf(qv[g][0].y, kv[u][0].y, p);
+          p = fmaf(qv[g][0].z, kv[u][0].z, p);
+          p = fmaf(qv[g][0].w, kv[u][0].w, p);
+          if (NV > 1) {
+            p = fmaf(qv[g][NV - 1].x, kv[u][NV - 1].x, p);
+            p = fmaf(qv[g][NV - 1].y, kv[u][NV - 1].y, p);
+            p = fmaf(qv[g][NV - 1].z, kv[u][NV - 1].z, p);
+            p = fmaf(qv[g][NV - 1].w, kv[u][NV - 1].w, p);
+          }
+          p = row16_sum(p);
           if (c == i0 + u) sreg[g] = key < k_end ? p * scale : -INFINITY;
         }
       }
@@ -106,54 +135,62 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       const float tmax = wave_max(sreg[g]);      // finite: the tile holds >= 1 live key
       const float mnew = fmaxf(m[g], tmax);
       const float corr = __expf(m[g] - mnew);    // 0 on the first tile (m = -inf)
-      const float p = __expf(sreg[g] - mnew);    // 0 for masked keys
+      const float p = __expf(sreg[g] - mnew);    // 0 for masked keys and idle lanes
       l[g] = fmaf(l[g], corr, p);
-      acc[g].x *= corr; acc[g].y *= corr; acc[g].z *= corr; acc[g].w *= corr;
+#pragma unroll
+      for (int v = 0; v < NV; v++) {
+        acc[g][v].x *= corr; acc[g][v].y *= corr; acc[g][v].z *= corr; acc[g][v].w *= corr;
+      }
       m[g] = mnew;
       pbuf[wave][g][lane] = p;
     }
     wave_lds_sync();
-    // ---- P.V: lane (slot,c) accumulates its 4 output columns over its slot's keys ----
-#pragma unroll
-    for (int i0 = 0; i0 < LPK; i0 += UNR) {
-      float4 vv[UNR];
+    // ---- P.V: lane (slot,c) accumulates its EPL output columns over its slot's keys ----
+    for (int i0 = 0; i0 < steps; i0 += UNR) {
+      float4 vv[UNR][NV];
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
-        const int key = kb + (i0 + u) * KPS + slot;
-        vv[u] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * 4)
-                            : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int key = kb + (i0 + u) * 4 + slot;
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+          vv[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+                                 : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int g = 0; g < G; g++) {
-        // key (i, slot) was parked in lane slot*LPK + i
-        const float4 p0 = *reinterpret_cast<const float4*>(&pbuf[wave][g][slot * LPK + i0]);
-        const float4 p1 = *reinterpret_cast<const float4*>(&pbuf[wave][g][slot * LPK + i0 + 4]);
-        const float pp[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+        // key (step i, slot) was parked in lane slot*16 + i
+        const float4 p4 = *reinterpret_cast<const float4*>(&pbuf[wave][g][slot * 16 + i0]);
+        const float pp[4] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
-        for (int u = 0; u < UNR; u++) {
-          acc[g].x = fmaf(pp[u], vv[u].x, acc[g].x);
-          acc[g].y = fmaf(pp[u], vv[u].y, acc[g].y);
-          acc[g].z = fmaf(pp[u], vv[u].z, acc[g].z);
-          acc[g].w = fmaf(pp[u], vv[u].w, acc[g].w);
-        }
+        for (int u = 0; u < UNR; u++)
+#pragma unroll
+          for (int v = 0; v < NV; v++) {
+            acc[g][v].x = fmaf(pp[u], vv[u][v].x, acc[g][v].x);
+            acc[g][v].y = fmaf(pp[u], vv[u][v].y, acc[g][v].y);
+            acc[g][v].z = fmaf(pp[u], vv[u][v].z, acc[g][v].z);
+            acc[g][v].w = fmaf(pp[u], vv[u][v].w, acc[g][v].w);
+          }
       }
     }
     wave_lds_sync();  // pbuf is rewritten by the next tile
   }
 
-  // ---- wave totals: sum l over lanes, acc over the key slots -----------------------------
+  // ---- wave totals: sum l over lanes, acc over the four key slots --------------------------
 #pragma unroll
   for (int g = 0; g < G; g++) {
     l[g] = wave_sum(l[g]);
 #pragma unroll
-    for (int msk = LPK; msk < 64; msk <<= 1) {
-      acc[g].x += __shfl_xor(acc[g].x, msk, kWave);
-      acc[g].y += __shfl_xor(acc[g].y, msk, kWave);
-      acc[g].z += __shfl_xor(acc[g].z, msk, kWave);
-      acc[g].w += __shfl_xor(acc[g].w, msk, kWave);
+    for (int v = 0; v < NV; v++) {
+#pragma unroll
+      for (int msk = 16; msk < 64; msk <<= 1) {
+        acc[g][v].x += __shfl_xor(acc[g][v].x, msk, kWave);
+        acc[g][v].y += __shfl_xor(acc[g][v].y, msk, kWave);
+        acc[g][v].z += __shfl_xor(acc[g][v].z, msk, kWave);
+        acc[g][v].w += __shfl_xor(acc[g][v].w, msk, kWave);
+      }
+      if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][c * EPL + v * 4]) = acc[g][v];
     }
     if (lane == 0) { st_m[wave][g] = m[g]; st_l[wave][g] = l[g]; }
-    if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][c * 4]) = acc[g];
   }
   __syncthreads();
 
@@ -179,42 +216,76 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// grid = Hq, block = D: merge the S split partials of one head.
-__global__ void attn_combine_kernel(const float* __restrict__ part_m,
-                                    const float* __restrict__ part_l,
-                                    const float* __restrict__ part_acc, float* __restrict__ out,
-                                    int S, int D) {
-  const int h = blockIdx.x, d = threadIdx.x;
+// grid = Hq, block = 256: merge the S split partials of one head. The split
+// weights exp(m_s - M) are formed once per split in LDS; the 256 threads are
+// D columns x (256/D) split groups, summed in a fixed order.
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part_m,
+                                                           const float* __restrict__ part_l,
+                                                           const float* __restrict__ part_acc,
+                                                           float* __restrict__ out, int S, int D) {
+  extern __shared__ float sm[];   // f[S] | red[256]
+  float* f = sm;
+  float* red = sm + S;
+  const int h = blockIdx.x, tid = threadIdx.x;
   const float* pm = part_m + (size_t)h * S;
   const float* pl = part_l + (size_t)h * S;
-  float M = pm[0];
-  for (int s = 1; s < S; s++) M = fmaxf(M, pm[s]);
-  float L = 0.f, A = 0.f;
-  for (int s = 0; s < S; s++) {
-    const float f = __expf(pm[s] - M);
-    L = fmaf(pl[s], f, L);
-    A = fmaf(part_acc[((size_t)h * S + s) * D + d], f, A);
+  float mx = -INFINITY;
+  for (int s = tid; s < S; s += 256) mx = fmaxf(mx, pm[s]);
+  mx = wave_max(mx);
+  if ((tid & 63) == 0) red[tid >> 6] = mx;
+  __syncthreads();
+  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float lsum = 0.f;
+  for (int s = tid; s < S; s += 256) {
+    const float w = __expf(pm[s] - M);
+    f[s] = w;
+    lsum = fmaf(pl[s], w, lsum);
   }
-  out[(size_t)h * D + d] = A / L;
+  lsum = wave_sum(lsum);
+  if ((tid & 63) == 0) red[tid >> 6] = lsum;
+  __syncthreads();
+  const float L = ((red[0] + red[1]) + red[2]) + red[3];
+  __syncthreads();
+  const int groups = 256 / D, d = tid % D, sg = tid / D;
+  const float* pa = part_acc + (size_t)h * S * D + d;
+  float a0 = 0.f, a1 = 0.f;
+  int s = sg;
+  for (; s + groups < S; s += 2 * groups) {
+    a0 = fmaf(f[s], pa[(size_t)s * D], a0);
+    a1 = fmaf(f[s + groups], pa[(size_t)(s + groups) * D], a1);
+  }
+  if (s < S) a0 = fmaf(f[s], pa[(size_t)s * D], a0);
+  red[tid] = a0 + a1;
+  __syncthreads();
+  if (sg == 0) {
+    float A = red[d];
+    for (int k = 1; k < groups; k++) A += red[k * D + d];
+    out[(size_t)h * D + d] = A / L;
+  }
 }
 
-struct AttnPlan { int G, gz, nw, S, chunk; };
+struct AttnPlan { int G, gz, nw, TK, S, chunk; };
 
-// Split-KV plan: enough blocks to cover the CUs about twice, and never less
-// than one 64-key tile per wavefront.
+// Split-KV plan. Work is cut into wave tiles of TK keys; the chip wants at least
+// ~4 wavefronts per CU, so short contexts use small tiles and 4-wave blocks, and
+// long contexts give every wavefront several 64-key tiles.
 static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus) {
   AttnPlan p{};
   p.G = group > 4 ? 8 : group > 2 ? 4 : group > 1 ? 2 : 1;
   p.gz = (group + p.G - 1) / p.G;
   const int base = Hkv * p.gz;
-  const int tiles = (ctx + 63) / 64;
-  int want = (2 * cus + base - 1) / base;  // splits wanted to fill the chip
-  if (want < 1) want = 1;
-  if (want > tiles) want = tiles;
-  int tiles_per_split = (tiles + want - 1) / want;
-  p.nw = tiles_per_split >= 4 ? 4 : tiles_per_split >= 2 ? 2 : 1;
-  tiles_per_split = (tiles_per_split + p.nw - 1) / p.nw * p.nw;
-  p.chunk = tiles_per_split * 64;
+  const int64_t want_waves = (int64_t)cus * 4;
+  p.TK = 64;
+  while (p.TK > 16 && (int64_t)base * ((ctx + p.TK - 1) / p.TK) < want_waves) p.TK >>= 1;
+  const int tiles = (ctx + p.TK - 1) / p.TK;
+  p.nw = tiles >= 4 ? 4 : tiles >= 2 ? 2 : 1;
+  const int block_tiles = (tiles + p.nw - 1) / p.nw;       // tiles per wave if S == 1
+  int want_s = (int)((want_waves + (int64_t)base * p.nw - 1) / ((int64_t)base * p.nw));
+  if (want_s < 1) want_s = 1;
+  if (want_s > block_tiles) want_s = block_tiles;
+  const int tiles_per_wave = (block_tiles + want_s - 1) / want_s;
+  p.chunk = tiles_per_wave * p.nw * p.TK;
   p.S = (ctx + p.chunk - 1) / p.chunk;
   return p;
 }
@@ -234,11 +305,12 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     pl = pm + hs;
     pacc = pl + hs;
   }
+  if (p.S > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode: context too long");
   const dim3 grid(Hkv, p.S, p.gz), block(p.nw * 64);
   const int64_t kv_stride = kv_max * D;
 #define TLHIP_ATTN(GG)                                                                         \
   hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT>), grid, block, 0, c.stream, q, K, V, out, \
-                     pm, pl, pacc, group, ctx, kv_stride, p.chunk, scale, p.S)
+                     pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S)
   switch (p.G) {
     case 1: TLHIP_ATTN(1); break;
     case 2: TLHIP_ATTN(2); break;
@@ -247,7 +319,8 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
   }
 #undef TLHIP_ATTN
   if (p.S > 1)
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(D), 0, c.stream, pm, pl, pacc, out, p.S, D);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(256), (size_t)(p.S + 256) * sizeof(float),
+                       c.stream, pm, pl, pacc, out, p.S, D);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
 }
 

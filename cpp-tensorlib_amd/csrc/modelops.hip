@@ -77,6 +77,72 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   for (int i = threadIdx.x; i < n; i += 256) hout[base + i] = (src[base + i] * inv) * w[i];
 }
 
+// Wide variant for rows that fit the registers of one 1024-thread block
+// (n % 4 == 0, n <= 4*1024*RV): every thread keeps its float4s of the row and of
+// the weight in VGPRs, so the row is read once and nothing waits on a second
+// pass. This is the decode-step shape (n = 896 ... 8192).
+template <bool RES, int RV>
+__global__ __launch_bounds__(1024) void rmsnorm_wide_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ delta,
+                                                            const float* __restrict__ w,
+                                                            float* __restrict__ xout,
+                                                            float* __restrict__ hout, int n,
+                                                            float eps) {
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * n;
+  const int n4 = n >> 2;
+  const float4* x4 = reinterpret_cast<const float4*>(x + base);
+  const float4* d4 = RES ? reinterpret_cast<const float4*>(delta + base) : nullptr;
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+  float4 v[RV], wv[RV];
+  float acc = 0.f;
+#pragma unroll
+  for (int k = 0; k < RV; k++) {
+    const int i = threadIdx.x + k * 1024;
+    if (i < n4) {
+      v[k] = x4[i];
+      wv[k] = w4[i];
+      if (RES) {
+        const float4 d = d4[i];
+        v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < RV; k++) {
+    const int i = threadIdx.x + k * 1024;
+    if (i < n4) {
+      if (RES) reinterpret_cast<float4*>(xout + base)[i] = v[k];
+      acc += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+    }
+  }
+  const float sum = block_sum<16>(acc, red);
+  const float inv = 1.0f / sqrtf(sum * (1.0f / (float)n) + eps);
+#pragma unroll
+  for (int k = 0; k < RV; k++) {
+    const int i = threadIdx.x + k * 1024;
+    if (i < n4) {
+      float4 o;
+      o.x = (v[k].x * inv) * wv[k].x; o.y = (v[k].y * inv) * wv[k].y;
+      o.z = (v[k].z * inv) * wv[k].z; o.w = (v[k].w * inv) * wv[k].w;
+      reinterpret_cast<float4*>(hout + base)[i] = o;
+    }
+  }
+}
+
+template <bool RES>
+static void launch_rmsnorm(const float* x, const float* delta, const float* w, float* xout,
+                           float* hout, int64_t n, float eps, int64_t rows) {
+  hipStream_t st = ctx().stream;
+  const bool wide_ok = (n % 4) == 0 && aligned16(w) && aligned16(hout) && rows <= 64;
+  if (wide_ok && n <= 4096)
+    rmsnorm_wide_kernel<RES, 1><<<dim3((unsigned)rows), dim3(1024), 0, st>>>(x, delta, w, xout, hout, (int)n, eps);
+  else if (wide_ok && n <= 8192)
+    rmsnorm_wide_kernel<RES, 2><<<dim3((unsigned)rows), dim3(1024), 0, st>>>(x, delta, w, xout, hout, (int)n, eps);
+  else
+    rmsnorm_kernel<RES><<<dim3((unsigned)rows), dim3(256), 0, st>>>(x, delta, w, xout, hout, (int)n, eps);
+}
+
 // ---- swiglu -----------------------------------------------------------------------
 // out = (g * sigmoid(g)) * u, the order of array.h:2435-2439.
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gu,
@@ -187,6 +253,48 @@ __global__ __launch_bounds__(256) void merge_heads_kernel(const float* __restric
   dst[i] = src[((size_t)h * T + t) * D + d];
 }
 
+// ---- fused q/k/v epilogue of a decode step --------------------------------------------
+// One launch for what the step otherwise does in four: q and k get their bias
+// and rotary embedding (written back in place), v gets its bias, and the new k, v
+// rows go straight into the cache at row `pos`. qkv = [q (Hq*D) | k (Hkv*D) | v (Hkv*D)].
+template <typename KT>
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(
+    float* __restrict__ qkv, const float* __restrict__ bq, const float* __restrict__ bk,
+    const float* __restrict__ bv, KT* __restrict__ Kc, KT* __restrict__ Vc, int Hq, int Hkv, int D,
+    int64_t pos, int64_t kv_max, float base) {
+  const int half = D >> 1;
+  const int n_rot = (Hq + Hkv) * half;       // rotary pairs of q and k
+  const int n_v = Hkv * D;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_rot) {
+    const int r = i / half, j = i - r * half;   // r: head row within [q heads | k heads]
+    const double theta = pow((double)base, -2.0 * (double)j / (double)D);
+    const double ang = (double)pos * theta;
+    const float c = (float)cos(ang), s = (float)sin(ang);
+    const size_t bi = (size_t)r * D;
+    const bool is_k = r >= Hq;
+    const float* bias = is_k ? (bk ? bk + (size_t)(r - Hq) * D : nullptr) : (bq ? bq + bi : nullptr);
+    float x0 = qkv[bi + j], x1 = qkv[bi + j + half];
+    if (bias) { x0 += bias[j]; x1 += bias[j + half]; }
+    const float o0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+    const float o1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+    qkv[bi + j] = o0;
+    qkv[bi + j + half] = o1;
+    if (is_k) {
+      const size_t dst = ((size_t)(r - Hq) * kv_max + pos) * D;
+      Kc[dst + j] = kv_narrow<KT>(o0);
+      Kc[dst + j + half] = kv_narrow<KT>(o1);
+    }
+  } else if (i < n_rot + n_v) {
+    const int e = i - n_rot, h = e / D, d = e - h * D;
+    float* vp = qkv + (size_t)(Hq + Hkv) * D;
+    float v = vp[e];
+    if (bv) v += bv[e];
+    vp[e] = v;
+    Vc[((size_t)h * kv_max + pos) * D + d] = kv_narrow<KT>(v);
+  }
+}
+
 static unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
 
 }  // namespace tlhip
@@ -215,9 +323,8 @@ int tlhip_rmsnorm(const void* x, const void* w, void* out, int64_t n, float eps,
   if (n <= 0 || rows <= 0 || n > 0x7fffffff || rows > 0x7fffffff)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_rmsnorm: n and rows must be positive");  // cuda.h:1290
   if (!aligned16(x) || !aligned16(out)) return fail(TLHIP_EINVAL, "tlhip_rmsnorm: misaligned");
-  rmsnorm_kernel<false><<<dim3((unsigned)rows), dim3(256), 0, ctx().stream>>>(
-      static_cast<const float*>(x), nullptr, static_cast<const float*>(w), nullptr,
-      static_cast<float*>(out), (int)n, eps);
+  launch_rmsnorm<false>(static_cast<const float*>(x), nullptr, static_cast<const float*>(w), nullptr,
+                        static_cast<float*>(out), n, eps, rows);
   TLHIP_CHECK_LAUNCH(TLHIP_C_RMSNORM);
 }
 
@@ -229,9 +336,9 @@ int tlhip_rmsnorm_res(const void* x, const void* delta, const void* w, void* xou
     return fail(TLHIP_EUNSUPPORTED, "tlhip_rmsnorm_res: n and rows must be positive");
   if (!aligned16(x) || !aligned16(delta) || !aligned16(xout))
     return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res: misaligned");
-  rmsnorm_kernel<true><<<dim3((unsigned)rows), dim3(256), 0, ctx().stream>>>(
-      static_cast<const float*>(x), static_cast<const float*>(delta), static_cast<const float*>(w),
-      static_cast<float*>(xout), static_cast<float*>(hout), (int)n, eps);
+  launch_rmsnorm<true>(static_cast<const float*>(x), static_cast<const float*>(delta),
+                       static_cast<const float*>(w), static_cast<float*>(xout),
+                       static_cast<float*>(hout), n, eps, rows);
   TLHIP_CHECK_LAUNCH(TLHIP_C_RMSNORM_RES);
 }
 
@@ -297,6 +404,34 @@ int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, in
   TLHIP_REQUIRE_READY();
   return kv_write(Kc, Vc, k_new, v_new, 1, kv_max, n_kv_heads, D, kv_bf16, pos, TLHIP_C_KV_APPEND,
                   "tlhip_kv_append");
+}
+
+int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                          void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                          int64_t kv_max, float base, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  if (!qkv || !Kc || !Vc) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: null pointer");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_append: head_dim must be 64 or 128");
+  if (n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads > 4096)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_append: bad head counts");
+  if (pos < 0 || pos >= kv_max) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: row %lld outside the cache of %lld",
+                                            (long long)pos, (long long)kv_max);
+  const int64_t total = (n_q_heads + n_kv_heads) * (D / 2) + n_kv_heads * D;
+  const float* pbq = static_cast<const float*>(bq);
+  const float* pbk = static_cast<const float*>(bk);
+  if (kv_bf16)
+    qkv_rope_append_kernel<uint16_t><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+        static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<uint16_t*>(Kc),
+        static_cast<uint16_t*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base);
+  else
+    qkv_rope_append_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
+        static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<float*>(Kc),
+        static_cast<float*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base);
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  ctx().census[TLHIP_C_ROPE]++;
+  ctx().census[TLHIP_C_KV_APPEND]++;
+  return TLHIP_OK;
 }
 
 int tlhip_kv_fill(void* Kc, void* Vc, const void* K, const void* V, int64_t T, int64_t kv_max,

@@ -84,6 +84,7 @@ int tlq_capture(void* hv, int64_t token, int64_t pos) {
   qwen::stage_embed(h->M, token);
   return h->cap.capture(h->M, pos) ? 0 : -1;
 }
+void tlq_set_fused(void* hv, int on) { static_cast<handle*>(hv)->M.fused = on != 0; }
 int tlq_replay(void* hv) { return static_cast<handle*>(hv)->cap.replay() ? 0 : -1; }
 void tlq_flush() { hip::flush(); }
 

@@ -108,6 +108,8 @@ struct api {
   int (*split_heads)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
                      int64_t) = nullptr;
   int (*merge_heads)(const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*qkv_rope_append)(void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
+                         int64_t, int64_t, int64_t, float, int) = nullptr;
 };
 
 struct context {
@@ -182,7 +184,8 @@ struct context {
               bind(f.swiglu, "tlhip_swiglu") && bind(f.argmax, "tlhip_argmax") &&
               bind(f.argmax_async, "tlhip_argmax_async") &&
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
-              bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads");
+              bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
+              bind(f.qkv_rope_append, "tlhip_qkv_rope_append");
     if (!ok) return;
     if (f.abi_version() != 1) {
       why = "libtensorlib_hip.so has a different ABI version";
@@ -589,6 +592,25 @@ inline bool merge_heads(void* src, void* dst, int64_t T, int64_t H, int64_t D) {
   return detail::done_(c, c.f.merge_heads(src, dst, T, H, D));
 }
 
+// One launch for the q/k/v epilogue of a decode step: rope(q,+bq), rope(k,+bk),
+// v += bv and the cache append at row pos — the four calls the reference's
+// run_layers_ issues per layer (qm:703-716), fused. qkv = [q | k | v] in place.
+inline bool qkv_rope_append(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
+                            int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                            int64_t kv_max, float base, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || pos < 0 || pos >= kv_max) return false;
+  c.device_read_(qkv);
+  if (bq) c.device_read_(bq);
+  if (bk) c.device_read_(bk);
+  if (bv) c.device_read_(bv);
+  c.device_write_(qkv);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.qkv_rope_append(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
+                                              kv_max, base, kv_bf16 ? 1 : 0));
+}
+
 // ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------
 inline bool graph_available() { return context::get().ready; }
 inline bool capture_begin() {
@@ -639,6 +661,14 @@ struct kv_cache {
   bool append(void* k_new, void* v_new) {
     if (pos >= max_ctx) return false;
     if (!kv_append(K, V, k_new, v_new, pos, max_ctx, n_kv_heads, D, kv_bf16)) return false;
+    pos++;
+    return true;
+  }
+  // fused epilogue + append of this step's [q|k|v] (see qkv_rope_append)
+  bool rope_append(void* qkv, void* bq, void* bk, void* bv, int64_t n_q_heads, float base) {
+    if (pos >= max_ctx) return false;
+    if (!qkv_rope_append(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, D, pos, max_ctx, base, kv_bf16))
+      return false;
     pos++;
     return true;
   }

@@ -87,6 +87,7 @@ struct model {
   std::vector<layer> layers;
   scratch s;
   bool ready = false;
+  bool fused = true;  // use the fused q/k/v epilogue launch (false: one launch per op)
 };
 
 namespace detail {
@@ -294,11 +295,15 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     void* qp = S.qkvb;
     void* kp = static_cast<char*>(S.qkvb) + QD * 4;
     void* vp = static_cast<char*>(S.qkvb) + (QD + KD) * 4;
-    ok &= hip::rope(qp, qp, d.n_q_heads, 1, d.head_dim, pos, d.rope_base, L.bq);
-    ok &= hip::rope(kp, kp, d.n_kv_heads, 1, d.head_dim, pos, d.rope_base, L.bk);
-    ok &= hip::binary(hip::kop::add, vp, 0, L.bv, 0, vp, 0, KD, 1.0f, 0.0f);
     L.cache.pos = pos;
-    ok &= L.cache.append(kp, vp);
+    if (M.fused) {
+      ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
+    } else {  // the reference's call sequence, one launch per op
+      ok &= hip::rope(qp, qp, d.n_q_heads, 1, d.head_dim, pos, d.rope_base, L.bq);
+      ok &= hip::rope(kp, kp, d.n_kv_heads, 1, d.head_dim, pos, d.rope_base, L.bk);
+      ok &= hip::binary(hip::kop::add, vp, 0, L.bv, 0, vp, 0, KD, 1.0f, 0.0f);
+      ok &= L.cache.append(kp, vp);
+    }
     ok &= L.cache.attn(qp, S.ab, d.n_q_heads, scale);
     ok &= gemv(L.wo, S.ab, ro);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, S.h2b, E, d.eps);

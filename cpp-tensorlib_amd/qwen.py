@@ -49,6 +49,7 @@ def _load():
             "tlq_argmax": (i64, [P]),
             "tlq_capture": (cint, [P, i64, i64]),
             "tlq_replay": (cint, [P]),
+            "tlq_set_fused": (None, [P, cint]),
             "tlq_flush": (None, []),
             "tlq_census": (cint, [C.POINTER(C.c_uint64), cint]),
         }
@@ -125,6 +126,9 @@ class QwenGPU:
     def replay(self):
         if self.L.tlq_replay(self.h) != 0:
             raise RuntimeError("graph replay failed")
+
+    def set_fused(self, on):
+        self.L.tlq_set_fused(self.h, 1 if on else 0)
 
     def flush(self):
         self.L.tlq_flush()

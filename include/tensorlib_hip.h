@@ -177,6 +177,16 @@ int tlhip_argmax(const void* in, int64_t n, int64_t* out_idx);
 /* same reduction, result left in a device int32 (no sync; capturable) */
 int tlhip_argmax_async(const void* in, int64_t n, void* out_idx_dev);
 
+/* ---- fused decode-step epilogues (no single reference counterpart) -------------
+ * q/k bias + rope, v bias and the cache append of one token in ONE launch; the
+ * arithmetic is that of tlhip_rope (bias form), tlhip_binary(ADD) and
+ * tlhip_kv_append, i.e. cuda.h:1203-1222, 640-654 and 1116-1138 as the reference's
+ * run_layers_ chains them (bench/cuda/qwen_model.h:703-716).
+ * qkv = [q (Hq*D) | k (Hkv*D) | v (Hkv*D)] f32, updated in place. */
+int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                          void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                          int64_t kv_max, float base, int kv_bf16);
+
 /* ---- prefill ------------------------------------------------------------------ */
 /* C[M,N] = A[M,K] f32 . W[N,K]^T bf16, fp32 accumulate; K % 8 == 0.  cuda.h:787-841 */
 int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K);

@@ -25,11 +25,13 @@ def _near_tie(logits, rtol=1e-4, atol=1e-5):
     return (top2[1] - top2[0]) <= atol + rtol * abs(top2[1])
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("dims,steps", [(SMALL, 40), (SMALL128, 270)])
-def test_decode_loop_matches_oracle(orc, dims, steps):
+def test_decode_loop_matches_oracle(orc, dims, steps, fused):
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     om = orc.qwen_create(dims, seed=3, q4=True)
     g = qwen.QwenGPU.from_oracle(om)
+    g.set_fused(fused)
     rng = np.random.default_rng(5)
     tok = int(rng.integers(0, dims["vocab"]))
     worst = 0.0

@@ -184,3 +184,28 @@ def test_gemm_seam(lib, orc, m, n, k, ta, tb):
     lib.gemm(da, As.shape[1], ta, db, Bs.shape[1], tb, do, m, n, k, 2.0, 1.0)
     want = orc.dot(A, B, 2.0, 1.0)
     assert allclose(do.numpy(), want, RTOL, 1e-4), maxrel(do.numpy(), want)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(14, 2, 64), (28, 4, 128)])
+def test_qkv_rope_append_equals_unfused(lib, orc, Hq, Hkv, D):
+    """The fused q/k/v epilogue is bit-identical to rope + rope + add + kv_append."""
+    kv_max, pos = 40, 17
+    n = (Hq + 2 * Hkv) * D
+    qkv = orc.normal(n, 80)
+    bq, bk, bv = orc.normal(Hq * D, 81, 0, 0.02), orc.normal(Hkv * D, 82, 0, 0.02), orc.normal(Hkv * D, 83, 0, 0.02)
+    zeros = np.zeros((Hkv, kv_max, D), np.float32)
+    d1, K1, V1 = lib.to_device(qkv), lib.to_device(zeros), lib.to_device(zeros)
+    dbq, dbk, dbv = lib.to_device(bq), lib.to_device(bk), lib.to_device(bv)
+    lib.qkv_rope_append(d1, dbq, dbk, dbv, K1, V1, Hq, Hkv, D, pos, kv_max, 1e6)
+    q = orc.rope(qkv[:Hq * D].reshape(Hq, D), pos, 1e6, bias=bq.reshape(Hq, D))
+    k = orc.rope(qkv[Hq * D:(Hq + Hkv) * D].reshape(Hkv, D), pos, 1e6, bias=bk.reshape(Hkv, D))
+    v = (qkv[(Hq + Hkv) * D:] + bv).reshape(Hkv, D)
+    got = d1.numpy()
+    assert allclose(got[:Hq * D], q.ravel(), RTOL, ATOL) and allclose(got[Hq * D:(Hq + Hkv) * D], k.ravel(), RTOL, ATOL)
+    assert np.array_equal(got[(Hq + Hkv) * D:], v.ravel())
+    Kc, Vc = K1.numpy(), V1.numpy()
+    assert np.array_equal(Kc[:, pos], got[Hq * D:(Hq + Hkv) * D].reshape(Hkv, D)) and np.array_equal(Vc[:, pos], v)
+    Kc[:, pos] = 0; Vc[:, pos] = 0
+    assert not Kc.any() and not Vc.any()
+    with pytest.raises(RuntimeError):
+        lib.qkv_rope_append(d1, dbq, dbk, dbv, K1, V1, Hq, Hkv, D, kv_max, kv_max, 1e6)
