@@ -80,8 +80,10 @@ class QwenGPU:
         self._keep = []
 
     @classmethod
-    def from_oracle(cls, om):
-        """Upload the very weight bytes an oracle model (tests/oraclelib.OracleQwen) holds."""
+    def from_blobs(cls, om):
+        """Build from a weight source: any object with `.d` (the dims) and
+        `.weight(layer, name)` returning the stored bytes of wq/wk/wv/wo/wg/wu/wd (q4
+        buffers), bq/bk/bv/an/fn (f32) and, for layer -1, embed (bf16), onorm, outw."""
         d = om.d
         g = cls(dict((f, getattr(d, f)) for f, _ in Dims._fields_))
         for li in range(d.n_layers):

@@ -30,7 +30,7 @@ def _near_tie(logits, rtol=1e-4, atol=1e-5):
 def test_decode_loop_matches_oracle(orc, dims, steps, fused):
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     om = orc.qwen_create(dims, seed=3, q4=True)
-    g = qwen.QwenGPU.from_oracle(om)
+    g = qwen.QwenGPU.from_blobs(om)
     g.set_fused(fused)
     rng = np.random.default_rng(5)
     tok = int(rng.integers(0, dims["vocab"]))
@@ -55,7 +55,7 @@ def test_graph_replay_equals_eager(orc):
     replays, reproduces the eager logits bit for bit every time."""
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     om = orc.qwen_create(SMALL, seed=4, q4=True)
-    g = qwen.QwenGPU.from_oracle(om)
+    g = qwen.QwenGPU.from_blobs(om)
     for pos in range(20):
         g.step(7 + pos, pos)
     pos, tok = 20, 123
