@@ -53,12 +53,18 @@ __device__ __forceinline__ float row16_sum(float v) {
 // A wavefront works on tiles of TK keys (16, 32 or 64): 4 keys per load step
 // (one per DPP row), each lane holding EPL = D/16 consecutive floats of its key.
 // part_m/part_l: [Hq*S], part_acc: [Hq*S*D]; used when S > 1, else `out` is final.
-template <int D, int G, typename KT>
+//
+// PRE = true is causal prefill over q/out [Hq, T, D]: grid = (Hq, 1, ceil(T/G)),
+// and the G rows of a block are G consecutive query positions of ONE head, which
+// share the K/V stream exactly like the query heads of a GQA group do in decode.
+// Row g of tile z sees keys [0, pos0 + z*G + g]; later keys of the tile are
+// masked per row. Tiles run longest-first. S is 1.
+template <int D, int G, typename KT, bool PRE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
     float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
     float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, int TK,
-    float scale, int S) {
+    float scale, int S, int T, int pos0) {
   constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
   constexpr int NV = EPL / 4;        // float4 loads per lane per key
   constexpr int UNR = 4;             // key steps in flight per lane
@@ -68,13 +74,29 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int slot = lane >> 4, c = lane & 15;     // DPP row = key slot, c = position in the row
-  const int kvh = blockIdx.x, split = blockIdx.y;
-  const int g0 = blockIdx.z * G;
-  const int ng = min(G, group - g0);
-  const int h0 = kvh * group + g0;
+  const int split = blockIdx.y;
+  int kvh, g0, ng, k_begin, k_end;
+  size_t row0;                                   // index of row g = 0 in q / out, in rows of D
+  if constexpr (PRE) {
+    const int h = blockIdx.x;
+    kvh = h / group;
+    g0 = (gridDim.z - 1 - blockIdx.z) * G;       // first query position of the tile
+    ng = min(G, T - g0);
+    row0 = (size_t)h * T + g0;
+    k_begin = 0;
+    k_end = pos0 + g0 + ng;                      // the last row's limit
+    TK = k_end >= 256 ? 64 : k_end >= 128 ? 32 : 16;
+  } else {
+    kvh = blockIdx.x;
+    g0 = blockIdx.z * G;
+    ng = min(G, group - g0);
+    row0 = (size_t)kvh * group + g0;
+    k_begin = split * chunk;
+    k_end = min(ctx, k_begin + chunk);
+  }
+  const int lim0 = pos0 + g0 + 1;                // PRE: row g sees keys < lim0 + g
   const KT* Kh = K + (size_t)kvh * kv_stride;
   const KT* Vh = V + (size_t)kvh * kv_stride;
-  const int k_begin = split * chunk, k_end = min(ctx, k_begin + chunk);
   const int steps = TK >> 2;                     // load steps per tile
 
   float4 qv[G][NV];
@@ -82,7 +104,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int g = 0; g < G; g++)
 #pragma unroll
     for (int v = 0; v < NV; v++)
-      qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (size_t)(h0 + g) * D + c * EPL + v * 4)
+      qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (row0 + g) * D + c * EPL + v * 4)
                         : make_float4(0.f, 0.f, 0.f, 0.f);
   float m[G], l[G];
   float4 acc[G][NV];
@@ -125,17 +147,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
             p = fmaf(qv[g][NV - 1].w, kv[u][NV - 1].w, p);
           }
           p = row16_sum(p);
-          if (c == i0 + u) sreg[g] = key < k_end ? p * scale : -INFINITY;
+          if (c == i0 + u) sreg[g] = key < (PRE ? min(k_end, lim0 + g) : k_end) ? p * scale : -INFINITY;
         }
       }
     }
     // ---- online softmax update for the tile ---------------------------------------
 #pragma unroll
     for (int g = 0; g < G; g++) {
-      const float tmax = wave_max(sreg[g]);      // finite: the tile holds >= 1 live key
+      const float tmax = wave_max(sreg[g]);      // decode: finite, the tile holds >= 1 live key
       const float mnew = fmaxf(m[g], tmax);
-      const float corr = __expf(m[g] - mnew);    // 0 on the first tile (m = -inf)
-      const float p = __expf(sreg[g] - mnew);    // 0 for masked keys and idle lanes
+      // prefill: a row may have seen no key yet (mnew = -inf); keep exp() away from inf - inf
+      const float mref = (PRE && mnew == -INFINITY) ? 0.f : mnew;
+      const float corr = __expf(m[g] - mref);    // 0 on the first tile (m = -inf)
+      const float p = __expf(sreg[g] - mref);    // 0 for masked keys and idle lanes
       l[g] = fmaf(l[g], corr, p);
 #pragma unroll
       for (int v = 0; v < NV; v++) {
@@ -205,11 +229,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       L = fmaf(st_l[w][g], f, L);
       A = fmaf(st_acc[w][g][d], f, A);
     }
-    const int h = h0 + g;
-    if (S == 1) {
-      out[(size_t)h * D + d] = A / L;
+    const size_t h = row0 + g;
+    if (PRE || S == 1) {
+      out[h * D + d] = A / L;
     } else {
-      const size_t ps = (size_t)h * S + split;
+      const size_t ps = h * S + split;
       part_acc[ps * D + d] = A;
       if (d == 0) { part_m[ps] = M; part_l[ps] = L; }
     }
@@ -309,8 +333,8 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
   const dim3 grid(Hkv, p.S, p.gz), block(p.nw * 64);
   const int64_t kv_stride = kv_max * D;
 #define TLHIP_ATTN(GG)                                                                         \
-  hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT>), grid, block, 0, c.stream, q, K, V, out, \
-                     pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S)
+  hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false>), grid, block, 0, c.stream, q, K, V, \
+                     out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0)
   switch (p.G) {
     case 1: TLHIP_ATTN(1); break;
     case 2: TLHIP_ATTN(2); break;
@@ -322,6 +346,18 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(256), (size_t)(p.S + 256) * sizeof(float),
                        c.stream, pm, pl, pacc, out, p.S, D);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
+}
+
+template <int D, typename KT>
+static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
+                          int T, int64_t kv_max, float scale, int pos0) {
+  Context& c = tlhip::ctx();
+  constexpr int G = 8;   // query positions per block
+  const dim3 grid(Hq, 1, (T + G - 1) / G), block(256);
+  hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
+                     (float*)nullptr, (float*)nullptr, (float*)nullptr, Hq / Hkv, pos0 + T,
+                     kv_max * D, 0, 64, scale, 1, T, pos0);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
 }
 
 }  // namespace tlhip
@@ -357,6 +393,36 @@ int tlhip_attn_decode(const void* q, const void* K, const void* V, void* out, in
   const float* pv = static_cast<const float*>(V);
   return D == 128 ? launch_attn<128, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale)
                   : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale);
+}
+
+int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                       int64_t n_kv_heads, int64_t T, int64_t kv_max, int64_t D, float scale,
+                       int kv_bf16, int64_t pos0) {
+  TLHIP_REQUIRE_READY();
+  if (!q || !K || !V || !out) return fail(TLHIP_EINVAL, "tlhip_attn_prefill: null pointer");
+  // the reference's gates (cuda.h:1171-1177)
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: head_dim must be 64 or 128");
+  if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: Hq must be a positive multiple of Hkv");
+  if (T <= 0 || T > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: need 0 < T <= 65535");
+  if (pos0 < 0 || pos0 + T > kv_max) return fail(TLHIP_EINVAL, "tlhip_attn_prefill: need 0 <= pos0, pos0 + T <= kv_max");
+  if (kv_max > 0x3fffffff || n_q_heads > 0x7fffffff || kv_max * D > ((int64_t)1 << 40))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: shape too large");
+  if (!aligned16(q) || !aligned16(K) || !aligned16(V) || !aligned16(out))
+    return fail(TLHIP_EINVAL, "tlhip_attn_prefill: operands must be 16-byte aligned");
+  const float* pq = static_cast<const float*>(q);
+  float* po = static_cast<float*>(out);
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads, t = (int)T, p0 = (int)pos0;
+  if (kv_bf16) {
+    const uint16_t* pk = static_cast<const uint16_t*>(K);
+    const uint16_t* pv = static_cast<const uint16_t*>(V);
+    return D == 128 ? launch_prefill<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0)
+                    : launch_prefill<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0);
+  }
+  const float* pk = static_cast<const float*>(K);
+  const float* pv = static_cast<const float*>(V);
+  return D == 128 ? launch_prefill<128, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0)
+                  : launch_prefill<64, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0);
 }
 
 }  // extern "C"

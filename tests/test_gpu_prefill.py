@@ -1,0 +1,209 @@
+"""GPU parity: the prefill pair (MFMA GEMM against bf16 weights, causal attention over a
+cache) through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+from oraclelib import allclose, maxrel
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _gemm(lib, A, Wb):
+    M, K = A.shape
+    N = Wb.shape[0]
+    da, dw, dc = lib.to_device(A), lib.to_device(Wb), lib.empty((M, N))
+    lib.gemm_bf16_nt(da, dw, dc, M, N, K)
+    out = dc.numpy()
+    for b in (da, dw, dc):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (512, 512, 3584),      # a prompt chunk against a kv-sized projection: 64x64 tiles
+    (512, 4608, 896),      # 64x128 tiles
+    (1024, 4864, 896),     # 128x128 tiles
+    (128, 1152, 896),      # 0.5B fused q|k|v
+    (33, 200, 40),         # ragged in M, N and K (K % 32 != 0)
+    (1, 64, 8),            # smallest legal
+    (257, 129, 264),
+])
+def test_gemm_bf16_nt_matches_oracle(lib, orc, M, N, K):
+    """out[M,N] = A[M,K] . W[N,K]^T, W bf16 (cuda.h:786-840). Weights N(0,0.02) as in the
+    decode model, A ~ N(0,1)."""
+    print("case gemm_bf16_nt", M, N, K, flush=True)
+    A = orc.normal(M * K, 11).reshape(M, K)
+    Wb = orc.to_bf16(orc.normal(N * K, 12, std=0.02)).reshape(N, K)
+    before = lib.census()["gemm_bf16_nt"]
+    got = _gemm(lib, A, Wb)
+    assert lib.census()["gemm_bf16_nt"] == before + 1
+    want = orc.gemm_bf16_nt(A, Wb)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_gemm_bf16_nt_exact_cases(lib, orc):
+    """What the arithmetic fixes without an oracle: the three-way bf16 split of A loses
+    nothing, so integer-valued operands give exact integers, and a one-hot A row copies
+    a weight column out bit for bit (a transposed operand or a wrong accumulator lane
+    map fails here)."""
+    M, N, K = 96, 160, 64
+    rng = np.random.default_rng(5)
+    A = rng.integers(-500, 500, (M, K)).astype(np.float32) + 0.5   # needs > 8 mantissa bits
+    Wf = rng.integers(-64, 64, (N, K)).astype(np.float32)
+    Wb = orc.to_bf16(Wf).reshape(N, K)
+    got = _gemm(lib, A, Wb)
+    want = (A.astype(np.float64) @ Wf.astype(np.float64).T)
+    assert np.array_equal(got.astype(np.float64), want)
+    # one-hot rows: out[m, n] == W[n, m % K]
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), np.arange(M) % K] = 1.0
+    Wf = orc.bf16_widen(orc.to_bf16(orc.normal(N * K, 3))).reshape(N, K)
+    got = _gemm(lib, A, orc.to_bf16(Wf).reshape(N, K))
+    assert np.array_equal(got, Wf[:, np.arange(M) % K].T)
+    # 24-bit mantissas survive: a = 1 + 2^-23, w = 1 -> the sum of K copies is exact in f32
+    A = np.full((32, 8), np.float32(1.0) + np.float32(2.0 ** -23), np.float32)
+    got = _gemm(lib, A, orc.to_bf16(np.ones((32, 8), np.float32)).reshape(32, 8))
+    assert np.all(got == np.float32(8.0 * (1.0 + 2.0 ** -23)))
+
+
+def test_gemm_bf16_nt_row_equals_gemv(lib, orc):
+    """Row m of the GEMM and the decode GEMV over the same [N,K] bf16 weights agree to
+    summation-order noise."""
+    M, N, K = 8, 1024, 896
+    A = orc.normal(M * K, 21).reshape(M, K)
+    Wb = orc.to_bf16(orc.normal(N * K, 22, std=0.02)).reshape(N, K)
+    got = _gemm(lib, A, Wb)
+    dw, dy = lib.to_device(Wb), lib.empty(N)
+    for m in (0, 7):
+        da = lib.to_device(A[m])
+        lib.gemv_bf16_row(da, dw, dy, N, K)
+        assert allclose(got[m], dy.numpy(), RTOL, ATOL)
+        da.free()
+    dw.free(), dy.free()
+
+
+def test_gemm_bf16_nt_declines(lib):
+    from importlib import import_module
+    err = import_module("cpp-tensorlib_amd.capi").TlHipError
+    a, w, c = lib.empty((4, 12)), lib.empty((4, 12), np.uint16), lib.empty((4, 4))
+    with pytest.raises(err):
+        lib.gemm_bf16_nt(a, w, c, 4, 4, 12)      # K % 8 != 0
+    for b in (a, w, c):
+        b.free()
+
+
+def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False):
+    Hq, T, D = q.shape
+    Hkv, kv_max, _ = K.shape
+    dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, T, D))
+    lib.attn_prefill(dq, dk, dv, do, Hq, Hkv, T, kv_max, D, scale, kv_bf16, pos0)
+    out = do.numpy()
+    for b in (dq, dk, dv, do):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("D,Hq,Hkv,T,pos0", [
+    (128, 28, 4, 64, 0), (64, 14, 2, 100, 0), (128, 4, 2, 7, 0), (128, 8, 8, 33, 300),
+    (64, 6, 2, 257, 19), (128, 2, 1, 1, 0), (128, 2, 1, 1, 77), (64, 4, 4, 130, 513),
+])
+def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0):
+    """Causal prefill over a cache: query p at absolute position pos0+p sees keys
+    0..pos0+p (cuda.h:1165-1200). Rows past pos0+T hold poison that must not leak; so
+    must, per query, the chunk's own later keys."""
+    print("case attn_prefill", D, Hq, Hkv, T, pos0, flush=True)
+    kv_max = pos0 + T + 5
+    q = orc.normal(Hq * T * D, 31).reshape(Hq, T, D)
+    K = orc.normal(Hkv * kv_max * D, 32).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 33).reshape(Hkv, kv_max, D)
+    K[:, pos0 + T:, :] = 1e30
+    V[:, pos0 + T:, :] = np.nan
+    scale = 1.0 / np.sqrt(float(D))
+    got = _prefill(lib, q, K, V, scale, pos0)
+    want = orc.attn_prefill(q, K, V, scale, pos0)
+    assert np.all(np.isfinite(got))
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_attn_prefill_rows_equal_decode(lib, orc):
+    """Row p of a prefill equals a decode step with ctx = pos0 + p + 1 (the equivalence the
+    reference's prefill bench relies on, bench_qwen_prefill.cpp:283-310), and the first query
+    of a fresh cache returns V[0] exactly."""
+    D, Hq, Hkv, T, pos0 = 128, 8, 2, 40, 24
+    kv_max = pos0 + T
+    q = orc.normal(Hq * T * D, 41).reshape(Hq, T, D)
+    K = orc.normal(Hkv * kv_max * D, 42).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 43).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    got = _prefill(lib, q, K, V, scale, pos0)
+    dk, dv, do = lib.to_device(K), lib.to_device(V), lib.empty((Hq, D))
+    for p in (0, 1, 17, T - 1):
+        dq = lib.to_device(np.ascontiguousarray(q[:, p, :]))
+        lib.attn_decode(dq, dk, dv, do, Hq, Hkv, pos0 + p + 1, kv_max, D, scale)
+        assert allclose(got[:, p, :], do.numpy(), RTOL, ATOL)
+        dq.free()
+    for b in (dk, dv, do):
+        b.free()
+    fresh = _prefill(lib, q, K, V, scale, 0)
+    assert np.array_equal(fresh[:, 0, :], np.repeat(V[:, 0, :], Hq // Hkv, axis=0))
+
+
+def test_attn_prefill_bf16_cache(lib, orc):
+    D, Hq, Hkv, T, pos0 = 128, 4, 2, 70, 10
+    kv_max = pos0 + T
+    q = orc.normal(Hq * T * D, 51).reshape(Hq, T, D)
+    Kb = orc.to_bf16(orc.normal(Hkv * kv_max * D, 52)).reshape(Hkv, kv_max, D)
+    Vb = orc.to_bf16(orc.normal(Hkv * kv_max * D, 53)).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    got = _prefill(lib, q, Kb, Vb, scale, pos0, kv_bf16=True)
+    want = orc.attn_prefill(q, orc.bf16_widen(Kb).reshape(Kb.shape),
+                            orc.bf16_widen(Vb).reshape(Vb.shape), scale, pos0)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+def test_prefill_chunk_pipeline(lib, orc):
+    """The attention half of a prompt chunk as the reference harness runs it
+    (bench/cuda/qwen_model.h:357-383): fused q|k|v GEMM -> split_heads (+bias) -> rope at pos0
+    -> kv_fill -> attn_prefill -> merge_heads, against the same chain in the oracle."""
+    D, Hq, Hkv, T, pos0, H = 64, 4, 2, 24, 8, 256
+    kv_max = 64
+    qd, kvd = Hq * D, Hkv * D
+    x = orc.normal(T * H, 61).reshape(T, H)
+    Wb = orc.to_bf16(orc.normal((qd + 2 * kvd) * H, 62, std=0.05)).reshape(qd + 2 * kvd, H)
+    bias = orc.normal(qd + 2 * kvd, 63, std=0.1)
+    Kc = orc.normal(Hkv * kv_max * D, 64).reshape(Hkv, kv_max, D)
+    Vc = orc.normal(Hkv * kv_max * D, 65).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    # oracle chain
+    qkv = orc.gemm_bf16_nt(x, Wb) + bias[None, :]
+    def heads(off, Hn):
+        return np.ascontiguousarray(qkv[:, off:off + Hn * D].reshape(T, Hn, D).transpose(1, 0, 2))
+    qh = orc.rope(heads(0, Hq), pos0, 1e6, T=T)
+    kh = orc.rope(heads(qd, Hkv), pos0, 1e6, T=T)
+    vh = heads(qd + kvd, Hkv)
+    Kw, Vw = Kc.copy(), Vc.copy()
+    Kw[:, pos0:pos0 + T] = kh
+    Vw[:, pos0:pos0 + T] = vh
+    want = orc.attn_prefill(qh, Kw, Vw, scale, pos0).transpose(1, 0, 2).reshape(T, qd)
+    # device chain
+    dx, dw = lib.to_device(x), lib.to_device(Wb)
+    dbq, dbk, dbv = (lib.to_device(bias[:qd]), lib.to_device(bias[qd:qd + kvd]),
+                     lib.to_device(bias[qd + kvd:]))
+    dqkv = lib.empty((T, qd + 2 * kvd))
+    dq, dk, dv = lib.empty((Hq, T, D)), lib.empty((Hkv, T, D)), lib.empty((Hkv, T, D))
+    dKc, dVc = lib.to_device(Kc), lib.to_device(Vc)
+    dah, dat = lib.empty((Hq, T, D)), lib.empty((T, qd))
+    lib.gemm_bf16_nt(dx, dw, dqkv, T, qd + 2 * kvd, H)
+    lib.split_heads(dqkv, dbq, dq, T, qd + 2 * kvd, 0, Hq, D)
+    lib.split_heads(dqkv, dbk, dk, T, qd + 2 * kvd, qd, Hkv, D)
+    lib.split_heads(dqkv, dbv, dv, T, qd + 2 * kvd, qd + kvd, Hkv, D)
+    lib.rope(dq, dq, Hq * T, T, D, pos0, 1e6)
+    lib.rope(dk, dk, Hkv * T, T, D, pos0, 1e6)
+    lib.kv_fill(dKc, dVc, dk, dv, T, kv_max, Hkv, D, False, pos0)
+    lib.attn_prefill(dq, dKc, dVc, dah, Hq, Hkv, T, kv_max, D, scale, False, pos0)
+    lib.merge_heads(dah, dat, T, Hq, D)
+    got = dat.numpy()
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    for b in (dx, dw, dbq, dbk, dbv, dqkv, dq, dk, dv, dKc, dVc, dah, dat):
+        b.free()
