@@ -18,6 +18,7 @@
 // fragment. Global loads of the next slab are in flight while the current one is
 // multiplied.
 #include "common.hpp"
+#include <cstdlib>
 
 namespace tlhip {
 
@@ -28,7 +29,7 @@ constexpr int kBK = 32;        // K slab
 constexpr int kLDK = kBK + 8;  // LDS row pitch in bf16 (80 B: 16-byte aligned, spreads banks)
 
 template <int TM, int TN>
-__global__ __launch_bounds__(256) void gemm_bf16_nt_kernel(const float* __restrict__ A,
+__global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
                                                            int K) {
@@ -40,7 +41,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_nt_kernel(const float* __restri
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // Block order. Hardware deals consecutive block ids round-robin to the 8 XCDs,
+  // each with a private L2. Give every XCD one contiguous run of tiles, M fastest,
+  // so the blocks that share a weight tile run together on one L2 and W is
+  // streamed from HBM once.
+  const int mt = (M + BM - 1) / BM;
+  const int nb = gridDim.x, xcd = blockIdx.x & 7, within = blockIdx.x >> 3;
+  const int q8 = nb >> 3, r8 = nb & 7;
+  const int lid = xcd * q8 + min(xcd, r8) + within;
+  const int m0 = (lid % mt) * BM, n0 = (lid / mt) * BN;
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -165,9 +174,15 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
   if (blocks(128, 128) >= want) { tm = 2; tn = 2; }
   else if (blocks(64, 128) >= want) { tm = 1; tn = 2; }
   else { tm = 1; tn = 1; }
-  const dim3 grid((unsigned)((N + 64 * tn - 1) / (64 * tn)), (unsigned)((M + 64 * tm - 1) / (64 * tm)));
-  if (grid.y > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: M too large for the grid");
-  if (tm == 2)
+  if (const char* e = getenv("TLHIP_GEMM_TILE")) { tm = e[0] - '0'; tn = e[1] - '0'; }
+  const int64_t nblk = ((N + 64 * tn - 1) / (64 * tn)) * ((M + 64 * tm - 1) / (64 * tm));
+  if (nblk > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
+  const dim3 grid((unsigned)nblk);
+  if (tm == 2 && tn == 4)
+    gemm_bf16_nt_kernel<2, 4><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
+  else if (tm == 1 && tn == 4)
+    gemm_bf16_nt_kernel<1, 4><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
+  else if (tm == 2)
     gemm_bf16_nt_kernel<2, 2><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
   else if (tn == 2)
     gemm_bf16_nt_kernel<1, 2><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);

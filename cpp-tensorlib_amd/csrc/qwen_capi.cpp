@@ -53,6 +53,46 @@ int tlq_set_random_q4(void* hv, uint32_t seed) {
   return qwen::set_random_q4(static_cast<handle*>(hv)->M, seed) ? 0 : -1;
 }
 
+// The same from bf16 blobs in the logical [K,N] layout.
+int tlq_set_layer_bf16(void* hv, int64_t li, const uint16_t* wq, const uint16_t* wk,
+                       const uint16_t* wv, const uint16_t* wo, const uint16_t* wg, const uint16_t* wu,
+                       const uint16_t* wd, const float* bq, const float* bk, const float* bv,
+                       const float* an, const float* fn) {
+  auto* h = static_cast<handle*>(hv);
+  qwen::layer_blobs_bf16 b{wq, wk, wv, wo, wg, wu, wd, bq, bk, bv, an, fn};
+  return qwen::set_layer_bf16(h->M, li, b) ? 0 : -1;
+}
+
+int tlq_set_head_bf16(void* hv, const uint16_t* embed, const float* onorm, const uint16_t* outw) {
+  return qwen::set_head_bf16(static_cast<handle*>(hv)->M, embed, onorm, outw) ? 0 : -1;
+}
+
+int tlq_set_random_bf16(void* hv, uint32_t seed) {
+  return qwen::set_random_bf16(static_cast<handle*>(hv)->M, seed) ? 0 : -1;
+}
+
+// Consume n prompt tokens in chunks, appending to the caches at their current
+// position; logits_out (may be NULL) receives the last token's [vocab] logits.
+int tlq_prefill(void* hv, const int64_t* tokens, int64_t n, int64_t chunk, float* logits_out) {
+  auto* h = static_cast<handle*>(hv);
+  if (!qwen::prefill(h->M, tokens, n, chunk)) return -1;
+  if (logits_out)
+    std::memcpy(logits_out, qwen::logits(h->M), (size_t)h->M.d.vocab * sizeof(float));
+  return 0;
+}
+
+// Throughput form: stage one chunk, then enqueue its layers with the caches
+// rewound to pos0, no lm_head and no sync.
+int tlq_stage_chunk(void* hv, const int64_t* tokens, int64_t T) {
+  return qwen::stage_chunk(static_cast<handle*>(hv)->M, tokens, T) ? 0 : -1;
+}
+int tlq_prefill_layers(void* hv, int64_t T, int64_t pos0) {
+  auto* h = static_cast<handle*>(hv);
+  qwen::set_cache_pos(h->M, pos0);
+  return qwen::prefill_layers(h->M, T) ? 0 : -1;
+}
+void tlq_set_cache_pos(void* hv, int64_t pos) { qwen::set_cache_pos(static_cast<handle*>(hv)->M, pos); }
+
 int tlq_fill_cache_random(void* hv, int64_t upto, uint32_t seed) {
   return qwen::fill_cache_random(static_cast<handle*>(hv)->M, upto, seed) ? 0 : -1;
 }

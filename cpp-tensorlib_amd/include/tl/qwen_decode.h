@@ -14,6 +14,12 @@
 //   -> swiglu -> down GEMV -> rmsnorm_res (x2 = x1 + mlp ; next layer's input norm)
 // then the lm_head GEMV and a device argmax whose 4-byte copy is the single
 // blocking call of the step.
+//
+// A prompt is consumed in chunks of T tokens (prefill_chunk, the counterpart of
+// qm:357-395): the same layer wiring with every GEMV replaced by the MFMA GEMM
+// over [T, hidden] activations, split_heads/rope/kv_fill/attn_prefill/merge_heads
+// around the cache, and multi-row norms. Like the reference's, it needs bf16
+// row-major weights.
 
 #include <algorithm>
 #include <cmath>
@@ -65,7 +71,8 @@ inline bool gemv(const linear& L, void* a, void* y) {
 
 struct layer {
   linear wqkv, wo, wgu, wd;          // fused [wq|wk|wv] and [wg|wu] (qm:188-199)
-  void *bq = nullptr, *bk = nullptr, *bv = nullptr;  // [q_dim], [kv_dim], [kv_dim]
+  void* bqkv = nullptr;                              // fused bias [q_dim + 2 kv_dim] (qm:196)
+  void *bq = nullptr, *bk = nullptr, *bv = nullptr;  // its three parts
   void *an = nullptr, *fn = nullptr;                 // attention / ffn norm weights [hidden]
   hip::kv_cache cache;
 };
@@ -79,8 +86,18 @@ struct scratch {
   float* logits_host = nullptr;
 };
 
+// Intermediates of a prompt chunk of up to T rows (qm:248-283), allocated on first use.
+struct prefill_scratch {
+  int64_t T = 0;
+  void *emb = nullptr, *h = nullptr, *h2 = nullptr, *qkv = nullptr, *qkvh = nullptr, *ah = nullptr,
+       *at = nullptr, *gu = nullptr, *mb = nullptr, *md = nullptr;
+  void* res[2] = {nullptr, nullptr};
+  float* emb_host = nullptr;
+};
+
 struct model {
   dims d{};
+  prefill_scratch ps;
   std::vector<uint16_t> embed;  // bf16 [vocab, hidden], gathered on the host (qm:530-535)
   void* onorm = nullptr;
   linear lm_head;
@@ -120,6 +137,12 @@ inline std::vector<uint8_t> fuse_q4(const std::vector<const uint8_t*>& parts,
   return out;
 }
 
+// [K,N] -> [N,K]
+inline void transpose_kn(const uint16_t* src, uint16_t* dst, int64_t K, int64_t N) {
+  for (int64_t k = 0; k < K; k++)
+    for (int64_t n = 0; n < N; n++) dst[n * K + k] = src[k * N + n];
+}
+
 }  // namespace detail
 
 // Host-side description of one layer's weights in the reference's storage
@@ -128,6 +151,26 @@ struct layer_blobs {
   const uint8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
   const float *bq, *bk, *bv, *an, *fn;
 };
+
+namespace detail {
+// Biases (one fused buffer, as the prefill path wants it) and norm weights.
+inline bool set_vectors(model& M, layer& L, const float* bq, const float* bk, const float* bv,
+                        const float* an, const float* fn) {
+  const dims& d = M.d;
+  std::vector<float> fused((size_t)d.qkv_dim());
+  std::memcpy(fused.data(), bq, (size_t)d.q_dim() * 4);
+  std::memcpy(fused.data() + d.q_dim(), bk, (size_t)d.kv_dim() * 4);
+  std::memcpy(fused.data() + d.q_dim() + d.kv_dim(), bv, (size_t)d.kv_dim() * 4);
+  L.bqkv = dev_from_host(fused.data(), d.qkv_dim() * 4);
+  if (!L.bqkv) return false;
+  L.bq = L.bqkv;
+  L.bk = static_cast<char*>(L.bqkv) + d.q_dim() * 4;
+  L.bv = static_cast<char*>(L.bqkv) + (d.q_dim() + d.kv_dim()) * 4;
+  L.an = dev_from_host(an, d.hidden * 4);
+  L.fn = dev_from_host(fn, d.hidden * 4);
+  return L.an && L.fn;
+}
+}  // namespace detail
 
 inline bool init(model& M, const dims& d) {
   if (!hip::available()) return false;
@@ -163,12 +206,53 @@ inline bool set_layer_q4(model& M, int64_t li, const layer_blobs& b) {
                  wfmt::q4};
   L.wo = linear{detail::dev_from_host(b.wo, q4_bytes(E, d.q_dim())), E, d.q_dim(), wfmt::q4};
   L.wd = linear{detail::dev_from_host(b.wd, q4_bytes(E, d.ff)), E, d.ff, wfmt::q4};
-  L.bq = detail::dev_from_host(b.bq, d.q_dim() * 4);
-  L.bk = detail::dev_from_host(b.bk, d.kv_dim() * 4);
-  L.bv = detail::dev_from_host(b.bv, d.kv_dim() * 4);
-  L.an = detail::dev_from_host(b.an, E * 4);
-  L.fn = detail::dev_from_host(b.fn, E * 4);
-  return L.wqkv.w && L.wgu.w && L.wo.w && L.wd.w && L.bq && L.bk && L.bv && L.an && L.fn;
+  return detail::set_vectors(M, L, b.bq, b.bk, b.bv, b.an, b.fn) && L.wqkv.w && L.wgu.w && L.wo.w &&
+         L.wd.w;
+}
+
+// The same layer from bf16 blobs in the reference's logical [K,N] layout
+// (array.h:639-658): transposed on the host to [N,K] rows, the layout the decode
+// GEMV and the prefill GEMM share (qm:118-146 does this transpose at load).
+struct layer_blobs_bf16 {
+  const uint16_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
+  const float *bq, *bk, *bv, *an, *fn;
+};
+
+inline bool set_layer_bf16(model& M, int64_t li, const layer_blobs_bf16& b) {
+  const dims& d = M.d;
+  layer& L = M.layers[(size_t)li];
+  const int64_t E = d.hidden;
+  std::vector<uint16_t> rows;
+  auto put = [&](std::vector<const uint16_t*> parts, std::vector<int64_t> Ns, int64_t K) {
+    int64_t N = 0;
+    for (auto n : Ns) N += n;
+    rows.resize((size_t)(N * K));
+    int64_t n0 = 0;
+    for (size_t i = 0; i < parts.size(); i++) {
+      detail::transpose_kn(parts[i], rows.data() + n0 * K, K, Ns[i]);
+      n0 += Ns[i];
+    }
+    return linear{detail::dev_from_host(rows.data(), N * K * 2), N, K, wfmt::bf16_row};
+  };
+  L.wqkv = put({b.wq, b.wk, b.wv}, {d.q_dim(), d.kv_dim(), d.kv_dim()}, E);
+  L.wgu = put({b.wg, b.wu}, {d.ff, d.ff}, E);
+  L.wo = put({b.wo}, {E}, d.q_dim());
+  L.wd = put({b.wd}, {E}, d.ff);
+  return detail::set_vectors(M, L, b.bq, b.bk, b.bv, b.an, b.fn) && L.wqkv.w && L.wgu.w && L.wo.w &&
+         L.wd.w;
+}
+
+inline bool set_head_bf16(model& M, const uint16_t* embed_bf16, const float* onorm,
+                          const uint16_t* outw_kn) {
+  const dims& d = M.d;
+  M.embed.assign(embed_bf16, embed_bf16 + d.vocab * d.hidden);
+  M.onorm = detail::dev_from_host(onorm, d.hidden * 4);
+  std::vector<uint16_t> rows((size_t)(d.vocab * d.hidden));
+  detail::transpose_kn(outw_kn, rows.data(), d.hidden, d.vocab);
+  M.lm_head = linear{detail::dev_from_host(rows.data(), d.vocab * d.hidden * 2), d.vocab, d.hidden,
+                     wfmt::bf16_row};
+  M.ready = M.onorm && M.lm_head.w;
+  return M.ready;
 }
 
 inline bool set_head_q4(model& M, const uint16_t* embed_bf16, const float* onorm,
@@ -186,7 +270,7 @@ inline bool set_head_q4(model& M, const uint16_t* embed_bf16, const float* onorm
 // one 32 MB block of seeded random nibbles and one of scales ~U(0.002,0.006) are
 // uploaded once and tiled into device-only weight buffers with device copies.
 // Values do not affect kernel time; they keep activations finite.
-inline bool set_random_q4(model& M, uint32_t seed) {
+inline bool set_random(model& M, uint32_t seed, wfmt fmt) {
   const dims& d = M.d;
   const int64_t blk = int64_t(32) << 20;
   std::vector<uint32_t> nib((size_t)blk / 4);
@@ -199,7 +283,19 @@ inline bool set_random_q4(model& M, uint32_t seed) {
   void* ds = detail::dev_from_host(scl.data(), blk);
   if (!dn || !ds) return false;
   bool ok = true;
+  // bf16: the scale block doubles as the weight pattern once its exponent bits are
+  // pinned to [2^-7, 2^-6) with random sign, so |w| ~ 0.01
+  std::vector<uint32_t> bfw((size_t)blk / 4);
+  for (auto& v : bfw) v = (next() & 0x807f807fu) | 0x3c003c00u;
+  void* db = fmt == wfmt::bf16_row ? detail::dev_from_host(bfw.data(), blk) : nullptr;
   auto make = [&](int64_t N, int64_t K) {
+    if (fmt == wfmt::bf16_row) {
+      linear L{hip::alloc_device(N * K * 2), N, K, wfmt::bf16_row};
+      if (!L.w || !db) { ok = false; return L; }
+      for (int64_t o = 0; o < N * K * 2; o += blk)
+        ok &= hip::copy_d2d(static_cast<char*>(L.w) + o, db, std::min(blk, N * K * 2 - o));
+      return L;
+    }
     linear L{hip::alloc_device(q4_bytes(N, K)), N, K, wfmt::q4};
     if (!L.w) { ok = false; return L; }
     const int64_t pb = N * K / 2, sb = N * (K / kQ4Group) * 4;
@@ -209,25 +305,23 @@ inline bool set_random_q4(model& M, uint32_t seed) {
       ok &= hip::copy_d2d(static_cast<char*>(L.w) + pb + o, ds, std::min(blk, sb - o));
     return L;
   };
-  auto vec = [&](int64_t n, float mean, float std_) {
+  auto hvec = [&](int64_t n, float mean, float std_) {
     std::vector<float> v((size_t)n);
     for (auto& e : v) e = mean + std_ * ((float)(int32_t)next() * (1.0f / 2147483648.0f));
-    return detail::dev_from_host(v.data(), n * 4);
+    return v;
   };
   for (auto& L : M.layers) {
     L.wqkv = make(d.qkv_dim(), d.hidden);
     L.wo = make(d.hidden, d.q_dim());
     L.wgu = make(2 * d.ff, d.hidden);
     L.wd = make(d.hidden, d.ff);
-    L.bq = vec(d.q_dim(), 0.f, 0.02f);
-    L.bk = vec(d.kv_dim(), 0.f, 0.02f);
-    L.bv = vec(d.kv_dim(), 0.f, 0.02f);
-    L.an = vec(d.hidden, 1.f, 0.02f);
-    L.fn = vec(d.hidden, 1.f, 0.02f);
-    ok = ok && L.bq && L.bk && L.bv && L.an && L.fn;
+    const auto bq = hvec(d.q_dim(), 0.f, 0.02f), bk = hvec(d.kv_dim(), 0.f, 0.02f),
+               bv = hvec(d.kv_dim(), 0.f, 0.02f), an = hvec(d.hidden, 1.f, 0.02f),
+               fn = hvec(d.hidden, 1.f, 0.02f);
+    ok = ok && detail::set_vectors(M, L, bq.data(), bk.data(), bv.data(), an.data(), fn.data());
   }
   M.lm_head = make(d.vocab, d.hidden);
-  M.onorm = vec(d.hidden, 1.f, 0.02f);
+  M.onorm = detail::dev_from_host(hvec(d.hidden, 1.f, 0.02f).data(), d.hidden * 4);
   M.embed.resize((size_t)(d.vocab * d.hidden));
   for (size_t i = 0; i < M.embed.size(); i++)
     M.embed[i] = f32_to_bf16(0.02f * ((float)(int32_t)next() * (1.0f / 2147483648.0f)));
@@ -235,6 +329,8 @@ inline bool set_random_q4(model& M, uint32_t seed) {
   M.ready = ok && M.onorm;
   return M.ready;
 }
+inline bool set_random_q4(model& M, uint32_t seed) { return set_random(M, seed, wfmt::q4); }
+inline bool set_random_bf16(model& M, uint32_t seed) { return set_random(M, seed, wfmt::bf16_row); }
 
 // Fill every layer's cache rows [0, upto) with seeded N(0,1)-like values so a
 // decode step at a deep position reads a realistic cache.
@@ -332,6 +428,101 @@ inline int64_t step_greedy(model& M, int64_t token, int64_t pos) {
 inline const float* logits(model& M) {
   hip::sync_to_host(M.s.logitsb, false);
   return M.s.logits_host;
+}
+
+// ---- prompt chunks ---------------------------------------------------------------------------
+
+inline bool prefill_reserve(model& M, int64_t T) {
+  prefill_scratch& P = M.ps;
+  if (P.T >= T) return true;
+  const dims& d = M.d;
+  auto A = [](int64_t n) { return hip::alloc_device(n * 4); };
+  for (void* b : {P.emb, P.h, P.h2, P.qkv, P.qkvh, P.ah, P.at, P.gu, P.mb, P.md, P.res[0], P.res[1]})
+    if (b) hip::release(b, 0, nullptr);
+  P.emb = hip::alloc(T * d.hidden * 4, &P.emb_host);
+  P.h = A(T * d.hidden);
+  P.h2 = A(T * d.hidden);
+  P.qkv = A(T * d.qkv_dim());
+  P.qkvh = A(T * d.qkv_dim());
+  P.ah = A(T * d.q_dim());
+  P.at = A(T * d.q_dim());
+  P.gu = A(T * 2 * d.ff);
+  P.mb = A(T * d.ff);
+  P.md = A(T * d.hidden);
+  P.res[0] = A(T * d.hidden);
+  P.res[1] = A(T * d.hidden);
+  const bool ok = P.emb && P.h && P.h2 && P.qkv && P.qkvh && P.ah && P.at && P.gu && P.mb && P.md &&
+                  P.res[0] && P.res[1];
+  P.T = ok ? T : 0;
+  return ok;
+}
+
+// All layers over the T rows staged in ps.emb, appended to the caches at their
+// current position (qm:357-395). Leaves the final norm of every row in ps.h.
+inline bool prefill_layers(model& M, int64_t T) {
+  const dims& d = M.d;
+  prefill_scratch& P = M.ps;
+  if (T <= 0 || T > P.T) return false;
+  for (const layer& L : M.layers)
+    if (L.wqkv.fmt != wfmt::bf16_row) return false;  // the MFMA GEMM reads bf16 rows only
+  const float scale = 1.0f / std::sqrt((float)d.head_dim);
+  const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim(), QKVN = d.qkv_dim(), HD = d.head_dim;
+  const int64_t pos0 = M.layers[0].cache.pos;
+  bool ok = true;
+  void* x = P.emb;
+  ok &= hip::rmsnorm(x, M.layers[0].an, P.h, E, d.eps, T);
+  for (int64_t l = 0; l < d.n_layers; l++) {
+    layer& L = M.layers[(size_t)l];
+    void* ro = P.res[l & 1];
+    ok &= hip::gemm_bf16_nt(P.h, L.wqkv.w, P.qkv, T, QKVN, E);
+    // [T, q|k|v] -> head-major [Hq + 2 Hkv, T, D], bias added on the way
+    ok &= hip::split_heads(P.qkv, L.bqkv, P.qkvh, T, QKVN, 0, d.n_q_heads + 2 * d.n_kv_heads, HD);
+    void* kh = static_cast<char*>(P.qkvh) + QD * T * 4;
+    void* vh = static_cast<char*>(P.qkvh) + (QD + KD) * T * 4;
+    // row r = h*T + t, so rope's position pos0 + r % T is pos0 + t
+    ok &= hip::rope(P.qkvh, P.qkvh, d.n_q_heads * T, T, HD, pos0, d.rope_base);
+    ok &= hip::rope(kh, kh, d.n_kv_heads * T, T, HD, pos0, d.rope_base);
+    L.cache.pos = pos0;
+    ok &= L.cache.prefill(P.qkvh, kh, vh, P.ah, T, d.n_q_heads, scale);
+    ok &= hip::merge_heads(P.ah, P.at, T, d.n_q_heads, HD);
+    ok &= hip::gemm_bf16_nt(P.at, L.wo.w, ro, T, E, QD);
+    ok &= hip::rmsnorm_res(ro, x, L.fn, ro, P.h2, E, d.eps, T);
+    ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);
+    ok &= hip::swiglu(P.gu, P.mb, d.ff, T);
+    ok &= hip::gemm_bf16_nt(P.mb, L.wd.w, P.md, T, E, d.ff);
+    void* nextw = (l + 1 < d.n_layers) ? M.layers[(size_t)l + 1].an : M.onorm;
+    ok &= hip::rmsnorm_res(ro, P.md, nextw, ro, P.h, E, d.eps, T);
+    x = ro;
+  }
+  return ok;
+}
+
+// Gather T embedding rows on the host and upload them as the chunk input.
+inline bool stage_chunk(model& M, const int64_t* tokens, int64_t T) {
+  if (!prefill_reserve(M, T)) return false;
+  const dims& d = M.d;
+  for (int64_t t = 0; t < T; t++) {
+    const uint16_t* r = M.embed.data() + (size_t)tokens[t] * d.hidden;
+    float* o = M.ps.emb_host + t * d.hidden;
+    for (int64_t j = 0; j < d.hidden; j++) o[j] = bf16_to_f32(r[j]);
+  }
+  hip::upload(M.ps.emb, M.ps.emb_host, T * d.hidden);
+  return true;
+}
+
+// Consume a prompt in chunks; logits of its LAST token land in s.logitsb (only
+// that row is ever read, so only it meets the lm_head: qm:396-401).
+inline bool prefill(model& M, const int64_t* tokens, int64_t n, int64_t chunk = 512) {
+  if (n <= 0 || chunk <= 0) return false;
+  bool ok = true;
+  int64_t last_T = 0;
+  for (int64_t t0 = 0; t0 < n && ok; t0 += chunk) {
+    last_T = std::min(chunk, n - t0);
+    ok = stage_chunk(M, tokens + t0, last_T) && prefill_layers(M, last_T);
+  }
+  if (!ok) return false;
+  void* last = static_cast<char*>(M.ps.h) + (last_T - 1) * M.d.hidden * 4;
+  return gemv(M.lm_head, last, M.s.logitsb);
 }
 
 // One decode step recorded as a hipGraph at a FIXED position (the throughput

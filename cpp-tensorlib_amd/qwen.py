@@ -43,6 +43,13 @@ def _load():
             "tlq_set_layer_q4": (cint, [P, i64] + [P] * 12),
             "tlq_set_head_q4": (cint, [P, P, P, P]),
             "tlq_set_random_q4": (cint, [P, u32]),
+            "tlq_set_layer_bf16": (cint, [P, i64] + [P] * 12),
+            "tlq_set_head_bf16": (cint, [P, P, P, P]),
+            "tlq_set_random_bf16": (cint, [P, u32]),
+            "tlq_prefill": (cint, [P, P, i64, i64, P]),
+            "tlq_stage_chunk": (cint, [P, P, i64]),
+            "tlq_prefill_layers": (cint, [P, i64, i64]),
+            "tlq_set_cache_pos": (None, [P, i64]),
             "tlq_fill_cache_random": (cint, [P, i64, u32]),
             "tlq_step": (i64, [P, i64, i64, P]),
             "tlq_run_layers": (cint, [P, i64, i64]),
@@ -80,28 +87,52 @@ class QwenGPU:
         self._keep = []
 
     @classmethod
-    def from_blobs(cls, om):
+    def from_blobs(cls, om, fmt="q4"):
         """Build from a weight source: any object with `.d` (the dims) and
         `.weight(layer, name)` returning the stored bytes of wq/wk/wv/wo/wg/wu/wd (q4
-        buffers), bq/bk/bv/an/fn (f32) and, for layer -1, embed (bf16), onorm, outw."""
+        buffers, or bf16 in the logical [K,N] layout when fmt == "bf16"), bq/bk/bv/an/fn
+        (f32) and, for layer -1, embed (bf16), onorm, outw."""
         d = om.d
         g = cls(dict((f, getattr(d, f)) for f, _ in Dims._fields_))
+        set_layer = g.L.tlq_set_layer_q4 if fmt == "q4" else g.L.tlq_set_layer_bf16
+        set_head = g.L.tlq_set_head_q4 if fmt == "q4" else g.L.tlq_set_head_bf16
         for li in range(d.n_layers):
             w = [np.ascontiguousarray(om.weight(li, n)) for n in ("wq", "wk", "wv", "wo", "wg", "wu", "wd")]
             v = [np.ascontiguousarray(om.weight(li, n)) for n in ("bq", "bk", "bv", "an", "fn")]
-            rc = g.L.tlq_set_layer_q4(g.h, li, *[_p(a) for a in w + v])
-            if rc != 0:
-                raise RuntimeError("tlq_set_layer_q4(%d) failed" % li)
+            if set_layer(g.h, li, *[_p(a) for a in w + v]) != 0:
+                raise RuntimeError("set_layer(%d) failed" % li)
         emb = np.ascontiguousarray(om.weight(-1, "embed"))
         onorm = np.ascontiguousarray(om.weight(-1, "onorm"))
         outw = np.ascontiguousarray(om.weight(-1, "outw"))
-        if g.L.tlq_set_head_q4(g.h, _p(emb), _p(onorm), _p(outw)) != 0:
-            raise RuntimeError("tlq_set_head_q4 failed")
+        if set_head(g.h, _p(emb), _p(onorm), _p(outw)) != 0:
+            raise RuntimeError("set_head failed")
         return g
 
-    def set_random(self, seed=1):
-        if self.L.tlq_set_random_q4(self.h, seed) != 0:
-            raise RuntimeError("tlq_set_random_q4 failed")
+    def set_random(self, seed=1, fmt="q4"):
+        fn = self.L.tlq_set_random_q4 if fmt == "q4" else self.L.tlq_set_random_bf16
+        if fn(self.h, seed) != 0:
+            raise RuntimeError("set_random failed")
+
+    def prefill(self, tokens, chunk=512, want_logits=True):
+        """Consume prompt tokens in chunks at the caches' current position; returns the
+        last token's logits."""
+        t = np.ascontiguousarray(tokens, np.int64)
+        logits = np.empty(self.d.vocab, np.float32) if want_logits else None
+        if self.L.tlq_prefill(self.h, _p(t), len(t), chunk, _p(logits) if want_logits else None) != 0:
+            raise RuntimeError("prefill declined by the backend")
+        return logits
+
+    def stage_chunk(self, tokens):
+        t = np.ascontiguousarray(tokens, np.int64)
+        if self.L.tlq_stage_chunk(self.h, _p(t), len(t)) != 0:
+            raise RuntimeError("stage_chunk failed")
+
+    def prefill_layers(self, T, pos0):
+        if self.L.tlq_prefill_layers(self.h, T, pos0) != 0:
+            raise RuntimeError("prefill_layers declined by the backend")
+
+    def set_cache_pos(self, pos):
+        self.L.tlq_set_cache_pos(self.h, pos)
 
     def fill_cache_random(self, upto, seed=2):
         if self.L.tlq_fill_cache_random(self.h, upto, seed) != 0:

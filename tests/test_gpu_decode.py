@@ -110,3 +110,61 @@ def test_config4_qwen05b_greedy_tokens_match_reference_golden(orc):
     assert maxrel(g2_logits, want_logits) < 2e-3
     assert mismatches == 0
     g.close(); om.close()
+
+
+def test_bf16_decode_loop_matches_oracle(orc):
+    """The same harness on bf16 weights (the decode GEMV over [N,K] rows, cuda.h:770-785):
+    blobs arrive in the logical [K,N] layout and are transposed at load."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(SMALL, seed=6, q4=False)
+    g = qwen.QwenGPU.from_blobs(om, fmt="bf16")
+    rng = np.random.default_rng(7)
+    for pos in range(24):
+        tok = int(rng.integers(0, SMALL["vocab"]))
+        want_tok, want_logits = om.step(tok, pos)
+        got_tok, got_logits = g.step(tok, pos, want_logits=True)
+        assert maxrel(got_logits, want_logits) < 2e-3, pos
+        assert got_tok == want_tok or _near_tie(want_logits), pos
+    assert g.census()["gemv_bf16_row"] >= 24 * (4 * SMALL["n_layers"] + 1)
+    g.close(); om.close()
+
+
+@pytest.mark.parametrize("dims,n_prompt,chunk", [(SMALL, 50, 32), (SMALL128, 130, 64), (SMALL, 40, 512)])
+def test_prefill_chunks_match_token_by_token_oracle(orc, dims, n_prompt, chunk):
+    """A prompt consumed in chunks through the MFMA GEMM + causal prefill attention
+    (bench/cuda/qwen_model.h:357-401) gives the logits of feeding the same tokens one at a
+    time to the oracle, and leaves caches from which decode continues identically."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(dims, seed=8, q4=False)
+    g = qwen.QwenGPU.from_blobs(om, fmt="bf16")
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, dims["vocab"], n_prompt)
+    for pos, tok in enumerate(prompt):
+        want_tok, want_logits = om.step(int(tok), pos)
+    before = g.census()
+    got_logits = g.prefill(prompt, chunk=chunk)
+    after = g.census()
+    n_chunks = -(-n_prompt // chunk)
+    assert after["gemm_bf16_nt"] - before["gemm_bf16_nt"] == 4 * dims["n_layers"] * n_chunks
+    assert after["attn_prefill"] - before["attn_prefill"] == dims["n_layers"] * n_chunks
+    assert maxrel(got_logits, want_logits) < 2e-3, maxrel(got_logits, want_logits)
+    assert int(np.argmax(got_logits)) == want_tok or _near_tie(want_logits)
+    tok = want_tok
+    for pos in range(n_prompt, n_prompt + 12):        # decode on top of the prefilled caches
+        want_tok, want_logits = om.step(tok, pos)
+        got_tok, got_logits = g.step(tok, pos, want_logits=True)
+        assert maxrel(got_logits, want_logits) < 2e-3, pos
+        assert got_tok == want_tok or _near_tie(want_logits), pos
+        tok = want_tok
+    g.close(); om.close()
+
+
+def test_prefill_declines_on_int4_weights(orc):
+    """Like the reference's, the chunked path needs bf16 rows; an int4 model must refuse
+    rather than compute something else."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(SMALL, seed=3, q4=True)
+    g = qwen.QwenGPU.from_blobs(om)
+    with pytest.raises(RuntimeError):
+        g.prefill(np.arange(8))
+    g.close(); om.close()
