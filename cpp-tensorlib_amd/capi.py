@@ -76,6 +76,10 @@ SIGNATURES = {
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
     "tlhip_qkv_rope_append": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
+    "tlhip_gemv_q4_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
+    "tlhip_gemv_bf16_row_swiglu": (cint, [P, P, P, i64, i64]),
+    "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
+    "tlhip_gemv_bf16_row_rmsnorm": (cint, [P, P, P, P, P, P, i64, i64, f32]),
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
@@ -286,6 +290,22 @@ class TlHip:
     def qkv_rope_append(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, D, pos, kv_max, base, kv_bf16=False):
         self._chk(self.c.tlhip_qkv_rope_append(qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None,
                                                Kc.ptr, Vc.ptr, Hq, Hkv, D, pos, kv_max, base, int(kv_bf16)))
+
+    def gemv_q4_swiglu(self, gu, wq, y, N, K, group=32):
+        self._chk(self.c.tlhip_gemv_q4_swiglu(gu.ptr, wq.ptr, wq.ptr + N * K // 2, y.ptr, N, K, group))
+
+    def gemv_bf16_row_swiglu(self, gu, W, y, N, K):
+        self._chk(self.c.tlhip_gemv_bf16_row_swiglu(gu.ptr, W.ptr, y.ptr, N, K))
+
+    def gemv_q4_rmsnorm(self, x, delta, norm_w, xout, wq, y, N, K, eps, group=32):
+        self._chk(self.c.tlhip_gemv_q4_rmsnorm(
+            x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
+            xout.ptr if xout is not None else None, wq.ptr, wq.ptr + N * K // 2, y.ptr, N, K, group, eps))
+
+    def gemv_bf16_row_rmsnorm(self, x, delta, norm_w, xout, W, y, N, K, eps):
+        self._chk(self.c.tlhip_gemv_bf16_row_rmsnorm(
+            x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
+            xout.ptr if xout is not None else None, W.ptr, y.ptr, N, K, eps))
 
     def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0):
         self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw))

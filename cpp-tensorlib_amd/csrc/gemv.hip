@@ -126,10 +126,26 @@ __device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __res
   }
 }
 
-template <typename Fmt, int R>
+// How a block obtains the activation vector while it stages it. Folding the
+// producer of x into the GEMV removes a launch and a round trip through memory;
+// every block recomputes the (tiny) producer redundantly.
+//   kPlain:   x is read as is.
+//   kSwiglu:  x[k] = (g*sigmoid(g))*u with g = in[k], u = in[K + k]   (array.h:2435-2439)
+//   kRmsnorm: s = in (+ delta); x = (s * 1/sqrt(mean(s*s) + eps)) * norm_w   (array.h:2429-2433);
+//             block 0 also writes s to xout (the residual stream), which therefore
+//             must not alias in or delta: other blocks still read them.
+enum { kPlain = 0, kSwiglu = 1, kRmsnorm = 2 };
+struct Producer {
+  const float* delta;
+  const float* norm_w;
+  float* xout;
+  float eps;
+};
+
+template <typename Fmt, int R, int PRO>
 __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
-    float* __restrict__ y, int N, int upr, int KW, int ntiles) {
+    float* __restrict__ y, int N, int upr, int KW, int ntiles, const Producer pro) {
   constexpr int J = Fmt::E / 4;
   extern __shared__ float4 smem4[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -156,9 +172,40 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const float4* x4 = reinterpret_cast<const float4*>(x);
     const int n4 = upr * J;
     const int n4_padded = (n4 + 63) & ~63;   // whole wavefronts take part in the shuffles
+    const float4* d4 = reinterpret_cast<const float4*>(pro.delta);
+    float inv = 0.f;
+    if (PRO == kRmsnorm) {   // mean square of the row, summed in a fixed order
+      float ss = 0.f;
+      for (int i = tid; i < n4; i += blockDim.x) {
+        float4 v = x4[i];
+        if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
+        ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+      }
+      ss = wave_sum(ss);
+      if (lane == 0) red[wave] = ss;
+      __syncthreads();
+      float tot = red[0];
+      for (int w = 1; w < nw; w++) tot += red[w];
+      inv = 1.0f / sqrtf(tot * (1.0f / (float)(n4 * 4)) + pro.eps);
+      // red is reused only after the barrier that ends the staging pass
+    }
     for (int i = tid; i < n4_padded; i += blockDim.x) {
       const bool live = i < n4;
-      const float4 v = live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      float4 v = live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (PRO == kSwiglu && live) {
+        const float4 up = x4[n4 + i];
+        v.x = (v.x * (1.0f / (1.0f + expf(-v.x)))) * up.x;
+        v.y = (v.y * (1.0f / (1.0f + expf(-v.y)))) * up.y;
+        v.z = (v.z * (1.0f / (1.0f + expf(-v.z)))) * up.z;
+        v.w = (v.w * (1.0f / (1.0f + expf(-v.w)))) * up.w;
+      }
+      if (PRO == kRmsnorm && live) {
+        if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
+        if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
+        const float4 w4 = reinterpret_cast<const float4*>(pro.norm_w)[i];
+        v.x = (v.x * inv) * w4.x; v.y = (v.y * inv) * w4.y;
+        v.z = (v.z * inv) * w4.z; v.w = (v.w * inv) * w4.w;
+      }
       const int u = i / J, j = i - u * J;
       if (live) xs[((u >> 6) * J + j) * 64 + (u & 63)] = Fmt::stage(v);
       if (Fmt::kScaled) {
@@ -407,21 +454,23 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   return c;
 }
 
-template <typename Fmt>
+template <typename Fmt, int PRO = kPlain>
 static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
-                       int64_t K, int census_id, int tR, int tKW, int tBPC, int tNW) {
+                       int64_t K, int census_id, int tR, int tKW, int tBPC, int tNW,
+                       const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
   Context& c = ctx();
   const int upr = (int)(K / Fmt::E);
   RowCfg cfg = pick_rows_cfg(N, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC, tNW);
   const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
   const int ntiles = (int)((N + rows_per_tile - 1) / rows_per_tile);
-  using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int);
+  using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int,
+                       const Producer);
   K_t fn = nullptr;
   switch (cfg.R) {
-    case 1: fn = gemv_rows_kernel<Fmt, 1>; break;
-    case 2: fn = gemv_rows_kernel<Fmt, 2>; break;
-    case 4: fn = gemv_rows_kernel<Fmt, 4>; break;
-    case 8: fn = gemv_rows_kernel<Fmt, 8>; break;
+    case 1: fn = gemv_rows_kernel<Fmt, 1, PRO>; break;
+    case 2: fn = gemv_rows_kernel<Fmt, 2, PRO>; break;
+    case 4: fn = gemv_rows_kernel<Fmt, 4, PRO>; break;
+    case 8: fn = gemv_rows_kernel<Fmt, 8, PRO>; break;
     default: return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
   }
   if (cfg.lds > 48 * 1024) {
@@ -430,7 +479,7 @@ static int launch_rows(const float* x, const void* W, const float* scales, float
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
   }
   hipLaunchKernelGGL(fn, dim3(cfg.blocks), dim3(cfg.nw * 64), cfg.lds, c.stream, x,
-                     static_cast<const uint4*>(W), scales, y, (int)N, upr, cfg.KW, ntiles);
+                     static_cast<const uint4*>(W), scales, y, (int)N, upr, cfg.KW, ntiles, pro);
   TLHIP_CHECK_LAUNCH(census_id);
 }
 
@@ -525,6 +574,85 @@ int tlhip_gemv_bf16(const void* a, const void* B, void* y, int64_t n, int64_t k)
   if (int rc = check_gemv_args(a, B, y, n, k, "tlhip_gemv_bf16")) return rc;
   return launch_cols<uint16_t>(static_cast<const float*>(a), static_cast<const uint16_t*>(B),
                                static_cast<float*>(y), n, k, TLHIP_C_GEMV_BF16);
+}
+
+// ---- GEMVs that produce their own activation vector ------------------------------------------
+
+static int check_fused_q4(const void* qw, const void* scales, int64_t K, int64_t group, size_t in_floats,
+                          const char* who) {
+  if (!scales) return fail(TLHIP_EINVAL, "%s: null scales", who);
+  if (group != 32 || (K % 32) != 0 || !aligned16(qw))
+    return fail(TLHIP_EUNSUPPORTED, "%s: fused form needs group 32, K %% 32 == 0, aligned weights", who);
+  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
+  if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
+    return fail(TLHIP_EUNSUPPORTED, "%s: K too large for the LDS-staged kernel", who);
+  (void)in_floats;
+  return 0;
+}
+
+static int check_fused_bf16(const void* W, int64_t K, const char* who) {
+  if ((K % 8) != 0 || !aligned16(W))
+    return fail(TLHIP_EUNSUPPORTED, "%s: need K %% 8 == 0 and aligned weights", who);
+  const size_t xbytes = (size_t)((K / 8 + 63) / 64) * 64 * 8 * 4;
+  if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
+    return fail(TLHIP_EUNSUPPORTED, "%s: K too large for the LDS-staged kernel", who);
+  return 0;
+}
+
+static int check_norm_args(const void* x, const void* delta, const void* norm_w, const void* xout,
+                           const char* who) {
+  if (!norm_w) return fail(TLHIP_EINVAL, "%s: null norm weight", who);
+  if (!aligned16(norm_w) || (delta && !aligned16(delta)) || (xout && !aligned16(xout)))
+    return fail(TLHIP_EINVAL, "%s: vectors must be 16-byte aligned", who);
+  if (xout && (xout == x || xout == delta))
+    return fail(TLHIP_EINVAL, "%s: xout must not alias x or delta (other blocks still read them)", who);
+  return 0;
+}
+
+int tlhip_gemv_q4_swiglu(const void* gu, const void* qw, const void* scales, void* y, int64_t N,
+                         int64_t K, int64_t group) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(gu, qw, y, N, K, "tlhip_gemv_q4_swiglu")) return rc;
+  if (int rc = check_fused_q4(qw, scales, K, group, 2 * K, "tlhip_gemv_q4_swiglu")) return rc;
+  Context& c = ctx();
+  return launch_rows<FmtQ4, kSwiglu>(static_cast<const float*>(gu), qw, static_cast<const float*>(scales),
+                                     static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
+                                     c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw);
+}
+
+int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
+                          const void* qw, const void* scales, void* y, int64_t N, int64_t K,
+                          int64_t group, float eps) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(x, qw, y, N, K, "tlhip_gemv_q4_rmsnorm")) return rc;
+  if (int rc = check_fused_q4(qw, scales, K, group, K, "tlhip_gemv_q4_rmsnorm")) return rc;
+  if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_q4_rmsnorm")) return rc;
+  Context& c = ctx();
+  const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
+                     static_cast<float*>(xout), eps};
+  return launch_rows<FmtQ4, kRmsnorm>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
+                                      static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
+                                      c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw, pro);
+}
+
+int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n, int64_t k) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(gu, W, y, n, k, "tlhip_gemv_bf16_row_swiglu")) return rc;
+  if (int rc = check_fused_bf16(W, k, "tlhip_gemv_bf16_row_swiglu")) return rc;
+  return launch_rows<FmtBf16, kSwiglu>(static_cast<const float*>(gu), W, nullptr, static_cast<float*>(y),
+                                       n, k, TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0);
+}
+
+int tlhip_gemv_bf16_row_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
+                                const void* W, void* y, int64_t n, int64_t k, float eps) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(x, W, y, n, k, "tlhip_gemv_bf16_row_rmsnorm")) return rc;
+  if (int rc = check_fused_bf16(W, k, "tlhip_gemv_bf16_row_rmsnorm")) return rc;
+  if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_bf16_row_rmsnorm")) return rc;
+  const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
+                     static_cast<float*>(xout), eps};
+  return launch_rows<FmtBf16, kRmsnorm>(static_cast<const float*>(x), W, nullptr, static_cast<float*>(y),
+                                        n, k, TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0, pro);
 }
 
 }  // extern "C"

@@ -110,6 +110,12 @@ struct api {
   int (*merge_heads)(const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*qkv_rope_append)(void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
                          int64_t, int64_t, int64_t, float, int) = nullptr;
+  int (*gemv_q4_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemv_bf16_row_swiglu)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
+  int (*gemv_q4_rmsnorm)(const void*, const void*, const void*, void*, const void*, const void*, void*,
+                         int64_t, int64_t, int64_t, float) = nullptr;
+  int (*gemv_bf16_row_rmsnorm)(const void*, const void*, const void*, void*, const void*, void*,
+                               int64_t, int64_t, float) = nullptr;
 };
 
 struct context {
@@ -185,7 +191,11 @@ struct context {
               bind(f.argmax_async, "tlhip_argmax_async") &&
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
-              bind(f.qkv_rope_append, "tlhip_qkv_rope_append");
+              bind(f.qkv_rope_append, "tlhip_qkv_rope_append") &&
+              bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
+              bind(f.gemv_bf16_row_swiglu, "tlhip_gemv_bf16_row_swiglu") &&
+              bind(f.gemv_q4_rmsnorm, "tlhip_gemv_q4_rmsnorm") &&
+              bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm");
     if (!ok) return;
     if (f.abi_version() != 1) {
       why = "libtensorlib_hip.so has a different ABI version";
@@ -609,6 +619,56 @@ inline bool qkv_rope_append(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
   c.device_write_(Vc);
   return detail::done_(c, c.f.qkv_rope_append(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
                                               kv_max, base, kv_bf16 ? 1 : 0));
+}
+
+// GEMVs that evaluate the producer of their activation vector while staging it:
+// swiglu(gu) -> GEMV and rmsnorm_res(x, delta) -> GEMV in one launch each. They
+// decline (false) on shapes the fused kernel does not take; the caller then
+// issues the two separate calls.
+inline bool gemv_q4_swiglu(void* gu, void* qw, void* scales, void* y, int64_t N, int64_t K,
+                           int64_t group) {
+  auto& c = context::get();
+  if (!c.ready || group != 32 || (K % 32) != 0) return false;
+  c.device_read_(gu);
+  c.device_read_(qw);
+  c.device_read_(scales);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_q4_swiglu(gu, qw, scales, y, N, K, group));
+}
+inline bool gemv_bf16_row_swiglu(void* gu, void* B, void* y, int64_t n, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0) return false;
+  c.device_read_(gu);
+  c.device_read_(B);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_bf16_row_swiglu(gu, B, y, n, k));
+}
+// s = x (+ delta); xout (optional, distinct from x and delta) receives s;
+// y = W . rmsnorm(s, norm_w, eps)
+inline bool gemv_q4_rmsnorm(void* x, void* delta, void* norm_w, void* xout, void* qw, void* scales,
+                            void* y, int64_t N, int64_t K, int64_t group, float eps) {
+  auto& c = context::get();
+  if (!c.ready || group != 32 || (K % 32) != 0 || (xout && (xout == x || xout == delta))) return false;
+  c.device_read_(x);
+  if (delta) c.device_read_(delta);
+  c.device_read_(norm_w);
+  c.device_read_(qw);
+  c.device_read_(scales);
+  if (xout) c.device_write_(xout);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_q4_rmsnorm(x, delta, norm_w, xout, qw, scales, y, N, K, group, eps));
+}
+inline bool gemv_bf16_row_rmsnorm(void* x, void* delta, void* norm_w, void* xout, void* B, void* y,
+                                  int64_t n, int64_t k, float eps) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0 || (xout && (xout == x || xout == delta))) return false;
+  c.device_read_(x);
+  if (delta) c.device_read_(delta);
+  c.device_read_(norm_w);
+  c.device_read_(B);
+  if (xout) c.device_write_(xout);
+  c.device_write_(y);
+  return detail::done_(c, c.f.gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, B, y, n, k, eps));
 }
 
 // ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------

@@ -13,7 +13,9 @@
 //   -> rmsnorm_res (x1 = x + attn ; h2 = norm(x1)) -> fused gate|up GEMV
 //   -> swiglu -> down GEMV -> rmsnorm_res (x2 = x1 + mlp ; next layer's input norm)
 // then the lm_head GEMV and a device argmax whose 4-byte copy is the single
-// blocking call of the step.
+// blocking call of the step. With model::fused (the default) the q/k/v epilogue is
+// one launch and the norms and swiglu are evaluated inside the GEMV that consumes
+// them: 6 launches per layer instead of 12.
 //
 // A prompt is consumed in chunks of T tokens (prefill_chunk, the counterpart of
 // qm:357-395): the same layer wiring with every GEMV replaced by the MFMA GEMM
@@ -69,6 +71,24 @@ inline bool gemv(const linear& L, void* a, void* y) {
   return hip::gemv_bf16_row(a, L.w, y, L.N, L.K);
 }
 
+// y = W . swiglu(gu)
+inline bool gemv_swiglu(const linear& L, void* gu, void* y) {
+  if (L.fmt == wfmt::q4) {
+    void* scales = static_cast<char*>(L.w) + L.N * L.K / 2;
+    return hip::gemv_q4_swiglu(gu, L.w, scales, y, L.N, L.K, kQ4Group);
+  }
+  return hip::gemv_bf16_row_swiglu(gu, L.w, y, L.N, L.K);
+}
+// s = x (+ delta) -> xout ; y = W . rmsnorm(s, norm_w)
+inline bool gemv_rmsnorm(const linear& L, void* x, void* delta, void* norm_w, void* xout, void* y,
+                         float eps) {
+  if (L.fmt == wfmt::q4) {
+    void* scales = static_cast<char*>(L.w) + L.N * L.K / 2;
+    return hip::gemv_q4_rmsnorm(x, delta, norm_w, xout, L.w, scales, y, L.N, L.K, kQ4Group, eps);
+  }
+  return hip::gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, L.w, y, L.N, L.K, eps);
+}
+
 struct layer {
   linear wqkv, wo, wgu, wd;          // fused [wq|wk|wv] and [wg|wu] (qm:188-199)
   void* bqkv = nullptr;                              // fused bias [q_dim + 2 kv_dim] (qm:196)
@@ -104,7 +124,9 @@ struct model {
   std::vector<layer> layers;
   scratch s;
   bool ready = false;
-  bool fused = true;  // use the fused q/k/v epilogue launch (false: one launch per op)
+  // true: fused launches (q/k/v epilogue + append; norms and swiglu evaluated inside the
+  // GEMV that consumes them). false: the reference's call sequence, one launch per op.
+  bool fused = true;
 };
 
 namespace detail {
@@ -382,6 +404,29 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
   const float scale = 1.0f / std::sqrt((float)d.head_dim);
   const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim();
   bool ok = true;
+  if (M.fused) {
+    // 6 launches per layer (+1 when attention splits the context):
+    //   [norm -> qkv GEMV] , q/k/v epilogue + append , attention , o-proj GEMV ,
+    //   [residual + norm -> gate|up GEMV] , [swiglu -> down GEMV]
+    // The residual stream ping-pongs between res[0] and res[1] because a fused GEMV
+    // may not write the residual over a vector its other blocks still read.
+    void* rin = x0;          // residual entering the layer
+    void* din = nullptr;     // MLP output of the previous layer, not yet added
+    for (int64_t l = 0; l < d.n_layers; l++) {
+      layer& L = M.layers[(size_t)l];
+      ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
+      L.cache.pos = pos;
+      ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
+      ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
+      ok &= gemv(L.wo, S.ab, S.hb);
+      ok &= gemv_rmsnorm(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.gub, d.eps);
+      ok &= gemv_swiglu(L.wd, S.gub, S.mdb);
+      rin = S.res[1];
+      din = S.mdb;
+    }
+    ok &= gemv_rmsnorm(M.lm_head, rin, din, M.onorm, nullptr, logits_out ? logits_out : S.logitsb, d.eps);
+    return ok;
+  }
   void* x = x0;
   ok &= hip::rmsnorm(x, M.layers[0].an, S.hb, E, d.eps);
   for (int64_t l = 0; l < d.n_layers; l++) {
@@ -392,14 +437,11 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     void* kp = static_cast<char*>(S.qkvb) + QD * 4;
     void* vp = static_cast<char*>(S.qkvb) + (QD + KD) * 4;
     L.cache.pos = pos;
-    if (M.fused) {
-      ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
-    } else {  // the reference's call sequence, one launch per op
-      ok &= hip::rope(qp, qp, d.n_q_heads, 1, d.head_dim, pos, d.rope_base, L.bq);
-      ok &= hip::rope(kp, kp, d.n_kv_heads, 1, d.head_dim, pos, d.rope_base, L.bk);
-      ok &= hip::binary(hip::kop::add, vp, 0, L.bv, 0, vp, 0, KD, 1.0f, 0.0f);
-      ok &= L.cache.append(kp, vp);
-    }
+    // the reference's call sequence, one launch per op (qm:703-716)
+    ok &= hip::rope(qp, qp, d.n_q_heads, 1, d.head_dim, pos, d.rope_base, L.bq);
+    ok &= hip::rope(kp, kp, d.n_kv_heads, 1, d.head_dim, pos, d.rope_base, L.bk);
+    ok &= hip::binary(hip::kop::add, vp, 0, L.bv, 0, vp, 0, KD, 1.0f, 0.0f);
+    ok &= L.cache.append(kp, vp);
     ok &= L.cache.attn(qp, S.ab, d.n_q_heads, scale);
     ok &= gemv(L.wo, S.ab, ro);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, S.h2b, E, d.eps);

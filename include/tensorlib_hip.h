@@ -187,6 +187,26 @@ int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void*
                           void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                           int64_t kv_max, float base, int kv_bf16);
 
+/* ---- GEMVs that produce their own activation vector (no single reference
+ * counterpart) -----------------------------------------------------------------
+ * The producer of x is evaluated by every block while it stages x, which removes a
+ * launch and a memory round trip per fused pair. Arithmetic is that of the separate
+ * entry points: tlhip_swiglu then tlhip_gemv_*, and tlhip_rmsnorm_res then
+ * tlhip_gemv_*, as run_layers_ chains them (bench/cuda/qwen_model.h:717-737).
+ * Row layouts only (int4 group 32, bf16 [N,K]); other shapes return
+ * TLHIP_EUNSUPPORTED and the caller issues the two separate calls. */
+/* y = W . swiglu(gu), gu = [gate (K) | up (K)] f32 */
+int tlhip_gemv_q4_swiglu(const void* gu, const void* qw, const void* scales, void* y, int64_t N,
+                         int64_t K, int64_t group);
+int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n, int64_t k);
+/* s = x (+ delta when non-NULL); xout (when non-NULL) receives s; y = W . rmsnorm(s, norm_w, eps).
+ * xout must not alias x or delta. */
+int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
+                          const void* qw, const void* scales, void* y, int64_t N, int64_t K,
+                          int64_t group, float eps);
+int tlhip_gemv_bf16_row_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
+                                const void* W, void* y, int64_t n, int64_t k, float eps);
+
 /* ---- prefill ------------------------------------------------------------------ */
 /* C[M,N] = A[M,K] f32 . W[N,K]^T bf16, fp32 accumulate; K % 8 == 0.  cuda.h:787-841 */
 int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K);

@@ -169,3 +169,78 @@ def test_census_counts_launches(lib, orc):
     lib.gemv_q4(dx, dw, dy, N, K)
     lib.gemv_q4(dx, dw, dy, N, K)
     assert lib.census()["gemv_q4"] == 2
+
+
+# ---- GEMVs that evaluate the producer of their activation vector ---------------------------
+
+@pytest.mark.parametrize("fmt", ["q4", "bf16"])
+@pytest.mark.parametrize("N,K", [(896, 4864), (3584, 18944), (40, 64), (777, 2048 + 32)])
+def test_gemv_swiglu_fused(lib, orc, fmt, N, K):
+    """y = W . swiglu(gu) in one launch equals swiglu (array.h:2435-2439) followed by the GEMV,
+    both taken from the oracle."""
+    print("case gemv_swiglu", fmt, N, K, flush=True)
+    gu = orc.normal(2 * K, 70 + N, 0.0, 1.5)
+    x = orc.swiglu_fused(gu, K).reshape(K)
+    dgu, dy = lib.to_device(gu), lib.empty(N)
+    if fmt == "q4":
+        buf = orc.to_q4(orc.normal(K * N, 71, 0.0, 0.02).reshape(K, N))
+        want = orc.gemv_q4(x, buf, N, K)
+        dw = lib.to_device(buf)
+        lib.gemv_q4_swiglu(dgu, dw, dy, N, K)
+    else:
+        w = orc.to_bf16(orc.normal(N * K, 72, 0.0, 0.02).reshape(N, K))
+        want = orc.gemv_bf16_row(x, w)
+        dw = lib.to_device(w)
+        lib.gemv_bf16_row_swiglu(dgu, dw, dy, N, K)
+    got = dy.numpy()
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    for b in (dgu, dw, dy):
+        b.free()
+
+
+@pytest.mark.parametrize("fmt", ["q4", "bf16"])
+@pytest.mark.parametrize("with_delta,with_xout", [(True, True), (False, True), (True, False), (False, False)])
+@pytest.mark.parametrize("N,K", [(4608, 3584), (1152, 896), (33, 160), (152064 // 16, 3584)])
+def test_gemv_rmsnorm_fused(lib, orc, fmt, N, K, with_delta, with_xout):
+    """s = x (+ delta) -> xout; y = W . rmsnorm(s) in one launch equals the oracle's rmsnorm_res
+    (array.h:2429-2433) followed by the GEMV; xout is the exact fp32 sum."""
+    print("case gemv_rmsnorm", fmt, N, K, with_delta, with_xout, flush=True)
+    eps = 1e-6
+    x = orc.normal(K, 80 + N, 0.0, 2.0)
+    delta = orc.normal(K, 81, 0.0, 0.5) if with_delta else np.zeros(K, np.float32)
+    nw = (1.0 + orc.normal(K, 82, 0.0, 0.1)).astype(np.float32)
+    s, h = orc.rmsnorm_res(x.reshape(1, K), delta.reshape(1, K), nw, eps)
+    dx, dn, dy = lib.to_device(x), lib.to_device(nw), lib.empty(N)
+    dd = lib.to_device(delta) if with_delta else None
+    dxo = lib.to_device(np.full(K, np.nan, np.float32)) if with_xout else None
+    if fmt == "q4":
+        buf = orc.to_q4(orc.normal(K * N, 83, 0.0, 0.02).reshape(K, N))
+        want = orc.gemv_q4(h.reshape(K), buf, N, K)
+        dw = lib.to_device(buf)
+        lib.gemv_q4_rmsnorm(dx, dd, dn, dxo, dw, dy, N, K, eps)
+    else:
+        w = orc.to_bf16(orc.normal(N * K, 84, 0.0, 0.02).reshape(N, K))
+        want = orc.gemv_bf16_row(h.reshape(K), w)
+        dw = lib.to_device(w)
+        lib.gemv_bf16_row_rmsnorm(dx, dd, dn, dxo, dw, dy, N, K, eps)
+    got = dy.numpy()
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    if with_xout:
+        assert np.array_equal(dxo.numpy(), s.reshape(K))
+    assert np.array_equal(dx.numpy(), x)          # inputs untouched
+    for b in (dx, dn, dy, dw, dd, dxo):
+        if b is not None:
+            b.free()
+
+
+def test_gemv_fused_rejects_aliasing_and_other_groups(lib, pkg):
+    x, n, y, w = lib.empty(64), lib.empty(64), lib.empty(8), lib.empty_bytes(4096)
+    with pytest.raises(pkg.TlHipError) as e:
+        lib.gemv_q4_rmsnorm(x, None, n, x, w, y, 8, 64, 1e-6)          # xout aliases x
+    assert e.value.code == -2
+    with pytest.raises(pkg.TlHipError) as e:
+        lib.gemv_q4_rmsnorm(x, None, n, None, w, y, 8, 64, 1e-6, group=16)
+    assert e.value.code == -3
+    with pytest.raises(pkg.TlHipError) as e:
+        lib.gemv_q4_swiglu(x, w, y, 8, 32, group=8)
+    assert e.value.code == -3
