@@ -121,6 +121,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     float sreg[G];
 #pragma unroll
     for (int g = 0; g < G; g++) sreg[g] = -INFINITY;
+    // The tile's first V rows do not depend on the scores: request them with the K
+    // rows so that one memory latency covers both.
+    float4 vfirst[UNR][NV];
     for (int i0 = 0; i0 < steps; i0 += UNR) {
       float4 kv[UNR][NV];
 #pragma unroll
@@ -130,6 +133,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         for (int v = 0; v < NV; v++)
           kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * EPL + v * 4)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      if (i0 == 0) {
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+          const int key = kb + u * 4 + slot;
+#pragma unroll
+          for (int v = 0; v < NV; v++)
+            vfirst[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+                                       : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
       }
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
@@ -177,8 +190,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         const int key = kb + (i0 + u) * 4 + slot;
 #pragma unroll
         for (int v = 0; v < NV; v++)
-          vv[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
-                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+          vv[u][v] = i0 == 0 ? vfirst[u][v]
+                     : key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int g = 0; g < G; g++) {
@@ -240,28 +254,31 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// grid = Hq, block = 256: merge the S split partials of one head. The split
-// weights exp(m_s - M) are formed once per split in LDS; the 256 threads are
-// D columns x (256/D) split groups, summed in a fixed order.
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part_m,
-                                                           const float* __restrict__ part_l,
-                                                           const float* __restrict__ part_acc,
-                                                           float* __restrict__ out, int S, int D) {
-  extern __shared__ float sm[];   // f[S] | red[256]
+// grid = Hq, block = 1024: merge the S split partials of one head. The split
+// weights exp(m_s - M) are formed once per split in LDS; the threads are D
+// columns x (1024/D) split groups, each summing its splits in a fixed order with
+// the loads of four splits in flight, then the groups are summed in a fixed order.
+__global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restrict__ part_m,
+                                                            const float* __restrict__ part_l,
+                                                            const float* __restrict__ part_acc,
+                                                            float* __restrict__ out, int S, int D) {
+  extern __shared__ float sm[];   // f[S] | red[1024]
   float* f = sm;
   float* red = sm + S;
   const int h = blockIdx.x, tid = threadIdx.x;
   const float* pm = part_m + (size_t)h * S;
   const float* pl = part_l + (size_t)h * S;
   float mx = -INFINITY;
-  for (int s = tid; s < S; s += 256) mx = fmaxf(mx, pm[s]);
+  for (int s = tid; s < S; s += 1024) mx = fmaxf(mx, pm[s]);
   mx = wave_max(mx);
   if ((tid & 63) == 0) red[tid >> 6] = mx;
   __syncthreads();
-  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float M = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) M = fmaxf(M, red[w]);
   __syncthreads();
   float lsum = 0.f;
-  for (int s = tid; s < S; s += 256) {
+  for (int s = tid; s < S; s += 1024) {
     const float w = __expf(pm[s] - M);
     f[s] = w;
     lsum = fmaf(pl[s], w, lsum);
@@ -269,18 +286,24 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   lsum = wave_sum(lsum);
   if ((tid & 63) == 0) red[tid >> 6] = lsum;
   __syncthreads();
-  const float L = ((red[0] + red[1]) + red[2]) + red[3];
+  float L = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; w++) L += red[w];
   __syncthreads();
-  const int groups = 256 / D, d = tid % D, sg = tid / D;
+  const int groups = 1024 / D, d = tid % D, sg = tid / D;
   const float* pa = part_acc + (size_t)h * S * D + d;
-  float a0 = 0.f, a1 = 0.f;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
   int s = sg;
-  for (; s + groups < S; s += 2 * groups) {
-    a0 = fmaf(f[s], pa[(size_t)s * D], a0);
-    a1 = fmaf(f[s + groups], pa[(size_t)(s + groups) * D], a1);
+  for (; s + 3 * groups < S; s += 4 * groups) {
+    const float v0 = pa[(size_t)s * D], v1 = pa[(size_t)(s + groups) * D],
+                v2 = pa[(size_t)(s + 2 * groups) * D], v3 = pa[(size_t)(s + 3 * groups) * D];
+    a0 = fmaf(f[s], v0, a0);
+    a1 = fmaf(f[s + groups], v1, a1);
+    a2 = fmaf(f[s + 2 * groups], v2, a2);
+    a3 = fmaf(f[s + 3 * groups], v3, a3);
   }
-  if (s < S) a0 = fmaf(f[s], pa[(size_t)s * D], a0);
-  red[tid] = a0 + a1;
+  for (; s < S; s += groups) a0 = fmaf(f[s], pa[(size_t)s * D], a0);
+  red[tid] = (a0 + a1) + (a2 + a3);
   __syncthreads();
   if (sg == 0) {
     float A = red[d];
@@ -296,7 +319,12 @@ struct AttnPlan { int G, gz, nw, TK, S, chunk; };
 // long contexts give every wavefront several 64-key tiles.
 static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus) {
   AttnPlan p{};
-  p.G = group > 4 ? 8 : group > 2 ? 4 : group > 1 ? 2 : 1;
+  // Query heads per block. A wavefront's instruction stream grows with G and, at
+  // short and medium contexts, that serial stream (not bandwidth) is what a step
+  // waits for: up to 4 heads per block there, and the whole group (up to 8) only
+  // when the context is long enough for K/V traffic to dominate.
+  const int gmax = ctx >= 16384 ? 8 : 4;
+  p.G = group > 4 ? gmax : group > 2 ? 4 : group > 1 ? 2 : 1;
   p.gz = (group + p.G - 1) / p.G;
   const int base = Hkv * p.gz;
   const int64_t want_waves = (int64_t)cus * 4;
@@ -343,7 +371,7 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
   }
 #undef TLHIP_ATTN
   if (p.S > 1)
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(256), (size_t)(p.S + 256) * sizeof(float),
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(1024), (size_t)(p.S + 1024) * sizeof(float),
                        c.stream, pm, pl, pacc, out, p.S, D);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
 }
