@@ -111,19 +111,65 @@ struct RowFrag {          // one (row tile, chunk) work item of a lane: R weight
   float sc[R];
 };
 
+// Weight and scale addresses are formed as a uniform base plus a 32-bit byte
+// offset per lane (the launcher checks that the matrix is below 4 GiB), which is
+// the cheapest global addressing form: one 24-bit multiply-add per row.
 template <typename Fmt, int R>
 __device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __restrict__ W,
                                           const float* __restrict__ scales, int N, int upr,
                                           int row0, int u) {
   if (u < upr) {
+    const char* wb = reinterpret_cast<const char*>(W);
+    const char* sb = reinterpret_cast<const char*>(scales);
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const int row = min(row0 + r, N - 1);
-      const size_t idx = (size_t)row * upr + u;
-      f.w[r] = load_stream16(&W[idx]);
-      if (Fmt::kScaled) f.sc[r] = __builtin_nontemporal_load(&scales[idx]);
+      const uint32_t row = (uint32_t)min(row0 + r, N - 1);
+      const uint32_t idx = __umul24(row, (uint32_t)upr) + (uint32_t)u;
+      f.w[r] = load_stream16(reinterpret_cast<const uint4*>(wb + (idx << 4)));
+      if (Fmt::kScaled)
+        f.sc[r] = __builtin_nontemporal_load(reinterpret_cast<const float*>(sb + (idx << 2)));
     }
   }
+}
+
+// ---- 16-lane sum on DPP: every lane of a DPP row ends up with the row's total ----
+template <int CTRL>
+__device__ __forceinline__ float dpp_add_f32(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+  return v + __int_as_float(t);
+}
+
+// Sum R per-lane partials over the wavefront at once. Halving steps trade
+// values for lanes (lane bit m clear keeps the lower half of the values and
+// receives the partner's contribution to them), so R values cost R-1 exchanges
+// instead of 6R; what is left is one value per lane, finished inside its lane
+// group on DPP. Returns, in every lane, the total of row (lane * R) >> 6.
+template <int N, int M, int R>
+__device__ __forceinline__ void halve_rows(float (&a)[R], int lane) {  // N live values -> N/2
+  const bool up = (lane & M) != 0;
+#pragma unroll
+  for (int i = 0; i < N / 2; i++) {
+    const float keep = up ? a[i + N / 2] : a[i];
+    const float send = up ? a[i] : a[i + N / 2];
+    a[i] = keep + __shfl_xor(send, M, kWave);
+  }
+}
+
+template <int R>
+__device__ __forceinline__ float wave_sum_rows(float (&a)[R], int lane) {
+  static_assert(R == 1 || R == 2 || R == 4 || R == 8, "rows per wavefront");
+  if constexpr (R == 8) { halve_rows<8, 32>(a, lane); halve_rows<4, 16>(a, lane); halve_rows<2, 8>(a, lane); }
+  if constexpr (R == 4) { halve_rows<4, 32>(a, lane); halve_rows<2, 16>(a, lane); }
+  if constexpr (R == 2) { halve_rows<2, 32>(a, lane); }
+  float v = a[0];
+  // lanes that differ only in bits below the last halving mask share a row
+  if (R <= 1) v += __shfl_xor(v, 32, kWave);
+  if (R <= 2) v += __shfl_xor(v, 16, kWave);
+  v = dpp_add_f32<0xB1>(v);                 // quad_perm [1,0,3,2]
+  v = dpp_add_f32<0x4E>(v);                 // quad_perm [2,3,0,1]
+  v = dpp_add_f32<0x141>(v);                // row_half_mirror: the two quads of 8 lanes
+  if (R <= 4) v = dpp_add_f32<0x140>(v);    // row_mirror: the two halves of 16 lanes
+  return v;
 }
 
 // How a block obtains the activation vector while it stages it. Folding the
@@ -163,7 +209,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   // The first work item's weights are requested before x is staged, so that the
   // HBM latency of the weights and the L2 latency of x overlap.
   int t = blockIdx.x, c = kw;
-  RowFrag<Fmt, R> cur, nxt;
+  RowFrag<Fmt, R> cur;
   if (t < ntiles) load_frag<Fmt, R>(cur, W, scales, N, upr, t * rows_per_tile + wn * R, (c << 6) + lane);
 
   {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
@@ -223,8 +269,9 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   for (int r = 0; r < R; r++) acc[r] = 0.f;
 
   // Software pipeline over this wavefront's (tile, chunk) items: the next item's
-  // loads are in flight while the current one is unpacked and accumulated.
-  while (t < ntiles) {
+  // loads are in flight while the current one is unpacked and accumulated. The
+  // two fragments swap roles every step (no register copies).
+  auto step = [&](const RowFrag<Fmt, R>& cur, RowFrag<Fmt, R>& nxt) -> bool {
     int nc = c + KW, nt = t;
     if (nc >= chunks) { nc = kw; nt = t + gridDim.x; }
     if (nt < ntiles)
@@ -247,33 +294,33 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
 
     if (nt != t) {  // last chunk of tile t for this wavefront: reduce and store
       const int row0 = t * rows_per_tile + wn * R;
-#pragma unroll
-      for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+      const float v = wave_sum_rows<R>(acc, lane);   // total of row (lane*R)>>6, in every lane
+      const int r = (lane * R) >> 6;
+      const bool writer = (lane & (64 / R - 1)) == 0;
       if (KW == 1) {
-        float v = acc[0];
-#pragma unroll
-        for (int r = 1; r < R; r++) v = (lane == r) ? acc[r] : v;
-        if (lane < R && row0 + lane < N) y[row0 + lane] = v;
+        if (writer && row0 + r < N) y[row0 + r] = v;
       } else {
         // every wavefront of the block passes these two barriers once per tile
-        if (lane == 0) {
-#pragma unroll
-          for (int r = 0; r < R; r++) red[(wn * KW + kw) * R + r] = acc[r];
-        }
+        if (writer) red[(wn * KW + kw) * R + r] = v;
         __syncthreads();
         if (kw == 0 && lane < R && row0 + lane < N) {
-          float v = 0.f;
-          for (int s = 0; s < KW; s++) v += red[(wn * KW + s) * R + lane];
-          y[row0 + lane] = v;
+          float sum = 0.f;
+          for (int sidx = 0; sidx < KW; sidx++) sum += red[(wn * KW + sidx) * R + lane];
+          y[row0 + lane] = sum;
         }
         __syncthreads();
       }
 #pragma unroll
-      for (int r = 0; r < R; r++) acc[r] = 0.f;
+      for (int r2 = 0; r2 < R; r2++) acc[r2] = 0.f;
     }
-    cur = nxt;
     t = nt;
     c = nc;
+    return t < ntiles;
+  };
+  RowFrag<Fmt, R> other;
+  if (t < ntiles) {
+    while (step(cur, other) && step(other, cur)) {
+    }
   }
 }
 
@@ -460,26 +507,38 @@ static int launch_rows(const float* x, const void* W, const float* scales, float
                        const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
   Context& c = ctx();
   const int upr = (int)(K / Fmt::E);
-  RowCfg cfg = pick_rows_cfg(N, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC, tNW);
-  const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
-  const int ntiles = (int)((N + rows_per_tile - 1) / rows_per_tile);
+  if (upr >= (1 << 24)) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large");
+  // The kernel addresses a matrix with 32-bit byte offsets and 24-bit row numbers:
+  // larger ones are walked in row ranges of < 4 GiB, one launch each.
+  int64_t max_rows = (((int64_t)1 << 32) - 16) / ((int64_t)upr * 16);
+  if (max_rows >= (1 << 24)) max_rows = (1 << 24) - 1;
+  max_rows &= ~(int64_t)63;
+  if (max_rows <= 0) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large");
   using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int,
                        const Producer);
-  K_t fn = nullptr;
-  switch (cfg.R) {
-    case 1: fn = gemv_rows_kernel<Fmt, 1, PRO>; break;
-    case 2: fn = gemv_rows_kernel<Fmt, 2, PRO>; break;
-    case 4: fn = gemv_rows_kernel<Fmt, 4, PRO>; break;
-    case 8: fn = gemv_rows_kernel<Fmt, 8, PRO>; break;
-    default: return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
+  for (int64_t n0 = 0; n0 < N; n0 += max_rows) {
+    const int64_t n = N - n0 < max_rows ? N - n0 : max_rows;
+    RowCfg cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC, tNW);
+    const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
+    const int ntiles = (int)((n + rows_per_tile - 1) / rows_per_tile);
+    K_t fn = nullptr;
+    switch (cfg.R) {
+      case 1: fn = gemv_rows_kernel<Fmt, 1, PRO>; break;
+      case 2: fn = gemv_rows_kernel<Fmt, 2, PRO>; break;
+      case 4: fn = gemv_rows_kernel<Fmt, 4, PRO>; break;
+      case 8: fn = gemv_rows_kernel<Fmt, 8, PRO>; break;
+      default: return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
+    }
+    if (cfg.lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)cfg.lds);
+      if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
+    }
+    const uint4* Wn = static_cast<const uint4*>(W) + (size_t)n0 * upr;
+    const float* sn = scales ? scales + (size_t)n0 * upr : nullptr;
+    hipLaunchKernelGGL(fn, dim3(cfg.blocks), dim3(cfg.nw * 64), cfg.lds, c.stream, x, Wn, sn, y + n0,
+                       (int)n, upr, cfg.KW, ntiles, pro);
   }
-  if (cfg.lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)cfg.lds);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  }
-  hipLaunchKernelGGL(fn, dim3(cfg.blocks), dim3(cfg.nw * 64), cfg.lds, c.stream, x,
-                     static_cast<const uint4*>(W), scales, y, (int)N, upr, cfg.KW, ntiles, pro);
   TLHIP_CHECK_LAUNCH(census_id);
 }
 
