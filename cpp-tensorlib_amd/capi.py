@@ -80,7 +80,7 @@ SIGNATURES = {
     "tlhip_gemv_bf16_row_swiglu": (cint, [P, P, P, i64, i64]),
     "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
     "tlhip_gemv_bf16_row_rmsnorm": (cint, [P, P, P, P, P, P, i64, i64, f32]),
-    "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint]),
+    "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
 }
@@ -307,8 +307,8 @@ class TlHip:
             x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
             xout.ptr if xout is not None else None, W.ptr, y.ptr, N, K, eps))
 
-    def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0):
-        self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw))
+    def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0, lpr=0):
+        self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw, lpr))
 
 
 _lib = None

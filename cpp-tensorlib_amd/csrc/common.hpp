@@ -29,7 +29,7 @@ struct Context {
   int* argmax_host = nullptr;     // pinned landing slot for the 4-byte result
   uint64_t census[TLHIP_C_COUNT] = {};
   // int4 GEMV launch-shape override (tlhip_tune_gemv_q4)
-  int tune_q4_rows = 0, tune_q4_kw = 0, tune_q4_bpc = 0, tune_q4_nw = 0;
+  int tune_q4_rows = 0, tune_q4_kw = 0, tune_q4_bpc = 0, tune_q4_nw = 0, tune_q4_lpr = 0;
 };
 
 Context& ctx();

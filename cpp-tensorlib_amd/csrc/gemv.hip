@@ -188,29 +188,38 @@ struct Producer {
   float eps;
 };
 
-template <typename Fmt, int R, int PRO>
+// LPR = lanes that share a weight row: 64 (a row segment of 64 units per
+// wavefront step) or 16 (the wavefront works on 4 row groups at once, 16 units
+// of each per step). Rows whose unit count is not close to a multiple of 64 leave
+// lanes idle in the 64-lane form (K = 3584 is 112 units: 12.5 % idle; K = 896 is
+// 28 units: 56 % idle); the 16-lane form wastes at most 15 units per row and
+// finishes a row sum inside one DPP row.
+template <typename Fmt, int R, int PRO, int LPR>
 __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
     float* __restrict__ y, int N, int upr, int KW, int ntiles, const Producer pro) {
   constexpr int J = Fmt::E / 4;
+  constexpr int QN = 64 / LPR;       // row groups a wavefront works on at once
   extern __shared__ float4 smem4[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & (LPR - 1), q = lane / LPR;
   const int nw = blockDim.x >> 6;
-  const int chunks = (upr + 63) >> 6;
+  const int chunks = (upr + LPR - 1) / LPR;
   float4* xs = smem4;
-  float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * 64);  // [chunks*64], int4 only
-  float* red = xsum + (Fmt::kScaled ? chunks * 64 : 0);
+  float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * LPR);  // [chunks*LPR], int4 only
+  float* red = xsum + (Fmt::kScaled ? chunks * LPR : 0);
 
   const int kw = wave % KW;          // which K split this wavefront takes
   const int wn = wave / KW;          // which row group of the block tile
-  const int groups = nw / KW;        // row groups per block tile
-  const int rows_per_tile = groups * R;
+  const int groups = nw / KW;        // wavefront row groups per block tile
+  const int rows_per_tile = groups * QN * R;
+  const int wrow = (wn * QN + q) * R;  // this lane's first row inside a tile
 
   // The first work item's weights are requested before x is staged, so that the
   // HBM latency of the weights and the L2 latency of x overlap.
   int t = blockIdx.x, c = kw;
   RowFrag<Fmt, R> cur;
-  if (t < ntiles) load_frag<Fmt, R>(cur, W, scales, N, upr, t * rows_per_tile + wn * R, (c << 6) + lane);
+  if (t < ntiles) load_frag<Fmt, R>(cur, W, scales, N, upr, t * rows_per_tile + wrow, c * LPR + li);
 
   {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
      // thread i owns float4 i; the J threads of a unit are adjacent lanes, so the
@@ -253,7 +262,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         v.z = (v.z * inv) * w4.z; v.w = (v.w * inv) * w4.w;
       }
       const int u = i / J, j = i - u * J;
-      if (live) xs[((u >> 6) * J + j) * 64 + (u & 63)] = Fmt::stage(v);
+      if (live) xs[((u / LPR) * J + j) * LPR + (u & (LPR - 1))] = Fmt::stage(v);
       if (Fmt::kScaled) {
         float sx = (v.x + v.y) + (v.z + v.w);
 #pragma unroll
@@ -275,13 +284,13 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     int nc = c + KW, nt = t;
     if (nc >= chunks) { nc = kw; nt = t + gridDim.x; }
     if (nt < ntiles)
-      load_frag<Fmt, R>(nxt, W, scales, N, upr, nt * rows_per_tile + wn * R, (nc << 6) + lane);
+      load_frag<Fmt, R>(nxt, W, scales, N, upr, nt * rows_per_tile + wrow, nc * LPR + li);
 
-    const int u = (c << 6) + lane;
+    const int u = c * LPR + li;
     if (u < upr) {
       float4 xv[J];
 #pragma unroll
-      for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * 64 + lane];
+      for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * LPR + li];
       if (Fmt::kScaled) {
         const float bias = xsum[u];
 #pragma unroll
@@ -293,20 +302,35 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     }
 
     if (nt != t) {  // last chunk of tile t for this wavefront: reduce and store
-      const int row0 = t * rows_per_tile + wn * R;
-      const float v = wave_sum_rows<R>(acc, lane);   // total of row (lane*R)>>6, in every lane
-      const int r = (lane * R) >> 6;
-      const bool writer = (lane & (64 / R - 1)) == 0;
+      const int row0 = t * rows_per_tile + wrow;
+      float v;
+      int r;
+      bool writer;
+      if constexpr (LPR == 64) {
+        v = wave_sum_rows<R>(acc, lane);   // total of row (lane*R)>>6, in every lane
+        r = (lane * R) >> 6;
+        writer = (lane & (64 / R - 1)) == 0;
+      } else {
+        // every lane of the DPP row gets every row total; lane r keeps row r
+        v = 0.f;
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) {
+          const float tot = dpp_add_f32<0x140>(dpp_add_f32<0x141>(dpp_add_f32<0x4E>(dpp_add_f32<0xB1>(acc[rr]))));
+          v = (li == rr) ? tot : v;
+        }
+        r = li;
+        writer = li < R;
+      }
       if (KW == 1) {
         if (writer && row0 + r < N) y[row0 + r] = v;
       } else {
         // every wavefront of the block passes these two barriers once per tile
-        if (writer) red[(wn * KW + kw) * R + r] = v;
+        if (writer) red[(wrow / R * KW + kw) * R + r] = v;
         __syncthreads();
-        if (kw == 0 && lane < R && row0 + lane < N) {
+        if (kw == 0 && li < R && row0 + li < N) {
           float sum = 0.f;
-          for (int sidx = 0; sidx < KW; sidx++) sum += red[(wn * KW + sidx) * R + lane];
-          y[row0 + lane] = sum;
+          for (int sidx = 0; sidx < KW; sidx++) sum += red[(wrow / R * KW + sidx) * R + li];
+          y[row0 + li] = sum;
         }
         __syncthreads();
       }
@@ -454,56 +478,84 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
 // host side
 // ---------------------------------------------------------------------------
 
-struct RowCfg { int R, KW, nw, blocks; size_t lds; };
+struct RowCfg { int R, KW, nw, lpr, blocks; size_t lds; };
+struct RowTune { int R, KW, bpc, nw, lpr; };
 
 // Launch shape for the row kernel, from sweeps on MI355X:
-//  * one fat block per CU (16 wavefronts) so x is staged once per CU; 8-wave
-//    blocks only when a row tile must be smaller than KW allows;
-//  * rows per block tile grow with the rows a CU owns, up to 64 (4 rows per
-//    wavefront: the x fragment held in VGPRs is reused 4 times);
+//  * lanes per row: 16 when the 64-lane form would leave a large part of the
+//    lanes without a unit (K = 896 is 28 units per row), else 64;
+//  * big matrices: two 8-wavefront blocks per CU, 4 rows per wavefront;
+//    otherwise one fat block per CU (16 wavefronts) so x is staged once per CU;
+//  * rows per block tile grow with the rows a CU owns (the x fragment held in
+//    VGPRs is reused for every row a lane group owns);
 //  * K is split over KW wavefronts of a block only when rows alone cannot give
 //    every CU a tile.
-static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, int tR, int tKW,
-                            int tBPC, int tNW) {
-  const int chunks = (upr + 63) / 64;
-  const size_t xbytes = (size_t)chunks * 64 * E * 4 + (size_t)chunks * 256;
+static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, const RowTune& tn) {
   RowCfg c{};
+  const double waste64 = (double)((upr + 63) / 64 * 64) / upr, waste16 = (double)((upr + 15) / 16 * 16) / upr;
+  int lpr = (waste64 >= 1.3 && waste16 < waste64) ? 16 : 64;
+  if (tn.lpr == 16 || tn.lpr == 64) lpr = tn.lpr;
+  const int qn = 64 / lpr;
+  const int chunks = (upr + lpr - 1) / lpr;
+  const size_t xbytes = (size_t)chunks * lpr * E * 4 + (size_t)chunks * lpr * 4;
   const int64_t rows_per_cu = N / cus;
   int nw = 16, R, KW;
-  if (rows_per_cu >= 128) { R = 4; KW = 1; }        // 64 rows per block tile
-  else if (rows_per_cu >= 32) { R = 2; KW = 1; }    // 32
-  else if (rows_per_cu >= 8) { R = 2; KW = 2; }     // 16
-  else { nw = 8; R = 1; KW = 2; }                   // 4
+  if (lpr == 64) {
+    if (rows_per_cu >= 128) { nw = 8; R = 4; KW = 1; }  // two 8-wave blocks per CU, 32-row tiles
+    else if (rows_per_cu >= 64) { nw = 8; R = 4; KW = 2; }  // same blocks, 16-row tiles
+    else if (rows_per_cu >= 32) { R = 2; KW = 1; }    // 32
+    else if (rows_per_cu >= 8) { R = 2; KW = 2; }     // 16
+    else { nw = 8; R = 1; KW = 2; }                   // 4
+  } else {
+    if (rows_per_cu >= 256) { R = 2; KW = 1; }        // 128 rows per block tile
+    else if (rows_per_cu >= 64) { R = 1; KW = 1; }    // 64
+    else if (rows_per_cu >= 16) { R = 1; KW = 2; }    // 32
+    else if (rows_per_cu >= 8) { R = 1; KW = 4; }     // 16
+    else { nw = 8; R = 1; KW = 4; }                   // 8
+  }
   while (KW > chunks) {  // not enough K to split that far: more row groups instead
     KW /= 2;
     if (R > 1) R /= 2; else if (nw > 4) nw /= 2;
   }
-  if (tNW > 0) nw = tNW;
-  if (tR > 0) R = tR;
-  if (tKW > 0) KW = tKW;
+  if (tn.nw > 0) nw = tn.nw;
+  if (tn.R > 0) R = tn.R;
+  if (tn.KW > 0) KW = tn.KW;
   if (R >= 8 && nw > 8) nw = 8;  // the 8-row variant is built for <= 512 threads
   if (KW > nw) KW = nw;
-  int bpc = (int)((size_t)lds_per_cu / (xbytes + 1024));
+  int bpc = (int)((size_t)lds_per_cu / (xbytes + 4096));
   const int max_by_waves = 32 / nw > 0 ? 32 / nw : 1;
   const int want_bpc = nw >= 16 ? 1 : nw == 8 ? 2 : 4;
   if (bpc > max_by_waves) bpc = max_by_waves;
   if (bpc > want_bpc) bpc = want_bpc;
   if (bpc < 1) bpc = 1;
-  if (tBPC > 0) bpc = tBPC;
+  if (tn.bpc > 0) bpc = tn.bpc;
   c.R = R;
   c.KW = KW;
   c.nw = nw;
-  const int rows_per_tile = (nw / KW) * R;
+  c.lpr = lpr;
+  const int rows_per_tile = (nw / KW) * qn * R;
   const int64_t ntiles = (N + rows_per_tile - 1) / rows_per_tile;
   const int64_t maxb = (int64_t)cus * bpc;
   c.blocks = (int)(ntiles < maxb ? ntiles : maxb);
-  c.lds = xbytes + (size_t)nw * 8 * 4 + 64;
+  c.lds = xbytes + (size_t)nw * qn * 8 * 4 + 64;   // x, per-unit sums, K-split partials
   return c;
+}
+
+template <typename Fmt, int PRO, int LPR>
+static auto pick_rows_fn(int R) -> void (*)(const float*, const uint4*, const float*, float*, int, int,
+                                            int, int, const Producer) {
+  switch (R) {
+    case 1: return gemv_rows_kernel<Fmt, 1, PRO, LPR>;
+    case 2: return gemv_rows_kernel<Fmt, 2, PRO, LPR>;
+    case 4: return gemv_rows_kernel<Fmt, 4, PRO, LPR>;
+    case 8: return gemv_rows_kernel<Fmt, 8, PRO, LPR>;
+    default: return nullptr;
+  }
 }
 
 template <typename Fmt, int PRO = kPlain>
 static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
-                       int64_t K, int census_id, int tR, int tKW, int tBPC, int tNW,
+                       int64_t K, int census_id, const RowTune tn = RowTune{0, 0, 0, 0, 0},
                        const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
   Context& c = ctx();
   const int upr = (int)(K / Fmt::E);
@@ -512,23 +564,16 @@ static int launch_rows(const float* x, const void* W, const float* scales, float
   // larger ones are walked in row ranges of < 4 GiB, one launch each.
   int64_t max_rows = (((int64_t)1 << 32) - 16) / ((int64_t)upr * 16);
   if (max_rows >= (1 << 24)) max_rows = (1 << 24) - 1;
-  max_rows &= ~(int64_t)63;
+  max_rows &= ~(int64_t)255;
   if (max_rows <= 0) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large");
-  using K_t = void (*)(const float*, const uint4*, const float*, float*, int, int, int, int,
-                       const Producer);
   for (int64_t n0 = 0; n0 < N; n0 += max_rows) {
     const int64_t n = N - n0 < max_rows ? N - n0 : max_rows;
-    RowCfg cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, tR, tKW, tBPC, tNW);
-    const int rows_per_tile = (cfg.nw / cfg.KW) * cfg.R;
+    RowCfg cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, tn);
+    if (cfg.lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large for the LDS-staged kernel");
+    const int rows_per_tile = (cfg.nw / cfg.KW) * (64 / cfg.lpr) * cfg.R;
     const int ntiles = (int)((n + rows_per_tile - 1) / rows_per_tile);
-    K_t fn = nullptr;
-    switch (cfg.R) {
-      case 1: fn = gemv_rows_kernel<Fmt, 1, PRO>; break;
-      case 2: fn = gemv_rows_kernel<Fmt, 2, PRO>; break;
-      case 4: fn = gemv_rows_kernel<Fmt, 4, PRO>; break;
-      case 8: fn = gemv_rows_kernel<Fmt, 8, PRO>; break;
-      default: return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
-    }
+    auto fn = cfg.lpr == 16 ? pick_rows_fn<Fmt, PRO, 16>(cfg.R) : pick_rows_fn<Fmt, PRO, 64>(cfg.R);
+    if (!fn) return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
     if (cfg.lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)cfg.lds);
@@ -572,6 +617,10 @@ static int launch_cols(const float* a, const T* B, float* y, int64_t N, int64_t 
   TLHIP_CHECK_LAUNCH(census_id);
 }
 
+static RowTune q4_tune(const Context& c) {
+  return RowTune{c.tune_q4_rows, c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw, c.tune_q4_lpr};
+}
+
 static int check_gemv_args(const void* a, const void* B, const void* y, int64_t n, int64_t k,
                            const char* who) {
   if (!a || !B || !y) return fail(TLHIP_EINVAL, "%s: null pointer", who);
@@ -600,8 +649,7 @@ int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, in
   const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
   if (group == 32 && aligned16(qw) && xbytes + 2048 <= (size_t)c.lds_per_cu)
     return launch_rows<FmtQ4>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
-                              static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
-                              c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw);
+                              static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c));
   hipLaunchKernelGGL(gemv_q4_generic_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, c.stream,
                      static_cast<const float*>(a), static_cast<const uint32_t*>(qw),
                      static_cast<const float*>(scales), static_cast<float*>(y), (int)N, (int)K,
@@ -618,7 +666,7 @@ int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_
   if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K too large for the LDS-staged kernel");
   return launch_rows<FmtBf16>(static_cast<const float*>(a), W, nullptr, static_cast<float*>(y), n, k,
-                              TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0);
+                              TLHIP_C_GEMV_BF16_ROW);
 }
 
 int tlhip_gemv_f32(const void* a, const void* B, void* y, int64_t n, int64_t k) {
@@ -675,8 +723,7 @@ int tlhip_gemv_q4_swiglu(const void* gu, const void* qw, const void* scales, voi
   if (int rc = check_fused_q4(qw, scales, K, group, 2 * K, "tlhip_gemv_q4_swiglu")) return rc;
   Context& c = ctx();
   return launch_rows<FmtQ4, kSwiglu>(static_cast<const float*>(gu), qw, static_cast<const float*>(scales),
-                                     static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
-                                     c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw);
+                                     static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c));
 }
 
 int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
@@ -690,8 +737,7 @@ int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, 
   const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
                      static_cast<float*>(xout), eps};
   return launch_rows<FmtQ4, kRmsnorm>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
-                                      static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, c.tune_q4_rows,
-                                      c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw, pro);
+                                      static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c), pro);
 }
 
 int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n, int64_t k) {
@@ -699,7 +745,7 @@ int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n
   if (int rc = check_gemv_args(gu, W, y, n, k, "tlhip_gemv_bf16_row_swiglu")) return rc;
   if (int rc = check_fused_bf16(W, k, "tlhip_gemv_bf16_row_swiglu")) return rc;
   return launch_rows<FmtBf16, kSwiglu>(static_cast<const float*>(gu), W, nullptr, static_cast<float*>(y),
-                                       n, k, TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0);
+                                       n, k, TLHIP_C_GEMV_BF16_ROW);
 }
 
 int tlhip_gemv_bf16_row_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
@@ -711,7 +757,7 @@ int tlhip_gemv_bf16_row_rmsnorm(const void* x, const void* delta, const void* no
   const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
                      static_cast<float*>(xout), eps};
   return launch_rows<FmtBf16, kRmsnorm>(static_cast<const float*>(x), W, nullptr, static_cast<float*>(y),
-                                        n, k, TLHIP_C_GEMV_BF16_ROW, 0, 0, 0, 0, pro);
+                                        n, k, TLHIP_C_GEMV_BF16_ROW, RowTune{0, 0, 0, 0, 0}, pro);
 }
 
 }  // extern "C"

@@ -328,12 +328,14 @@ int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks) {
   return e == hipSuccess ? TLHIP_OK : hip_fail(e, "read kernel");
 }
 
-int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block) {
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
+                       int lanes_per_row) {
   Context& c = ctx();
   c.tune_q4_rows = rows_per_wave;
   c.tune_q4_kw = k_waves;
   c.tune_q4_bpc = blocks_per_cu;
   c.tune_q4_nw = waves_per_block;
+  c.tune_q4_lpr = lanes_per_row;
   return TLHIP_OK;
 }
 

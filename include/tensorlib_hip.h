@@ -226,10 +226,12 @@ int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
 
 /* ---- tuning hook (benchmarks only) --------------------------------------------
  * Overrides the int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts
- * sharing one row's K range (a power of two), resident blocks per CU and
- * wavefronts per block (<= 16); 0 restores the built-in choice for that field.
+ * sharing one row's K range (a power of two), resident blocks per CU,
+ * wavefronts per block (<= 16) and lanes that share a weight row (64 or 16);
+ * 0 restores the built-in choice for that field.
  * Results do not depend on it beyond fp32 summation order. */
-int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block);
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
+                       int lanes_per_row);
 
 #ifdef __cplusplus
 }

@@ -44,16 +44,17 @@ def test_gemv_q4_ragged(lib, orc, N, K):
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
+@pytest.mark.parametrize("lpr", [64, 16])
 @pytest.mark.parametrize("rows,kw", [(1, 1), (2, 1), (4, 1), (8, 1), (1, 2), (2, 4), (1, 8), (4, 2)])
-def test_gemv_q4_every_launch_shape(lib, orc, rows, kw):
-    """All (rows per wavefront, K-split) variants compute the same product."""
+def test_gemv_q4_every_launch_shape(lib, orc, rows, kw, lpr):
+    """All (rows per wavefront, K-split, lanes per row) variants compute the same product."""
     N, K = 777, 3584
-    print("case gemv_q4 tuned", rows, kw, flush=True)
-    lib.tune_gemv_q4(rows, kw, 0)
+    print("case gemv_q4 tuned", rows, kw, lpr, flush=True)
+    lib.tune_gemv_q4(rows, kw, 0, 0, lpr)
     try:
         got, want = _q4_case(lib, orc, N, K, 31, from_weights=True)
     finally:
-        lib.tune_gemv_q4(0, 0, 0)
+        lib.tune_gemv_q4(0, 0, 0, 0, 0)
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
