@@ -13,31 +13,40 @@
 // Tiling: a block of 4 wavefronts (2x2) owns a (64*TM) x (64*TN) tile of C; each
 // wavefront TM x TN MFMA tiles of 32x32. K advances in slabs of 32 through LDS:
 // the A slab is split into its three bf16 planes while it is written to LDS, the
-// W slab is copied as is. Both operands are K-contiguous per lane (A is [M,K],
+// W slab is copied as is (rows XOR-swizzled against bank conflicts). Both operands are K-contiguous per lane (A is [M,K],
 // W is [N,K]), which is exactly the MFMA operand layout: one ds_read_b128 per
 // fragment. Global loads of the next slab are in flight while the current one is
 // multiplied.
 #include "common.hpp"
-#include <cstdlib>
 
 namespace tlhip {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kBK = 32;        // K slab
-constexpr int kLDK = kBK + 8;  // LDS row pitch in bf16 (80 B: 16-byte aligned, spreads banks)
+constexpr int kBK = 32;        // K slab: an LDS row is 32 bf16 = four 16-byte chunks
 
+// LDS rows are not padded; instead the 16-byte chunk index is XORed with bits of
+// the row number. Both the fragment reads (8 consecutive rows, same chunk) and the
+// tile stores (consecutive chunks of one row, then the next row) then spread over
+// all 32 banks.
+__device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elements
+  return row * kBK + ((chunk ^ ((row >> 1) & 3)) << 3);
+}
+
+// gridDim.y > 1 is split-K: block row y takes K range [y*kchunk, (y+1)*kchunk) and
+// writes its partial product to C + y*M*N (a scratch area); splitk_sum_kernel adds
+// the parts in a fixed order.
 template <int TM, int TN>
 __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
-                                                           int K) {
+                                                           int K, int kchunk) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   constexpr int A_LOADS = BM * kBK / 4 / 256;   // float4 per thread per slab
   constexpr int B_LOADS = BN * kBK / 8 / 256;   // uint4 (8 bf16) per thread per slab
-  __shared__ __attribute__((aligned(16))) uint16_t As[3][BM][kLDK];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[BN][kLDK];
+  __shared__ __attribute__((aligned(16))) uint16_t As[3][BM * kBK];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * kBK];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -50,6 +59,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
   const int q8 = nb >> 3, r8 = nb & 7;
   const int lid = xcd * q8 + min(xcd, r8) + within;
   const int m0 = (lid % mt) * BM, n0 = (lid / mt) * BN;
+  const int kbeg = blockIdx.y * kchunk, kend = min(K, kbeg + kchunk);
+  C += (size_t)blockIdx.y * M * N;
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -66,14 +77,14 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
     for (int i = 0; i < A_LOADS; i++) {
       const int idx = tid + i * 256, row = idx >> 3, c4 = idx & 7;
       const int gm = m0 + row, gk = k0 + c4 * 4;
-      ra[i] = (gm < M && gk < K) ? *reinterpret_cast<const float4*>(A + (size_t)gm * K + gk)
+      ra[i] = (gm < M && gk < kend) ? *reinterpret_cast<const float4*>(A + (size_t)gm * K + gk)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * 256, row = idx >> 2, c8 = idx & 3;
       const int gn = n0 + row, gk = k0 + c8 * 8;
-      rb[i] = (gn < N && gk < K) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
+      rb[i] = (gn < N && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
                                  : make_uint4(0u, 0u, 0u, 0u);
     }
   };
@@ -95,36 +106,37 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
       split3(ra[i].y, h[1], m[1], l[1]);
       split3(ra[i].z, h[2], m[2], l[2]);
       split3(ra[i].w, h[3], m[3], l[3]);
-      *reinterpret_cast<uint2*>(&As[0][row][c4 * 4]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-      *reinterpret_cast<uint2*>(&As[1][row][c4 * 4]) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
-      *reinterpret_cast<uint2*>(&As[2][row][c4 * 4]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+      const int o = lds_off(row, c4 >> 1) + (c4 & 1) * 4;
+      *reinterpret_cast<uint2*>(&As[0][o]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+      *reinterpret_cast<uint2*>(&As[1][o]) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
+      *reinterpret_cast<uint2*>(&As[2][o]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * 256, row = idx >> 2, c8 = idx & 3;
-      *reinterpret_cast<uint4*>(&Bs[row][c8 * 8]) = rb[i];
+      *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8)]) = rb[i];
     }
   };
 
-  gload(0);
-  for (int k0 = 0; k0 < K; k0 += kBK) {
+  gload(kbeg);
+  for (int k0 = kbeg; k0 < kend; k0 += kBK) {
     __syncthreads();          // the previous slab has been consumed
     lstore();
     __syncthreads();
-    if (k0 + kBK < K) gload(k0 + kBK);
+    if (k0 + kBK < kend) gload(k0 + kBK);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ks++) {
-      const int kk = ks * 16 + (lane >> 5) * 8;
+      const int kc = ks * 2 + (lane >> 5);   // 16-byte chunk of the slab this lane multiplies
       bf16x8 bfrag[TN];
 #pragma unroll
       for (int j = 0; j < TN; j++)
-        bfrag[j] = *reinterpret_cast<const bf16x8*>(&Bs[wn * 32 * TN + j * 32 + (lane & 31)][kk]);
+        bfrag[j] = *reinterpret_cast<const bf16x8*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
 #pragma unroll
       for (int i = 0; i < TM; i++) {
         const int row = wm * 32 * TM + i * 32 + (lane & 31);
 #pragma unroll
         for (int p = 0; p < 3; p++) {
-          const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][row][kk]);
+          const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
 #pragma unroll
           for (int j = 0; j < TN; j++)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
@@ -148,6 +160,19 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
     }
 }
 
+// C[i] = sum_s part[s][i], s in ascending order; n4 = M*N/4 float4s per part.
+__global__ __launch_bounds__(256) void splitk_sum_kernel(const float4* __restrict__ part,
+                                                         float4* __restrict__ C, size_t n4, int S) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  float4 a = part[i];
+  for (int sidx = 1; sidx < S; sidx++) {
+    const float4 b = part[(size_t)sidx * n4 + i];
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+  }
+  C[i] = a;
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;
@@ -167,27 +192,46 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
   const float* pa = static_cast<const float*>(A);
   const uint16_t* pw = static_cast<const uint16_t*>(W);
   float* pc = static_cast<float*>(C);
-  // largest tile that still gives every CU about two blocks
+  // Largest tile that still gives every CU about two blocks. When even 128x128
+  // tiles are too few (M of one prompt chunk against a narrow N), K is split over
+  // gridDim.y instead of shrinking the tile: small tiles re-read both operands
+  // through L2 far more often per MFMA.
   auto blocks = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   const int64_t want = (int64_t)c.cus * 2;
-  int tm, tn;
-  if (blocks(128, 128) >= want) { tm = 2; tn = 2; }
-  else if (blocks(64, 128) >= want) { tm = 1; tn = 2; }
-  else { tm = 1; tn = 1; }
-  if (const char* e = getenv("TLHIP_GEMM_TILE")) { tm = e[0] - '0'; tn = e[1] - '0'; }
+  int tm = 2, tn = 2, S = 1;
+  if (blocks(128, 128) < want) {
+    S = (int)((want + blocks(128, 128) - 1) / blocks(128, 128));
+    if (S > 8) S = 8;
+    while (S > 1 && K / S < 512) S--;
+    if ((M * N) % 4 != 0 || !aligned16(C)) S = 1;   // the part sum works on float4s
+    if (S == 1) {
+      if (blocks(64, 128) >= want) { tm = 1; tn = 2; }
+      else { tm = 1; tn = 1; }
+    }
+  }
+  int kchunk = (int)K;
+  float* dst = pc;
+  if (S > 1) {
+    kchunk = (int)(((K + S - 1) / S + kBK - 1) / kBK * kBK);
+    S = (int)((K + kchunk - 1) / kchunk);
+    dst = static_cast<float*>(scratch((size_t)S * M * N * sizeof(float)));
+    if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
+  }
   const int64_t nblk = ((N + 64 * tn - 1) / (64 * tn)) * ((M + 64 * tm - 1) / (64 * tm));
   if (nblk > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
-  const dim3 grid((unsigned)nblk);
-  if (tm == 2 && tn == 4)
-    gemm_bf16_nt_kernel<2, 4><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
-  else if (tm == 1 && tn == 4)
-    gemm_bf16_nt_kernel<1, 4><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
-  else if (tm == 2)
-    gemm_bf16_nt_kernel<2, 2><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
-  else if (tn == 2)
-    gemm_bf16_nt_kernel<1, 2><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
-  else
-    gemm_bf16_nt_kernel<1, 1><<<grid, dim3(256), 0, c.stream>>>(pa, pw, pc, (int)M, (int)N, (int)K);
+  const dim3 grid((unsigned)nblk, (unsigned)S);
+#define TLHIP_GEMM(TM_, TN_)                                                                     \
+  gemm_bf16_nt_kernel<TM_, TN_><<<grid, dim3(256), 0, c.stream>>>(pa, pw, dst, (int)M, (int)N, \
+                                                                   (int)K, kchunk)
+  if (tm == 2) TLHIP_GEMM(2, 2);
+  else if (tn == 2) TLHIP_GEMM(1, 2);
+  else TLHIP_GEMM(1, 1);
+#undef TLHIP_GEMM
+  if (S > 1) {
+    const size_t n4 = (size_t)M * N / 4;
+    splitk_sum_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, c.stream>>>(
+        reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc), n4, S);
+  }
   TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
 }
 
