@@ -31,7 +31,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 SHAPES = [(3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584)]  # (N, K)
 HBM_PEAK_GBS = 8000.0
 RING_BYTES = 1.2e9      # distinct weight bytes per shape, > 4x the Infinity Cache
-LMHEAD_HBM_BYTES_PER_LAUNCH = 356_616_000   # (173831.6 KiB * 2.000 + 595.4 KiB) * 1024
+LMHEAD_HBM_BYTES_PER_LAUNCH = 356_657_000   # (173851.3 KiB * 2.000 + 595.6 KiB) * 1024
 
 
 def q4_nbytes(N, K):
@@ -327,7 +327,7 @@ def main():
                    "per_shape": per_shape},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_rows_kernel<FmtQ4,4> on 152064x3584 (LM head)",
+                     "kernel": "gemv_rows_kernel<FmtQ4,4,0,64> on 152064x3584 (LM head)",
                      "bytes_per_launch": dom["nb"], "avg_launch_us": round(dom_ms * 1e3, 2),
                      "avg_us_between_events_inside_step": round(in_step_ms * 1e3, 2)},
     }
