@@ -130,11 +130,38 @@ def decode_7b(lib, steps, eager=False):
         lib.record(e1)
         ms = lib.elapsed_ms(e0, e1) / steps
         best = ms if best is None else min(best, ms)
+    # The real loop: ONE graph recorded with the position on the device, replayed for
+    # successive tokens ending at position 4095 (ctx 4096); each token stages its embedding
+    # row (host gather + 14 KB copy) and, in the greedy form, reads the argmax back.
+    n_loop = max(steps, 32)
+    start = ctx - 2 * n_loop
+    g.set_cache_pos(start - 1)
+    captured = g.decoder_init(11, start - 1)
+    g.decoder_feed(11)                      # the first launch of a new graph pays its upload
+    g.flush()
     t = time.perf_counter()
-    for _ in range(steps):
-        g.replay()
-        g.argmax()                           # the per-token sync + 4-byte copy
-    with_argmax = (time.perf_counter() - t) / steps * 1e3
+    for i in range(n_loop):
+        g.decoder_feed(11 + i)
+    g.flush()
+    loop_feed = (time.perf_counter() - t) / n_loop * 1e3
+    tok = 11
+    t = time.perf_counter()
+    for i in range(n_loop):
+        tok = g.decoder_step(tok)
+    with_argmax = (time.perf_counter() - t) / n_loop * 1e3
+    assert g.decoder_pos() == ctx
+    # Greedy decoding with the token loop on the device: embedding gather, argmax and the
+    # token hand-over are kernels of the recorded step, so n tokens are queued back to back
+    # and the ids are read once at the end.
+    g.set_cache_pos(start - 1)
+    g.greedy_init(11, start - 1)
+    g.greedy_run(1)
+    g.flush()
+    t = time.perf_counter()
+    queued = g.greedy_run(2 * n_loop)
+    ids = g.greedy_tokens(start, queued)          # blocks until the last token exists
+    greedy_dev = (time.perf_counter() - t) / queued * 1e3
+    assert queued == 2 * n_loop and len(ids) == queued
     d = g.d
     wbytes = 0.625 * (d.n_layers * (d.hidden * (d.n_q_heads + 2 * d.n_kv_heads) * d.head_dim
                                     + d.hidden * d.n_q_heads * d.head_dim + 3 * d.hidden * d.ff)
@@ -144,10 +171,74 @@ def decode_7b(lib, steps, eager=False):
     return {
         "workload": "Qwen2.5-7B-shape int4 decode step, ctx 4096, f32 KV, hipGraph replay",
         "ms_per_token": round(best, 4), "tok_s": round(1e3 / best, 1),
-        "ms_per_token_with_argmax_sync": round(with_argmax, 4),
+        "loop": {"what": "one recorded graph, position on the device, %d successive tokens ending at "
+                         "ctx 4096, wall clock incl. embedding staging" % n_loop,
+                 "graph_captured": bool(captured),
+                 "ms_per_token_feed_only": round(loop_feed, 4),
+                 "ms_per_token_greedy_with_argmax_readback": round(with_argmax, 4),
+                 "tok_s_greedy": round(1e3 / with_argmax, 1),
+                 "ms_per_token_greedy_token_loop_on_device": round(greedy_dev, 4),
+                 "tok_s_greedy_token_loop_on_device": round(1e3 / greedy_dev, 1)},
         "algorithmic_bytes": int(wbytes + kvbytes),
         "hbm_frac": round((wbytes + kvbytes) / (best * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
     }
+
+
+def side_kernels(lib, orc):
+    """The other bandwidth-bound kernels of the path at their BASELINE shapes: the bf16 GEMV in
+    both layouts (configs[1] weights as bf16; [N,K] rows for the harness, [K,N] at the array
+    seam) and decode attention (configs[2]: q[28,128], K/V[28,ctx,128] f32). Bytes counted the
+    reference's way: 2*N*K per GEMV (bench_bf16_gemv.cpp:119), 2*H*ctx*D*4 per attention call
+    (bench_attn_decode.cpp:129). Buffers rotate so that no call re-reads what the previous one
+    left in the caches."""
+    rng = np.random.default_rng(7)
+    e0, e1 = lib.event(), lib.event()
+    out = {"gemv_bf16_row": {}, "gemv_bf16_kn": {}, "attn_decode_f32": {}}
+
+    def timed(calls, n):
+        for i in range(min(n, 3)):
+            calls(i)
+        lib.record(e0)
+        for i in range(n):
+            calls(i)
+        lib.record(e1)
+        return lib.elapsed_ms(e0, e1) / n
+
+    for (N, K) in [(3584, 3584), (18944, 3584), (3584, 18944), (152064, 3584)]:
+        nb = 2 * N * K
+        copies = max(2, int(1.2e9 // nb) + 1)
+        w = lib.empty_bytes(nb * copies)
+        host = (rng.integers(0, 65536, N * K, dtype=np.uint16) & 0x807f) | 0x3c00
+        w.upload(host)
+        for c in range(1, copies):
+            lib._chk(lib.c.tlhip_memcpy_d2d_async(w.ptr + c * nb, w.ptr, nb))
+        x, y = lib.to_device(orc.normal(K, 5)), lib.empty(N)
+        for name, fn in (("gemv_bf16_row", lib.c.tlhip_gemv_bf16_row), ("gemv_bf16_kn", lib.c.tlhip_gemv_bf16)):
+            ms = timed(lambda i: lib._chk(fn(x.ptr, w.ptr + (i % copies) * nb, y.ptr, N, K)), max(10, copies))
+            out[name]["%dx%d" % (N, K)] = {"us": round(ms * 1e3, 2), "GB/s": round(nb / ms / 1e6, 1)}
+        for b in (w, x, y):
+            b.free()
+
+    H, D = 28, 128
+    for ctx in (512, 2048, 8192, 32768):
+        per = H * ctx * D
+        copies = max(2, min(8, int(1.2e9 // (8 * per)) + 1))
+        Ks, Vs = lib.empty(per * copies), lib.empty(per * copies)
+        blk = orc.normal(min(per, 1 << 22), 9)
+        for b in (Ks, Vs):
+            for o in range(0, per * copies, len(blk)):
+                n = min(len(blk), per * copies - o)
+                lib._chk(lib.c.tlhip_memcpy_h2d(b.ptr + o * 4, blk.ctypes.data, n * 4))
+        q, o_ = lib.to_device(orc.normal(H * D, 10)), lib.empty(H * D)
+        scale = 1.0 / np.sqrt(128.0)
+        ms = timed(lambda i: lib._chk(lib.c.tlhip_attn_decode(
+            q.ptr, Ks.ptr + (i % copies) * per * 4, Vs.ptr + (i % copies) * per * 4, o_.ptr,
+            H, H, ctx, ctx, D, scale, 0)), 20)
+        nb = 2 * per * 4
+        out["attn_decode_f32"]["ctx%d" % ctx] = {"us": round(ms * 1e3, 2), "GB/s": round(nb / ms / 1e6, 1)}
+        for b in (Ks, Vs, q, o_):
+            b.free()
+    return out
 
 
 def prefill_7b(lib, rounds=3):
@@ -221,6 +312,8 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode leg")
     ap.add_argument("--eager-decode", action="store_true",
                     help="decode leg without the hipGraph (for kernel traces)")
+    ap.add_argument("--no-side", action="store_true",
+                    help="skip the bf16 GEMV and decode attention legs")
     ap.add_argument("--no-prefill", action="store_true", help="skip the 7B-shape prompt-chunk leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch the plain 1 GiB copy kernel 3 times (scale for --pmc runs)")
@@ -345,6 +438,8 @@ def main():
             cpu_ms = d["algorithmic_bytes"] / (cpu_gbs * 1e9) * 1e3
             d["cpu_reference_ms_per_token_est"] = round(cpu_ms, 1)
             d["speedup_vs_cpu_reference_est"] = round(cpu_ms / d["ms_per_token"], 1)
+    if not a.no_side:
+        out["side_kernels"] = side_kernels(lib, orc)
     if not a.no_prefill:
         out["prefill"] = prefill_7b(lib)
     print(json.dumps(out))

@@ -76,6 +76,14 @@ SIGNATURES = {
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
     "tlhip_qkv_rope_append": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
+    "tlhip_rope_dpos": (cint, [P, P, i64, i64, i64, P, f32, P]),
+    "tlhip_incr_u32": (cint, [P]),
+    "tlhip_kv_append_dpos": (cint, [P, P, P, P, P, i64, i64, i64, cint]),
+    "tlhip_attn_partials_bytes": (i64, [i64, i64, i64, i64]),
+    "tlhip_attn_decode_dpos": (cint, [P, P, P, P, i64, i64, P, i64, i64, f32, cint, P, i64]),
+    "tlhip_qkv_rope_append_dpos": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, f32, cint]),
+    "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
+    "tlhip_token_advance": (cint, [P, P, P, i64]),
     "tlhip_gemv_q4_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
     "tlhip_gemv_bf16_row_swiglu": (cint, [P, P, P, i64, i64]),
     "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
@@ -290,6 +298,36 @@ class TlHip:
     def qkv_rope_append(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, D, pos, kv_max, base, kv_bf16=False):
         self._chk(self.c.tlhip_qkv_rope_append(qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None,
                                                Kc.ptr, Vc.ptr, Hq, Hkv, D, pos, kv_max, base, int(kv_bf16)))
+
+    def rope_dpos(self, x, out, rows, T, D, d_pos, base, bias=None):
+        self._chk(self.c.tlhip_rope_dpos(x.ptr, out.ptr, rows, T, D, d_pos.ptr, base,
+                                         bias.ptr if bias is not None else None))
+
+    def incr_u32(self, d_pos):
+        self._chk(self.c.tlhip_incr_u32(d_pos.ptr))
+
+    def kv_append_dpos(self, Kc, Vc, k, v, d_pos, kv_max, Hkv, D, kv_bf16=False):
+        self._chk(self.c.tlhip_kv_append_dpos(Kc.ptr, Vc.ptr, k.ptr, v.ptr, d_pos.ptr, kv_max, Hkv, D,
+                                              int(kv_bf16)))
+
+    def attn_partials_bytes(self, Hq, Hkv, kv_max, D):
+        return int(self.c.tlhip_attn_partials_bytes(Hq, Hkv, kv_max, D))
+
+    def attn_decode_dpos(self, q, K, V, out, Hq, Hkv, d_pos, kv_max, D, scale, partials, kv_bf16=False):
+        self._chk(self.c.tlhip_attn_decode_dpos(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, d_pos.ptr, kv_max,
+                                                D, scale, int(kv_bf16), partials.ptr, partials.nbytes))
+
+    def qkv_rope_append_dpos(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, D, d_pos, kv_max, base, kv_bf16=False):
+        self._chk(self.c.tlhip_qkv_rope_append_dpos(
+            qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None, Kc.ptr, Vc.ptr, Hq, Hkv, D,
+            d_pos.ptr, kv_max, base, int(kv_bf16)))
+
+    def embed_gather_bf16(self, table, d_token, out, hidden, vocab):
+        self._chk(self.c.tlhip_embed_gather_bf16(table.ptr, d_token.ptr, out.ptr, hidden, vocab))
+
+    def token_advance(self, d_pos, d_token, history, capacity):
+        self._chk(self.c.tlhip_token_advance(d_pos.ptr, d_token.ptr,
+                                             history.ptr if history is not None else None, capacity))
 
     def gemv_q4_swiglu(self, gu, wq, y, N, K, group=32):
         self._chk(self.c.tlhip_gemv_q4_swiglu(gu.ptr, wq.ptr, wq.ptr + N * K // 2, y.ptr, N, K, group))

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
     float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
     float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, int TK,
-    float scale, int S, int T, int pos0) {
+    float scale, int S, int T, int pos0, const uint32_t* __restrict__ dpos) {
   constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
   constexpr int NV = EPL / 4;        // float4 loads per lane per key
   constexpr int UNR = 4;             // key steps in flight per lane
@@ -75,6 +75,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int slot = lane >> 4, c = lane & 15;     // DPP row = key slot, c = position in the row
   const int split = blockIdx.y;
+  // Position kept on the device (captured decode loops): the grid was planned for
+  // the cache capacity, the live context is *dpos + 1. Splits past it find no keys
+  // and write neutral partials (m = -inf, l = 0, acc = 0).
+  if (!PRE && dpos) ctx = min(ctx, (int)*dpos + 1);
   int kvh, g0, ng, k_begin, k_end;
   size_t row0;                                   // index of row g = 0 in q / out, in rows of D
   if constexpr (PRE) {
@@ -239,7 +243,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     for (int w = 1; w < nw; w++) M = fmaxf(M, st_m[w][g]);
     float L = 0.f, A = 0.f;
     for (int w = 0; w < nw; w++) {
-      const float f = __expf(st_m[w][g] - M);   // idle waves: exp(-inf) = 0
+      // waves (or whole blocks, with a device-side position) that saw no key weigh 0
+      const float f = st_m[w][g] == -INFINITY ? 0.f : __expf(st_m[w][g] - M);
       L = fmaf(st_l[w][g], f, L);
       A = fmaf(st_acc[w][g][d], f, A);
     }
@@ -336,22 +341,42 @@ static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus) {
   int want_s = (int)((want_waves + (int64_t)base * p.nw - 1) / ((int64_t)base * p.nw));
   if (want_s < 1) want_s = 1;
   if (want_s > block_tiles) want_s = block_tiles;
-  const int tiles_per_wave = (block_tiles + want_s - 1) / want_s;
+  // nearest, not ceiling: 34 tiles for 32 wanted splits is 34 splits of one tile per
+  // wave, not 17 of two
+  int tiles_per_wave = (block_tiles + want_s / 2) / want_s;
+  if (tiles_per_wave < 1) tiles_per_wave = 1;
   p.chunk = tiles_per_wave * p.nw * p.TK;
   p.S = (ctx + p.chunk - 1) / p.chunk;
   return p;
 }
 
+static size_t attn_partials_floats(int Hq, int S, int D) {
+  const size_t hs = (size_t)Hq * S;
+  return hs * 2 + hs * D;
+}
+
+// dpos != nullptr: ctx is the cache CAPACITY the grid is planned for, the live
+// context is read from the device, and the split partials live in a buffer the
+// caller owns (a captured graph bakes the address in).
 template <int D, typename KT>
 static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
-                       int ctx, int64_t kv_max, float scale) {
+                       int ctx, int64_t kv_max, float scale, const uint32_t* dpos = nullptr,
+                       float* partials = nullptr, size_t partials_bytes = 0) {
   Context& c = tlhip::ctx();
   const int group = Hq / Hkv;
   const AttnPlan p = plan_attn(Hkv, group, ctx, c.cus);
   float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
   if (p.S > 1) {
     const size_t hs = (size_t)Hq * p.S;
-    float* base = static_cast<float*>(scratch((hs * 2 + hs * D) * sizeof(float)));
+    const size_t need = attn_partials_floats(Hq, p.S, D) * sizeof(float);
+    float* base;
+    if (dpos) {
+      if (!partials || partials_bytes < need)
+        return fail(TLHIP_EINVAL, "tlhip_attn_decode_dpos: partials buffer of %zu bytes needed", need);
+      base = partials;
+    } else {
+      base = static_cast<float*>(scratch(need));
+    }
     if (!base) return fail(TLHIP_ENOMEM, "tlhip_attn_decode: no scratch for %d splits", p.S);
     pm = base;
     pl = pm + hs;
@@ -362,7 +387,7 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
   const int64_t kv_stride = kv_max * D;
 #define TLHIP_ATTN(GG)                                                                         \
   hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false>), grid, block, 0, c.stream, q, K, V, \
-                     out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0)
+                     out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0, dpos)
   switch (p.G) {
     case 1: TLHIP_ATTN(1); break;
     case 2: TLHIP_ATTN(2); break;
@@ -384,7 +409,7 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
   const dim3 grid(Hq, 1, (T + G - 1) / G), block(256);
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
                      (float*)nullptr, (float*)nullptr, (float*)nullptr, Hq / Hkv, pos0 + T,
-                     kv_max * D, 0, 64, scale, 1, T, pos0);
+                     kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
 }
 
@@ -451,6 +476,44 @@ int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out, i
   const float* pv = static_cast<const float*>(V);
   return D == 128 ? launch_prefill<128, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0)
                   : launch_prefill<64, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0);
+}
+
+int64_t tlhip_attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_max, int64_t D) {
+  if (!ctx().ready || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || kv_max <= 0 ||
+      kv_max > 0x3fffffff || (D != 64 && D != 128))
+    return 0;
+  const AttnPlan p = plan_attn((int)n_kv_heads, (int)(n_q_heads / n_kv_heads), (int)kv_max, ctx().cus);
+  return (int64_t)(attn_partials_floats((int)n_q_heads, p.S, (int)D) * sizeof(float)) + 16;
+}
+
+int tlhip_attn_decode_dpos(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                           int64_t n_kv_heads, const void* d_pos, int64_t kv_max, int64_t D,
+                           float scale, int kv_bf16, void* partials, int64_t partials_bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!q || !K || !V || !out || !d_pos) return fail(TLHIP_EINVAL, "tlhip_attn_decode_dpos: null pointer");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_dpos: head_dim must be 64 or 128");
+  if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_dpos: Hq must be a positive multiple of Hkv");
+  if (kv_max <= 0 || kv_max > 0x3fffffff || n_kv_heads > 65535 || kv_max * D > ((int64_t)1 << 40))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_dpos: shape too large");
+  if (!aligned16(q) || !aligned16(K) || !aligned16(V) || !aligned16(out) || (partials && !aligned16(partials)))
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_dpos: operands must be 16-byte aligned");
+  const float* pq = static_cast<const float*>(q);
+  float* po = static_cast<float*>(out);
+  const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
+  float* pp = static_cast<float*>(partials);
+  const size_t pb = partials_bytes > 0 ? (size_t)partials_bytes : 0;
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads, cap = (int)kv_max;
+  if (kv_bf16) {
+    const uint16_t* pk = static_cast<const uint16_t*>(K);
+    const uint16_t* pv = static_cast<const uint16_t*>(V);
+    return D == 128 ? launch_attn<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb)
+                    : launch_attn<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb);
+  }
+  const float* pk = static_cast<const float*>(K);
+  const float* pv = static_cast<const float*>(V);
+  return D == 128 ? launch_attn<128, float>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb)
+                  : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb);
 }
 
 }  // extern "C"

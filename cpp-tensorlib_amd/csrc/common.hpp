@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <vector>
 
 #include <cstdarg>
 #include <cstdint>
@@ -25,6 +26,10 @@ struct Context {
   // grow-only device scratch (split-K / split-KV partials, argmax partials)
   void* scratch = nullptr;
   size_t scratch_bytes = 0;
+  // A recorded graph bakes the scratch address into its kernel nodes: once any graph
+  // exists, an outgrown scratch buffer is retired (kept allocated), never freed.
+  int graphs_recorded = 0;
+  std::vector<void*> retired_scratch;
   int* argmax_dev = nullptr;      // one int32 result slot
   int* argmax_host = nullptr;     // pinned landing slot for the 4-byte result
   uint64_t census[TLHIP_C_COUNT] = {};

@@ -14,10 +14,12 @@ namespace tlhip {
 __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x,
                                                    const float* __restrict__ bias,
                                                    float* __restrict__ out, int64_t rows, int T,
-                                                   int D, int64_t pos, float base) {
+                                                   int D, int64_t pos, float base,
+                                                   const uint32_t* __restrict__ dpos) {
   const int half = D >> 1;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= rows * half) return;
+  if (dpos) pos = (int64_t)*dpos;   // position kept on the device (captured decode loops)
   const int64_t r = i / half;
   const int j = (int)(i - r * half);
   const int64_t t = T ? r % T : 0;
@@ -216,9 +218,14 @@ __global__ __launch_bounds__(256) void kv_write_kernel(KT* __restrict__ Kc, KT* 
                                                        const float* __restrict__ k,
                                                        const float* __restrict__ v, int64_t T,
                                                        int64_t kv_max, int D, int64_t pos0,
-                                                       int64_t total) {
+                                                       int64_t total,
+                                                       const uint32_t* __restrict__ dpos) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
+  if (dpos) {
+    pos0 = (int64_t)*dpos;
+    if (pos0 + T > kv_max) return;   // a full cache drops the write instead of leaving it
+  }
   const int d = (int)(i % D);
   const int64_t hp = i / D;
   const int64_t p = hp % T, h = hp / T;
@@ -261,7 +268,11 @@ template <typename KT>
 __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
     float* __restrict__ qkv, const float* __restrict__ bq, const float* __restrict__ bk,
     const float* __restrict__ bv, KT* __restrict__ Kc, KT* __restrict__ Vc, int Hq, int Hkv, int D,
-    int64_t pos, int64_t kv_max, float base) {
+    int64_t pos, int64_t kv_max, float base, const uint32_t* __restrict__ dpos) {
+  if (dpos) {   // position kept on the device; a full cache drops the step's writes
+    pos = (int64_t)*dpos;
+    if (pos >= kv_max) return;
+  }
   const int half = D >> 1;
   const int n_rot = (Hq + Hkv) * half;       // rotary pairs of q and k
   const int n_v = Hkv * D;
@@ -295,6 +306,28 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
   }
 }
 
+__global__ void incr_u32_kernel(uint32_t* p) { *p += 1u; }
+
+// ---- device-resident greedy loop --------------------------------------------------------
+// out[j] = widen(table[tok][j]) with tok read from the device (the previous step's argmax).
+__global__ __launch_bounds__(256) void embed_gather_bf16_kernel(const uint16_t* __restrict__ table,
+                                                                const int* __restrict__ d_token,
+                                                                float* __restrict__ out, int hidden,
+                                                                int vocab) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= hidden) return;
+  int tok = *d_token;
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  out[j] = __uint_as_float((uint32_t)table[(size_t)tok * hidden + j] << 16);
+}
+
+// history[*d_pos] = *d_token (when it fits), then *d_pos += 1: the tail of a recorded greedy step.
+__global__ void token_advance_kernel(uint32_t* d_pos, const int* d_token, int* history, uint32_t capacity) {
+  const uint32_t p = *d_pos;
+  if (history && p < capacity) history[p] = *d_token;
+  *d_pos = p + 1u;
+}
+
 static unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
 
 }  // namespace tlhip
@@ -303,9 +336,8 @@ using namespace tlhip;
 
 extern "C" {
 
-int tlhip_rope(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos,
-               float base, const void* bias) {
-  TLHIP_REQUIRE_READY();
+static int rope_launch(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos,
+                       float base, const void* bias, const void* d_pos) {
   if (!x || !out || rows < 0 || T < 0) return fail(TLHIP_EINVAL, "tlhip_rope: bad arguments");
   if (D <= 0 || (D & 1)) return fail(TLHIP_EUNSUPPORTED, "tlhip_rope: head_dim must be even");  // cuda.h:1208
   if (rows == 0) return TLHIP_OK;
@@ -313,8 +345,30 @@ int tlhip_rope(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int
   if (n > (int64_t)0x7fffffff * 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_rope: too large");
   rope_kernel<<<dim3(blocks_for(n)), dim3(256), 0, ctx().stream>>>(
       static_cast<const float*>(x), static_cast<const float*>(bias), static_cast<float*>(out), rows,
-      (int)T, (int)D, pos, base);
+      (int)T, (int)D, pos, base, static_cast<const uint32_t*>(d_pos));
   TLHIP_CHECK_LAUNCH(TLHIP_C_ROPE);
+}
+
+int tlhip_rope(const void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos,
+               float base, const void* bias) {
+  TLHIP_REQUIRE_READY();
+  return rope_launch(x, out, rows, T, D, pos, base, bias, nullptr);
+}
+
+int tlhip_rope_dpos(const void* x, void* out, int64_t rows, int64_t T, int64_t D, const void* d_pos,
+                    float base, const void* bias) {
+  TLHIP_REQUIRE_READY();
+  if (!d_pos) return fail(TLHIP_EINVAL, "tlhip_rope_dpos: null position pointer");
+  return rope_launch(x, out, rows, T, D, 0, base, bias, d_pos);
+}
+
+int tlhip_incr_u32(void* d_pos) {
+  TLHIP_REQUIRE_READY();
+  if (!d_pos) return fail(TLHIP_EINVAL, "tlhip_incr_u32: null pointer");
+  incr_u32_kernel<<<dim3(1), dim3(1), 0, ctx().stream>>>(static_cast<uint32_t*>(d_pos));
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  return TLHIP_OK;
 }
 
 int tlhip_rmsnorm(const void* x, const void* w, void* out, int64_t n, float eps, int64_t rows) {
@@ -381,8 +435,9 @@ int tlhip_argmax(const void* in, int64_t n, int64_t* out_idx) {
 
 static int kv_write(void* Kc, void* Vc, const void* k, const void* v, int64_t T, int64_t kv_max,
                     int64_t n_kv_heads, int64_t D, int kv_bf16, int64_t pos0, int census_id,
-                    const char* who) {
+                    const char* who, const void* d_pos = nullptr) {
   if (!Kc || !Vc || !k || !v) return fail(TLHIP_EINVAL, "%s: null pointer", who);
+  const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
   if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "%s: head_dim must be 64 or 128", who);  // cuda.h:1122
   if (T <= 0 || n_kv_heads <= 0 || pos0 < 0 || pos0 + T > kv_max)
     return fail(TLHIP_EINVAL, "%s: rows [%lld,%lld) outside the cache of %lld", who, (long long)pos0,
@@ -391,12 +446,46 @@ static int kv_write(void* Kc, void* Vc, const void* k, const void* v, int64_t T,
   if (kv_bf16)
     kv_write_kernel<uint16_t><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<uint16_t*>(Kc), static_cast<uint16_t*>(Vc), static_cast<const float*>(k),
-        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total);
+        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total, dp);
   else
     kv_write_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<float*>(Kc), static_cast<float*>(Vc), static_cast<const float*>(k),
-        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total);
+        static_cast<const float*>(v), T, kv_max, (int)D, pos0, total, dp);
   TLHIP_CHECK_LAUNCH(census_id);
+}
+
+int tlhip_embed_gather_bf16(const void* table, const void* d_token, void* out, int64_t hidden,
+                            int64_t vocab) {
+  TLHIP_REQUIRE_READY();
+  if (!table || !d_token || !out) return fail(TLHIP_EINVAL, "tlhip_embed_gather_bf16: null pointer");
+  if (hidden <= 0 || vocab <= 0 || hidden > 0x7fffffff || vocab > 0x7fffffff)
+    return fail(TLHIP_EINVAL, "tlhip_embed_gather_bf16: bad sizes");
+  embed_gather_bf16_kernel<<<dim3(blocks_for(hidden)), dim3(256), 0, ctx().stream>>>(
+      static_cast<const uint16_t*>(table), static_cast<const int*>(d_token), static_cast<float*>(out),
+      (int)hidden, (int)vocab);
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  return TLHIP_OK;
+}
+
+int tlhip_token_advance(void* d_pos, const void* d_token, void* history, int64_t capacity) {
+  TLHIP_REQUIRE_READY();
+  if (!d_pos || !d_token) return fail(TLHIP_EINVAL, "tlhip_token_advance: null pointer");
+  if (capacity < 0 || capacity > 0xffffffffll) return fail(TLHIP_EINVAL, "tlhip_token_advance: bad capacity");
+  token_advance_kernel<<<dim3(1), dim3(1), 0, ctx().stream>>>(
+      static_cast<uint32_t*>(d_pos), static_cast<const int*>(d_token), static_cast<int*>(history),
+      (uint32_t)capacity);
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  return TLHIP_OK;
+}
+
+int tlhip_kv_append_dpos(void* Kc, void* Vc, const void* k_new, const void* v_new, const void* d_pos,
+                         int64_t kv_max, int64_t n_kv_heads, int64_t D, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  if (!d_pos) return fail(TLHIP_EINVAL, "tlhip_kv_append_dpos: null position pointer");
+  return kv_write(Kc, Vc, k_new, v_new, 1, kv_max, n_kv_heads, D, kv_bf16, 0, TLHIP_C_KV_APPEND,
+                  "tlhip_kv_append_dpos", d_pos);
 }
 
 int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, int64_t pos,
@@ -406,32 +495,51 @@ int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, in
                   "tlhip_kv_append");
 }
 
-int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
-                          void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
-                          int64_t kv_max, float base, int kv_bf16) {
-  TLHIP_REQUIRE_READY();
+static int qkv_rope_append_launch(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                                  void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
+                                  int64_t pos, int64_t kv_max, float base, int kv_bf16,
+                                  const void* d_pos) {
   if (!qkv || !Kc || !Vc) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: null pointer");
   if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_append: head_dim must be 64 or 128");
   if (n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads > 4096)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_append: bad head counts");
-  if (pos < 0 || pos >= kv_max) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: row %lld outside the cache of %lld",
-                                            (long long)pos, (long long)kv_max);
+  if (!d_pos && (pos < 0 || pos >= kv_max))
+    return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: row %lld outside the cache of %lld",
+                (long long)pos, (long long)kv_max);
   const int64_t total = (n_q_heads + n_kv_heads) * (D / 2) + n_kv_heads * D;
   const float* pbq = static_cast<const float*>(bq);
   const float* pbk = static_cast<const float*>(bk);
+  const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
   if (kv_bf16)
     qkv_rope_append_kernel<uint16_t><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<uint16_t*>(Kc),
-        static_cast<uint16_t*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base);
+        static_cast<uint16_t*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp);
   else
     qkv_rope_append_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<float*>(Kc),
-        static_cast<float*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base);
+        static_cast<float*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp);
   hipError_t e_ = hipGetLastError();
   if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
   ctx().census[TLHIP_C_ROPE]++;
   ctx().census[TLHIP_C_KV_APPEND]++;
   return TLHIP_OK;
+}
+
+int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                          void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                          int64_t kv_max, float base, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  return qkv_rope_append_launch(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos, kv_max, base,
+                                kv_bf16, nullptr);
+}
+
+int tlhip_qkv_rope_append_dpos(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                               void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
+                               const void* d_pos, int64_t kv_max, float base, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  if (!d_pos) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append_dpos: null position pointer");
+  return qkv_rope_append_launch(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, 0, kv_max, base,
+                                kv_bf16, d_pos);
 }
 
 int tlhip_kv_fill(void* Kc, void* Vc, const void* K, const void* V, int64_t T, int64_t kv_max,

@@ -15,6 +15,8 @@ namespace {
 struct handle {
   qwen::model M;
   qwen::captured_step cap;
+  qwen::captured_decoder dec;
+  qwen::greedy_loop loop;
   std::map<std::string, const void*> pending;  // weight blobs of the layer being assembled
 };
 }  // namespace
@@ -124,6 +126,50 @@ int tlq_capture(void* hv, int64_t token, int64_t pos) {
   qwen::stage_embed(h->M, token);
   return h->cap.capture(h->M, pos) ? 0 : -1;
 }
+// A decode loop on one recorded graph with the position on the device.
+int tlq_decoder_init(void* hv, int64_t first_id, int64_t pos) {
+  auto* h = static_cast<handle*>(hv);
+  h->dec.destroy();
+  return h->dec.init(h->M, first_id, pos) ? 0 : -1;
+}
+int tlq_decoder_feed(void* hv, int64_t id) {
+  auto* h = static_cast<handle*>(hv);
+  return h->dec.feed(h->M, id) ? 0 : -1;
+}
+int64_t tlq_decoder_step(void* hv, int64_t id, float* logits_out) {
+  auto* h = static_cast<handle*>(hv);
+  const int64_t tok = h->dec.step(h->M, id);
+  if (tok >= 0 && logits_out)
+    std::memcpy(logits_out, qwen::logits(h->M), (size_t)h->M.d.vocab * sizeof(float));
+  return tok;
+}
+int64_t tlq_decoder_pos(void* hv) { return static_cast<handle*>(hv)->dec.cur_pos; }
+int tlq_decoder_captured(void* hv) { return static_cast<handle*>(hv)->dec.ok() ? 1 : 0; }
+void tlq_decoder_sync_host_pos(void* hv) {
+  auto* h = static_cast<handle*>(hv);
+  h->dec.sync_host_pos(h->M);
+}
+
+// Greedy decoding with the token loop on the device.
+int tlq_greedy_init(void* hv, int64_t first_id, int64_t pos) {
+  auto* h = static_cast<handle*>(hv);
+  h->loop.destroy();
+  return h->loop.init(h->M, first_id, pos) ? 0 : -1;
+}
+int64_t tlq_greedy_run(void* hv, int64_t n) { return static_cast<handle*>(hv)->loop.run(n); }
+// Copies the tokens generated at positions [from, from + n) into out (blocks until done).
+int tlq_greedy_tokens(void* hv, int64_t from, int64_t n, int32_t* out) {
+  auto* h = static_cast<handle*>(hv);
+  if (from < 0 || from + n > h->loop.cur_pos) return -1;
+  const int32_t* t = h->loop.tokens();
+  std::memcpy(out, t + from, (size_t)n * sizeof(int32_t));
+  return 0;
+}
+void tlq_greedy_sync_host_pos(void* hv) {
+  auto* h = static_cast<handle*>(hv);
+  h->loop.sync_host_pos(h->M);
+}
+
 void tlq_set_fused(void* hv, int on) { static_cast<handle*>(hv)->M.fused = on != 0; }
 int tlq_replay(void* hv) { return static_cast<handle*>(hv)->cap.replay() ? 0 : -1; }
 void tlq_flush() { hip::flush(); }

@@ -32,7 +32,8 @@ void* scratch(size_t bytes) {
   if (c.capturing) return nullptr;  // growing would synchronise mid-capture
   if (c.scratch) {
     (void)hipStreamSynchronize(c.stream);
-    (void)hipFree(c.scratch);
+    if (c.graphs_recorded > 0) c.retired_scratch.push_back(c.scratch);  // a graph may still point at it
+    else (void)hipFree(c.scratch);
     c.scratch = nullptr;
     c.scratch_bytes = 0;
   }
@@ -245,6 +246,7 @@ int tlhip_graph_end(void** graph_exec) {
   e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
   (void)hipGraphDestroy(g);
   if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+  c.graphs_recorded++;
   *graph_exec = ex;
   return TLHIP_OK;
 }

@@ -25,6 +25,7 @@
 #include <dlfcn.h>
 
 #include <cstdint>
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -110,6 +111,17 @@ struct api {
   int (*merge_heads)(const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*qkv_rope_append)(void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
                          int64_t, int64_t, int64_t, float, int) = nullptr;
+  int (*rope_dpos)(const void*, void*, int64_t, int64_t, int64_t, const void*, float, const void*) = nullptr;
+  int (*incr_u32)(void*) = nullptr;
+  int (*kv_append_dpos)(void*, void*, const void*, const void*, const void*, int64_t, int64_t, int64_t,
+                        int) = nullptr;
+  int64_t (*attn_partials_bytes)(int64_t, int64_t, int64_t, int64_t) = nullptr;
+  int (*attn_decode_dpos)(const void*, const void*, const void*, void*, int64_t, int64_t, const void*,
+                          int64_t, int64_t, float, int, void*, int64_t) = nullptr;
+  int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
+                              int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
+  int (*embed_gather_bf16)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
+  int (*token_advance)(void*, const void*, void*, int64_t) = nullptr;
   int (*gemv_q4_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*gemv_bf16_row_swiglu)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
   int (*gemv_q4_rmsnorm)(const void*, const void*, const void*, void*, const void*, const void*, void*,
@@ -124,6 +136,11 @@ struct context {
   bool ready = false;
   bool pending = false;
   bool capturing = false;
+  // Buffers a capture recorded writes to. A replay runs no launcher, so it is
+  // graph_launch that marks them device-owned again: a host reader after a replay
+  // must fetch, not trust the copy it made after the previous one.
+  std::vector<uintptr_t> capture_writes;
+  std::unordered_map<void*, std::vector<uintptr_t>> graph_writes;
   std::string why;  // why the backend is unavailable (diagnostics only)
 
   // Host/device mirror per allocation, keyed by the device pointer (== the
@@ -192,6 +209,13 @@ struct context {
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
               bind(f.qkv_rope_append, "tlhip_qkv_rope_append") &&
+              bind(f.rope_dpos, "tlhip_rope_dpos") && bind(f.incr_u32, "tlhip_incr_u32") &&
+              bind(f.kv_append_dpos, "tlhip_kv_append_dpos") &&
+              bind(f.attn_partials_bytes, "tlhip_attn_partials_bytes") &&
+              bind(f.attn_decode_dpos, "tlhip_attn_decode_dpos") &&
+              bind(f.qkv_rope_append_dpos, "tlhip_qkv_rope_append_dpos") &&
+              bind(f.embed_gather_bf16, "tlhip_embed_gather_bf16") &&
+              bind(f.token_advance, "tlhip_token_advance") &&
               bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
               bind(f.gemv_bf16_row_swiglu, "tlhip_gemv_bf16_row_swiglu") &&
               bind(f.gemv_q4_rmsnorm, "tlhip_gemv_q4_rmsnorm") &&
@@ -236,6 +260,7 @@ struct context {
       f.memcpy_h2d(m->dev, m->host, m->bytes);
     }
     m->where = DEVICE;
+    if (capturing) capture_writes.push_back(reinterpret_cast<uintptr_t>(m->dev));
   }
 };
 
@@ -621,6 +646,105 @@ inline bool qkv_rope_append(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
                                               kv_max, base, kv_bf16 ? 1 : 0));
 }
 
+// ---- device-side position (cuda.h:1011-1114) ------------------------------------------
+// Twins of rope / kv_append / attn_decode that take the position from a 4-byte
+// device scalar `d_pos`, on grids that do not depend on it, so one recorded graph
+// serves every token of a decode loop.
+inline bool rope_dpos(void* x, void* out, int64_t rows, int64_t T, int64_t D, void* d_pos, float base,
+                      void* bias = nullptr) {
+  auto& c = context::get();
+  if (!c.ready || D <= 0 || (D & 1) || !d_pos) return false;
+  c.device_read_(x);
+  if (bias) c.device_read_(bias);
+  c.device_read_(d_pos);
+  c.device_write_(out);
+  return detail::done_(c, c.f.rope_dpos(x, out, rows, T, D, d_pos, base, bias));
+}
+inline bool incr_u32(void* d_pos) {
+  auto& c = context::get();
+  if (!c.ready || !d_pos) return false;
+  c.device_read_(d_pos);
+  c.device_write_(d_pos);
+  return detail::done_(c, c.f.incr_u32(d_pos));
+}
+inline bool kv_append_dpos(void* Kc, void* Vc, void* k_new, void* v_new, void* d_pos, int64_t kv_max,
+                           int64_t n_kv_heads, int64_t D, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || !d_pos) return false;
+  c.device_read_(k_new);
+  c.device_read_(v_new);
+  c.device_read_(d_pos);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.kv_append_dpos(Kc, Vc, k_new, v_new, d_pos, kv_max, n_kv_heads, D,
+                                             kv_bf16 ? 1 : 0));
+}
+// Bytes of the caller-owned split-partials buffer attn_decode_dpos needs for a cache.
+inline int64_t attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_max, int64_t D) {
+  auto& c = context::get();
+  return c.ready ? c.f.attn_partials_bytes(n_q_heads, n_kv_heads, kv_max, D) : 0;
+}
+inline bool attn_decode_dpos(void* q, void* K, void* V, void* out, int64_t n_q_heads,
+                             int64_t n_kv_heads, void* d_pos, int64_t kv_max, int64_t D, float scale,
+                             void* partials, int64_t partials_bytes, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || !partials || !d_pos) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  c.device_read_(q);
+  c.device_read_(K);
+  c.device_read_(V);
+  c.device_read_(d_pos);
+  c.device_write_(out);
+  c.device_write_(partials);
+  return detail::done_(c, c.f.attn_decode_dpos(q, K, V, out, n_q_heads, n_kv_heads, d_pos, kv_max, D,
+                                               scale, kv_bf16 ? 1 : 0, partials, partials_bytes));
+}
+inline bool qkv_rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
+                                 int64_t n_q_heads, int64_t n_kv_heads, int64_t D, void* d_pos,
+                                 int64_t kv_max, float base, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || !d_pos) return false;
+  c.device_read_(qkv);
+  if (bq) c.device_read_(bq);
+  if (bk) c.device_read_(bk);
+  if (bv) c.device_read_(bv);
+  c.device_read_(d_pos);
+  c.device_write_(qkv);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.qkv_rope_append_dpos(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D,
+                                                   d_pos, kv_max, base, kv_bf16 ? 1 : 0));
+}
+
+// ---- device-resident greedy loop -----------------------------------------------------------
+// The next token never visits the host: the embedding row of *d_token (a device
+// int32, what argmax_async wrote) is gathered on the device, and the step's tail
+// appends the token to a device history and advances the position.
+inline bool embed_gather_bf16(void* table, void* d_token, void* out, int64_t hidden, int64_t vocab) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(table);
+  c.device_read_(d_token);
+  c.device_write_(out);
+  return detail::done_(c, c.f.embed_gather_bf16(table, d_token, out, hidden, vocab));
+}
+inline bool argmax_async(void* in, int64_t n, void* d_token) {
+  auto& c = context::get();
+  if (!c.ready || !d_token) return false;
+  c.device_read_(in);
+  c.device_write_(d_token);
+  return detail::done_(c, c.f.argmax_async(in, n, d_token));
+}
+inline bool token_advance(void* d_pos, void* d_token, void* history, int64_t capacity) {
+  auto& c = context::get();
+  if (!c.ready || !d_pos || !d_token) return false;
+  c.device_read_(d_pos);
+  c.device_read_(d_token);
+  c.device_write_(d_pos);
+  if (history) c.device_write_(history);
+  return detail::done_(c, c.f.token_advance(d_pos, d_token, history, capacity));
+}
+
 // GEMVs that evaluate the producer of their activation vector while staging it:
 // swiglu(gu) -> GEMV and rmsnorm_res(x, delta) -> GEMV in one launch each. They
 // decline (false) on shapes the fused kernel does not take; the caller then
@@ -679,6 +803,7 @@ inline bool capture_begin() {
   if (c.pending) flush();
   if (c.f.graph_begin() != 0) return false;
   c.capturing = true;
+  c.capture_writes.clear();
   return true;
 }
 inline void* capture_end() {
@@ -688,16 +813,31 @@ inline void* capture_end() {
   int rc = c.f.graph_end(&g);
   c.capturing = false;
   c.pending = false;  // recorded launches did not run
-  return rc == 0 ? g : nullptr;
+  if (rc != 0 || !g) return nullptr;
+  std::sort(c.capture_writes.begin(), c.capture_writes.end());
+  c.capture_writes.erase(std::unique(c.capture_writes.begin(), c.capture_writes.end()),
+                         c.capture_writes.end());
+  c.graph_writes[g] = std::move(c.capture_writes);
+  c.capture_writes.clear();
+  return g;
 }
 inline bool graph_launch(void* g) {
   auto& c = context::get();
   if (!c.ready || !g) return false;
-  return detail::done_(c, c.f.graph_launch(g));
+  if (!detail::done_(c, c.f.graph_launch(g))) return false;
+  auto it = c.graph_writes.find(g);
+  if (it != c.graph_writes.end())
+    for (uintptr_t a : it->second) {
+      auto m = c.mirrors.find(a);
+      if (m != c.mirrors.end()) m->second.where = context::DEVICE;
+    }
+  return true;
 }
 inline void graph_destroy(void* g) {
   auto& c = context::get();
-  if (c.ready && g) c.f.graph_destroy(g);
+  if (!c.ready || !g) return;
+  c.graph_writes.erase(g);
+  c.f.graph_destroy(g);
 }
 
 // ---- persistent KV cache (cuda.h:1321-1405) --------------------------------------
@@ -734,6 +874,18 @@ struct kv_cache {
   }
   bool attn(void* q, void* out, int64_t n_q_heads, float scale) {
     return attn_decode(q, K, V, out, n_q_heads, n_kv_heads, pos, max_ctx, D, scale, kv_bf16);
+  }
+  // The same two with the position on the device (the host pos is NOT advanced:
+  // a recorded graph replays these; captured_decoder reconciles pos afterwards).
+  bool rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, int64_t n_q_heads, float base,
+                        void* d_pos) {
+    return qkv_rope_append_dpos(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, D, d_pos, max_ctx, base,
+                                kv_bf16);
+  }
+  bool attn_dpos(void* q, void* out, int64_t n_q_heads, float scale, void* d_pos, void* partials,
+                 int64_t partials_bytes) {
+    return attn_decode_dpos(q, K, V, out, n_q_heads, n_kv_heads, d_pos, max_ctx, D, scale, partials,
+                            partials_bytes, kv_bf16);
   }
   bool prefill(void* q, void* k_src, void* v_src, void* out, int64_t T, int64_t n_q_heads,
                float scale) {

@@ -123,6 +123,9 @@ struct model {
   linear lm_head;
   std::vector<layer> layers;
   scratch s;
+  void* embed_dev = nullptr;           // the embedding table on the device (greedy_loop only)
+  void* attn_partials = nullptr;       // split partials of the device-position attention
+  int64_t attn_partials_bytes = 0;
   bool ready = false;
   // true: fused launches (q/k/v epilogue + append; norms and swiglu evaluated inside the
   // GEMV that consumes them). false: the reference's call sequence, one launch per op.
@@ -398,7 +401,12 @@ inline void stage_embed(model& M, int64_t token) {
 // All layers + final norm + lm_head on the scratch buffers, no allocation, no
 // sync: capturable as one graph. Reads the layer-0 residual from x0, writes
 // logits to S.logitsb (or logits_out).
-inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullptr) {
+// With d_pos (a 4-byte device scalar holding the position) the cache append and the
+// attention take the position from the device on position-independent grids, and the
+// scalar is advanced at the end: the launch sequence is then the same for every
+// token and one recorded graph serves a whole decode loop (qm:673-740 with d_pos).
+inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullptr,
+                       void* d_pos = nullptr, bool advance = true) {
   const dims& d = M.d;
   scratch& S = M.s;
   const float scale = 1.0f / std::sqrt((float)d.head_dim);
@@ -415,9 +423,15 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     for (int64_t l = 0; l < d.n_layers; l++) {
       layer& L = M.layers[(size_t)l];
       ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
-      L.cache.pos = pos;
-      ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
-      ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
+      if (d_pos) {
+        ok &= L.cache.rope_append_dpos(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base, d_pos);
+        ok &= L.cache.attn_dpos(S.qkvb, S.ab, d.n_q_heads, scale, d_pos, M.attn_partials,
+                                M.attn_partials_bytes);
+      } else {
+        L.cache.pos = pos;
+        ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
+        ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
+      }
       ok &= gemv(L.wo, S.ab, S.hb);
       ok &= gemv_rmsnorm(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.gub, d.eps);
       ok &= gemv_swiglu(L.wd, S.gub, S.mdb);
@@ -425,8 +439,10 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
       din = S.mdb;
     }
     ok &= gemv_rmsnorm(M.lm_head, rin, din, M.onorm, nullptr, logits_out ? logits_out : S.logitsb, d.eps);
+    if (d_pos && advance) ok &= hip::incr_u32(d_pos);
     return ok;
   }
+  if (d_pos) return false;  // the one-launch-per-op sequence is kept on the host position
   void* x = x0;
   ok &= hip::rmsnorm(x, M.layers[0].an, S.hb, E, d.eps);
   for (int64_t l = 0; l < d.n_layers; l++) {
@@ -584,6 +600,162 @@ struct captured_step {
   void destroy() {
     hip::graph_destroy(graph);
     graph = nullptr;
+  }
+};
+
+// Copy the host embedding table to the device once, through a pinned staging block.
+inline bool upload_embed(model& M) {
+  if (M.embed_dev) return true;
+  const int64_t bytes = (int64_t)M.embed.size() * 2;
+  if (bytes <= 0) return false;
+  M.embed_dev = hip::alloc_device(bytes);
+  if (!M.embed_dev) return false;
+  const int64_t blk = int64_t(32) << 20;
+  float* stage_host = nullptr;
+  void* stage = hip::alloc(blk, &stage_host);
+  if (!stage) return false;
+  bool ok = true;
+  for (int64_t o = 0; o < bytes && ok; o += blk) {
+    const int64_t n = std::min(blk, bytes - o);
+    std::memcpy(stage_host, reinterpret_cast<const char*>(M.embed.data()) + o, (size_t)n);
+    hip::upload(stage, stage_host, (n + 3) / 4);
+    ok = hip::copy_d2d(static_cast<char*>(M.embed_dev) + o, stage, n);
+    hip::flush();   // the staging block is reused
+  }
+  hip::release(stage, blk, stage_host);
+  return ok;
+}
+
+// Greedy decoding with the whole token loop on the device: one recorded graph does
+//   embedding gather of *d_tok -> layers at *d_pos -> lm_head -> argmax -> *d_tok,
+//   history[*d_pos] = *d_tok, *d_pos += 1
+// so consecutive tokens are queued back to back with no host round trip between them
+// (the reference stages each embedding on the host and reads every argmax back:
+// qm:530-535, 642-647). The host reads the generated ids from the history afterwards.
+struct greedy_loop {
+  void *d_pos = nullptr, *d_tok = nullptr, *history = nullptr, *graph = nullptr;
+  float* history_host = nullptr;
+  int64_t cur_pos = 0, max_ctx = 0;
+
+  bool init(model& M, int64_t first_id, int64_t pos) {
+    if (M.layers.empty() || !M.fused || !hip::graph_available()) return false;
+    const dims& d = M.d;
+    max_ctx = M.layers[0].cache.max_ctx;
+    cur_pos = pos;
+    if (!upload_embed(M)) return false;
+    if (!M.attn_partials) {
+      M.attn_partials_bytes = hip::attn_partials_bytes(d.n_q_heads, d.n_kv_heads, max_ctx, d.head_dim);
+      M.attn_partials = hip::alloc_device(M.attn_partials_bytes);
+      if (!M.attn_partials) return false;
+    }
+    d_pos = hip::alloc(4, nullptr);
+    d_tok = hip::alloc(4, nullptr);
+    history = hip::alloc(max_ctx * 4, &history_host);
+    if (!d_pos || !d_tok || !history) return false;
+    auto one = [&]() {
+      bool ok = hip::embed_gather_bf16(M.embed_dev, d_tok, M.s.embedb, d.hidden, d.vocab);
+      ok = ok && run_layers(M, M.s.embedb, 0, nullptr, d_pos, /*advance=*/false);
+      ok = ok && hip::argmax_async(M.s.logitsb, d.vocab, d_tok);
+      return ok && hip::token_advance(d_pos, d_tok, history, max_ctx);
+    };
+    hip::upload_u32(d_pos, (unsigned)pos);
+    hip::upload_u32(d_tok, (unsigned)first_id);
+    if (!one()) return false;            // warm run (sizes the library's scratch)
+    hip::flush();
+    hip::upload_u32(d_pos, (unsigned)pos);
+    hip::upload_u32(d_tok, (unsigned)first_id);
+    if (!hip::capture_begin()) return false;
+    const bool ok = one();
+    graph = hip::capture_end();
+    if (!ok && graph) { hip::graph_destroy(graph); graph = nullptr; }
+    return graph != nullptr;
+  }
+  // Queue n greedy steps (no sync). Returns how many were queued before the cache filled.
+  int64_t run(int64_t n) {
+    int64_t done = 0;
+    while (done < n && cur_pos < max_ctx && graph && hip::graph_launch(graph)) {
+      cur_pos++;
+      done++;
+    }
+    return done;
+  }
+  // The token generated at position p (p in [first pos, cur_pos)); blocks until the queue drained.
+  const int32_t* tokens() {
+    hip::sync_to_host(history, false);
+    return reinterpret_cast<const int32_t*>(history_host);
+  }
+  void sync_host_pos(model& M) const { set_cache_pos(M, cur_pos); }
+  void destroy() {
+    if (graph) hip::graph_destroy(graph);
+    for (void* b : {d_pos, d_tok, history})
+      if (b) hip::release(b, 0, nullptr);
+    graph = d_pos = d_tok = history = nullptr;
+  }
+};
+
+// A decode loop on ONE recorded graph (qm:791-905): the position lives in a device
+// scalar that the recorded forward advances itself, so feed()/step() replay the same
+// graph for every token. Falls back to the imperative path when capture is not
+// available; callers never branch on ok().
+struct captured_decoder {
+  void* d_pos = nullptr;
+  void* graph = nullptr;
+  int64_t cur_pos = 0, max_ctx = 0;
+
+  // Record the forward at `pos` (the first position this decoder will process).
+  bool init(model& M, int64_t first_id, int64_t pos) {
+    if (M.layers.empty()) return false;
+    max_ctx = M.layers[0].cache.max_ctx;
+    cur_pos = pos;
+    if (!hip::graph_available() || !M.fused) return false;
+    const dims& d = M.d;
+    if (!M.attn_partials) {
+      M.attn_partials_bytes = hip::attn_partials_bytes(d.n_q_heads, d.n_kv_heads, max_ctx, d.head_dim);
+      M.attn_partials = hip::alloc_device(M.attn_partials_bytes);
+      if (!M.attn_partials) return false;
+    }
+    d_pos = hip::alloc(4, nullptr);
+    if (!d_pos) return false;
+    stage_embed(M, first_id);
+    hip::upload_u32(d_pos, (unsigned)pos);
+    // warm run: real launches (they also size the library's scratch); it advances d_pos
+    // and writes cache row pos, which the first recorded step rewrites identically
+    if (!run_layers(M, M.s.embedb, pos, nullptr, d_pos)) return false;
+    hip::flush();
+    hip::upload_u32(d_pos, (unsigned)pos);
+    if (!hip::capture_begin()) return false;
+    const bool ok = run_layers(M, M.s.embedb, pos, nullptr, d_pos);  // recorded, not executed
+    graph = hip::capture_end();
+    if (!ok && graph) { hip::graph_destroy(graph); graph = nullptr; }
+    return graph != nullptr;
+  }
+  // Feed token `id` at the current position without reading a token back.
+  bool feed(model& M, int64_t id) {
+    if (cur_pos >= max_ctx) return false;
+    stage_embed(M, id);
+    bool ok;
+    if (graph) ok = hip::graph_launch(graph);
+    else ok = run_layers(M, M.s.embedb, cur_pos);
+    cur_pos++;
+    return ok;
+  }
+  // One decode step: feed + greedy token (-1 when the cache is full or a launch failed).
+  int64_t step(model& M, int64_t id) {
+    if (!feed(M, id)) return -1;
+    int64_t idx = -1;
+    return hip::argmax(M.s.logitsb, M.d.vocab, &idx) ? idx : -1;
+  }
+  // Replays advance only the device counter; bring the host cache position up to date
+  // before switching to a host-position call.
+  void sync_host_pos(model& M) const {
+    if (graph) set_cache_pos(M, cur_pos);
+  }
+  bool ok() const { return graph != nullptr; }
+  void destroy() {
+    if (graph) hip::graph_destroy(graph);
+    if (d_pos) hip::release(d_pos, 0, nullptr);
+    graph = nullptr;
+    d_pos = nullptr;
   }
 };
 

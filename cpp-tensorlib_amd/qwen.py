@@ -57,6 +57,16 @@ def _load():
             "tlq_capture": (cint, [P, i64, i64]),
             "tlq_replay": (cint, [P]),
             "tlq_set_fused": (None, [P, cint]),
+            "tlq_greedy_init": (cint, [P, i64, i64]),
+            "tlq_greedy_run": (i64, [P, i64]),
+            "tlq_greedy_tokens": (cint, [P, i64, i64, P]),
+            "tlq_greedy_sync_host_pos": (None, [P]),
+            "tlq_decoder_init": (cint, [P, i64, i64]),
+            "tlq_decoder_feed": (cint, [P, i64]),
+            "tlq_decoder_step": (i64, [P, i64, P]),
+            "tlq_decoder_pos": (i64, [P]),
+            "tlq_decoder_captured": (cint, [P]),
+            "tlq_decoder_sync_host_pos": (None, [P]),
             "tlq_flush": (None, []),
             "tlq_census": (cint, [C.POINTER(C.c_uint64), cint]),
         }
@@ -159,6 +169,51 @@ class QwenGPU:
     def replay(self):
         if self.L.tlq_replay(self.h) != 0:
             raise RuntimeError("graph replay failed")
+
+    # ---- greedy decoding with the token loop on the device -----------------------------
+    def greedy_init(self, first_id, pos):
+        """Record ONE graph: embedding gather of the device token -> layers -> lm_head ->
+        argmax -> device token; position and token history stay on the device."""
+        if self.L.tlq_greedy_init(self.h, first_id, pos) != 0:
+            raise RuntimeError("greedy loop: graph capture failed")
+
+    def greedy_run(self, n):
+        """Queue n greedy steps back to back (no sync); returns how many were queued."""
+        return int(self.L.tlq_greedy_run(self.h, n))
+
+    def greedy_tokens(self, start, n):
+        """Tokens generated at positions [start, start+n) (blocks until they exist)."""
+        out = np.empty(n, np.int32)
+        if self.L.tlq_greedy_tokens(self.h, start, n, _p(out)) != 0:
+            raise RuntimeError("greedy_tokens: range not generated yet")
+        return out
+
+    def greedy_sync_host_pos(self):
+        self.L.tlq_greedy_sync_host_pos(self.h)
+
+    # ---- a decode loop on ONE recorded graph, position kept on the device ----------
+    def decoder_init(self, first_id, pos):
+        """Record the forward at `pos`; returns True when a graph was captured (otherwise
+        feed/step run the imperative path)."""
+        self.L.tlq_decoder_init(self.h, first_id, pos)
+        return bool(self.L.tlq_decoder_captured(self.h))
+
+    def decoder_feed(self, token):
+        if self.L.tlq_decoder_feed(self.h, token) != 0:
+            raise RuntimeError("decoder feed failed (cache full or launch declined)")
+
+    def decoder_step(self, token, want_logits=False):
+        logits = np.empty(self.d.vocab, np.float32) if want_logits else None
+        tok = self.L.tlq_decoder_step(self.h, token, _p(logits) if want_logits else None)
+        if tok < 0:
+            raise RuntimeError("decoder step failed (cache full or launch declined)")
+        return (int(tok), logits) if want_logits else int(tok)
+
+    def decoder_pos(self):
+        return int(self.L.tlq_decoder_pos(self.h))
+
+    def decoder_sync_host_pos(self):
+        self.L.tlq_decoder_sync_host_pos(self.h)
 
     def set_fused(self, on):
         self.L.tlq_set_fused(self.h, 1 if on else 0)

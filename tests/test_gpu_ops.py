@@ -209,3 +209,49 @@ def test_qkv_rope_append_equals_unfused(lib, orc, Hq, Hkv, D):
     assert not Kc.any() and not Vc.any()
     with pytest.raises(RuntimeError):
         lib.qkv_rope_append(d1, dbq, dbk, dbv, K1, V1, Hq, Hkv, D, kv_max, kv_max, 1e6)
+
+
+def test_device_position_twins_equal_host_position_calls(lib, orc):
+    """rope_dpos / kv_append_dpos / qkv_rope_append_dpos read the position from a device
+    scalar and are otherwise the host-position kernels: bit-identical results, and
+    incr_u32 advances the scalar (cuda.h:1011-1060)."""
+    Hq, Hkv, D, kv_max, base = 6, 2, 64, 50, 1e6
+    dpos = lib.to_device(np.array([0], np.uint32))
+    for pos in (0, 7, 49):
+        dpos.upload(np.array([pos], np.uint32))
+        x = orc.normal(Hq * D, 300 + pos).reshape(Hq, D)
+        bias = orc.normal(Hq * D, 301).reshape(Hq, D)
+        dx, db, o1, o2 = lib.to_device(x), lib.to_device(bias), lib.empty((Hq, D)), lib.empty((Hq, D))
+        lib.rope(dx, o1, Hq, 1, D, pos, base, bias=db)
+        lib.rope_dpos(dx, o2, Hq, 1, D, dpos, base, bias=db)
+        assert np.array_equal(o1.numpy(), o2.numpy())
+        k, v = orc.normal(Hkv * D, 302).reshape(Hkv, D), orc.normal(Hkv * D, 303).reshape(Hkv, D)
+        dk, dv = lib.to_device(k), lib.to_device(v)
+        caches = [lib.to_device(np.zeros((Hkv, kv_max, D), np.float32)) for _ in range(4)]
+        lib.kv_append(caches[0], caches[1], dk, dv, pos, kv_max, Hkv, D)
+        lib.kv_append_dpos(caches[2], caches[3], dk, dv, dpos, kv_max, Hkv, D)
+        assert np.array_equal(caches[0].numpy(), caches[2].numpy())
+        assert np.array_equal(caches[1].numpy(), caches[3].numpy())
+        assert np.array_equal(caches[0].numpy()[:, pos, :], k)
+        qkv = orc.normal((Hq + 2 * Hkv) * D, 304)
+        bq, bk, bv = (lib.to_device(orc.normal(n, 305 + i)) for i, n in enumerate((Hq * D, Hkv * D, Hkv * D)))
+        q1, q2 = lib.to_device(qkv), lib.to_device(qkv)
+        lib.qkv_rope_append(q1, bq, bk, bv, caches[0], caches[1], Hq, Hkv, D, pos, kv_max, base)
+        lib.qkv_rope_append_dpos(q2, bq, bk, bv, caches[2], caches[3], Hq, Hkv, D, dpos, kv_max, base)
+        assert np.array_equal(q1.numpy(), q2.numpy())
+        assert np.array_equal(caches[0].numpy(), caches[2].numpy())
+        assert np.array_equal(caches[1].numpy(), caches[3].numpy())
+        for b in [dx, db, o1, o2, dk, dv, q1, q2, bq, bk, bv] + caches:
+            b.free()
+    dpos.upload(np.array([41], np.uint32))
+    lib.incr_u32(dpos)
+    lib.incr_u32(dpos)
+    assert int(dpos.numpy()[0]) == 43
+    # a full cache drops the write instead of running past the end
+    dpos.upload(np.array([kv_max], np.uint32))
+    Kc, Vc = lib.to_device(np.zeros((Hkv, kv_max, D), np.float32)), lib.to_device(np.zeros((Hkv, kv_max, D), np.float32))
+    dk = lib.to_device(np.ones((Hkv, D), np.float32))
+    lib.kv_append_dpos(Kc, Vc, dk, dk, dpos, kv_max, Hkv, D)
+    assert not Kc.numpy().any() and not Vc.numpy().any()
+    for b in (dpos, Kc, Vc, dk):
+        b.free()
