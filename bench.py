@@ -53,16 +53,21 @@ def make_q4_host(orc, N, K, seed):
     return out
 
 
-def cpu_baseline(orc, refl, budget_s=20.0):
+def cpu_baseline(orc, refl, budget_s=25.0):
     """The reference CPU path (x.dot(Wq) in use_cpu() mode: per-call widening to f32
-    plus cpu::sgemm on ONE thread, array.h:1980-1984, cpu.h:436-438) on a bounded
-    sample: the 512x3584 and 3584x3584 GEMVs of the sweep, median of 3 after a warm-up.
-    Falls back to the plain-C restatement when oracle/_ref was not built."""
+    plus cpu::sgemm on ONE thread, array.h:1980-1984, cpu.h:436-438) on the sweep's own
+    shapes, smallest first: median of 3 calls after a warm-up for the four smaller ones,
+    one call for the LM head; a shape is skipped once the time budget is spent (the sample
+    says which were timed). Falls back to the plain-C restatement when oracle/_ref was
+    not built."""
     import ctypes as C
-    sample = [(512, 3584), (3584, 3584)]
-    total_bytes, total_s = 0, 0.0
+    total_bytes, total_s, timed = 0, 0.0, []
     t_start = time.time()
-    for (N, K) in sample:
+    for (N, K) in sorted(SHAPES, key=lambda s: s[0] * s[1]):
+        big = N * K > 10 ** 8
+        est = 0.62 * N * K / 0.1e9 * (1.3 if big else 4.2)     # ~0.1 GB/s, calls incl. warm-up
+        if time.time() - t_start + est > budget_s and timed:
+            continue
         buf = orc.fill_q4(N, K, 77)
         x = orc.normal(K, 78)
         y = np.empty(N, np.float32)
@@ -74,24 +79,26 @@ def cpu_baseline(orc, refl, budget_s=20.0):
             run = lambda: orc.lib.orc_gemv_q4(x.ctypes.data_as(C.c_void_p), buf.ctypes.data_as(C.c_void_p),
                                               y.ctypes.data_as(C.c_void_p), N, K, 1.0, 0.0,
                                               ws.ctypes.data_as(C.c_void_p))
-        run()
         ts = []
-        for _ in range(3):
+        if not big:
+            run()
+        for _ in range(1 if big else 3):
             t = time.perf_counter()
             run()
             ts.append(time.perf_counter() - t)
-            if time.time() - t_start > budget_s:
-                break
         if refl is not None:
             refl.lib.tlref_gemv_free(h)
         total_bytes += q4_nbytes(N, K)
         total_s += float(np.median(ts))
+        timed.append("%dx%d" % (N, K))
     return {
         "value": round(total_bytes / total_s / 1e9, 4), "unit": "GB/s", "cores": 1,
         "kind": "reference" if refl is not None else "port",
-        "sample": "int4 x.dot(Wq) at 512x3584 and 3584x3584 (2 of the 5 sweep shapes), median of 3; "
-                  "the reference's dot at M=1 runs on one thread whatever the core count",
-        "ms": round(total_s * 1e3, 2), "host_cores_online": os.cpu_count(),
+        "sample": "int4 x.dot(Wq) at %s (%d of the 5 sweep shapes; median of 3 calls, one call for "
+                  "the LM head); the reference's dot at M=1 runs on one thread whatever the core "
+                  "count" % (", ".join(timed), len(timed)),
+        "ms": round(total_s * 1e3, 2), "cpu_seconds_spent": round(time.time() - t_start, 1),
+        "host_cores_online": os.cpu_count(),
     }
 
 
