@@ -19,7 +19,7 @@ def _run(lib, q, K, V, ctx, scale, kv_bf16=False):
     return out
 
 
-@pytest.mark.parametrize("ctx", [512, 2048, 8192])
+@pytest.mark.parametrize("ctx", [512, 2048, 8192, 32768])
 def test_attn_config3(lib, orc, ctx):
     """BASELINE config 3: q[28,128], K/V[28,ctx,128] ~ N(0,1), scale 1/sqrt(128)."""
     H, D = 28, 128
@@ -131,3 +131,22 @@ def test_attn_decode_device_position(lib, orc, D, Hq, Hkv, kv_max):
         small.free()
     for b in (dq, dk, dv, do, part, dpos):
         b.free()
+
+
+def test_attn_full_size_properties(lib, orc):
+    """BASELINE config 3 at its largest context (ctx 32768, 0.94 GB of f32 K/V) through
+    properties that need no oracle run: constant keys make the output the plain mean of V
+    for every head; adding a constant to all scores (a key offset along q) leaves the
+    output unchanged; the result does not depend on rows of the cache past ctx."""
+    H, D, ctx = 28, 128, 32768
+    q = orc.normal(H * D, 1).reshape(H, D)
+    V = orc.normal(H * ctx * D, 3).reshape(H, ctx, D)
+    K = np.tile(orc.normal(H * D, 2).reshape(H, 1, D), (1, ctx, 1))       # every key of a head identical
+    scale = 1.0 / np.sqrt(128.0)
+    got = _run(lib, q, K, V, ctx, scale)
+    want = V.astype(np.float64).mean(axis=1)
+    assert allclose(got, want, 1e-4, 2e-5), maxrel(got, want)
+    K2 = orc.normal(H * ctx * D, 4).reshape(H, ctx, D)
+    base = _run(lib, q, K2, V, ctx, scale)
+    shifted = _run(lib, q, K2 + (q / np.sum(q * q, axis=1, keepdims=True))[:, None, :] * 3.0, V, ctx, scale)
+    assert allclose(shifted, base, 2e-4, 2e-5), maxrel(shifted, base)

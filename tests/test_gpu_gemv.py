@@ -245,3 +245,34 @@ def test_gemv_fused_rejects_aliasing_and_other_groups(lib, pkg):
     with pytest.raises(pkg.TlHipError) as e:
         lib.gemv_q4_swiglu(x, w, y, 8, 32, group=8)
     assert e.value.code == -3
+
+
+def test_gemv_q4_full_size_linearity(lib, orc):
+    """The LM-head shape of BASELINE config 2 (152064x3584, 340 MB) through size-independent
+    properties: y(a + b) = y(a) + y(b), y(2a) = 2 y(a) exactly, y(0) = 0 exactly, and a one-hot
+    a picks column k of the dequantised matrix (checked against the stored nibbles and scales
+    of a few rows)."""
+    N, K = 152064, 3584
+    buf = orc.fill_q4(N, K, 5)
+    dw = lib.to_device(buf)
+    def run(a):
+        da, dy = lib.to_device(a.astype(np.float32)), lib.empty(N)
+        lib.gemv_q4(da, dw, dy, N, K)
+        out = dy.numpy()
+        da.free(); dy.free()
+        return out
+    a, b = orc.normal(K, 6), orc.normal(K, 7)
+    ya, yb, yab = run(a), run(b), run(a + b)
+    assert allclose(yab, ya + yb, 1e-4, 2e-5), maxrel(yab, ya + yb)
+    assert np.array_equal(run(2.0 * a), 2.0 * ya)
+    assert not run(np.zeros(K)).any()
+    k = 1234
+    col = run(np.eye(1, K, k).reshape(K))
+    packed = buf[:N * K // 2].reshape(N, K // 2)
+    scales = buf[N * K // 2:].view(np.float32).reshape(N, K // 32)
+    rows = np.array([0, 1, 77, N // 2, N - 1])
+    byte = packed[rows, k // 2]
+    nib = (byte >> 4) if (k & 1) else (byte & 15)
+    want = scales[rows, k // 32] * (nib.astype(np.float32) - 8.0)
+    assert np.allclose(col[rows], want, rtol=1e-6, atol=1e-7)
+    dw.free()
