@@ -418,15 +418,12 @@ __global__ __launch_bounds__(256) void gemv_cols_kernel(const float* __restrict_
   if (col < N) {  // N % V == 0 is guaranteed by the launcher
     const T* bp = B + col;
     int k = k0 + w;
-    for (; k + 12 < k1; k += 16) {  // 4 rows in flight per lane
-      const Raw b0 = *reinterpret_cast<const Raw*>(bp + (size_t)k * N);
-      const Raw b1 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 4) * N);
-      const Raw b2 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 8) * N);
-      const Raw b3 = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 12) * N);
-      ColVec<T>::fma(acc, a[k], b0);
-      ColVec<T>::fma(acc, a[k + 4], b1);
-      ColVec<T>::fma(acc, a[k + 8], b2);
-      ColVec<T>::fma(acc, a[k + 12], b3);
+    for (; k + 28 < k1; k += 32) {  // 8 rows in flight per lane
+      Raw b[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) b[u] = *reinterpret_cast<const Raw*>(bp + (size_t)(k + 4 * u) * N);
+#pragma unroll
+      for (int u = 0; u < 8; u++) ColVec<T>::fma(acc, a[k + 4 * u], b[u]);
     }
     for (; k < k1; k += 4) {
       const Raw b0 = *reinterpret_cast<const Raw*>(bp + (size_t)k * N);
@@ -593,9 +590,9 @@ static int launch_cols(const float* a, const T* B, float* y, int64_t N, int64_t 
   constexpr int V = ColVec<T>::V;
   const bool vec = (N % V) == 0 && aligned16(B);
   const int64_t ctiles = vec ? (N + 64 * V - 1) / (64 * V) : (N + 255) / 256;
-  // K splits: fill ~8 blocks per CU, keep >= 64 rows per split
-  int64_t S = ((int64_t)c.cus * 8 + ctiles - 1) / ctiles;
-  if (S > K / 64) S = K / 64;
+  // K splits: fill ~4 blocks per CU, keep >= 128 rows per split (32 per wavefront)
+  int64_t S = ((int64_t)c.cus * 4 + ctiles - 1) / ctiles;
+  if (S > K / 128) S = K / 128;
   if (S < 1) S = 1;
   int kchunk = (int)((K + S - 1) / S);
   kchunk = (kchunk + 3) & ~3;
