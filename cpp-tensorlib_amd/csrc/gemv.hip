@@ -229,11 +229,17 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const int n4_padded = (n4 + 63) & ~63;   // whole wavefronts take part in the shuffles
     const float4* d4 = reinterpret_cast<const float4*>(pro.delta);
     float inv = 0.f;
+    // the first two float4s a thread owns (all of them for rows up to 2 * blockDim * 4
+    // floats) stay in registers between the two passes of the norm
+    float4 kept0 = make_float4(0.f, 0.f, 0.f, 0.f), kept1 = kept0;
     if (PRO == kRmsnorm) {   // mean square of the row, summed in a fixed order
       float ss = 0.f;
-      for (int i = tid; i < n4; i += blockDim.x) {
+      int it = 0;
+      for (int i = tid; i < n4; i += blockDim.x, it++) {
         float4 v = x4[i];
         if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
+        if (it == 0) kept0 = v;
+        if (it == 1) kept1 = v;
         ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
       }
       ss = wave_sum(ss);
@@ -244,9 +250,12 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       inv = 1.0f / sqrtf(tot * (1.0f / (float)(n4 * 4)) + pro.eps);
       // red is reused only after the barrier that ends the staging pass
     }
-    for (int i = tid; i < n4_padded; i += blockDim.x) {
+    int it2 = 0;
+    for (int i = tid; i < n4_padded; i += blockDim.x, it2++) {
       const bool live = i < n4;
-      float4 v = live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      const bool have = PRO == kRmsnorm && it2 < 2;   // already summed with delta, in registers
+      float4 v = have ? (it2 == 0 ? kept0 : kept1)
+                      : live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
       if (PRO == kSwiglu && live) {
         const float4 up = x4[n4 + i];
         v.x = (v.x * (1.0f / (1.0f + expf(-v.x)))) * up.x;
@@ -255,7 +264,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         v.w = (v.w * (1.0f / (1.0f + expf(-v.w)))) * up.w;
       }
       if (PRO == kRmsnorm && live) {
-        if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
+        if (d4 && !have) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
         if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
         const float4 w4 = reinterpret_cast<const float4*>(pro.norm_w)[i];
         v.x = (v.x * inv) * w4.x; v.y = (v.y * inv) * w4.y;
