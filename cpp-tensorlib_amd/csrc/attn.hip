@@ -54,11 +54,11 @@ __device__ __forceinline__ float row16_sum(float v) {
 // (one per DPP row), each lane holding EPL = D/16 consecutive floats of its key.
 // part_m/part_l: [Hq*S], part_acc: [Hq*S*D]; used when S > 1, else `out` is final.
 //
-// PRE = true is causal prefill over q/out [Hq, T, D]: grid = (Hq, 1, ceil(T/G)),
-// and the G rows of a block are G consecutive query positions of ONE head, which
-// share the K/V stream exactly like the query heads of a GQA group do in decode.
-// Row g of tile z sees keys [0, pos0 + z*G + g]; later keys of the tile are
-// masked per row. Tiles run longest-first. S is 1.
+// PRE = true is causal prefill over q/out [Hq, T, D]: grid = (Hq, 1, ceil(T/(4G))).
+// A WAVEFRONT owns G consecutive query positions of one head, which share the K/V
+// stream exactly like the query heads of a GQA group do in decode, and walks all
+// of their keys itself (no merge between wavefronts). Row g sees keys
+// [0, pos0 + p_g]; later keys of a tile are masked per row. Longest rows first.
 template <int D, int G, typename KT, bool PRE>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
@@ -84,12 +84,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   if constexpr (PRE) {
     const int h = blockIdx.x;
     kvh = h / group;
-    g0 = (gridDim.z - 1 - blockIdx.z) * G;       // first query position of the tile
+    // every wavefront owns G query rows of its own and walks ALL of their keys: no
+    // merge between wavefronts, and the four of a block read the same K/V rows at
+    // about the same time (the later ones hit in L1/L2)
+    g0 = ((gridDim.z - 1 - blockIdx.z) * nw + wave) * G;   // first query position of this wavefront
+    if (g0 >= T) return;                                   // (no block-wide barrier follows in this mode)
     ng = min(G, T - g0);
     row0 = (size_t)h * T + g0;
     k_begin = 0;
     k_end = pos0 + g0 + ng;                      // the last row's limit
-    TK = k_end >= 256 ? 64 : k_end >= 128 ? 32 : 16;
+    TK = k_end >= 64 ? 64 : k_end >= 32 ? 32 : 16;
   } else {
     kvh = blockIdx.x;
     g0 = blockIdx.z * G;
@@ -120,7 +124,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     for (int v = 0; v < NV; v++) acc[g][v] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
 
-  for (int kb = k_begin + wave * TK; kb < k_end; kb += nw * TK) {
+  const int kb_first = PRE ? 0 : k_begin + wave * TK, kb_step = PRE ? TK : nw * TK;
+  for (int kb = kb_first; kb < k_end; kb += kb_step) {
     // ---- scores: lane (slot,c) ends up holding key kb + c*4 + slot (c < steps) ----
     float sreg[G];
 #pragma unroll
@@ -230,10 +235,20 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         acc[g][v].z += __shfl_xor(acc[g][v].z, msk, kWave);
         acc[g][v].w += __shfl_xor(acc[g][v].w, msk, kWave);
       }
-      if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][c * EPL + v * 4]) = acc[g][v];
+      if constexpr (PRE) {   // this wavefront's rows are complete: normalise and store
+        if (slot == 0 && g < ng) {
+          const float inv = 1.0f / l[g];
+          float4 o = acc[g][v];
+          o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
+          *reinterpret_cast<float4*>(out + (row0 + g) * D + c * EPL + v * 4) = o;
+        }
+      } else {
+        if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][c * EPL + v * 4]) = acc[g][v];
+      }
     }
-    if (lane == 0) { st_m[wave][g] = m[g]; st_l[wave][g] = l[g]; }
+    if (!PRE && lane == 0) { st_m[wave][g] = m[g]; st_l[wave][g] = l[g]; }
   }
+  if constexpr (PRE) return;
   __syncthreads();
 
   // ---- block merge (fixed wave order) and store ---------------------------------------------
@@ -406,7 +421,7 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
                           int T, int64_t kv_max, float scale, int pos0) {
   Context& c = tlhip::ctx();
   constexpr int G = 8;   // query positions per block
-  const dim3 grid(Hq, 1, (T + G - 1) / G), block(256);
+  const dim3 grid(Hq, 1, (T + 4 * G - 1) / (4 * G)), block(256);   // 4 wavefronts x G query rows
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
                      (float*)nullptr, (float*)nullptr, (float*)nullptr, Hq / Hkv, pos0 + T,
                      kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr);
