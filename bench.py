@@ -31,7 +31,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 SHAPES = [(3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584)]  # (N, K)
 HBM_PEAK_GBS = 8000.0
 RING_BYTES = 1.2e9      # distinct weight bytes per shape, > 4x the Infinity Cache
-LMHEAD_HBM_BYTES_PER_LAUNCH = 356_657_000   # (173851.3 KiB * 2.000 + 595.6 KiB) * 1024
+LMHEAD_HBM_BYTES_PER_LAUNCH = 356_645_000   # (173845.2 KiB * 2.000 + 595.6 KiB) * 1024
 
 
 def q4_nbytes(N, K):
