@@ -82,6 +82,8 @@ SIGNATURES = {
     "tlhip_attn_partials_bytes": (i64, [i64, i64, i64, i64]),
     "tlhip_attn_decode_dpos": (cint, [P, P, P, P, i64, i64, P, i64, i64, f32, cint, P, i64]),
     "tlhip_qkv_rope_append_dpos": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, f32, cint]),
+    "tlhip_rope_table": (cint, [P, i64, i64, P, f32]),
+    "tlhip_qkv_rope_append_tab": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, P, i64, P, cint]),
     "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
     "tlhip_token_advance": (cint, [P, P, P, i64]),
     "tlhip_gemv_q4_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
@@ -321,6 +323,15 @@ class TlHip:
         self._chk(self.c.tlhip_qkv_rope_append_dpos(
             qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None, Kc.ptr, Vc.ptr, Hq, Hkv, D,
             d_pos.ptr, kv_max, base, int(kv_bf16)))
+
+    def rope_table(self, table, D, pos, base, d_pos=None):
+        self._chk(self.c.tlhip_rope_table(table.ptr, D, pos, d_pos.ptr if d_pos is not None else None, base))
+
+    def qkv_rope_append_tab(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, D, pos, kv_max, table, d_pos=None,
+                            kv_bf16=False):
+        self._chk(self.c.tlhip_qkv_rope_append_tab(
+            qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None, Kc.ptr, Vc.ptr, Hq, Hkv, D, pos,
+            d_pos.ptr if d_pos is not None else None, kv_max, table.ptr, int(kv_bf16)))
 
     def embed_gather_bf16(self, table, d_token, out, hidden, vocab):
         self._chk(self.c.tlhip_embed_gather_bf16(table.ptr, d_token.ptr, out.ptr, hidden, vocab))

@@ -268,7 +268,8 @@ template <typename KT>
 __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
     float* __restrict__ qkv, const float* __restrict__ bq, const float* __restrict__ bk,
     const float* __restrict__ bv, KT* __restrict__ Kc, KT* __restrict__ Vc, int Hq, int Hkv, int D,
-    int64_t pos, int64_t kv_max, float base, const uint32_t* __restrict__ dpos) {
+    int64_t pos, int64_t kv_max, float base, const uint32_t* __restrict__ dpos,
+    const float2* __restrict__ table) {
   if (dpos) {   // position kept on the device; a full cache drops the step's writes
     pos = (int64_t)*dpos;
     if (pos >= kv_max) return;
@@ -279,9 +280,17 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_rot) {
     const int r = i / half, j = i - r * half;   // r: head row within [q heads | k heads]
-    const double theta = pow((double)base, -2.0 * (double)j / (double)D);
-    const double ang = (double)pos * theta;
-    const float c = (float)cos(ang), s = (float)sin(ang);
+    float c, s;
+    if (table) {   // (cos, sin) of this step's position, formed once per step by rope_table_kernel
+      const float2 cs = table[j];
+      c = cs.x;
+      s = cs.y;
+    } else {
+      const double theta = pow((double)base, -2.0 * (double)j / (double)D);
+      const double ang = (double)pos * theta;
+      c = (float)cos(ang);
+      s = (float)sin(ang);
+    }
     const size_t bi = (size_t)r * D;
     const bool is_k = r >= Hq;
     const float* bias = is_k ? (bk ? bk + (size_t)(r - Hq) * D : nullptr) : (bq ? bq + bi : nullptr);
@@ -307,6 +316,18 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
 }
 
 __global__ void incr_u32_kernel(uint32_t* p) { *p += 1u; }
+
+// table[j] = (cos, sin)(pos * base^(-2j/D)), the same fp64 expression as rope_kernel:
+// every layer of a decode step rotates by the same angles, so a step forms them once.
+__global__ void rope_table_kernel(float2* __restrict__ table, int D, int64_t pos, float base,
+                                  const uint32_t* __restrict__ dpos) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= (D >> 1)) return;
+  if (dpos) pos = (int64_t)*dpos;
+  const double theta = pow((double)base, -2.0 * (double)j / (double)D);
+  const double ang = (double)pos * theta;
+  table[j] = make_float2((float)cos(ang), (float)sin(ang));
+}
 
 // ---- device-resident greedy loop --------------------------------------------------------
 // out[j] = widen(table[tok][j]) with tok read from the device (the previous step's argmax).
@@ -498,7 +519,7 @@ int tlhip_kv_append(void* Kc, void* Vc, const void* k_new, const void* v_new, in
 static int qkv_rope_append_launch(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
                                   void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
                                   int64_t pos, int64_t kv_max, float base, int kv_bf16,
-                                  const void* d_pos) {
+                                  const void* d_pos, const void* table = nullptr) {
   if (!qkv || !Kc || !Vc) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append: null pointer");
   if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_append: head_dim must be 64 or 128");
   if (n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads > 4096)
@@ -510,14 +531,15 @@ static int qkv_rope_append_launch(void* qkv, const void* bq, const void* bk, con
   const float* pbq = static_cast<const float*>(bq);
   const float* pbk = static_cast<const float*>(bk);
   const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
+  const float2* tb = static_cast<const float2*>(table);
   if (kv_bf16)
     qkv_rope_append_kernel<uint16_t><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<uint16_t*>(Kc),
-        static_cast<uint16_t*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp);
+        static_cast<uint16_t*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp, tb);
   else
     qkv_rope_append_kernel<float><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(
         static_cast<float*>(qkv), pbq, pbk, static_cast<const float*>(bv), static_cast<float*>(Kc),
-        static_cast<float*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp);
+        static_cast<float*>(Vc), (int)n_q_heads, (int)n_kv_heads, (int)D, pos, kv_max, base, dp, tb);
   hipError_t e_ = hipGetLastError();
   if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
   ctx().census[TLHIP_C_ROPE]++;
@@ -531,6 +553,25 @@ int tlhip_qkv_rope_append(void* qkv, const void* bq, const void* bk, const void*
   TLHIP_REQUIRE_READY();
   return qkv_rope_append_launch(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos, kv_max, base,
                                 kv_bf16, nullptr);
+}
+
+int tlhip_rope_table(void* table, int64_t D, int64_t pos, const void* d_pos, float base) {
+  TLHIP_REQUIRE_READY();
+  if (!table || D <= 0 || (D & 1) || D > 65536) return fail(TLHIP_EINVAL, "tlhip_rope_table: bad arguments");
+  rope_table_kernel<<<dim3(blocks_for(D / 2)), dim3(256), 0, ctx().stream>>>(
+      static_cast<float2*>(table), (int)D, pos, base, static_cast<const uint32_t*>(d_pos));
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  return TLHIP_OK;
+}
+
+int tlhip_qkv_rope_append_tab(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                              void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                              const void* d_pos, int64_t kv_max, const void* table, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  if (!table) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_append_tab: null table");
+  return qkv_rope_append_launch(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos, kv_max, 0.f,
+                                kv_bf16, d_pos, table);
 }
 
 int tlhip_qkv_rope_append_dpos(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,

@@ -120,6 +120,9 @@ struct api {
                           int64_t, int64_t, float, int, void*, int64_t) = nullptr;
   int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
+  int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
+  int (*qkv_rope_append_tab)(void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
+                             int64_t, int64_t, const void*, int64_t, const void*, int) = nullptr;
   int (*embed_gather_bf16)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
   int (*token_advance)(void*, const void*, void*, int64_t) = nullptr;
   int (*gemv_q4_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
@@ -214,6 +217,8 @@ struct context {
               bind(f.attn_partials_bytes, "tlhip_attn_partials_bytes") &&
               bind(f.attn_decode_dpos, "tlhip_attn_decode_dpos") &&
               bind(f.qkv_rope_append_dpos, "tlhip_qkv_rope_append_dpos") &&
+              bind(f.rope_table, "tlhip_rope_table") &&
+              bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
               bind(f.embed_gather_bf16, "tlhip_embed_gather_bf16") &&
               bind(f.token_advance, "tlhip_token_advance") &&
               bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
@@ -716,6 +721,36 @@ inline bool qkv_rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, void* 
                                                    d_pos, kv_max, base, kv_bf16 ? 1 : 0));
 }
 
+// ---- rotary angles formed once per step -------------------------------------------------------
+// All layers of a decode step rotate by the same angles: rope_table writes (cos, sin)
+// for position pos (or *d_pos) once, qkv_rope_append_tab reads them instead of
+// evaluating fp64 pow/cos/sin per layer. Bit-identical to qkv_rope_append.
+inline bool rope_table(void* table, int64_t D, int64_t pos, void* d_pos, float base) {
+  auto& c = context::get();
+  if (!c.ready || !table) return false;
+  if (d_pos) c.device_read_(d_pos);
+  c.device_write_(table);
+  return detail::done_(c, c.f.rope_table(table, D, pos, d_pos, base));
+}
+inline bool qkv_rope_append_tab(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
+                                int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                                void* d_pos, int64_t kv_max, void* table, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || !table) return false;
+  if (!d_pos && (pos < 0 || pos >= kv_max)) return false;
+  c.device_read_(qkv);
+  if (bq) c.device_read_(bq);
+  if (bk) c.device_read_(bk);
+  if (bv) c.device_read_(bv);
+  if (d_pos) c.device_read_(d_pos);
+  c.device_read_(table);
+  c.device_write_(qkv);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.qkv_rope_append_tab(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
+                                                  d_pos, kv_max, table, kv_bf16 ? 1 : 0));
+}
+
 // ---- device-resident greedy loop -----------------------------------------------------------
 // The next token never visits the host: the embedding row of *d_token (a device
 // int32, what argmax_async wrote) is gathered on the device, and the step's tail
@@ -874,6 +909,16 @@ struct kv_cache {
   }
   bool attn(void* q, void* out, int64_t n_q_heads, float scale) {
     return attn_decode(q, K, V, out, n_q_heads, n_kv_heads, pos, max_ctx, D, scale, kv_bf16);
+  }
+  // fused epilogue reading this step's rotary table; position on the host or (d_pos) the device
+  bool rope_append_tab(void* qkv, void* bq, void* bk, void* bv, int64_t n_q_heads, void* table,
+                       void* d_pos = nullptr) {
+    if (!d_pos && pos >= max_ctx) return false;
+    if (!qkv_rope_append_tab(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, D, pos, d_pos, max_ctx, table,
+                             kv_bf16))
+      return false;
+    if (!d_pos) pos++;
+    return true;
   }
   // The same two with the position on the device (the host pos is NOT advanced:
   // a recorded graph replays these; captured_decoder reconciles pos afterwards).

@@ -123,6 +123,7 @@ struct model {
   linear lm_head;
   std::vector<layer> layers;
   scratch s;
+  void* rope_tab = nullptr;            // (cos, sin)[head_dim/2] of the step being run
   void* embed_dev = nullptr;           // the embedding table on the device (greedy_loop only)
   void* attn_partials = nullptr;       // split partials of the device-position attention
   int64_t attn_partials_bytes = 0;
@@ -420,16 +421,18 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     // may not write the residual over a vector its other blocks still read.
     void* rin = x0;          // residual entering the layer
     void* din = nullptr;     // MLP output of the previous layer, not yet added
+    if (!M.rope_tab) M.rope_tab = hip::alloc_device(d.head_dim * 4);
+    ok &= M.rope_tab && hip::rope_table(M.rope_tab, d.head_dim, pos, d_pos, d.rope_base);
     for (int64_t l = 0; l < d.n_layers; l++) {
       layer& L = M.layers[(size_t)l];
       ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
       if (d_pos) {
-        ok &= L.cache.rope_append_dpos(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base, d_pos);
+        ok &= L.cache.rope_append_tab(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, M.rope_tab, d_pos);
         ok &= L.cache.attn_dpos(S.qkvb, S.ab, d.n_q_heads, scale, d_pos, M.attn_partials,
                                 M.attn_partials_bytes);
       } else {
         L.cache.pos = pos;
-        ok &= L.cache.rope_append(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, d.rope_base);
+        ok &= L.cache.rope_append_tab(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, M.rope_tab);
         ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
       }
       ok &= gemv(L.wo, S.ab, S.hb);

@@ -209,6 +209,16 @@ int tlhip_qkv_rope_append_dpos(void* qkv, const void* bq, const void* bk, const 
                                void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
                                const void* d_pos, int64_t kv_max, float base, int kv_bf16);
 
+/* ---- rotary angles formed once per step (no reference counterpart) -------------------
+ * table[D/2] of float2 (cos, sin) at position pos (or *d_pos when d_pos is non-NULL), the fp64
+ * expression of tlhip_rope. All layers of a decode step rotate by the same angles. */
+int tlhip_rope_table(void* table, int64_t D, int64_t pos, const void* d_pos, float base);
+/* tlhip_qkv_rope_append(_dpos) reading the angles from such a table; the cache row is pos, or
+ * *d_pos when d_pos is non-NULL. Bit-identical to the table-less forms. */
+int tlhip_qkv_rope_append_tab(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                              void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
+                              const void* d_pos, int64_t kv_max, const void* table, int kv_bf16);
+
 /* ---- device-resident greedy loop (no reference counterpart: the reference gathers the
  * embedding row on the host and reads every token back, qwen_model.h:530-535, 642-647) ----
  * out[hidden] f32 = widened row *d_token of a bf16 [vocab, hidden] table; d_token is a device

@@ -255,3 +255,33 @@ def test_device_position_twins_equal_host_position_calls(lib, orc):
     assert not Kc.numpy().any() and not Vc.numpy().any()
     for b in (dpos, Kc, Vc, dk):
         b.free()
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_rope_table_form_is_bit_identical(lib, orc, D):
+    """The per-step rotary table (cos, sin formed once, fp64 like array.h:1719-1727) and the fused
+    epilogue that reads it give exactly what the table-less epilogue gives, with the position on
+    the host or on the device."""
+    Hq, Hkv, kv_max, base = 6, 2, 5000, 1e6
+    dpos = lib.to_device(np.array([0], np.uint32))
+    tab = lib.empty(D)                       # D/2 float2
+    for pos in (0, 1, 777, 4095):
+        qkv = orc.normal((Hq + 2 * Hkv) * D, 400 + pos)
+        bq, bk, bv = (lib.to_device(orc.normal(n, 401 + i)) for i, n in enumerate((Hq * D, Hkv * D, Hkv * D)))
+        q1, q2, q3 = lib.to_device(qkv), lib.to_device(qkv), lib.to_device(qkv)
+        big = [lib.to_device(np.zeros((Hkv, kv_max, D), np.float32)) for _ in range(6)]
+        lib.qkv_rope_append(q1, bq, bk, bv, big[0], big[1], Hq, Hkv, D, pos, kv_max, base)
+        lib.rope_table(tab, D, pos, base)
+        lib.qkv_rope_append_tab(q2, bq, bk, bv, big[2], big[3], Hq, Hkv, D, pos, kv_max, tab)
+        dpos.upload(np.array([pos], np.uint32))
+        lib.rope_table(tab, D, 0, base, d_pos=dpos)
+        lib.qkv_rope_append_tab(q3, bq, bk, bv, big[4], big[5], Hq, Hkv, D, 0, kv_max, tab, d_pos=dpos)
+        a = q1.numpy()
+        assert np.array_equal(a, q2.numpy()) and np.array_equal(a, q3.numpy())
+        k1, v1 = big[0].numpy(), big[1].numpy()
+        assert np.array_equal(k1, big[2].numpy()) and np.array_equal(k1, big[4].numpy())
+        assert np.array_equal(v1, big[3].numpy()) and np.array_equal(v1, big[5].numpy())
+        assert k1[:, pos, :].any()
+        for b in [q1, q2, q3, bq, bk, bv] + big:
+            b.free()
+    dpos.free(); tab.free()
