@@ -84,6 +84,7 @@ SIGNATURES = {
     "tlhip_qkv_rope_append_dpos": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, f32, cint]),
     "tlhip_rope_table": (cint, [P, i64, i64, P, f32]),
     "tlhip_qkv_rope_append_tab": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, P, i64, P, cint]),
+    "tlhip_attn_decode_qkv": (cint, [P, P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, cint, P, i64]),
     "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
     "tlhip_token_advance": (cint, [P, P, P, i64]),
     "tlhip_gemv_q4_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
@@ -332,6 +333,13 @@ class TlHip:
         self._chk(self.c.tlhip_qkv_rope_append_tab(
             qkv.ptr, bq.ptr, bk.ptr, bv.ptr if bv is not None else None, Kc.ptr, Vc.ptr, Hq, Hkv, D, pos,
             d_pos.ptr if d_pos is not None else None, kv_max, table.ptr, int(kv_bf16)))
+
+    def attn_decode_qkv(self, qkv, bq, bk, bv, Kc, Vc, out, Hq, Hkv, pos, kv_max, D, scale, table,
+                        d_pos=None, partials=None, kv_bf16=False):
+        opt = lambda b: b.ptr if b is not None else None
+        self._chk(self.c.tlhip_attn_decode_qkv(
+            qkv.ptr, opt(bq), opt(bk), opt(bv), Kc.ptr, Vc.ptr, out.ptr, Hq, Hkv, pos, opt(d_pos), kv_max,
+            D, scale, table.ptr, int(kv_bf16), opt(partials), partials.nbytes if partials is not None else 0))
 
     def embed_gather_bf16(self, table, d_token, out, hidden, vocab):
         self._chk(self.c.tlhip_embed_gather_bf16(table.ptr, d_token.ptr, out.ptr, hidden, vocab))

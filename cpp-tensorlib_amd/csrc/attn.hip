@@ -49,6 +49,77 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// ---- fused step prologue (QKV = true) ------------------------------------------------------
+// The kernel then takes the raw [q | k | v] vector of the step's projection instead of a
+// finished q: every block adds the bias to its own query heads and rotates them in
+// registers, and the step's new key/value row (bias, rotation, narrowing to the cache
+// type) is formed in registers by wavefront 0 of split 0, which starts its running
+// softmax state from it as key number one; its loads are requested together with the
+// query's, so the row costs that wavefront some arithmetic and no extra memory latency.
+// The block of head group 0 stores the row into the cache. Keys [0, pos) come from the cache as usual, so no block
+// reads the row that is being written. The arithmetic (unfused multiplies, then one add/sub) is that of
+// qkv_rope_append_kernel, so the rotated values are bit-identical to the two-kernel path.
+struct QkvFuse {
+  const float *bq, *bk, *bv;   // biases or nullptr
+  const float2* table;         // (cos, sin) of this step's position, D/2 entries
+  void *Kw, *Vw;               // the caches, writable
+  int64_t kv_max;
+};
+
+// Rotates elements [d0, d0+4) of a head row that is spread over the 16 lanes of a DPP
+// row (lane c holds D/16 consecutive elements). `own` holds this lane's elements with
+// the bias added; the rotation partner, element d +- D/2, sits in lane c ^ 8 of the
+// same row, which is a rotation of the row by 8 lanes (DPP row_ror:8).
+__device__ __forceinline__ float dpp_ror8(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, true));
+}
+template <int D>
+__device__ __forceinline__ float4 rope4(float4 own, const float2* __restrict__ table, int d0) {
+  constexpr int half = D / 2;
+  const bool lo = d0 < half;
+  const int j0 = lo ? d0 : d0 - half;
+  const float4 oth = make_float4(dpp_ror8(own.x), dpp_ror8(own.y), dpp_ror8(own.z), dpp_ror8(own.w));
+  const float4 a = lo ? own : oth;   // x0: elements j
+  const float4 b = lo ? oth : own;   // x1: elements j + half
+  const float4 t0 = *reinterpret_cast<const float4*>(table + j0);       // (c0, s0, c1, s1)
+  const float4 t1 = *reinterpret_cast<const float4*>(table + j0 + 2);   // (c2, s2, c3, s3)
+  float4 o;
+  if (lo) {
+    o.x = __fsub_rn(__fmul_rn(a.x, t0.x), __fmul_rn(b.x, t0.y));
+    o.y = __fsub_rn(__fmul_rn(a.y, t0.z), __fmul_rn(b.y, t0.w));
+    o.z = __fsub_rn(__fmul_rn(a.z, t1.x), __fmul_rn(b.z, t1.y));
+    o.w = __fsub_rn(__fmul_rn(a.w, t1.z), __fmul_rn(b.w, t1.w));
+  } else {
+    o.x = __fadd_rn(__fmul_rn(a.x, t0.y), __fmul_rn(b.x, t0.x));
+    o.y = __fadd_rn(__fmul_rn(a.y, t0.w), __fmul_rn(b.y, t0.z));
+    o.z = __fadd_rn(__fmul_rn(a.z, t1.y), __fmul_rn(b.z, t1.x));
+    o.w = __fadd_rn(__fmul_rn(a.w, t1.w), __fmul_rn(b.w, t1.z));
+  }
+  return o;
+}
+// x[d0..d0+4) + bias[d0..d0+4) (bias may be nullptr)
+__device__ __forceinline__ float4 load_biased4(const float* __restrict__ x, const float* __restrict__ bias, int d0) {
+  float4 a = *reinterpret_cast<const float4*>(x + d0);
+  if (bias) {
+    const float4 b4 = *reinterpret_cast<const float4*>(bias + d0);
+    a.x += b4.x; a.y += b4.y; a.z += b4.z; a.w += b4.w;
+  }
+  return a;
+}
+
+// Stores four consecutive elements into a cache row and returns them as the cache holds them.
+__device__ __forceinline__ float4 kv_store4(float* p, float4 v, bool store) {
+  if (store) *reinterpret_cast<float4*>(p) = v;
+  return v;
+}
+__device__ __forceinline__ float4 kv_store4(uint16_t* p, float4 v, bool store) {
+  const uint32_t a = f32_to_bf16_rne(v.x), b = f32_to_bf16_rne(v.y), c = f32_to_bf16_rne(v.z),
+                 d = f32_to_bf16_rne(v.w);
+  const uint2 r = make_uint2(a | (b << 16), c | (d << 16));
+  if (store) *reinterpret_cast<uint2*>(p) = r;
+  return make_float4(bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y));
+}
+
 // grid = (Hkv, S, ceil(group/G)); block = nw*64 threads (nw in 1,2,4).
 // A wavefront works on tiles of TK keys (16, 32 or 64): 4 keys per load step
 // (one per DPP row), each lane holding EPL = D/16 consecutive floats of its key.
@@ -59,26 +130,45 @@ __device__ __forceinline__ float row16_sum(float v) {
 // stream exactly like the query heads of a GQA group do in decode, and walks all
 // of their keys itself (no merge between wavefronts). Row g sees keys
 // [0, pos0 + p_g]; later keys of a tile are masked per row. Longest rows first.
-template <int D, int G, typename KT, bool PRE>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
+template <int D, int G, typename KT, bool PRE, bool QKV = false>
+__global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kernel(
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
     float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
     float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, int TK,
-    float scale, int S, int T, int pos0, const uint32_t* __restrict__ dpos) {
+    float scale, int S, int T, int pos0, const uint32_t* __restrict__ dpos, QkvFuse fz, int kv_rows) {
   constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
   constexpr int NV = EPL / 4;        // float4 loads per lane per key
   constexpr int UNR = 4;             // key steps in flight per lane
-  __shared__ float pbuf[4][G][64];               // per-wave probabilities of the current tile
-  __shared__ float st_m[4][G], st_l[4][G];       // per-wave softmax state for the block merge
-  __shared__ float st_acc[4][G][D];
+  // Decode at short and medium contexts gives a wavefront one or two tiles, and the step
+  // is a chain of memory latencies. The first K and V rows of the wavefront's first tile
+  // depend on nothing but the block and wave indices (rows are clamped to the cache's
+  // capacity, which is mapped memory whatever it holds), so they are requested at the very
+  // top, ahead of the device-side position and of the query prologue, and masked when used.
+  constexpr bool kPre = !PRE && G <= 4;
+  constexpr int NWMAX = (!PRE && G <= 4) ? 8 : 4;   // wavefronts per block, at most
+  __shared__ float pbuf[NWMAX][G][64];              // per-wave probabilities of the current tile
+  __shared__ float st_m[NWMAX][G], st_l[NWMAX][G];  // per-wave softmax state for the block merge
+  __shared__ float st_acc[NWMAX][G][D];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int slot = lane >> 4, c = lane & 15;     // DPP row = key slot, c = position in the row
   const int split = blockIdx.y;
-  // Position kept on the device (captured decode loops): the grid was planned for
-  // the cache capacity, the live context is *dpos + 1. Splits past it find no keys
-  // and write neutral partials (m = -inf, l = 0, acc = 0).
-  if (!PRE && dpos) ctx = min(ctx, (int)*dpos + 1);
+  float4 kpre[UNR][NV], vpre[UNR][NV];
+  if constexpr (kPre) {
+    const size_t hoff = (size_t)blockIdx.x * kv_stride;
+    const int kb0 = chunk ? split * chunk + wave * TK : (split * nw + wave) * TK;
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      const int key = min(kb0 + u * 4 + slot, kv_rows - 1);
+#pragma unroll
+      for (int v = 0; v < NV; v++) {
+        kpre[u][v] = KvLoad<KT>::ld(K + hoff + (size_t)key * D + c * EPL + v * 4);
+        vpre[u][v] = KvLoad<KT>::ld(V + hoff + (size_t)key * D + c * EPL + v * 4);
+      }
+    }
+  }
+  // (the query rows first: nothing about them depends on the position, and with the
+  // position on the device its load should not stand in front of theirs)
   int kvh, g0, ng, k_begin, k_end;
   size_t row0;                                   // index of row g = 0 in q / out, in rows of D
   if constexpr (PRE) {
@@ -99,8 +189,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     g0 = blockIdx.z * G;
     ng = min(G, group - g0);
     row0 = (size_t)kvh * group + g0;
-    k_begin = split * chunk;
-    k_end = min(ctx, k_begin + chunk);
+    k_begin = k_end = 0;                         // set below, once the position is known
   }
   const int lim0 = pos0 + g0 + 1;                // PRE: row g sees keys < lim0 + g
   const KT* Kh = K + (size_t)kvh * kv_stride;
@@ -112,8 +201,38 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int g = 0; g < G; g++)
 #pragma unroll
     for (int v = 0; v < NV; v++)
-      qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (row0 + g) * D + c * EPL + v * 4)
-                        : make_float4(0.f, 0.f, 0.f, 0.f);
+      if constexpr (QKV)
+        // (rows g >= ng rotate zeros: the DPP exchange needs every lane of the row)
+        qv[g][v] = rope4<D>(g < ng ? load_biased4(q + (row0 + g) * D,
+                                                  fz.bq ? fz.bq + (row0 + g) * D : nullptr, c * EPL + v * 4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f),
+                            fz.table, c * EPL + v * 4);
+      else
+        qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (row0 + g) * D + c * EPL + v * 4)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+  // Position kept on the device (captured decode loops): the grid was planned for
+  // the cache capacity, the live context is *dpos + 1. Splits past it find no keys
+  // and write neutral partials (m = -inf, l = 0, acc = 0).
+  if (!PRE && !QKV && dpos) ctx = min(ctx, (int)*dpos + 1);
+  // QKV: the step's position; keys [0, pos) are in the cache, key pos is formed here
+  // (a full cache takes no new row: the step attends to what the cache holds).
+  int64_t new_pos = 0;
+  bool has_new = false;
+  if constexpr (QKV) {
+    new_pos = dpos ? (int64_t)*dpos : (int64_t)ctx - 1;
+    has_new = new_pos < fz.kv_max;
+    ctx = (int)min(new_pos, fz.kv_max);
+  }
+  if constexpr (!PRE) {
+    // Two ways to deal tiles. chunk > 0: split s owns keys [s * chunk, (s + 1) * chunk) and its
+    // wavefronts alternate over the tiles of that range (long per-head streams read best
+    // this way). chunk == 0: round-robin over all wavefronts of all splits, wavefront w of
+    // split s takes tiles (s * nw + w) + j * (S * nw); that deal does not depend on the
+    // context length, so a grid planned for the cache capacity (position on the device)
+    // keeps every split busy at any live context.
+    k_begin = split * chunk;
+    k_end = chunk ? min(ctx, k_begin + chunk) : ctx;
+  }
   float m[G], l[G];
   float4 acc[G][NV];
 #pragma unroll
@@ -124,7 +243,51 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     for (int v = 0; v < NV; v++) acc[g][v] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
 
-  const int kb_first = PRE ? 0 : k_begin + wave * TK, kb_step = PRE ? TK : nw * TK;
+  // ---- the step's own key/value row: the first key of split 0's first wavefront -----------
+  // (its loads travel with the query's, so it costs that wavefront arithmetic only)
+  if constexpr (QKV) {
+    if (split == 0 && wave == 0 && has_new) {
+      const int Hkv = gridDim.x, Hq = Hkv * group;
+      const float* kraw = q + (size_t)(Hq + kvh) * D;
+      const float* vraw = q + (size_t)(Hq + Hkv + kvh) * D;
+      KT* krow = static_cast<KT*>(fz.Kw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
+      KT* vrow = static_cast<KT*>(fz.Vw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
+      const bool store = blockIdx.z == 0 && slot == 0;
+      float4 kn[NV], vn[NV];
+#pragma unroll
+      for (int v = 0; v < NV; v++) {
+        const int d0 = c * EPL + v * 4;
+        const float4 kr =
+            rope4<D>(load_biased4(kraw, fz.bk ? fz.bk + (size_t)kvh * D : nullptr, d0), fz.table, d0);
+        const float4 vr = load_biased4(vraw, fz.bv ? fz.bv + (size_t)kvh * D : nullptr, d0);
+        kn[v] = kv_store4(krow + d0, kr, store);
+        vn[v] = kv_store4(vrow + d0, vr, store);
+      }
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        float p = qv[g][0].x * kn[0].x;
+        p = fmaf(qv[g][0].y, kn[0].y, p);
+        p = fmaf(qv[g][0].z, kn[0].z, p);
+        p = fmaf(qv[g][0].w, kn[0].w, p);
+        if (NV > 1) {
+          p = fmaf(qv[g][NV - 1].x, kn[NV - 1].x, p);
+          p = fmaf(qv[g][NV - 1].y, kn[NV - 1].y, p);
+          p = fmaf(qv[g][NV - 1].z, kn[NV - 1].z, p);
+          p = fmaf(qv[g][NV - 1].w, kn[NV - 1].w, p);
+        }
+        // the state is still empty: the key's weight is exp(0) = 1 (l, acc are per-lane and
+        // per-slot partials that are summed later, so one lane and one slot carry it)
+        m[g] = row16_sum(p) * scale;               // the same in all four slots
+        l[g] = lane == 0 ? 1.f : 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+          acc[g][v] = slot == 0 ? vn[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  }
+
+  const int kb_first = PRE ? 0 : chunk ? k_begin + wave * TK : (split * nw + wave) * TK;
+  const int kb_step = PRE ? TK : chunk ? nw * TK : S * nw * TK;
   for (int kb = kb_first; kb < k_end; kb += kb_step) {
     // ---- scores: lane (slot,c) ends up holding key kb + c*4 + slot (c < steps) ----
     float sreg[G];
@@ -133,24 +296,37 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     // The tile's first V rows do not depend on the scores: request them with the K
     // rows so that one memory latency covers both.
     float4 vfirst[UNR][NV];
+    const bool pre_tile = kPre && kb == kb_first;   // its first rows were requested at the top
     for (int i0 = 0; i0 < steps; i0 += UNR) {
       float4 kv[UNR][NV];
-#pragma unroll
-      for (int u = 0; u < UNR; u++) {
-        const int key = kb + (i0 + u) * 4 + slot;
-#pragma unroll
-        for (int v = 0; v < NV; v++)
-          kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * EPL + v * 4)
-                                 : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-      if (i0 == 0) {
+      if (pre_tile && i0 == 0) {
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
-          const int key = kb + u * 4 + slot;
+          const bool live = kb + u * 4 + slot < k_end;   // masked keys: finite K, zero V
+#pragma unroll
+          for (int v = 0; v < NV; v++) {
+            kv[u][v] = live ? kpre[u][v] : make_float4(0.f, 0.f, 0.f, 0.f);
+            vfirst[u][v] = live ? vpre[u][v] : make_float4(0.f, 0.f, 0.f, 0.f);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+          const int key = kb + (i0 + u) * 4 + slot;
 #pragma unroll
           for (int v = 0; v < NV; v++)
-            vfirst[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
-                                       : make_float4(0.f, 0.f, 0.f, 0.f);
+            kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * EPL + v * 4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        if (i0 == 0) {
+#pragma unroll
+          for (int u = 0; u < UNR; u++) {
+            const int key = kb + u * 4 + slot;
+#pragma unroll
+            for (int v = 0; v < NV; v++)
+              vfirst[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);
+          }
         }
       }
 #pragma unroll
@@ -274,10 +450,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
 }
 
-// grid = Hq, block = 1024: merge the S split partials of one head. The split
-// weights exp(m_s - M) are formed once per split in LDS; the threads are D
-// columns x (1024/D) split groups, each summing its splits in a fixed order with
-// the loads of four splits in flight, then the groups are summed in a fixed order.
+// grid = Hq, block = 1024: merge the S split partials of one head. The threads are D
+// columns x (1024/D) split groups. The kernel is a chain of memory latencies and little
+// else, so with up to 8 splits per group (S <= 64 at D = 128) every load - the partial
+// maxima and sums and the thread's own accumulator values - is requested at the top and
+// waited for once; the split weights exp(m_s - M) are formed once per split in LDS, each
+// thread sums its splits in a fixed order and the groups are summed in a fixed order.
 __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restrict__ part_m,
                                                             const float* __restrict__ part_l,
                                                             const float* __restrict__ part_acc,
@@ -285,11 +463,25 @@ __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restr
   extern __shared__ float sm[];   // f[S] | red[1024]
   float* f = sm;
   float* red = sm + S;
+  constexpr int kUp = 8;          // accumulator loads a thread issues up front
   const int h = blockIdx.x, tid = threadIdx.x;
   const float* pm = part_m + (size_t)h * S;
   const float* pl = part_l + (size_t)h * S;
-  float mx = -INFINITY;
-  for (int s = tid; s < S; s += 1024) mx = fmaxf(mx, pm[s]);
+  const int groups = 1024 / D, d = tid % D, sg = tid / D;
+  const float* pa = part_acc + (size_t)h * S * D + d;
+  const bool upfront = S <= kUp * groups;        // (then S <= 1024 as well)
+  float pv[kUp], my_m = -INFINITY, my_l = 0.f;
+  if (upfront) {
+#pragma unroll
+    for (int u = 0; u < kUp; u++) {
+      const int s = sg + u * groups;
+      pv[u] = s < S ? pa[(size_t)s * D] : 0.f;
+    }
+    if (tid < S) { my_m = pm[tid]; my_l = pl[tid]; }
+  }
+  float mx = my_m;
+  if (!upfront)
+    for (int s = tid; s < S; s += 1024) mx = fmaxf(mx, pm[s]);
   mx = wave_max(mx);
   if ((tid & 63) == 0) red[tid >> 6] = mx;
   __syncthreads();
@@ -298,10 +490,18 @@ __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restr
   for (int w = 1; w < 16; w++) M = fmaxf(M, red[w]);
   __syncthreads();
   float lsum = 0.f;
-  for (int s = tid; s < S; s += 1024) {
-    const float w = __expf(pm[s] - M);
-    f[s] = w;
-    lsum = fmaf(pl[s], w, lsum);
+  if (upfront) {
+    if (tid < S) {
+      const float w = __expf(my_m - M);
+      f[tid] = w;
+      lsum = my_l * w;
+    }
+  } else {
+    for (int s = tid; s < S; s += 1024) {
+      const float w = __expf(pm[s] - M);
+      f[s] = w;
+      lsum = fmaf(pl[s], w, lsum);
+    }
   }
   lsum = wave_sum(lsum);
   if ((tid & 63) == 0) red[tid >> 6] = lsum;
@@ -310,19 +510,28 @@ __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restr
 #pragma unroll
   for (int w = 1; w < 16; w++) L += red[w];
   __syncthreads();
-  const int groups = 1024 / D, d = tid % D, sg = tid / D;
-  const float* pa = part_acc + (size_t)h * S * D + d;
   float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-  int s = sg;
-  for (; s + 3 * groups < S; s += 4 * groups) {
-    const float v0 = pa[(size_t)s * D], v1 = pa[(size_t)(s + groups) * D],
-                v2 = pa[(size_t)(s + 2 * groups) * D], v3 = pa[(size_t)(s + 3 * groups) * D];
-    a0 = fmaf(f[s], v0, a0);
-    a1 = fmaf(f[s + groups], v1, a1);
-    a2 = fmaf(f[s + 2 * groups], v2, a2);
-    a3 = fmaf(f[s + 3 * groups], v3, a3);
+  if (upfront) {
+#pragma unroll
+    for (int u = 0; u < kUp; u += 4) {
+      const int s = sg + u * groups;
+      a0 = fmaf(s < S ? f[s] : 0.f, pv[u], a0);
+      a1 = fmaf(s + groups < S ? f[s + groups] : 0.f, pv[u + 1], a1);
+      a2 = fmaf(s + 2 * groups < S ? f[s + 2 * groups] : 0.f, pv[u + 2], a2);
+      a3 = fmaf(s + 3 * groups < S ? f[s + 3 * groups] : 0.f, pv[u + 3], a3);
+    }
+  } else {
+    int s = sg;
+    for (; s + 3 * groups < S; s += 4 * groups) {
+      const float v0 = pa[(size_t)s * D], v1 = pa[(size_t)(s + groups) * D],
+                  v2 = pa[(size_t)(s + 2 * groups) * D], v3 = pa[(size_t)(s + 3 * groups) * D];
+      a0 = fmaf(f[s], v0, a0);
+      a1 = fmaf(f[s + groups], v1, a1);
+      a2 = fmaf(f[s + 2 * groups], v2, a2);
+      a3 = fmaf(f[s + 3 * groups], v3, a3);
+    }
+    for (; s < S; s += groups) a0 = fmaf(f[s], pa[(size_t)s * D], a0);
   }
-  for (; s < S; s += groups) a0 = fmaf(f[s], pa[(size_t)s * D], a0);
   red[tid] = (a0 + a1) + (a2 + a3);
   __syncthreads();
   if (sg == 0) {
@@ -334,10 +543,11 @@ __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restr
 
 struct AttnPlan { int G, gz, nw, TK, S, chunk; };
 
-// Split-KV plan. Work is cut into wave tiles of TK keys; the chip wants at least
-// ~4 wavefronts per CU, so short contexts use small tiles and 4-wave blocks, and
-// long contexts give every wavefront several 64-key tiles.
-static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus) {
+// Split-KV plan. Work is cut into wave tiles of TK keys; the chip wants 4 to 8
+// wavefronts per CU, so short contexts use small tiles and 4-wave blocks, and
+// long contexts give every wavefront several 64-key tiles. chunk == 0: tiles are
+// dealt round-robin over the S * nw wavefronts of a kv head.
+static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus, bool fixed_grid) {
   AttnPlan p{};
   // Query heads per block. A wavefront's instruction stream grows with G and, at
   // short and medium contexts, that serial stream (not bandwidth) is what a step
@@ -347,21 +557,41 @@ static AttnPlan plan_attn(int Hkv, int group, int ctx, int cus) {
   p.G = group > 4 ? gmax : group > 2 ? 4 : group > 1 ? 2 : 1;
   p.gz = (group + p.G - 1) / p.G;
   const int base = Hkv * p.gz;
-  const int64_t want_waves = (int64_t)cus * 4;
+  // 8-wavefront blocks of 16-key tiles (every K/V row of a tile is then requested at the
+  // top of the kernel and the tile costs one memory latency) once such blocks still cover
+  // every CU; below that, 4-wavefront blocks spread a short context over more CUs.
+  const bool wide = p.G <= 4 && (int64_t)base * ((ctx + 127) / 128) >= cus;
+  const int64_t want_waves = (int64_t)cus * (wide ? 8 : 4);
   p.TK = 64;
   while (p.TK > 16 && (int64_t)base * ((ctx + p.TK - 1) / p.TK) < want_waves) p.TK >>= 1;
   const int tiles = (ctx + p.TK - 1) / p.TK;
-  p.nw = tiles >= 4 ? 4 : tiles >= 2 ? 2 : 1;
-  const int block_tiles = (tiles + p.nw - 1) / p.nw;       // tiles per wave if S == 1
-  int want_s = (int)((want_waves + (int64_t)base * p.nw - 1) / ((int64_t)base * p.nw));
-  if (want_s < 1) want_s = 1;
-  if (want_s > block_tiles) want_s = block_tiles;
-  // nearest, not ceiling: 34 tiles for 32 wanted splits is 34 splits of one tile per
-  // wave, not 17 of two
-  int tiles_per_wave = (block_tiles + want_s / 2) / want_s;
-  if (tiles_per_wave < 1) tiles_per_wave = 1;
-  p.chunk = tiles_per_wave * p.nw * p.TK;
-  p.S = (ctx + p.chunk - 1) / p.chunk;
+  p.nw = wide && tiles >= 8 ? 8 : tiles >= 4 ? 4 : tiles >= 2 ? 2 : 1;
+  // Splits: enough for want_waves wavefronts, no more than there are rows of nw tiles, and
+  // no more blocks than run at once (a block left for a second round would double the
+  // step): 8-wavefront blocks and the 8-head kernel fill a CU's registers alone, the
+  // smaller 4-wavefront blocks fit two to a CU.
+  const int tile_rows = (tiles + p.nw - 1) / p.nw;
+  const int at_once = cus * ((wide || p.G > 4) ? 1 : 2);
+  int S = (int)((want_waves + (int64_t)base * p.nw - 1) / ((int64_t)base * p.nw));
+  if (S > tile_rows) S = tile_rows;
+  if (S > at_once / base) S = at_once / base;
+  p.S = S < 1 ? 1 : S;
+  // Many kv heads with one query head each (no GQA sharing) at a long context is a plain
+  // bandwidth problem, and there long contiguous per-split streams measured best: 8 x 64-key
+  // tiles per block round, at least 1024 keys per split, at most two blocks per CU. (Needs
+  // the context length when the grid is built, so not with a device-side position.)
+  if (!fixed_grid && p.G == 1 && wide && ctx >= 4096 && (int64_t)base * (ctx / 1024) >= cus / 2) {
+    p.TK = 64;
+    p.nw = 8;
+    const int rows = (ctx + 511) / 512;                        // rounds of 8 tiles
+    int want = ctx / 1024 < 2 * cus / base ? ctx / 1024 : 2 * cus / base;
+    const int one_round = rows < cus / base ? rows : cus / base;
+    if (want < one_round) want = one_round;
+    if (want < 1) want = 1;
+    const int per_split = (rows + want - 1) / want;
+    p.chunk = per_split * 512;
+    p.S = (ctx + p.chunk - 1) / p.chunk;
+  }
   return p;
 }
 
@@ -376,14 +606,16 @@ static size_t attn_partials_floats(int Hq, int S, int D) {
 template <int D, typename KT>
 static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
                        int ctx, int64_t kv_max, float scale, const uint32_t* dpos = nullptr,
-                       float* partials = nullptr, size_t partials_bytes = 0) {
+                       float* partials = nullptr, size_t partials_bytes = 0,
+                       const QkvFuse* fuse = nullptr) {
   Context& c = tlhip::ctx();
   const int group = Hq / Hkv;
-  const AttnPlan p = plan_attn(Hkv, group, ctx, c.cus);
+  const AttnPlan p = plan_attn(Hkv, group, ctx, c.cus, dpos != nullptr);
   float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
-  if (p.S > 1) {
-    const size_t hs = (size_t)Hq * p.S;
-    const size_t need = attn_partials_floats(Hq, p.S, D) * sizeof(float);
+  const int S = p.S;
+  if (S > 1) {
+    const size_t hs = (size_t)Hq * S;
+    const size_t need = attn_partials_floats(Hq, S, D) * sizeof(float);
     float* base;
     if (dpos) {
       if (!partials || partials_bytes < need)
@@ -397,12 +629,19 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     pl = pm + hs;
     pacc = pl + hs;
   }
-  if (p.S > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode: context too long");
-  const dim3 grid(Hkv, p.S, p.gz), block(p.nw * 64);
+  if (S > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode: context too long");
+  const dim3 grid(Hkv, S, p.gz), block(p.nw * 64);
   const int64_t kv_stride = kv_max * D;
-#define TLHIP_ATTN(GG)                                                                         \
-  hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false>), grid, block, 0, c.stream, q, K, V, \
-                     out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0, dpos)
+  const QkvFuse fz = fuse ? *fuse : QkvFuse{};
+#define TLHIP_ATTN(GG)                                                                            \
+  if (fuse)                                                                                       \
+    hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false, true>), grid, block, 0, c.stream, q, \
+                       K, V, out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, S,   \
+                       1, 0, dpos, fz, (int)kv_max);                                              \
+  else                                                                                            \
+    hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false>), grid, block, 0, c.stream, q, K, V, \
+                       out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0, \
+                       dpos, fz, (int)kv_max)
   switch (p.G) {
     case 1: TLHIP_ATTN(1); break;
     case 2: TLHIP_ATTN(2); break;
@@ -410,9 +649,9 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     default: TLHIP_ATTN(8); break;
   }
 #undef TLHIP_ATTN
-  if (p.S > 1)
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(1024), (size_t)(p.S + 1024) * sizeof(float),
-                       c.stream, pm, pl, pacc, out, p.S, D);
+  if (S > 1)
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(1024), (size_t)(S + 1024) * sizeof(float),
+                       c.stream, pm, pl, pacc, out, S, D);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
 }
 
@@ -424,7 +663,7 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
   const dim3 grid(Hq, 1, (T + 4 * G - 1) / (4 * G)), block(256);   // 4 wavefronts x G query rows
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
                      (float*)nullptr, (float*)nullptr, (float*)nullptr, Hq / Hkv, pos0 + T,
-                     kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr);
+                     kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr, QkvFuse{}, (int)kv_max);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
 }
 
@@ -497,7 +736,7 @@ int64_t tlhip_attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t
   if (!ctx().ready || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || kv_max <= 0 ||
       kv_max > 0x3fffffff || (D != 64 && D != 128))
     return 0;
-  const AttnPlan p = plan_attn((int)n_kv_heads, (int)(n_q_heads / n_kv_heads), (int)kv_max, ctx().cus);
+  const AttnPlan p = plan_attn((int)n_kv_heads, (int)(n_q_heads / n_kv_heads), (int)kv_max, ctx().cus, true);
   return (int64_t)(attn_partials_floats((int)n_q_heads, p.S, (int)D) * sizeof(float)) + 16;
 }
 
@@ -529,6 +768,52 @@ int tlhip_attn_decode_dpos(const void* q, const void* K, const void* V, void* ou
   const float* pv = static_cast<const float*>(V);
   return D == 128 ? launch_attn<128, float>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb)
                   : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cap, kv_max, scale, dp, pp, pb);
+}
+
+// The step's raw [q | k | v] projection goes in; bias, rotation, the cache append
+// and the attention over keys [0, pos] happen in one launch (plus the split merge).
+int tlhip_attn_decode_qkv(const void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                          void* Vc, void* out, int64_t n_q_heads, int64_t n_kv_heads, int64_t pos,
+                          const void* d_pos, int64_t kv_max, int64_t D, float scale,
+                          const void* table, int kv_bf16, void* partials, int64_t partials_bytes) {
+  TLHIP_REQUIRE_READY();
+  if (!qkv || !Kc || !Vc || !out || !table) return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv: null pointer");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv: head_dim must be 64 or 128");
+  if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv: Hq must be a positive multiple of Hkv");
+  if (kv_max <= 0 || kv_max > 0x3fffffff || n_kv_heads > 65535 || kv_max * D > ((int64_t)1 << 40))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv: shape too large");
+  if (!d_pos && (pos < 0 || pos >= kv_max)) return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv: need 0 <= pos < kv_max");
+  if (!aligned16(qkv) || !aligned16(Kc) || !aligned16(Vc) || !aligned16(out) || !aligned16(table) ||
+      (bq && !aligned16(bq)) || (bk && !aligned16(bk)) || (bv && !aligned16(bv)) ||
+      (partials && !aligned16(partials)))
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv: operands must be 16-byte aligned");
+  const QkvFuse fz{static_cast<const float*>(bq), static_cast<const float*>(bk),
+                   static_cast<const float*>(bv), static_cast<const float2*>(table), Kc, Vc, kv_max};
+  const float* pq = static_cast<const float*>(qkv);
+  float* po = static_cast<float*>(out);
+  const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
+  float* pp = static_cast<float*>(partials);
+  const size_t pb = partials_bytes > 0 ? (size_t)partials_bytes : 0;
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads;
+  const int cx = dp ? (int)kv_max : (int)pos + 1;   // the grid is planned for this many keys
+  int rc;
+  if (kv_bf16) {
+    const uint16_t* pk = static_cast<const uint16_t*>(Kc);
+    const uint16_t* pv = static_cast<const uint16_t*>(Vc);
+    rc = D == 128 ? launch_attn<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz)
+                  : launch_attn<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz);
+  } else {
+    const float* pk = static_cast<const float*>(Kc);
+    const float* pv = static_cast<const float*>(Vc);
+    rc = D == 128 ? launch_attn<128, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz)
+                  : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz);
+  }
+  if (rc == TLHIP_OK) {
+    ctx().census[TLHIP_C_ROPE]++;
+    ctx().census[TLHIP_C_KV_APPEND]++;
+  }
+  return rc;
 }
 
 }  // extern "C"

@@ -121,6 +121,9 @@ struct api {
   int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
   int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
+  int (*attn_decode_qkv)(const void*, const void*, const void*, const void*, void*, void*, void*, int64_t,
+                        int64_t, int64_t, const void*, int64_t, int64_t, float, const void*, int, void*,
+                        int64_t);
   int (*qkv_rope_append_tab)(void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
                              int64_t, int64_t, const void*, int64_t, const void*, int) = nullptr;
   int (*embed_gather_bf16)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
@@ -219,6 +222,7 @@ struct context {
               bind(f.qkv_rope_append_dpos, "tlhip_qkv_rope_append_dpos") &&
               bind(f.rope_table, "tlhip_rope_table") &&
               bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
+              bind(f.attn_decode_qkv, "tlhip_attn_decode_qkv") &&
               bind(f.embed_gather_bf16, "tlhip_embed_gather_bf16") &&
               bind(f.token_advance, "tlhip_token_advance") &&
               bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
@@ -751,6 +755,31 @@ inline bool qkv_rope_append_tab(void* qkv, void* bq, void* bk, void* bv, void* K
                                                   d_pos, kv_max, table, kv_bf16 ? 1 : 0));
 }
 
+// Bias + rotation of the raw [q|k|v] projection, the cache append and the attention over
+// keys [0, pos] in one launch (plus the split merge). qkv itself is left untouched.
+inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc, void* out,
+                            int64_t n_q_heads, int64_t n_kv_heads, int64_t pos, void* d_pos,
+                            int64_t kv_max, int64_t D, float scale, void* table, void* partials,
+                            int64_t partials_bytes, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64) || !table) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  if (d_pos ? !partials : (pos < 0 || pos >= kv_max)) return false;
+  c.device_read_(qkv);
+  if (bq) c.device_read_(bq);
+  if (bk) c.device_read_(bk);
+  if (bv) c.device_read_(bv);
+  if (d_pos) c.device_read_(d_pos);
+  c.device_read_(table);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  c.device_write_(out);
+  if (partials) c.device_write_(partials);
+  return detail::done_(c, c.f.attn_decode_qkv(qkv, bq, bk, bv, Kc, Vc, out, n_q_heads, n_kv_heads, pos,
+                                              d_pos, kv_max, D, scale, table, kv_bf16 ? 1 : 0, partials,
+                                              partials_bytes));
+}
+
 // ---- device-resident greedy loop -----------------------------------------------------------
 // The next token never visits the host: the embedding row of *d_token (a device
 // int32, what argmax_async wrote) is gathered on the device, and the step's tail
@@ -916,6 +945,18 @@ struct kv_cache {
     if (!d_pos && pos >= max_ctx) return false;
     if (!qkv_rope_append_tab(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, D, pos, d_pos, max_ctx, table,
                              kv_bf16))
+      return false;
+    if (!d_pos) pos++;
+    return true;
+  }
+  // rope_append_tab + attn in one launch: out = attention of this step's rotated q over the
+  // cache plus the step's own row, which is appended on the way.
+  bool attn_qkv(void* qkv, void* bq, void* bk, void* bv, void* out, int64_t n_q_heads, float scale,
+                void* table, void* d_pos = nullptr, void* partials = nullptr,
+                int64_t partials_bytes = 0) {
+    if (!d_pos && pos >= max_ctx) return false;
+    if (!attn_decode_qkv(qkv, bq, bk, bv, K, V, out, n_q_heads, n_kv_heads, pos, d_pos, max_ctx, D,
+                         scale, table, partials, partials_bytes, kv_bf16))
       return false;
     if (!d_pos) pos++;
     return true;

@@ -131,6 +131,7 @@ struct model {
   // true: fused launches (q/k/v epilogue + append; norms and swiglu evaluated inside the
   // GEMV that consumes them). false: the reference's call sequence, one launch per op.
   bool fused = true;
+  bool fused_attn = true;   // within the fused path: q/k/v epilogue + append inside the attention launch
 };
 
 namespace detail {
@@ -414,9 +415,10 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
   const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim();
   bool ok = true;
   if (M.fused) {
-    // 6 launches per layer (+1 when attention splits the context):
-    //   [norm -> qkv GEMV] , q/k/v epilogue + append , attention , o-proj GEMV ,
+    // 5 launches per layer (+1 when attention splits the context):
+    //   [norm -> qkv GEMV] , [q/k/v epilogue + append -> attention] , o-proj GEMV ,
     //   [residual + norm -> gate|up GEMV] , [swiglu -> down GEMV]
+    // (fused_attn = false runs the q/k/v epilogue as a launch of its own)
     // The residual stream ping-pongs between res[0] and res[1] because a fused GEMV
     // may not write the residual over a vector its other blocks still read.
     void* rin = x0;          // residual entering the layer
@@ -426,7 +428,11 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     for (int64_t l = 0; l < d.n_layers; l++) {
       layer& L = M.layers[(size_t)l];
       ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
-      if (d_pos) {
+      if (M.fused_attn) {
+        if (!d_pos) L.cache.pos = pos;
+        ok &= L.cache.attn_qkv(S.qkvb, L.bq, L.bk, L.bv, S.ab, d.n_q_heads, scale, M.rope_tab, d_pos,
+                               d_pos ? M.attn_partials : nullptr, d_pos ? M.attn_partials_bytes : 0);
+      } else if (d_pos) {
         ok &= L.cache.rope_append_tab(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, M.rope_tab, d_pos);
         ok &= L.cache.attn_dpos(S.qkvb, S.ab, d.n_q_heads, scale, d_pos, M.attn_partials,
                                 M.attn_partials_bytes);

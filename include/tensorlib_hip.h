@@ -219,6 +219,20 @@ int tlhip_qkv_rope_append_tab(void* qkv, const void* bq, const void* bk, const v
                               void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                               const void* d_pos, int64_t kv_max, const void* table, int kv_bf16);
 
+/* ---- decode attention with the step's prologue fused in (no reference counterpart: the
+ * reference runs bias, rope, cache append and attention as separate ops, qwen_model.h:560-600) --
+ * qkv = the step's raw [q (Hq*D) | k (Hkv*D) | v (Hkv*D)] projection, left untouched. Adds the
+ * biases (each may be NULL), rotates q and k by `table` (tlhip_rope_table), stores the new k, v
+ * row at cache row pos (or *d_pos when d_pos is non-NULL; a full cache takes no row) and writes
+ * out[Hq*D] = attention of the rotated q over keys [0, pos]. Same values as
+ * tlhip_qkv_rope_append_tab followed by tlhip_attn_decode(_dpos); the new key enters the softmax
+ * in a different position of the summation order. With d_pos the grid is planned for kv_max and
+ * `partials` (tlhip_attn_partials_bytes) is required; without it partials may be NULL. */
+int tlhip_attn_decode_qkv(const void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                          void* Vc, void* out, int64_t n_q_heads, int64_t n_kv_heads, int64_t pos,
+                          const void* d_pos, int64_t kv_max, int64_t D, float scale,
+                          const void* table, int kv_bf16, void* partials, int64_t partials_bytes);
+
 /* ---- device-resident greedy loop (no reference counterpart: the reference gathers the
  * embedding row on the host and reads every token back, qwen_model.h:530-535, 642-647) ----
  * out[hidden] f32 = widened row *d_token of a bf16 [vocab, hidden] table; d_token is a device

@@ -150,3 +150,83 @@ def test_attn_full_size_properties(lib, orc):
     base = _run(lib, q, K2, V, ctx, scale)
     shifted = _run(lib, q, K2 + (q / np.sum(q * q, axis=1, keepdims=True))[:, None, :] * 3.0, V, ctx, scale)
     assert allclose(shifted, base, 2e-4, 2e-5), maxrel(shifted, base)
+
+
+@pytest.mark.parametrize("kv_bf16", [False, True])
+@pytest.mark.parametrize("D,Hq,Hkv,kv_max", [(128, 28, 4, 4352), (64, 14, 2, 700), (128, 4, 4, 96),
+                                             (64, 16, 1, 300), (128, 3, 1, 130)])
+def test_attn_decode_qkv_fused_prologue(lib, orc, D, Hq, Hkv, kv_max, kv_bf16):
+    """Bias + rope + cache append + attention in one launch (the raw [q|k|v] projection goes in)
+    against the oracle's rope and attention, and against the two-launch path: the appended cache
+    rows are bit-identical, no other cache row changes, the projection is left untouched and the
+    output agrees to the attention tolerance. Position on the host and on the device; the last
+    case has a full cache (device position == capacity: no row is taken)."""
+    base, scale = 1e6, 1.0 / np.sqrt(float(D))
+    n = (Hq + 2 * Hkv) * D
+    cache_dt = np.uint16 if kv_bf16 else np.float32
+    K0 = orc.normal(Hkv * kv_max * D, 501).reshape(Hkv, kv_max, D)
+    V0 = orc.normal(Hkv * kv_max * D, 502).reshape(Hkv, kv_max, D)
+    if kv_bf16:
+        K0, V0 = orc.to_bf16(K0), orc.to_bf16(V0)
+    widen = (lambda a: orc.bf16_widen(a)) if kv_bf16 else (lambda a: a)
+    bq, bk, bv = orc.normal(Hq * D, 503, 0, 0.5), orc.normal(Hkv * D, 504, 0, 0.5), orc.normal(Hkv * D, 505, 0, 0.5)
+    dbq, dbk, dbv = lib.to_device(bq), lib.to_device(bk), lib.to_device(bv)
+    tab = lib.empty(D)
+    dpos = lib.to_device(np.zeros(1, np.uint32))
+    part = lib.empty_bytes(lib.attn_partials_bytes(Hq, Hkv, kv_max, D))
+    positions = sorted(set([0, 1, 15, 16, 63, 64, 65, 127, 128, kv_max // 2, kv_max - 2, kv_max - 1]))
+    for pos in [p for p in positions if 0 <= p < kv_max]:
+        for on_device, with_bias in ((False, True), (True, True), (True, False)):
+            print("case attn qkv", D, Hq, Hkv, kv_max, kv_bf16, pos, on_device, with_bias, flush=True)
+            qkv = orc.normal(n, 510 + pos)
+            b3 = (dbq, dbk, dbv) if with_bias else (None, None, None)
+            # two launches
+            q1, K1, V1, o1 = lib.to_device(qkv), lib.to_device(K0), lib.to_device(V0), lib.empty((Hq, D))
+            lib.rope_table(tab, D, pos, base)
+            if with_bias:
+                lib.qkv_rope_append_tab(q1, dbq, dbk, dbv, K1, V1, Hq, Hkv, D, pos, kv_max, tab, kv_bf16=kv_bf16)
+            else:
+                zq, zk, zv = (lib.to_device(np.zeros(m, np.float32)) for m in (Hq * D, Hkv * D, Hkv * D))
+                lib.qkv_rope_append_tab(q1, zq, zk, zv, K1, V1, Hq, Hkv, D, pos, kv_max, tab, kv_bf16=kv_bf16)
+                for z in (zq, zk, zv):
+                    z.free()
+            lib.attn_decode(q1, K1, V1, o1, Hq, Hkv, pos + 1, kv_max, D, scale, kv_bf16)
+            # one launch
+            q2, K2, V2, o2 = lib.to_device(qkv), lib.to_device(K0), lib.to_device(V0), lib.empty((Hq, D))
+            o2.upload(np.full((Hq, D), np.nan, np.float32))
+            if on_device:
+                dpos.upload(np.array([pos], np.uint32))
+                lib.rope_table(tab, D, 0, base, d_pos=dpos)
+                lib.attn_decode_qkv(q2, *b3, K2, V2, o2, Hq, Hkv, 0, kv_max, D, scale, tab, d_pos=dpos,
+                                    partials=part, kv_bf16=kv_bf16)
+            else:
+                lib.attn_decode_qkv(q2, *b3, K2, V2, o2, Hq, Hkv, pos, kv_max, D, scale, tab, kv_bf16=kv_bf16)
+            k1, v1, k2, v2 = K1.numpy(cache_dt), V1.numpy(cache_dt), K2.numpy(cache_dt), V2.numpy(cache_dt)
+            assert np.array_equal(k1, k2) and np.array_equal(v1, v2), pos
+            assert not np.array_equal(k2[:, pos], K0[:, pos])
+            assert np.array_equal(q2.numpy(), qkv)
+            got, two = o2.numpy(), o1.numpy()
+            assert np.all(np.isfinite(got)), pos
+            assert allclose(got, two, RTOL, ATOL), (pos, maxrel(got, two))
+            # the oracle on the same cache contents
+            zero = np.zeros_like
+            qr = orc.rope(qkv[:Hq * D].reshape(Hq, D), pos, base, bias=(bq if with_bias else zero(bq)).reshape(Hq, D))
+            want = orc.attn_decode(qr, widen(k2), widen(v2), scale, ctx=pos + 1)
+            assert allclose(got, want, RTOL, ATOL), (pos, maxrel(got, want))
+            for b in (q1, K1, V1, o1, q2, K2, V2, o2):
+                b.free()
+    # full cache: the device position has run past the capacity
+    qkv = orc.normal(n, 599)
+    q2, K2, V2, o2 = lib.to_device(qkv), lib.to_device(K0), lib.to_device(V0), lib.empty((Hq, D))
+    dpos.upload(np.array([kv_max], np.uint32))
+    lib.rope_table(tab, D, 0, base, d_pos=dpos)
+    lib.attn_decode_qkv(q2, dbq, dbk, dbv, K2, V2, o2, Hq, Hkv, 0, kv_max, D, scale, tab, d_pos=dpos,
+                        partials=part, kv_bf16=kv_bf16)
+    assert np.array_equal(K2.numpy(cache_dt), K0) and np.array_equal(V2.numpy(cache_dt), V0)
+    qr = orc.rope(qkv[:Hq * D].reshape(Hq, D), kv_max, base, bias=bq.reshape(Hq, D))
+    want = orc.attn_decode(qr, widen(K0), widen(V0), scale, ctx=kv_max)
+    assert allclose(o2.numpy(), want, RTOL, ATOL)
+    with pytest.raises(Exception):
+        lib.attn_decode_qkv(q2, dbq, dbk, dbv, K2, V2, o2, Hq, Hkv, kv_max, kv_max, D, scale, tab, kv_bf16=kv_bf16)
+    for b in (q2, K2, V2, o2, dbq, dbk, dbv, tab, dpos, part):
+        b.free()
