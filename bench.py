@@ -200,7 +200,7 @@ def side_kernels(lib, orc):
     left in the caches."""
     rng = np.random.default_rng(7)
     e0, e1 = lib.event(), lib.event()
-    out = {"gemv_bf16_row": {}, "gemv_bf16_kn": {}, "attn_decode_f32": {}}
+    out = {"gemv_bf16_row": {}, "gemv_bf16_kn": {}, "attn_decode_f32": {}, "load_convert_f16": {}}
 
     def timed(calls, n):
         for i in range(min(n, 3)):
@@ -225,6 +225,22 @@ def side_kernels(lib, orc):
             out[name]["%dx%d" % (N, K)] = {"us": round(ms * 1e3, 2), "GB/s": round(nb / ms / 1e6, 1)}
         for b in (w, x, y):
             b.free()
+
+    # Load-time conversion of a model file's f16 rows (the 7B LM head, 1.09 GB of f16): into the
+    # int4 group format and into bf16 rows. GB/s over bytes read + bytes written.
+    N, K = 152064, 3584
+    src = lib.empty_bytes(2 * N * K)
+    host = (rng.integers(0, 65536, 1 << 22, dtype=np.uint16) & 0x83ff) | 0x2000      # |w| ~ 0.01
+    for o in range(0, 2 * N * K, host.nbytes):
+        lib._chk(lib.c.tlhip_memcpy_h2d(src.ptr + o, host.ctypes.data, min(host.nbytes, 2 * N * K - o)))
+    q4, b16 = lib.empty_bytes(N * K // 2 + N * (K // 32) * 4), lib.empty_bytes(2 * N * K)
+    ms = timed(lambda i: lib.quantize_q4(src, lib.T_F16, q4, N, K), 5)
+    nb = 2 * N * K + q4.nbytes
+    out["load_convert_f16"]["to_q4_152064x3584"] = {"us": round(ms * 1e3, 1), "GB/s": round(nb / ms / 1e6, 1)}
+    ms = timed(lambda i: lib.convert(src, lib.T_F16, b16, lib.T_BF16, N * K), 5)
+    out["load_convert_f16"]["to_bf16_152064x3584"] = {"us": round(ms * 1e3, 1), "GB/s": round(4 * N * K / ms / 1e6, 1)}
+    for b in (src, q4, b16):
+        b.free()
 
     H, D = 28, 128
     for ctx in (512, 2048, 8192, 32768):

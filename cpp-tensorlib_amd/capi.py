@@ -24,7 +24,8 @@ OPS = dict(add=0, sub=1, mul=2, div=3, pow=4, exp=5, log=6, sqrt=7, sigmoid=8, r
 
 CENSUS = ["binary", "bcast", "unary", "row_op", "gemm", "gemv_f32", "gemv_bf16", "gemv_bf16_row",
           "gemv_q4", "attn_decode", "rope", "rmsnorm", "rmsnorm_res", "swiglu", "argmax",
-          "kv_append", "kv_fill", "split_heads", "merge_heads", "gemm_bf16_nt", "attn_prefill"]
+          "kv_append", "kv_fill", "split_heads", "merge_heads", "gemm_bf16_nt", "attn_prefill",
+          "convert", "quantize_q4"]
 
 # name -> (restype, argtypes): exactly the declarations of include/tensorlib_hip.h
 SIGNATURES = {
@@ -84,6 +85,10 @@ SIGNATURES = {
     "tlhip_qkv_rope_append_dpos": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, f32, cint]),
     "tlhip_rope_table": (cint, [P, i64, i64, P, f32]),
     "tlhip_qkv_rope_append_tab": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, P, i64, P, cint]),
+    "tlhip_convert": (cint, [P, cint, P, cint, i64]),
+    "tlhip_convert_transpose": (cint, [P, cint, P, cint, i64, i64, i64, i64]),
+    "tlhip_quantize_q4": (cint, [P, cint, P, P, i64, i64, i64]),
+    "tlhip_embed_gather_f16": (cint, [P, P, P, i64, i64]),
     "tlhip_attn_decode_qkv": (cint, [P, P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, cint, P, i64]),
     "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
     "tlhip_token_advance": (cint, [P, P, P, i64]),
@@ -340,6 +345,24 @@ class TlHip:
         self._chk(self.c.tlhip_attn_decode_qkv(
             qkv.ptr, opt(bq), opt(bk), opt(bv), Kc.ptr, Vc.ptr, out.ptr, Hq, Hkv, pos, opt(d_pos), kv_max,
             D, scale, table.ptr, int(kv_bf16), opt(partials), partials.nbytes if partials is not None else 0))
+
+    # element types of the load-time converters
+    T_F32, T_F16, T_BF16 = 0, 1, 2
+
+    def convert(self, src, src_type, dst, dst_type, n):
+        self._chk(self.c.tlhip_convert(src.ptr, src_type, dst.ptr, dst_type, n))
+
+    def convert_transpose(self, src, src_type, dst, dst_type, rows, cols, ld_dst, col_base=0):
+        self._chk(self.c.tlhip_convert_transpose(src.ptr, src_type, dst.ptr, dst_type, rows, cols, ld_dst, col_base))
+
+    def quantize_q4(self, src, src_type, q4buf, rows, K, row_base=0, total_rows=None, group=32):
+        """Quantise `rows` file rows into rows [row_base, row_base + rows) of a q4 buffer of total_rows."""
+        total = rows if total_rows is None else total_rows
+        self._chk(self.c.tlhip_quantize_q4(src.ptr, src_type, q4buf.ptr + row_base * K // 2,
+                                           q4buf.ptr + total * K // 2 + row_base * (K // 32) * 4, rows, K, group))
+
+    def embed_gather_f16(self, table, d_token, out, hidden, vocab):
+        self._chk(self.c.tlhip_embed_gather_f16(table.ptr, d_token.ptr, out.ptr, hidden, vocab))
 
     def embed_gather_bf16(self, table, d_token, out, hidden, vocab):
         self._chk(self.c.tlhip_embed_gather_bf16(table.ptr, d_token.ptr, out.ptr, hidden, vocab))

@@ -7,7 +7,9 @@
 #include <map>
 #include <string>
 
+#include "../include/tl/gguf_dump.h"
 #include "../include/tl/qwen_decode.h"
+#include "../include/tl/tokenizer.h"
 
 using namespace tl;
 
@@ -36,6 +38,95 @@ void* tlq_create(const qwen::dims* d) {
 }
 
 void tlq_destroy(void* hv) { delete static_cast<handle*>(hv); }
+
+// ---- model files ------------------------------------------------------------------------------
+// The last error of tlq_gguf_* / tlq_create_from_gguf on this thread ("" when none).
+static thread_local std::string g_file_error;
+const char* tlq_file_error() { return g_file_error.c_str(); }
+
+// Parses a GGUF file on the host (no GPU involved). NULL on error.
+void* tlq_gguf_open(const char* path) {
+  g_file_error.clear();
+  try {
+    return new gguf::model(path);
+  } catch (const std::exception& e) {
+    g_file_error = e.what();
+    return nullptr;
+  }
+}
+void tlq_gguf_close(void* g) { delete static_cast<gguf::model*>(g); }
+// Writes the canonical rendering (tl/gguf_dump.h) into buf (cap bytes, NUL-terminated when it
+// fits) and returns its length without the NUL.
+int64_t tlq_gguf_dump(void* g, char* buf, int64_t cap) {
+  const std::string text = gguf_dump::render(*static_cast<gguf::model*>(g));
+  if (buf && cap > (int64_t)text.size()) std::memcpy(buf, text.c_str(), text.size() + 1);
+  return (int64_t)text.size();
+}
+// Hyperparameters a loader would use; 0 on success.
+int tlq_gguf_dims(void* g, int64_t max_ctx, qwen::dims* out) {
+  g_file_error.clear();
+  return qwen::dims_from_gguf(*static_cast<gguf::model*>(g), max_ctx, *out, &g_file_error) ? 0 : -1;
+}
+
+// ---- tokenizer (host only) --------------------------------------------------------------------
+void* tlq_tok_open(const char* path) {
+  g_file_error.clear();
+  try {
+    return new tokenizer(std::string(path));
+  } catch (const std::exception& e) {
+    g_file_error = e.what();
+    return nullptr;
+  }
+}
+void tlq_tok_close(void* t) { delete static_cast<tokenizer*>(t); }
+void tlq_tok_special_ids(void* t, int* bos, int* eos) {
+  *bos = static_cast<tokenizer*>(t)->bos_id();
+  *eos = static_cast<tokenizer*>(t)->eos_id();
+}
+// ids of text[0, n) into out (cap entries); returns the count, or -1 when encode throws.
+int64_t tlq_tok_encode(void* t, const char* text, int64_t n, int32_t* out, int64_t cap) {
+  g_file_error.clear();
+  try {
+    const std::vector<int> ids = static_cast<tokenizer*>(t)->encode(std::string(text, (size_t)n));
+    for (size_t i = 0; i < ids.size() && (int64_t)i < cap; i++) out[i] = ids[i];
+    return (int64_t)ids.size();
+  } catch (const std::exception& e) {
+    g_file_error = e.what();
+    return -1;
+  }
+}
+// bytes of ids[0, n) into out (cap bytes); returns the length, or -1 when decode throws.
+int64_t tlq_tok_decode(void* t, const int32_t* ids, int64_t n, char* out, int64_t cap) {
+  g_file_error.clear();
+  try {
+    const std::string s = static_cast<tokenizer*>(t)->decode(std::vector<int>(ids, ids + n));
+    std::memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
+    return (int64_t)s.size();
+  } catch (const std::exception& e) {
+    g_file_error = e.what();
+    return -1;
+  }
+}
+// bit 0: letter, bit 1: number, bit 2: whitespace - the classes the pre-tokenizer uses
+int tlq_unicode_class(uint32_t cp) {
+  return (unicode::is_letter(cp) ? 1 : 0) | (unicode::is_number(cp) ? 2 : 0) | (unicode::is_space(cp) ? 4 : 0);
+}
+
+// A model built from a GGUF file: fmt 0 = int4 groups, 1 = bf16 rows. NULL on error.
+void* tlq_create_from_gguf(const char* path, int fmt, int64_t max_ctx) {
+  g_file_error.clear();
+  auto* h = new handle();
+  try {
+    gguf::model g(path);
+    if (qwen::load_gguf(h->M, g, fmt == 0 ? qwen::wfmt::q4 : qwen::wfmt::bf16_row, max_ctx, &g_file_error))
+      return h;
+  } catch (const std::exception& e) {
+    g_file_error = e.what();
+  }
+  delete h;
+  return nullptr;
+}
+void tlq_get_dims(void* hv, qwen::dims* out) { *out = static_cast<handle*>(hv)->M.d; }
 
 // One layer's blobs in the reference's storage forms (q4 buffers, f32 vectors).
 int tlq_set_layer_q4(void* hv, int64_t li, const uint8_t* wq, const uint8_t* wk, const uint8_t* wv,

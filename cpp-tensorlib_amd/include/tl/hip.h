@@ -121,6 +121,10 @@ struct api {
   int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
   int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
+  int (*convert)(const void*, int, void*, int, int64_t) = nullptr;
+  int (*convert_transpose)(const void*, int, void*, int, int64_t, int64_t, int64_t, int64_t) = nullptr;
+  int (*quantize_q4)(const void*, int, void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*embed_gather_f16)(const void*, const void*, void*, int64_t, int64_t) = nullptr;
   int (*attn_decode_qkv)(const void*, const void*, const void*, const void*, void*, void*, void*, int64_t,
                         int64_t, int64_t, const void*, int64_t, int64_t, float, const void*, int, void*,
                         int64_t);
@@ -223,6 +227,8 @@ struct context {
               bind(f.rope_table, "tlhip_rope_table") &&
               bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
               bind(f.attn_decode_qkv, "tlhip_attn_decode_qkv") &&
+              bind(f.convert, "tlhip_convert") && bind(f.convert_transpose, "tlhip_convert_transpose") &&
+              bind(f.quantize_q4, "tlhip_quantize_q4") && bind(f.embed_gather_f16, "tlhip_embed_gather_f16") &&
               bind(f.embed_gather_bf16, "tlhip_embed_gather_bf16") &&
               bind(f.token_advance, "tlhip_token_advance") &&
               bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
@@ -388,6 +394,14 @@ inline void upload(void* native, const float* src, int64_t n) {
   if (src != m->host) std::memcpy(m->host, src, bytes);
   c.f.memcpy_h2d(m->dev, m->host, bytes);
   m->where = context::BOTH;
+}
+
+// Blocking H2D from any host memory (pageable or a file mapping) to a device address, which
+// may lie inside a managed buffer; ordered after the launches queued so far.
+inline bool upload_raw(void* dst_dev, const void* src_host, int64_t bytes) {
+  auto& c = context::get();
+  if (!c.ready || !dst_dev || !src_host || bytes < 0) return false;
+  return bytes == 0 || c.f.memcpy_h2d(dst_dev, src_host, (size_t)bytes) == 0;
 }
 
 inline void upload_u32(void* native, unsigned val) {
@@ -778,6 +792,43 @@ inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
   return detail::done_(c, c.f.attn_decode_qkv(qkv, bq, bk, bv, Kc, Vc, out, n_q_heads, n_kv_heads, pos,
                                               d_pos, kv_max, D, scale, table, kv_bf16 ? 1 : 0, partials,
                                               partials_bytes));
+}
+
+// ---- load-time weight conversion on the device ---------------------------------------------
+// The file's element types as the converters number them.
+enum class elem : int { f32 = 0, f16 = 1, bf16 = 2 };
+// dst[i] = narrow(widen(src[i])): file rows [out, in] into bf16 (or f32) rows [N, K].
+inline bool convert(void* src, elem st, void* dst, elem dt, int64_t n) {
+  auto& c = context::get();
+  if (!c.ready || !src || !dst || n <= 0) return false;
+  c.device_read_(src);
+  c.device_write_(dst);
+  return detail::done_(c, c.f.convert(src, (int)st, dst, (int)dt, n));
+}
+// file rows [out = rows, in = cols] into the seam's [K, N] layout at columns [col_base, col_base + rows)
+inline bool convert_transpose(void* src, elem st, void* dst, elem dt, int64_t rows, int64_t cols,
+                              int64_t ld_dst, int64_t col_base) {
+  auto& c = context::get();
+  if (!c.ready || !src || !dst) return false;
+  c.device_read_(src);
+  c.device_write_(dst);
+  return detail::done_(c, c.f.convert_transpose(src, (int)st, dst, (int)dt, rows, cols, ld_dst, col_base));
+}
+// array::to_q4 of the widened rows, written into the packed and scale sections given
+inline bool quantize_q4(void* src, elem st, void* packed, void* scales, int64_t rows, int64_t K) {
+  auto& c = context::get();
+  if (!c.ready || !src || !packed || !scales) return false;
+  c.device_read_(src);
+  c.device_write_(packed);
+  return detail::done_(c, c.f.quantize_q4(src, (int)st, packed, scales, rows, K, kQ4Group));
+}
+inline bool embed_gather_f16(void* table, void* d_token, void* out, int64_t hidden, int64_t vocab) {
+  auto& c = context::get();
+  if (!c.ready) return false;
+  c.device_read_(table);
+  c.device_read_(d_token);
+  c.device_write_(out);
+  return detail::done_(c, c.f.embed_gather_f16(table, d_token, out, hidden, vocab));
 }
 
 // ---- device-resident greedy loop -----------------------------------------------------------

@@ -5,7 +5,8 @@
 // (Layer/Scratch/Model: 175-308; run_layers_: 673-740; step_imperative:
 // 747-752; captured_decoder: 791-905), with two differences that the task
 // asks for: the dimensions are parameters (0.5B and 7B shapes), and weights
-// come from memory blobs instead of a GGUF file.
+// come from memory blobs or from a GGUF file whose tensors are converted on the
+// device (load_gguf).
 //
 // Per token and layer the step issues, in stream order and with no host sync:
 //   fused QKV GEMV -> rope(q,+bias) , rope(k,+bias) , v += bias -> cache append
@@ -30,6 +31,7 @@
 #include <string>
 #include <vector>
 
+#include "gguf.h"
 #include "hip.h"
 #include "types.h"
 
@@ -118,7 +120,8 @@ struct prefill_scratch {
 struct model {
   dims d{};
   prefill_scratch ps;
-  std::vector<uint16_t> embed;  // bf16 [vocab, hidden], gathered on the host (qm:530-535)
+  std::vector<uint16_t> embed;  // [vocab, hidden] bf16 or f16 rows, gathered on the host (qm:530-535)
+  bool embed_f16 = false;       // rows are IEEE half, as a model file stores token_embd (qm:297)
   void* onorm = nullptr;
   linear lm_head;
   std::vector<layer> layers;
@@ -385,6 +388,200 @@ inline bool fill_cache_random(model& M, int64_t upto, uint32_t seed) {
   return ok;
 }
 
+// ---- a model file as the source of the weights (qm:449-505 build) ---------------------------
+// The reference widens every f16 tensor to f32 on the host, transposes or stacks it there,
+// narrows to bf16 / quantises to int4 and uploads the result. Here the mapped file bytes go
+// to the device as they are, through one staging buffer, and tlhip_convert /
+// tlhip_quantize_q4 write the decode formats straight into the fused weight buffers:
+// the same values bit for bit, with the element loops on the GPU.
+namespace detail {
+
+inline bool why_(std::string* why, const std::string& msg) {
+  if (why) *why = msg;
+  return false;
+}
+
+inline bool elem_of(gguf::ggml_type t, hip::elem& e) {
+  switch (t) {
+    case gguf::ggml_type::f32: e = hip::elem::f32; return true;
+    case gguf::ggml_type::f16: e = hip::elem::f16; return true;
+    case gguf::ggml_type::bf16: e = hip::elem::bf16; return true;
+    default: return false;   // block-quantised files: dequantisation is the consumer's job, not built
+  }
+}
+inline int64_t elem_bytes(hip::elem e) { return e == hip::elem::f32 ? 4 : 2; }
+
+// Uploads file tensors through one device staging buffer and converts them in place.
+struct converter {
+  void* stage = nullptr;
+  int64_t stage_bytes = 0;
+  bool init(int64_t bytes = int64_t(64) << 20) {
+    stage_bytes = bytes;
+    stage = hip::alloc_device(bytes);
+    return stage != nullptr;
+  }
+  void destroy() {
+    if (stage) hip::release(stage, 0, nullptr);
+    stage = nullptr;
+  }
+  // Rows [out, in] of one file tensor into rows [row_base, row_base + out) of `dst`.
+  bool rows_into(const gguf::tensor_info& t, int64_t out, int64_t in, const linear& dst, int64_t row_base) {
+    hip::elem e;
+    if (!elem_of(t.type, e)) return false;
+    const int64_t row_bytes = in * elem_bytes(e);
+    int64_t per = stage_bytes / row_bytes;      // whole rows per staged piece
+    if (per < 1) return false;
+    const char* src = static_cast<const char*>(t.data);
+    char* w = static_cast<char*>(dst.w);
+    for (int64_t r = 0; r < out; r += per) {
+      const int64_t n = std::min(per, out - r);
+      if (!hip::upload_raw(stage, src + r * row_bytes, n * row_bytes)) return false;
+      const int64_t row = row_base + r;
+      bool ok;
+      if (dst.fmt == wfmt::q4)
+        ok = hip::quantize_q4(stage, e, w + row * in / 2,
+                              w + dst.N * in / 2 + row * (in / kQ4Group) * 4, n, in);
+      else
+        ok = hip::convert(stage, e, w + row * in * 2, hip::elem::bf16, n * in);
+      if (!ok) return false;
+    }
+    return true;
+  }
+};
+
+// A linear layer's file tensor must be 2-D with dims {in, out} (dims[0] is the contiguous axis).
+inline const gguf::tensor_info* linear_tensor(const gguf::model& g, const std::string& name, int64_t in,
+                                              int64_t out, std::string* why) {
+  const gguf::tensor_info* t = g.tensor(name);
+  if (!t) { why_(why, "missing tensor " + name); return nullptr; }
+  hip::elem e;
+  if (!elem_of(t->type, e)) { why_(why, name + ": storage type not supported (f32, f16, bf16 only)"); return nullptr; }
+  if (t->dims.size() != 2 || (int64_t)t->dims[0] != in || (int64_t)t->dims[1] != out) {
+    why_(why, name + ": shape does not match the hyperparameters");
+    return nullptr;
+  }
+  return t;
+}
+
+// An f32 vector of the file (norm weights, biases); `optional` ones default to a constant.
+inline bool vector_f32(const gguf::model& g, const std::string& name, int64_t len, bool optional,
+                       float fill, std::vector<float>& out, std::string* why) {
+  out.assign((size_t)len, fill);
+  const gguf::tensor_info* t = g.tensor(name);
+  if (!t) return optional ? true : why_(why, "missing tensor " + name);
+  if (t->type != gguf::ggml_type::f32 || (int64_t)t->n_elements() != len)
+    return why_(why, name + ": expected " + std::to_string(len) + " f32 values");
+  std::memcpy(out.data(), t->data, (size_t)len * 4);
+  return true;
+}
+
+}  // namespace detail
+
+// Hyperparameters from the metadata (`<arch>.block_count` ..., arch = general.architecture,
+// "qwen2" when absent: qm:918-922 checks exactly these keys) and from token_embd's shape.
+inline bool dims_from_gguf(const gguf::model& g, int64_t max_ctx, dims& d, std::string* why = nullptr) {
+  try {
+    const std::string a = (g.has("general.architecture") ? g.kv("general.architecture").as_str() : "qwen2") + ".";
+    d.n_layers = (int64_t)g.kv(a + "block_count").as_count();
+    d.hidden = (int64_t)g.kv(a + "embedding_length").as_count();
+    d.ff = (int64_t)g.kv(a + "feed_forward_length").as_count();
+    d.n_q_heads = (int64_t)g.kv(a + "attention.head_count").as_count();
+    d.n_kv_heads = g.has(a + "attention.head_count_kv") ? (int64_t)g.kv(a + "attention.head_count_kv").as_count()
+                                                         : d.n_q_heads;
+    if (d.n_q_heads <= 0) return detail::why_(why, "attention.head_count is zero");
+    d.head_dim = g.has(a + "attention.key_length") ? (int64_t)g.kv(a + "attention.key_length").as_count()
+                                                   : d.hidden / d.n_q_heads;
+    d.eps = g.has(a + "attention.layer_norm_rms_epsilon") ? g.kv(a + "attention.layer_norm_rms_epsilon").as_f32() : 1e-6f;
+    d.rope_base = g.has(a + "rope.freq_base") ? g.kv(a + "rope.freq_base").as_f32() : 1e6f;
+    const gguf::tensor_info* emb = g.tensor("token_embd.weight");
+    if (!emb || emb->dims.size() != 2 || (int64_t)emb->dims[0] != d.hidden)
+      return detail::why_(why, "token_embd.weight missing or not [vocab, hidden]");
+    d.vocab = (int64_t)emb->dims[1];
+    d.max_ctx = max_ctx;
+    if (g.has(a + "context_length")) d.max_ctx = std::min<int64_t>(max_ctx, (int64_t)g.kv(a + "context_length").as_count());
+  } catch (const std::exception& e) {
+    return detail::why_(why, e.what());
+  }
+  if (d.n_layers <= 0 || d.hidden <= 0 || d.ff <= 0 || d.n_kv_heads <= 0 || d.n_q_heads % d.n_kv_heads != 0 ||
+      (d.head_dim != 64 && d.head_dim != 128) || d.max_ctx <= 0 || d.hidden % kQ4Group != 0 ||
+      d.ff % kQ4Group != 0 || d.q_dim() % kQ4Group != 0)
+    return detail::why_(why, "hyperparameters outside what the decode path takes");
+  return true;
+}
+
+// Builds the model from a mapped file: linear layers into `fmt` (int4 groups or bf16 rows),
+// fused [q|k|v] and [gate|up] by stacking row blocks; norms and biases f32; the embedding
+// stays in the file's f16 (bf16 accepted) and is gathered per token. output.weight may be
+// absent (tied to token_embd.weight).
+inline bool load_gguf(model& M, const gguf::model& g, wfmt fmt, int64_t max_ctx = 4096,
+                      std::string* why = nullptr) {
+  dims d{};
+  if (!dims_from_gguf(g, max_ctx, d, why)) return false;
+  if (!init(M, d)) return detail::why_(why, "GPU backend unavailable or out of memory");
+  detail::converter cv;
+  if (!cv.init()) return detail::why_(why, "no staging buffer");
+  const int64_t E = d.hidden;
+  auto make = [&](int64_t N, int64_t K) {
+    linear L{nullptr, N, K, fmt};
+    L.w = hip::alloc_device(L.bytes());
+    return L;
+  };
+  struct part { std::string name; int64_t out; };
+  auto fill = [&](linear& L, std::vector<part> parts) {
+    if (!L.w) return detail::why_(why, "out of device memory");
+    int64_t row = 0;
+    for (const auto& p : parts) {
+      const gguf::tensor_info* t = detail::linear_tensor(g, p.name, L.K, p.out, why);
+      if (!t) return false;
+      if (!cv.rows_into(*t, p.out, L.K, L, row)) return detail::why_(why, p.name + ": conversion failed");
+      row += p.out;
+    }
+    return true;
+  };
+  bool ok = true;
+  std::vector<float> bq, bk, bv, an, fn;
+  for (int64_t l = 0; l < d.n_layers && ok; l++) {
+    layer& L = M.layers[(size_t)l];
+    const std::string p = "blk." + std::to_string(l) + ".";
+    L.wqkv = make(d.qkv_dim(), E);
+    L.wo = make(E, d.q_dim());
+    L.wgu = make(2 * d.ff, E);
+    L.wd = make(E, d.ff);
+    ok = fill(L.wqkv, {{p + "attn_q.weight", d.q_dim()}, {p + "attn_k.weight", d.kv_dim()}, {p + "attn_v.weight", d.kv_dim()}}) &&
+         fill(L.wo, {{p + "attn_output.weight", E}}) &&
+         fill(L.wgu, {{p + "ffn_gate.weight", d.ff}, {p + "ffn_up.weight", d.ff}}) &&
+         fill(L.wd, {{p + "ffn_down.weight", E}}) &&
+         detail::vector_f32(g, p + "attn_q.bias", d.q_dim(), true, 0.f, bq, why) &&
+         detail::vector_f32(g, p + "attn_k.bias", d.kv_dim(), true, 0.f, bk, why) &&
+         detail::vector_f32(g, p + "attn_v.bias", d.kv_dim(), true, 0.f, bv, why) &&
+         detail::vector_f32(g, p + "attn_norm.weight", E, false, 1.f, an, why) &&
+         detail::vector_f32(g, p + "ffn_norm.weight", E, false, 1.f, fn, why) &&
+         detail::set_vectors(M, L, bq.data(), bk.data(), bv.data(), an.data(), fn.data());
+  }
+  if (ok) {
+    std::vector<float> on;
+    ok = detail::vector_f32(g, "output_norm.weight", E, false, 1.f, on, why);
+    if (ok) M.onorm = detail::dev_from_host(on.data(), E * 4);
+    M.lm_head = make(d.vocab, E);
+    const char* head = g.tensor("output.weight") ? "output.weight" : "token_embd.weight";
+    ok = ok && M.onorm && fill(M.lm_head, {{head, d.vocab}});
+  }
+  if (ok) {
+    const gguf::tensor_info* emb = g.tensor("token_embd.weight");
+    if (emb->type == gguf::ggml_type::f16) M.embed_f16 = true;
+    else if (emb->type == gguf::ggml_type::bf16) M.embed_f16 = false;
+    else ok = detail::why_(why, "token_embd.weight: f16 or bf16 expected");
+    if (ok) {
+      const uint16_t* rows = static_cast<const uint16_t*>(emb->data);
+      M.embed.assign(rows, rows + d.vocab * E);
+    }
+  }
+  hip::flush();
+  cv.destroy();
+  M.ready = ok;
+  return ok;
+}
+
 inline void reset_cache(model& M) {
   for (auto& L : M.layers) L.cache.pos = 0;
 }
@@ -396,7 +593,10 @@ inline void set_cache_pos(model& M, int64_t p) {
 inline void stage_embed(model& M, int64_t token) {
   const dims& d = M.d;
   const uint16_t* r = M.embed.data() + (size_t)token * d.hidden;
-  for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = bf16_to_f32(r[j]);
+  if (M.embed_f16)
+    for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = f16_to_f32(r[j]);
+  else
+    for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = bf16_to_f32(r[j]);
   hip::upload(M.s.embedb, M.s.embed_host, d.hidden);
 }
 
@@ -571,7 +771,10 @@ inline bool stage_chunk(model& M, const int64_t* tokens, int64_t T) {
   for (int64_t t = 0; t < T; t++) {
     const uint16_t* r = M.embed.data() + (size_t)tokens[t] * d.hidden;
     float* o = M.ps.emb_host + t * d.hidden;
-    for (int64_t j = 0; j < d.hidden; j++) o[j] = bf16_to_f32(r[j]);
+    if (M.embed_f16)
+      for (int64_t j = 0; j < d.hidden; j++) o[j] = f16_to_f32(r[j]);
+    else
+      for (int64_t j = 0; j < d.hidden; j++) o[j] = bf16_to_f32(r[j]);
   }
   hip::upload(M.ps.emb, M.ps.emb_host, T * d.hidden);
   return true;
@@ -662,7 +865,8 @@ struct greedy_loop {
     history = hip::alloc(max_ctx * 4, &history_host);
     if (!d_pos || !d_tok || !history) return false;
     auto one = [&]() {
-      bool ok = hip::embed_gather_bf16(M.embed_dev, d_tok, M.s.embedb, d.hidden, d.vocab);
+      bool ok = M.embed_f16 ? hip::embed_gather_f16(M.embed_dev, d_tok, M.s.embedb, d.hidden, d.vocab)
+                            : hip::embed_gather_bf16(M.embed_dev, d_tok, M.s.embedb, d.hidden, d.vocab);
       ok = ok && run_layers(M, M.s.embedb, 0, nullptr, d_pos, /*advance=*/false);
       ok = ok && hip::argmax_async(M.s.logitsb, d.vocab, d_tok);
       return ok && hip::token_advance(d_pos, d_tok, history, max_ctx);

@@ -38,6 +38,25 @@ inline float bf16_to_f32(uint16_t h) {
   return f;
 }
 
+// IEEE half -> float, exact for every bit pattern (model files store f16): a subnormal
+// is mantissa * 2^-24, a NaN keeps its payload.
+inline float f16_to_f32(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16, exp = (h >> 10) & 31u, man = h & 0x3ffu;
+  uint32_t bits;
+  if (exp == 0) {
+    const float sub = static_cast<float>(man) * 5.9604644775390625e-8f;   // exact, and a normal f32
+    std::memcpy(&bits, &sub, sizeof bits);
+  } else if (exp == 31) {
+    bits = 0x7f800000u | (man << 13);
+  } else {
+    bits = ((exp + 112u) << 23) | (man << 13);
+  }
+  bits |= sign;
+  float f;
+  std::memcpy(&f, &bits, sizeof f);
+  return f;
+}
+
 enum class device_type { cpu, gpu, auto_ };
 inline device_type device_ = device_type::cpu;
 inline void use_cpu() { device_ = device_type::cpu; }

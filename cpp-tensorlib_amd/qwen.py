@@ -70,6 +70,19 @@ def _load():
             "tlq_decoder_sync_host_pos": (None, [P]),
             "tlq_flush": (None, []),
             "tlq_census": (cint, [C.POINTER(C.c_uint64), cint]),
+            "tlq_file_error": (C.c_char_p, []),
+            "tlq_gguf_open": (P, [C.c_char_p]),
+            "tlq_gguf_close": (None, [P]),
+            "tlq_gguf_dump": (i64, [P, C.c_char_p, i64]),
+            "tlq_gguf_dims": (cint, [P, i64, C.POINTER(Dims)]),
+            "tlq_create_from_gguf": (P, [C.c_char_p, cint, i64]),
+            "tlq_tok_open": (P, [C.c_char_p]),
+            "tlq_tok_close": (None, [P]),
+            "tlq_tok_special_ids": (None, [P, C.POINTER(cint), C.POINTER(cint)]),
+            "tlq_tok_encode": (i64, [P, C.c_char_p, i64, P, i64]),
+            "tlq_tok_decode": (i64, [P, P, i64, C.c_char_p, i64]),
+            "tlq_unicode_class": (cint, [u32]),
+            "tlq_get_dims": (None, [P, C.POINTER(Dims)]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -81,6 +94,71 @@ def _load():
 def _p(a):
     assert a.flags["C_CONTIGUOUS"]
     return a.ctypes.data_as(P)
+
+
+class GgufFile:
+    """A GGUF v3 file parsed by tl/gguf.h (host only: no GPU is needed to read a file)."""
+
+    def __init__(self, path):
+        self.L = _load()
+        self.h = self.L.tlq_gguf_open(os.fsencode(path))
+        if not self.h:
+            raise RuntimeError(self.L.tlq_file_error().decode())
+
+    def dump(self):
+        """Canonical rendering of header, metadata and tensor directory (tl/gguf_dump.h)."""
+        n = self.L.tlq_gguf_dump(self.h, None, 0)
+        buf = C.create_string_buffer(n + 1)
+        self.L.tlq_gguf_dump(self.h, buf, n + 1)
+        return buf.value.decode("latin-1")
+
+    def dims(self, max_ctx=4096):
+        d = Dims()
+        if self.L.tlq_gguf_dims(self.h, max_ctx, C.byref(d)) != 0:
+            raise RuntimeError(self.L.tlq_file_error().decode())
+        return d
+
+    def close(self):
+        if self.h:
+            self.L.tlq_gguf_close(self.h)
+            self.h = None
+
+
+class Tokenizer:
+    """tl::tokenizer (byte-level BPE, vocabulary from a GGUF file's metadata). Host only."""
+
+    def __init__(self, path):
+        self.L = _load()
+        self.h = self.L.tlq_tok_open(os.fsencode(path))
+        if not self.h:
+            raise RuntimeError(self.L.tlq_file_error().decode("latin-1"))
+        bos, eos = cint(), cint()
+        self.L.tlq_tok_special_ids(self.h, C.byref(bos), C.byref(eos))
+        self.bos_id, self.eos_id = bos.value, eos.value
+
+    def encode(self, text):
+        raw = text.encode() if isinstance(text, str) else bytes(text)
+        cap = 4 * len(raw) + 16
+        out = np.empty(cap, np.int32)
+        n = self.L.tlq_tok_encode(self.h, raw, len(raw), _p(out), cap)
+        if n < 0:
+            raise RuntimeError(self.L.tlq_file_error().decode("latin-1"))
+        return [int(v) for v in out[:n]]
+
+    def decode(self, ids):
+        a = np.ascontiguousarray(ids, np.int32)
+        cap = 64 * max(1, len(a)) + 64
+        buf = C.create_string_buffer(cap)
+        n = self.L.tlq_tok_decode(self.h, _p(a), len(a), buf, cap)
+        if n < 0:
+            raise RuntimeError(self.L.tlq_file_error().decode("latin-1"))
+        assert n <= cap
+        return buf.raw[:n]
+
+    def close(self):
+        if self.h:
+            self.L.tlq_tok_close(self.h)
+            self.h = None
 
 
 class QwenGPU:
@@ -117,6 +195,22 @@ class QwenGPU:
         outw = np.ascontiguousarray(om.weight(-1, "outw"))
         if set_head(g.h, _p(emb), _p(onorm), _p(outw)) != 0:
             raise RuntimeError("set_head failed")
+        return g
+
+    @classmethod
+    def from_gguf(cls, path, fmt="q4", max_ctx=4096):
+        """Build from a GGUF file: f16 / f32 / bf16 tensors are uploaded as stored and converted to
+        int4 groups (fmt "q4") or bf16 rows (fmt "bf16") on the device."""
+        g = cls.__new__(cls)
+        g.L = _load()
+        if not g.L.tlq_available():
+            raise RuntimeError("tl::hip backend unavailable: %s" % g.L.tlq_unavailable_reason().decode())
+        g.h = g.L.tlq_create_from_gguf(os.fsencode(path), 0 if fmt == "q4" else 1, max_ctx)
+        if not g.h:
+            raise RuntimeError("load_gguf failed: %s" % g.L.tlq_file_error().decode())
+        g.d = Dims()
+        g.L.tlq_get_dims(g.h, C.byref(g.d))
+        g._keep = []
         return g
 
     def set_random(self, seed=1, fmt="q4"):

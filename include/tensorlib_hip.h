@@ -97,7 +97,8 @@ typedef enum {
   TLHIP_C_GEMV_F32, TLHIP_C_GEMV_BF16, TLHIP_C_GEMV_BF16_ROW, TLHIP_C_GEMV_Q4,
   TLHIP_C_ATTN_DECODE, TLHIP_C_ROPE, TLHIP_C_RMSNORM, TLHIP_C_RMSNORM_RES, TLHIP_C_SWIGLU,
   TLHIP_C_ARGMAX, TLHIP_C_KV_APPEND, TLHIP_C_KV_FILL, TLHIP_C_SPLIT_HEADS,
-  TLHIP_C_MERGE_HEADS, TLHIP_C_GEMM_BF16_NT, TLHIP_C_ATTN_PREFILL, TLHIP_C_COUNT
+  TLHIP_C_MERGE_HEADS, TLHIP_C_GEMM_BF16_NT, TLHIP_C_ATTN_PREFILL, TLHIP_C_CONVERT,
+  TLHIP_C_QUANTIZE_Q4, TLHIP_C_COUNT
 } tlhip_census_id;
 int tlhip_census(uint64_t* counts, int n);  /* copies min(n, TLHIP_C_COUNT) counters */
 int tlhip_census_reset(void);
@@ -241,6 +242,33 @@ int tlhip_embed_gather_bf16(const void* table, const void* d_token, void* out, i
                             int64_t vocab);
 /* history[*d_pos] = *d_token when *d_pos < capacity (history may be NULL), then *d_pos += 1 */
 int tlhip_token_advance(void* d_pos, const void* d_token, void* history, int64_t capacity);
+
+/* ---- load-time weight conversion on the device ------------------------------------------
+ * A model file (GGUF) stores linear layers as f16 / f32 / bf16 rows [out, in]. The reference
+ * widens, transposes, narrows and quantises them on the host, element by element, and
+ * uploads the result (bench/cuda/qwen_model.h:40-131); here the file's bytes are uploaded as
+ * they are and converted on the device, bit-identically to that host arithmetic. */
+typedef enum { TLHIP_T_F32 = 0, TLHIP_T_F16 = 1, TLHIP_T_BF16 = 2 } tlhip_elem_type;
+/* dst[i] = narrow(widen(src[i])), i < n; dst_type f32 or bf16 (round to nearest even,
+ * types.h:35-41); f16 widening is exact for every bit pattern (qwen_model.h:41-60). Same
+ * layout both sides: file rows [out, in] ARE the row layout [N, K] of tlhip_gemv_bf16_row
+ * (qwen_model.h:114-131 load_w_T_cat_row; stack parts by pointing dst at their row block). */
+int tlhip_convert(const void* src, int src_type, void* dst, int dst_type, int64_t n);
+/* dst[c * ld_dst + col_base + r] = src[r * cols + c]: file rows [out = rows, in = cols] into the
+ * seam's [K, N] layout, N = ld_dst, this tensor's outputs at columns [col_base, col_base + rows)
+ * (qwen_model.h:88-106 load_w_T_cat). dst_type f32 or bf16. */
+int tlhip_convert_transpose(const void* src, int src_type, void* dst, int dst_type, int64_t rows,
+                            int64_t cols, int64_t ld_dst, int64_t col_base);
+/* array::to_q4 (array.h:703-742) applied to the widened rows: per group of 32 consecutive k of a
+ * row, scale = max(1e-8, maxabs) / 7, q = clamp(lround(w / scale), -8, 7), nibble q + 8, even k
+ * low. packed: rows x K/2 bytes, scales: rows x K/32 floats - the two sections of a q4 buffer
+ * (point them at a row block of a fused buffer to stack parts). group must be 32. */
+int tlhip_quantize_q4(const void* src, int src_type, void* packed, void* scales, int64_t rows,
+                      int64_t K, int64_t group);
+/* tlhip_embed_gather_bf16 for an f16 [vocab, hidden] table, as the file stores token_embd and
+ * the reference gathers it (qwen_model.h:297, 531-540). */
+int tlhip_embed_gather_f16(const void* table, const void* d_token, void* out, int64_t hidden,
+                           int64_t vocab);
 
 /* ---- GEMVs that produce their own activation vector (no single reference
  * counterpart) -----------------------------------------------------------------

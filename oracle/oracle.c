@@ -120,6 +120,36 @@ void orc_bf16_widen(const uint16_t* src, float* dst, int64_t n) {
   for (int64_t i = 0; i < n; i++) dst[i] = orc_bf16_to_f32(src[i]);
 }
 
+/* IEEE half -> float as the model loader widens GGUF F16 tensors
+ * (bench/cuda/qwen_model.h:41-60): subnormals are renormalised by shifting the
+ * mantissa up, inf/nan keep their mantissa bits, everything else rebiases the
+ * exponent by 127 - 15. */
+float orc_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1Fu, mant = h & 0x3FFu, bits;
+  if (e == 0x1Fu) {
+    bits = sign | 0x7F800000u | (mant << 13);
+  } else if (e != 0) {
+    bits = sign | ((e + 112u) << 23) | (mant << 13);
+  } else if (mant == 0) {
+    bits = sign;
+  } else {
+    e = 113; /* 127 - 15 + 1 */
+    while (!(mant & 0x400u)) {
+      mant <<= 1;
+      e--;
+    }
+    bits = sign | (e << 23) | ((mant & 0x3FFu) << 13);
+  }
+  float out;
+  memcpy(&out, &bits, 4);
+  return out;
+}
+
+void orc_f16_widen(const uint16_t* src, float* dst, int64_t n) {
+  for (int64_t i = 0; i < n; i++) dst[i] = orc_f16_to_f32(src[i]);
+}
+
 int64_t orc_q4_bytes(int64_t N, int64_t K) { return N * K / 2 + N * (K / 32) * 4; }
 
 int orc_to_q4(const float* w, int64_t s0, int64_t s1, int64_t K, int64_t N, uint8_t* out) {
@@ -574,6 +604,7 @@ struct orc_qwen {
   orc_qwen_dims d;
   int q4;
   uint16_t* embed; /* bf16 [vocab, hidden] */
+  float* embed_f32; /* when set (a model file's f16 table, widened): used instead of embed */
   float* onorm;
   orc_lin outw; /* [hidden, vocab] */
   orc_layer* layers;
@@ -656,6 +687,7 @@ void orc_qwen_destroy(orc_qwen* m) {
   lin_free(&m->outw);
   free(m->onorm);
   free(m->embed);
+  free(m->embed_f32);
   free(m);
 }
 
@@ -684,7 +716,8 @@ int64_t orc_qwen_step(orc_qwen* m, int64_t token, int64_t pos, float* logits) {
   float* g = (float*)malloc((size_t)FF * 4);
   float* u = (float*)malloc((size_t)FF * 4);
   float* mm = (float*)malloc((size_t)FF * 4);
-  orc_bf16_widen(m->embed + token * E, x, E);
+  if (m->embed_f32) memcpy(x, m->embed_f32 + token * E, (size_t)E * 4);
+  else orc_bf16_widen(m->embed + token * E, x, E);
   for (int64_t l = 0; l < d->n_layers; l++) {
     orc_layer* L = &m->layers[l];
     orc_rmsnorm(x, L->an, h, 1, E, d->eps);
@@ -713,6 +746,50 @@ int64_t orc_qwen_step(orc_qwen* m, int64_t token, int64_t pos, float* logits) {
   free(x); free(h); free(x1); free(q); free(k); free(v); free(a); free(t);
   free(g); free(u); free(mm);
   return id;
+}
+
+/* Replace one weight of the model with caller data (a model built from a file instead
+ * of from the seeded generator). Linear weights come as f32 in the logical [K,N] layout and are
+ * stored in the model's format exactly as lin_init does: to_q4 / to_bf16, then widened back
+ * (what the reference's build() does with the widened file tensors,
+ * bench/cuda/qwen_model.h:449-505). Vectors are copied. "embed" takes f32 [vocab, hidden]. */
+static void lin_set(orc_lin* L, const float* w_kn, int q4) {
+  const int64_t K = L->K, N = L->N;
+  memcpy(L->f32, w_kn, (size_t)(K * N) * 4);
+  if (q4) {
+    orc_to_q4(L->f32, N, 1, K, N, (uint8_t*)L->stored);
+    orc_q4_to_f32((const uint8_t*)L->stored, K, N, L->f32);
+  } else {
+    orc_to_bf16(L->f32, (uint16_t*)L->stored, K * N);
+    orc_bf16_widen((const uint16_t*)L->stored, L->f32, K * N);
+  }
+}
+
+int orc_qwen_set(orc_qwen* m, int64_t layer, const char* name, const float* data) {
+  const orc_qwen_dims* d = &m->d;
+  const int64_t E = d->hidden, QD = d->n_q_heads * d->head_dim, KD = d->n_kv_heads * d->head_dim;
+  if (layer < 0) {
+    if (!strcmp(name, "embed")) {
+      if (!m->embed_f32) m->embed_f32 = (float*)malloc((size_t)(d->vocab * E) * 4);
+      memcpy(m->embed_f32, data, (size_t)(d->vocab * E) * 4);
+      return 0;
+    }
+    if (!strcmp(name, "onorm")) { memcpy(m->onorm, data, (size_t)E * 4); return 0; }
+    if (!strcmp(name, "outw")) { lin_set(&m->outw, data, m->q4); return 0; }
+    return -1;
+  }
+  if (layer >= d->n_layers) return -1;
+  orc_layer* L = &m->layers[layer];
+  orc_lin* lin = !strcmp(name, "wq") ? &L->wq : !strcmp(name, "wk") ? &L->wk : !strcmp(name, "wv") ? &L->wv
+               : !strcmp(name, "wo") ? &L->wo : !strcmp(name, "wg") ? &L->wg : !strcmp(name, "wu") ? &L->wu
+               : !strcmp(name, "wd") ? &L->wd : NULL;
+  if (lin) { lin_set(lin, data, m->q4); return 0; }
+  if (!strcmp(name, "bq")) { memcpy(L->bq, data, (size_t)QD * 4); return 0; }
+  if (!strcmp(name, "bk")) { memcpy(L->bk, data, (size_t)KD * 4); return 0; }
+  if (!strcmp(name, "bv")) { memcpy(L->bv, data, (size_t)KD * 4); return 0; }
+  if (!strcmp(name, "an")) { memcpy(L->an, data, (size_t)E * 4); return 0; }
+  if (!strcmp(name, "fn")) { memcpy(L->fn, data, (size_t)E * 4); return 0; }
+  return -1;
 }
 
 const void* orc_qwen_weight(const orc_qwen* m, int64_t layer, const char* name,

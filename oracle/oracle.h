@@ -38,6 +38,10 @@ uint16_t orc_f32_to_bf16(float f);                  /* types.h:35-40, RNE */
 float    orc_bf16_to_f32(uint16_t h);               /* types.h:41-46 */
 void     orc_to_bf16(const float* src, uint16_t* dst, int64_t n);   /* array.h:639-658 */
 void     orc_bf16_widen(const uint16_t* src, float* dst, int64_t n);/* array.h:685-697 */
+/* GGUF F16 widening of the model loader; pinned exhaustively (2^16 patterns) against an
+ * independent IEEE half implementation (numpy float16) in tests/test_oracle_pins.py */
+float    orc_f16_to_f32(uint16_t h);                                 /* bench/cuda/qwen_model.h:41-60 */
+void     orc_f16_widen(const uint16_t* src, float* dst, int64_t n);
 int64_t  orc_q4_bytes(int64_t N, int64_t K);        /* types.h:28-31 */
 /* w is logical [K,N] with element strides (s0,s1); out = packed [N][K/2] bytes
  * then f32 scales [N][K/32]. array.h:703-742 */
@@ -137,6 +141,7 @@ void      orc_qwen_reset(orc_qwen* m);
 /* one decode step at position pos; logits [vocab] out; returns greedy id */
 int64_t   orc_qwen_step(orc_qwen* m, int64_t token, int64_t pos, float* logits);
 /* accessors so the GPU harness can upload the very same weight bytes */
+int       orc_qwen_set(orc_qwen* m, int64_t layer, const char* name, const float* data);
 const void*  orc_qwen_weight(const orc_qwen* m, int64_t layer, const char* name, int64_t* bytes);
 
 #ifdef __cplusplus

@@ -30,6 +30,12 @@
 #include <tensorlib.h>
 #undef private
 
+// The reference's GGUF reader, parsed results rendered by the same generic text dump the
+// product's reader is rendered with (the dump touches only the surface both share).
+#include <gguf.h>
+#include <tokenizer.h>
+#include <tl/gguf_dump.h>
+
 using tl::array;
 
 namespace {
@@ -321,6 +327,64 @@ int64_t tlref_qwen_step(void* h, int64_t token, int64_t pos, float* logits) {
   for (int64_t i = 1; i < d.vocab; i++)
     if (p[i] > p[bi]) bi = i;
   return bi;
+}
+
+}  // extern "C"
+
+extern "C" {
+
+// Canonical rendering of a GGUF file as the REFERENCE's reader parses it. Returns the text
+// length (buf is filled and NUL-terminated when it fits), or -1 with the exception text in
+// buf when the reader throws.
+int64_t tlref_gguf_dump(const char* path, char* buf, int64_t cap) {
+  try {
+    tl::gguf::model m(path);
+    const std::string text = tl::gguf_dump::render(m);
+    if (buf && cap > (int64_t)text.size()) std::memcpy(buf, text.c_str(), text.size() + 1);
+    return (int64_t)text.size();
+  } catch (const std::exception& e) {
+    if (buf && cap > 0) {
+      std::strncpy(buf, e.what(), (size_t)cap - 1);
+      buf[cap - 1] = 0;
+    }
+    return -1;
+  }
+}
+
+
+// The REFERENCE's tokenizer (include/tokenizer.h) and its code-point classes.
+void* tlref_tok_open(const char* path) {
+  try {
+    return new tl::tokenizer(std::string(path));
+  } catch (const std::exception&) {
+    return nullptr;
+  }
+}
+void tlref_tok_close(void* t) { delete static_cast<tl::tokenizer*>(t); }
+void tlref_tok_special_ids(void* t, int* bos, int* eos) {
+  *bos = static_cast<tl::tokenizer*>(t)->bos_id();
+  *eos = static_cast<tl::tokenizer*>(t)->eos_id();
+}
+int64_t tlref_tok_encode(void* t, const char* text, int64_t n, int32_t* out, int64_t cap) {
+  try {
+    const std::vector<int> ids = static_cast<tl::tokenizer*>(t)->encode(std::string(text, (size_t)n));
+    for (size_t i = 0; i < ids.size() && (int64_t)i < cap; i++) out[i] = ids[i];
+    return (int64_t)ids.size();
+  } catch (const std::exception&) {
+    return -1;
+  }
+}
+int64_t tlref_tok_decode(void* t, const int32_t* ids, int64_t n, char* out, int64_t cap) {
+  try {
+    const std::string s = static_cast<tl::tokenizer*>(t)->decode(std::vector<int>(ids, ids + n));
+    std::memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
+    return (int64_t)s.size();
+  } catch (const std::exception&) {
+    return -1;
+  }
+}
+int tlref_unicode_class(uint32_t cp) {
+  return (tl::tokdata::is_L(cp) ? 1 : 0) | (tl::tokdata::is_N(cp) ? 2 : 0) | (tl::tokdata::is_WS(cp) ? 4 : 0);
 }
 
 }  // extern "C"

@@ -8,6 +8,8 @@ here. Outputs are stored as float32 (sub-sampled where large).
 
     python tests/golden/make_golden.py            # everything but the 0.5B decode
     python tests/golden/make_golden.py qwen05b     # BASELINE config 4 token sequence (~10 min)
+    python tests/golden/make_golden.py gguf        # a small GGUF file + the reference reader's view of it
+    python tests/golden/make_golden.py tokenizer   # a synthetic BPE vocabulary + the reference tokenizer's ids
 """
 import json
 import os
@@ -129,8 +131,49 @@ def qwen05b():
          top1=np.array(top1, np.float32))
 
 
+def gguf():
+    """gguf_small.gguf (written by tests/ggufwriter.py) and gguf_small.dump.txt: what the
+    REFERENCE's reader (include/gguf.h) reports for it, rendered by tl/gguf_dump.h."""
+    sys.path.insert(0, os.path.join(HERE, ".."))
+    import ggufwriter as W
+    from test_gguf_reader import rich_file
+    kv, t = rich_file()
+    path = os.path.join(HERE, "gguf_small.gguf")
+    W.write(path, kv, t, alignment=64)
+    text = R.gguf_dump(path)
+    assert text is not None
+    with open(os.path.join(HERE, "gguf_small.dump.txt"), "w", encoding="latin-1") as f:
+        f.write(text)
+    print("wrote gguf_small.gguf (%d bytes) and its reference dump (%d chars)" % (os.path.getsize(path), len(text)))
+
+
+def tokenizer():
+    """tok_vocab.gguf (the synthetic vocabulary of tests/test_tokenizer.py) and tok_cases.json: ids
+    the REFERENCE's tokenizer (include/tokenizer.h) gives for that file's CASES plus byte strings
+    with malformed UTF-8."""
+    sys.path.insert(0, os.path.join(HERE, ".."))
+    import test_tokenizer as T
+    path = os.path.join(HERE, "tok_vocab.gguf")
+    T.write_vocab(path)
+    tok = R.tokenizer(path)
+    rng = np.random.default_rng(3)
+    raws = [t.encode() for t in T.CASES] + [b"\x80", b"\xc3", b"\xe3\x81", b"\xaa\xb5 x", b"ok \xe2\x82 ok"]
+    raws += [bytes(rng.integers(0, 256, int(rng.integers(1, 40)), dtype=np.uint8)) for _ in range(40)]
+    cases = []
+    for raw in raws:
+        ids = tok.encode(raw)
+        assert ids is not None and tok.decode(ids) == raw
+        cases.append({"text_hex": raw.hex(), "ids": ids})
+    json.dump(cases, open(os.path.join(HERE, "tok_cases.json"), "w"))
+    print("wrote tok_vocab.gguf (%d bytes) and %d cases" % (os.path.getsize(path), len(cases)))
+
+
 if __name__ == "__main__":
-    if "qwen05b" in sys.argv[1:]:
+    if "tokenizer" in sys.argv[1:]:
+        tokenizer()
+    elif "gguf" in sys.argv[1:]:
+        gguf()
+    elif "qwen05b" in sys.argv[1:]:
         qwen05b()
     else:
         gemv_cases(); attn_cases(); op_cases(); decode_small()

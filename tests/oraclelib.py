@@ -90,6 +90,8 @@ class Oracle:
             "orc_qwen_destroy": (None, [P]),
             "orc_qwen_step": (i64, [P, i64, i64, P]),
             "orc_qwen_weight": (P, [P, i64, C.c_char_p, C.POINTER(i64)]),
+            "orc_qwen_set": (cint, [P, i64, C.c_char_p, P]),
+            "orc_f16_widen": (None, [P, P, i64]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -138,6 +140,13 @@ class Oracle:
         a = np.ascontiguousarray(a, np.float32)
         out = np.empty(a.shape, np.uint16)
         self.lib.orc_to_bf16(_ptr(a), _ptr(out), a.size)
+        return out
+
+    def f16_widen(self, a):
+        """IEEE half bit patterns (uint16) -> float32, the model loader's widening."""
+        a = np.ascontiguousarray(a, np.uint16)
+        out = np.empty(a.shape, np.float32)
+        self.lib.orc_f16_widen(_ptr(a), _ptr(out), a.size)
         return out
 
     def bf16_widen(self, a):
@@ -315,6 +324,13 @@ class OracleQwen:
         tok = self.orc.lib.orc_qwen_step(self.h, token, pos, _ptr(logits))
         return int(tok), logits
 
+    def set(self, layer, name, data):
+        """Replace a weight: linear layers as f32 in the logical [K,N] layout (stored in the model's
+        format like the seeded ones), vectors f32, layer -1: embed f32 [vocab, hidden], onorm, outw."""
+        a = np.ascontiguousarray(data, np.float32)
+        if self.orc.lib.orc_qwen_set(self.h, layer, name.encode(), _ptr(a)) != 0:
+            raise KeyError(name)
+
     def weight(self, layer, name):
         """Stored bytes of a weight as a numpy view (uint8 for linear weights and the
         bf16 embedding, float32 for vectors)."""
@@ -372,11 +388,33 @@ class Ref:
             "tlref_qwen_destroy": (None, [P]),
             "tlref_qwen_set": (cint, [P, i64, C.c_char_p, P, cint, i64, i64, cint]),
             "tlref_qwen_step": (i64, [P, i64, i64, P]),
+            "tlref_gguf_dump": (i64, [C.c_char_p, C.c_char_p, i64]),
+            "tlref_tok_open": (P, [C.c_char_p]),
+            "tlref_tok_close": (None, [P]),
+            "tlref_tok_special_ids": (None, [P, C.POINTER(cint), C.POINTER(cint)]),
+            "tlref_tok_encode": (i64, [P, C.c_char_p, i64, P, i64]),
+            "tlref_tok_decode": (i64, [P, P, i64, C.c_char_p, i64]),
+            "tlref_unicode_class": (cint, [u32]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
             fn.restype, fn.argtypes = res, args
         L.tlref_init()
+
+    def tokenizer(self, path):
+        return RefTokenizer(self, path)
+
+    def unicode_class(self, cp):
+        return int(self.lib.tlref_unicode_class(cp))
+
+    def gguf_dump(self, path):
+        """Canonical text of a GGUF file as the reference's reader parses it; None when it throws."""
+        n = self.lib.tlref_gguf_dump(os.fsencode(path), None, 0)
+        if n < 0:
+            return None
+        buf = C.create_string_buffer(n + 1)
+        self.lib.tlref_gguf_dump(os.fsencode(path), buf, n + 1)
+        return buf.value.decode("latin-1")
 
     def to_q4(self, w):
         w = np.ascontiguousarray(w, np.float32)
@@ -513,6 +551,35 @@ class Ref:
                 v = om.weight(li, nm).copy()
                 put(li, nm, v, 0, 0, v.size)
         return RefQwen(self, h, d)
+
+
+class RefTokenizer:
+    """The reference's tl::tokenizer; encode / decode return None where it throws."""
+
+    def __init__(self, ref, path):
+        self.lib = ref.lib
+        self.h = self.lib.tlref_tok_open(os.fsencode(path))
+        if not self.h:
+            raise RuntimeError("reference tokenizer rejected " + path)
+        bos, eos = cint(), cint()
+        self.lib.tlref_tok_special_ids(self.h, C.byref(bos), C.byref(eos))
+        self.bos_id, self.eos_id = bos.value, eos.value
+
+    def encode(self, raw):
+        cap = 4 * len(raw) + 16
+        out = np.empty(cap, np.int32)
+        n = self.lib.tlref_tok_encode(self.h, raw, len(raw), _ptr(out), cap)
+        return None if n < 0 else [int(v) for v in out[:n]]
+
+    def decode(self, ids):
+        a = np.ascontiguousarray(ids, np.int32)
+        cap = 64 * max(1, len(a)) + 64
+        buf = C.create_string_buffer(cap)
+        n = self.lib.tlref_tok_decode(self.h, _ptr(a), len(a), buf, cap)
+        return None if n < 0 else buf.raw[:n]
+
+    def close(self):
+        self.lib.tlref_tok_close(self.h)
 
 
 class RefQwen:

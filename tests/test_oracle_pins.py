@@ -24,6 +24,23 @@ def test_bf16_exhaustive_roundtrip(orc):
 
 
 # ---- q4 (array.h:703-742; test_array.cpp:809-856) --------------------------------------
+def test_f16_widen_exhaustive(orc):
+    """orc_f16_to_f32 (the model loader's widening, qwen_model.h:41-60) on all 2^16 patterns
+    against an independent IEEE half implementation (numpy's float16): equal bits for every
+    number incl. subnormals, zeros and infinities; a NaN keeps sign and mantissa bits (payload
+    shifted up by 13, no quieting)."""
+    h = np.arange(65536, dtype=np.uint16)
+    got = orc.f16_widen(h).view(np.uint32)
+    want = h.view(np.float16).astype(np.float32).view(np.uint32)
+    nan = ((h >> 10) & 31 == 31) & (h & 0x3ff != 0)
+    assert np.array_equal(got[~nan], want[~nan])
+    hn = h[nan].astype(np.uint32)
+    assert np.array_equal(got[nan], ((hn & 0x8000) << 16) | 0x7f800000 | ((hn & 0x3ff) << 13))
+    # known answers: 1.0, -2.0, the largest half, the smallest subnormal, the smallest normal
+    ka = orc.f16_widen(np.array([0x3c00, 0xc000, 0x7bff, 0x0001, 0x0400], np.uint16))
+    assert list(ka) == [1.0, -2.0, 65504.0, 2.0 ** -24, 2.0 ** -14]
+
+
 def test_q4_bytes_and_layout(orc):
     assert orc.q4_bytes(48, 256) == 48 * 128 + 48 * 8 * 4 == 7680
     K, N = 64, 3
