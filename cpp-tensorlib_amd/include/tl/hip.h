@@ -1014,6 +1014,22 @@ struct kv_cache {
   }
   // The same two with the position on the device (the host pos is NOT advanced:
   // a recorded graph replays these; captured_decoder reconciles pos afterwards).
+  // Reference forms (cuda.h:1370-1388): the cache owns the split-partials buffer of its
+  // device-position attention, sized once for the capacity on the first (warm) call.
+  bool append_dpos(void* k_new, void* v_new, void* d_pos) {
+    return kv_append_dpos(K, V, k_new, v_new, d_pos, max_ctx, n_kv_heads, D, kv_bf16);
+  }
+  void* dpos_partials = nullptr;
+  int64_t dpos_partials_bytes = 0;
+  bool attn_dpos(void* q, void* out, int64_t n_q_heads, void* d_pos, float scale) {
+    if (!dpos_partials) {
+      dpos_partials_bytes = attn_partials_bytes(n_q_heads, n_kv_heads, max_ctx, D);
+      dpos_partials = alloc_device(dpos_partials_bytes);
+      if (!dpos_partials) return false;
+    }
+    return attn_decode_dpos(q, K, V, out, n_q_heads, n_kv_heads, d_pos, max_ctx, D, scale, dpos_partials,
+                            dpos_partials_bytes, kv_bf16);
+  }
   bool rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, int64_t n_q_heads, float base,
                         void* d_pos) {
     return qkv_rope_append_dpos(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, D, d_pos, max_ctx, base,
@@ -1035,7 +1051,8 @@ struct kv_cache {
   void destroy() {
     if (K) release(K, 0, nullptr);
     if (V) release(V, 0, nullptr);
-    K = V = nullptr;
+    if (dpos_partials) release(dpos_partials, 0, nullptr);
+    K = V = dpos_partials = nullptr;
   }
 };
 

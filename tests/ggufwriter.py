@@ -56,6 +56,33 @@ def write(path, kv, tensors, **kw):
     return data
 
 
+def write_streaming(path, kv, tensors, alignment=32):
+    """Like write() for files too large to assemble in memory: tensors = [(name, storage_code,
+    dims_ne, ndarray)], each array written straight to the file."""
+    sizes = [int(a.nbytes) for _, _, _, a in tensors]
+    directory = [(n, c, d, b"") for n, c, d, _ in tensors]
+    head = bytearray(build(kv, directory, alignment=alignment))
+    # build() laid the (empty) tensors out at offset 0: patch the real offsets in
+    offsets, at = [], 0
+    for nb in sizes:
+        offsets.append(at)
+        at = (at + nb + alignment - 1) // alignment * alignment
+    pos = 24
+    for key, t, v in kv:
+        pos += len(_string(key)) + 4 + len(_value(t, v))
+    for (name, _, dims, _), off in zip(tensors, offsets):
+        pos += len(_string(name)) + 4 + 8 * len(dims) + 4
+        head[pos:pos + 8] = struct.pack("<Q", off)
+        pos += 8
+    with open(path, "wb") as f:
+        f.write(head)
+        written = 0
+        for (_, _, _, a), off in zip(tensors, offsets):
+            f.write(b"\0" * (off - written))
+            f.write(np.ascontiguousarray(a).data)
+            written = off + int(a.nbytes)
+
+
 def qwen2_file(path, dims, weights, arch="qwen2", tied=False, with_bias=True, linear_type="f16",
                extra_kv=()):
     """A Qwen2-architecture file. weights: dict name -> ndarray in the FILE's layout: linear layers
