@@ -97,6 +97,7 @@ SIGNATURES = {
     "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
     "tlhip_gemv_bf16_row_rmsnorm": (cint, [P, P, P, P, P, P, i64, i64, f32]),
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
+    "tlhip_tune_gemv_cols": (cint, [cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
 }

@@ -602,6 +602,7 @@ static int launch_cols(const float* a, const T* B, float* y, int64_t N, int64_t 
   // K splits: fill ~4 blocks per CU, keep >= 128 rows per split (32 per wavefront)
   int64_t S = ((int64_t)c.cus * 4 + ctiles - 1) / ctiles;
   if (S > K / 128) S = K / 128;
+  if (c.tune_cols_max_splits > 0 && S > c.tune_cols_max_splits) S = c.tune_cols_max_splits;
   if (S < 1) S = 1;
   int kchunk = (int)((K + S - 1) / S);
   kchunk = (kchunk + 3) & ~3;

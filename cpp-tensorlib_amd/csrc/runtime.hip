@@ -341,4 +341,9 @@ int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int wa
   return TLHIP_OK;
 }
 
+int tlhip_tune_gemv_cols(int max_k_splits) {
+  ctx().tune_cols_max_splits = max_k_splits > 0 ? max_k_splits : 0;
+  return TLHIP_OK;
+}
+
 }  // extern "C"

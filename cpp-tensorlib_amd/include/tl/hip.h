@@ -121,6 +121,7 @@ struct api {
   int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
   int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
+  int (*tune_gemv_cols)(int) = nullptr;
   int (*convert)(const void*, int, void*, int, int64_t) = nullptr;
   int (*convert_transpose)(const void*, int, void*, int, int64_t, int64_t, int64_t, int64_t) = nullptr;
   int (*quantize_q4)(const void*, int, void*, void*, int64_t, int64_t, int64_t) = nullptr;
@@ -227,7 +228,7 @@ struct context {
               bind(f.rope_table, "tlhip_rope_table") &&
               bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
               bind(f.attn_decode_qkv, "tlhip_attn_decode_qkv") &&
-              bind(f.convert, "tlhip_convert") && bind(f.convert_transpose, "tlhip_convert_transpose") &&
+              bind(f.tune_gemv_cols, "tlhip_tune_gemv_cols") && bind(f.convert, "tlhip_convert") && bind(f.convert_transpose, "tlhip_convert_transpose") &&
               bind(f.quantize_q4, "tlhip_quantize_q4") && bind(f.embed_gather_f16, "tlhip_embed_gather_f16") &&
               bind(f.embed_gather_bf16, "tlhip_embed_gather_bf16") &&
               bind(f.token_advance, "tlhip_token_advance") &&
@@ -289,6 +290,13 @@ inline void flush() {
   if (!c.ready || !c.pending) return;
   c.f.sync();
   c.pending = false;
+}
+
+// Diagnostic knob of the reference (cuda.h:496-497): true forces the [K,N] GEMVs to run
+// without K splits, false restores the built-in choice.
+inline void set_no_splitk(bool v) {
+  auto& c = context::get();
+  if (c.ready) c.f.tune_gemv_cols(v ? 1 : 0);
 }
 
 inline void cpu_barrier() {

@@ -315,6 +315,10 @@ int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
  * Results do not depend on it beyond fp32 summation order. */
 int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
                        int lanes_per_row);
+/* Upper bound on the K splits of the [K,N] GEMVs (tlhip_gemv_f32 / tlhip_gemv_bf16); 1 = no
+ * split, 0 = the built-in choice. The reference's diagnostic knob set_no_splitk (cuda.h:193-197,
+ * 496-497), which its GEMV benchmark toggles. */
+int tlhip_tune_gemv_cols(int max_k_splits);
 
 #ifdef __cplusplus
 }

@@ -110,3 +110,34 @@ def qwen2_file(path, dims, weights, arch="qwen2", tied=False, with_bias=True, li
             code = {np.dtype(np.float32): GGML["f32"], np.dtype(np.float16): GGML["f16"]}[a.dtype]
         tensors.append((name, code, list(a.shape[::-1]), a.tobytes()))
     return write(path, kv, tensors)
+
+
+def qwen05b_synthetic(path, seed=17):
+    """A Qwen2.5-0.5B-shaped F16 file (24 layers, hidden 896, 14/2 heads of 64, FF 4864, vocab 151936;
+    1.26 GB) with seeded ~N(0, 0.02) weights: the shape the reference's harness hard-codes
+    (bench/cuda/qwen_model.h:27-28). Tensors are tiled from one random block, each at its own shift."""
+    NL, E, NH, NKV, HD, FF, V = 24, 896, 14, 2, 64, 4864, 151936
+    rng = np.random.default_rng(seed)
+    block = (rng.standard_normal(1 << 21) * 0.02).astype(np.float16)
+
+    def lin(out, inn, k):
+        return np.resize(np.roll(block, 7919 * k), out * inn).reshape(out, inn)
+
+    def vec(n, mean, k):
+        return (mean + np.resize(np.roll(block, 104729 * k), n).astype(np.float32)).astype(np.float32)
+    kv = [("general.architecture", STRING, "qwen2"), ("qwen2.block_count", U32, NL),
+          ("qwen2.embedding_length", U32, E), ("qwen2.feed_forward_length", U32, FF),
+          ("qwen2.attention.head_count", U32, NH), ("qwen2.attention.head_count_kv", U32, NKV)]
+    f16, f32 = GGML["f16"], GGML["f32"]
+    t = [("token_embd.weight", f16, [E, V], lin(V, E, 1)), ("output.weight", f16, [E, V], lin(V, E, 2)),
+         ("output_norm.weight", f32, [E], vec(E, 1.0, 3))]
+    for l in range(NL):
+        p, k = "blk.%d." % l, 10 * l + 5
+        t += [(p + "attn_q.weight", f16, [E, NH * HD], lin(NH * HD, E, k)), (p + "attn_q.bias", f32, [NH * HD], vec(NH * HD, 0.0, k + 1)),
+              (p + "attn_k.weight", f16, [E, NKV * HD], lin(NKV * HD, E, k + 2)), (p + "attn_k.bias", f32, [NKV * HD], vec(NKV * HD, 0.0, k + 3)),
+              (p + "attn_v.weight", f16, [E, NKV * HD], lin(NKV * HD, E, k + 4)), (p + "attn_v.bias", f32, [NKV * HD], vec(NKV * HD, 0.0, k + 5)),
+              (p + "attn_output.weight", f16, [NH * HD, E], lin(E, NH * HD, k + 6)),
+              (p + "ffn_gate.weight", f16, [E, FF], lin(FF, E, k + 7)), (p + "ffn_up.weight", f16, [E, FF], lin(FF, E, k + 8)),
+              (p + "ffn_down.weight", f16, [FF, E], lin(E, FF, k + 9)),
+              (p + "attn_norm.weight", f32, [E], vec(E, 1.0, k + 10)), (p + "ffn_norm.weight", f32, [E], vec(E, 1.0, k + 11))]
+    write_streaming(path, kv, t)
