@@ -470,14 +470,36 @@ __global__ __launch_bounds__(256) void gemv_cols_scalar_kernel(const float* __re
   out[(size_t)blockIdx.y * N + col] = acc;
 }
 
-__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part,
-                                                              float* __restrict__ y, int N,
-                                                              int S) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= N) return;
-  float v = part[i];
-  for (int s = 1; s < S; s++) v += part[(size_t)s * N + i];
-  y[i] = v;
+// y[i] = sum over s of part[s][i], fixed order. The kernel is latency, not bytes: a block is
+// 64 columns x 16 split groups, a thread requests up to eight of its splits at once (s = g,
+// g + 16, ...), and the 16 group sums meet in LDS in group order.
+__global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __restrict__ part,
+                                                               float* __restrict__ y, int N,
+                                                               int S) {
+  __shared__ float red[16][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  float acc = 0.f;
+  if (i < N) {
+    for (int s0 = g; s0 < S; s0 += 128) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int s = s0 + 16 * u;
+        v[u] = s < S ? part[(size_t)s * N + i] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc += v[u];
+    }
+  }
+  red[g][lane] = acc;
+  __syncthreads();
+  if (g == 0 && i < N) {
+    float t = red[0][lane];
+#pragma unroll
+    for (int k = 1; k < 16; k++) t += red[k][lane];
+    y[i] = t;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -619,7 +641,7 @@ static int launch_cols(const float* a, const T* B, float* y, int64_t N, int64_t 
     hipLaunchKernelGGL(gemv_cols_scalar_kernel<T>, dim3((unsigned)ctiles, (unsigned)S), dim3(256),
                        0, c.stream, a, B, out, (int)N, (int)K, kchunk);
   if (S > 1)
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)((N + 63) / 64)), dim3(1024), 0,
                        c.stream, out, y, (int)N, (int)S);
   TLHIP_CHECK_LAUNCH(census_id);
 }
