@@ -191,6 +191,48 @@ def decode_7b(lib, steps, eager=False):
     }
 
 
+def decode_05b(lib, steps):
+    """Qwen2.5-0.5B-shape decode (BASELINE configs[3]'s architecture; the shape the reference's
+    published RTX 3090 figures are quoted on, README.md:310-311) through tl/qwen_decode.h's fused
+    step: graph replay at a fixed position after a 128-token context, and the greedy loop with
+    an argmax read-back per token (one recorded graph, position on the device)."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    out = {"workload": "Qwen2.5-0.5B-shape decode after a 128-token context, f32 KV"}
+    e0, e1 = lib.event(), lib.event()
+    for fmt in ("q4", "bf16"):
+        g = qwen.QwenGPU(dict(qwen.QWEN_05B))
+        g.set_random(5, fmt=fmt)
+        g.fill_cache_random(127, 6)
+        for _ in range(2):
+            g.step(11, 127)
+        g.capture(11, 127)
+        for _ in range(3):
+            g.replay()
+        g.flush()
+        best = None
+        for _ in range(3):
+            lib.record(e0)
+            for _ in range(steps):
+                g.replay()
+            lib.record(e1)
+            ms = lib.elapsed_ms(e0, e1) / steps
+            best = ms if best is None else min(best, ms)
+        n_loop = 64
+        g.set_cache_pos(127)
+        g.decoder_init(11, 127)
+        g.decoder_feed(11)
+        g.flush()
+        tok = 11
+        t = time.perf_counter()
+        for _ in range(n_loop):
+            tok = g.decoder_step(tok)
+        loop = (time.perf_counter() - t) / n_loop * 1e3
+        g.close()
+        out[fmt] = {"ms_per_token_graph_replay": round(best, 4), "tok_s_graph_replay": round(1e3 / best, 1),
+                    "ms_per_token_greedy_with_argmax_readback": round(loop, 4), "tok_s_greedy": round(1e3 / loop, 1)}
+    return out
+
+
 def side_kernels(lib, orc):
     """The other bandwidth-bound kernels of the path at their BASELINE shapes: the bf16 GEMV in
     both layouts (configs[1] weights as bf16; [N,K] rows for the harness, [K,N] at the array
@@ -501,6 +543,8 @@ def main():
             cpu_ms = d["algorithmic_bytes"] / (cpu_gbs * 1e9) * 1e3
             d["cpu_reference_ms_per_token_est"] = round(cpu_ms, 1)
             d["speedup_vs_cpu_reference_est"] = round(cpu_ms / d["ms_per_token"], 1)
+        if not a.eager_decode:
+            out["decode_05b"] = decode_05b(lib, max(20, a.steps))
     if not a.no_side:
         out["side_kernels"] = side_kernels(lib, orc)
     if not a.no_prefill:
