@@ -166,8 +166,9 @@ def decode_7b(lib, steps, eager=False):
     g.flush()
     t = time.perf_counter()
     queued = g.greedy_run(2 * n_loop)
-    ids = g.greedy_tokens(start, queued)          # blocks until the last token exists
+    g.flush()                                     # the last token exists
     greedy_dev = (time.perf_counter() - t) / queued * 1e3
+    ids = g.greedy_tokens(start, queued)          # one read-back of the whole history
     assert queued == 2 * n_loop and len(ids) == queued
     d = g.d
     wbytes = 0.625 * (d.n_layers * (d.hidden * (d.n_q_heads + 2 * d.n_kv_heads) * d.head_dim
