@@ -70,15 +70,21 @@ inline bool use_accelerate_ = true;
 
 enum class kernel_class { elementwise, reduction, matmul };
 
-// auto_ mode: the op size from which GPU-total (launch + flush) beats this
-// host layer's CPU loops on an MI355X box. A launch plus a flush costs ~10 us
-// here, the CPU loops run at a few GFLOP/s on one core, so the GPU wins from
-// small sizes; the matmul figure is M*N*K.
+// auto_ mode: the op size from which GPU-total (single op + flush) beats the CPU path.
+// MI355X census with the reference's own tool (misc/census.cpp compiled against this backend,
+// host = the GPU box's Xeon cores, CPU side = the reference's blocked SGEMM / loops); a
+// launch plus a flush costs ~12 us here:
+//   matmul      64^3 = 2.6e5 already GPU (0.022 vs cpu 0.035 ms), 512^3 0.091 vs 0.446 ms:
+//               the crossover lies at or below the smallest measured size.
+//   elementwise 16K cpu (0.004 vs 0.012 ms), 64K GPU (0.012 vs 0.014), 256K 0.012 vs 0.055
+//               -> ~5e4.
+//   reduction   softmax 64x256 = 16K already GPU (0.013 vs 0.054 ms): GPU from the smallest
+//               measured size.
 inline int64_t auto_threshold_(kernel_class kc) {
   switch (kc) {
-    case kernel_class::matmul: return 100'000;
-    case kernel_class::elementwise: return 200'000;
-    case kernel_class::reduction: return 16'000;
+    case kernel_class::matmul: return 200'000;        // ~58^3; GPU by 64^3
+    case kernel_class::elementwise: return 50'000;    // cpu at 16K, GPU from 64K
+    case kernel_class::reduction: return 16'000;      // GPU from ~16K
   }
   return INT64_MAX;
 }
