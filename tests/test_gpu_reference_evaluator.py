@@ -79,3 +79,21 @@ def test_reference_own_checks_pass_on_the_hip_backend(prog, needle):
     print(out, flush=True)
     assert r.returncode == 0, out[-3000:]
     assert needle in out and "skipping" not in out.lower()
+
+
+@pytest.mark.parametrize("mode", ["--gpu", "--auto", "--cpu"])
+def test_reference_unit_suite_passes_on_the_hip_backend(mode):
+    """The reference's doctest unit suite (test/test_basic.cpp + test/test_array.cpp, the ctest
+    entries `gpu`, `auto` and `cpu` of its CMakeLists.txt:293-295), compiled unmodified on this
+    backend: every test case passes in all three device modes, and with a GPU present the suite
+    runs its GPU-vs-oracle assertions (335 assertions instead of 275)."""
+    exe = os.path.join(PROGS, "tensorlib_test")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/refprogs not built (needs /root/reference at build time: make -C oracle refprogs)")
+    print("running", exe, mode, flush=True)
+    r = subprocess.run([exe, mode], env=dict(os.environ, TENSORLIB_HIP_LIB=LIB), stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, timeout=150)
+    out = r.stdout.decode(errors="replace")
+    print(out[-1500:], flush=True)
+    assert r.returncode == 0, out[-3000:]
+    assert "gpu_available=1" in out and "Status: SUCCESS!" in out and "0 failed" in out
