@@ -392,7 +392,7 @@ def reference_benches():
         text = r.stdout.decode(errors="replace")
         print(text, flush=True)
         out[" ".join([name] + [os.path.basename(a) for a in args])] = {"rc": r.returncode, "output": text}
-    for name in ("bench_q4_gemv", "bench_bf16_gemv", "bench_qwen_gemv", "bench_attn_decode"):
+    for name in ("bench_q4_gemv", "bench_bf16_gemv", "bench_qwen_gemv", "bench_attn_decode", "bench_llm"):
         run(name)
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(d, "qwen05b_synthetic_f16.gguf")

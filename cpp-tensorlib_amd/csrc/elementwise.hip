@@ -115,9 +115,9 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ 
   for (int64_t c = threadIdx.x; c < cols; c += 256) dst[c] = dst[c] / s;
 }
 
-// General f32 GEMM with transposed-view operands and an affine epilogue.
-// 64x64 tile, 16-wide K slab through LDS, 4x4 outputs per thread. Not a
-// roofline kernel: the decode path only reaches it for M>1 `dot` nodes.
+// General f32 GEMM with transposed-view operands and an affine epilogue, VALU form:
+// 64x64 tile, 16-wide K slab through LDS, 4x4 outputs per thread. Serves the small
+// products; from 128 x 128 outputs on the matrix-pipe kernel of sgemm.hip takes over.
 __global__ __launch_bounds__(256) void sgemm_kernel(const float* __restrict__ A, int64_t lda,
                                                     int ta, const float* __restrict__ B,
                                                     int64_t ldb, int tb, float* __restrict__ C,
@@ -162,6 +162,9 @@ __global__ __launch_bounds__(256) void sgemm_kernel(const float* __restrict__ A,
     }
   }
 }
+
+int launch_sgemm_mfma(const float* pa, int64_t lda, int ta, const float* pb, int64_t ldb, int tb, float* pc,
+                      int M, int N, int K, float scale, float offset, int epi);   // sgemm.hip
 
 static unsigned grid1d(int64_t n) {
   int64_t b = (n + 255) / 256;
@@ -281,6 +284,10 @@ int tlhip_gemm(const void* a, int64_t a_off, int64_t lda, int ta, const void* b,
   const float* pb = reinterpret_cast<const float*>(at(b, b_off));
   float* po = reinterpret_cast<float*>(at(out, out_off));
   const int epi = !(scale == 1.0f && offset == 0.0f);
+  if (m >= 128 && n >= 128 && k >= 16 && (m + 127) / 128 <= 65535) {
+    launch_sgemm_mfma(pa, lda, ta, pb, ldb, tb, po, (int)m, (int)n, (int)k, scale, offset, epi);
+    TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM);
+  }
   dim3 g((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64));
   if (g.y > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm: M too large for the grid");
   sgemm_kernel<<<g, dim3(256), 0, ctx().stream>>>(pa, lda, ta, pb, ldb, tb, po, (int)m, (int)n,

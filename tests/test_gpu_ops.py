@@ -175,7 +175,13 @@ def test_row_ops(lib, orc):
 
 
 @pytest.mark.parametrize("m,n,k,ta,tb", [(3, 40, 100, 0, 0), (2, 300, 700, 0, 1), (65, 64, 1030, 1, 0),
-                                         (1, 17, 33, 1, 1)])
+                                         (1, 17, 33, 1, 1),
+                                         # from 128 x 128 outputs on: the fp32 matrix-pipe kernel, all four
+                                         # operand forms, whole tiles and ragged edges, K not a slab multiple
+                                         (128, 128, 16, 0, 0), (256, 384, 512, 0, 0), (256, 384, 512, 0, 1),
+                                         (256, 384, 512, 1, 0), (256, 384, 512, 1, 1), (130, 257, 75, 0, 0),
+                                         (130, 257, 75, 0, 1), (131, 258, 77, 1, 0), (129, 129, 17, 1, 1),
+                                         (512, 640, 1001, 0, 1), (300, 128, 19, 0, 0)])
 def test_gemm_seam(lib, orc, m, n, k, ta, tb):
     A = orc.normal(m * k, 70).reshape(m, k); B = orc.normal(k * n, 71).reshape(k, n)
     As = np.ascontiguousarray(A.T) if ta else A
@@ -184,6 +190,27 @@ def test_gemm_seam(lib, orc, m, n, k, ta, tb):
     lib.gemm(da, As.shape[1], ta, db, Bs.shape[1], tb, do, m, n, k, 2.0, 1.0)
     want = orc.dot(A, B, 2.0, 1.0)
     assert allclose(do.numpy(), want, RTOL, 1e-4), maxrel(do.numpy(), want)
+    lib.gemm(da, As.shape[1], ta, db, Bs.shape[1], tb, do, m, n, k)          # identity epilogue
+    assert allclose(do.numpy(), orc.dot(A, B), RTOL, 1e-4)
+
+
+def test_gemm_seam_exact_and_strided(lib, orc):
+    """Integer-valued operands make every partial sum exact, so any summation order gives the same
+    bits: the matrix-pipe GEMM must equal the integer product exactly. Then operands that are
+    views into larger buffers (row strides larger than the row, byte offsets, unaligned bases)."""
+    rng = np.random.default_rng(4)
+    m, n, k = 256, 256, 96
+    A = rng.integers(-8, 9, (m, k)).astype(np.float32); B = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    da, db, do = lib.to_device(A), lib.to_device(B), lib.empty((m, n))
+    lib.gemm(da, k, 0, db, n, 0, do, m, n, k)
+    assert np.array_equal(do.numpy(), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32))
+    # A = rows 3.. of a [m+5, k+7] buffer starting at column 1 (unaligned, lda = k + 7); B transposed view
+    big = orc.normal((m + 5) * (k + 7), 72).reshape(m + 5, k + 7)
+    Bt = orc.normal(n * (k + 4), 73).reshape(n, k + 4)
+    dbig, dbt = lib.to_device(big), lib.to_device(Bt)
+    lib._chk(lib.c.tlhip_gemm(dbig.ptr, (3 * (k + 7) + 1) * 4, k + 7, 0, dbt.ptr, 2 * 4, k + 4, 1, do.ptr, 0, m, n, k, 1.0, 0.0))
+    want = orc.dot(np.ascontiguousarray(big[3:3 + m, 1:1 + k]), np.ascontiguousarray(Bt[:, 2:2 + k].T))
+    assert allclose(do.numpy(), want, RTOL, 1e-4)
 
 
 @pytest.mark.parametrize("Hq,Hkv,D", [(14, 2, 64), (28, 4, 128)])
