@@ -285,7 +285,8 @@ int tlhip_gemm(const void* a, int64_t a_off, int64_t lda, int ta, const void* b,
   float* po = reinterpret_cast<float*>(at(out, out_off));
   const int epi = !(scale == 1.0f && offset == 0.0f);
   if (m >= 128 && n >= 128 && k >= 16 && (m + 127) / 128 <= 65535) {
-    launch_sgemm_mfma(pa, lda, ta, pb, ldb, tb, po, (int)m, (int)n, (int)k, scale, offset, epi);
+    const int rc = launch_sgemm_mfma(pa, lda, ta, pb, ldb, tb, po, (int)m, (int)n, (int)k, scale, offset, epi);
+    if (rc != 0) return rc;
     TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM);
   }
   dim3 g((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64));

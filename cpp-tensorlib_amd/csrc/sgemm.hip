@@ -85,13 +85,19 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const float* __restr
                                                            const float* __restrict__ B, int64_t ldb,
                                                            float* __restrict__ C, int M, int N, int K,
                                                            float scale, float offset, int epi,
-                                                           int aligned) {
+                                                           int aligned, int kchunk) {
   __shared__ __attribute__((aligned(16))) float As[kSgBK][kSgBM + kSgPad];
   __shared__ __attribute__((aligned(16))) float Bs[kSgBK][kSgBN + kSgPad];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int m0 = blockIdx.y * kSgBM, n0 = blockIdx.x * kSgBN;
   const bool inside = aligned && m0 + kSgBM <= M && n0 + kSgBN <= N;
+  // gridDim.z > 1 is split-K: slice z takes K range [z * kchunk, (z + 1) * kchunk) (kchunk a
+  // multiple of the slab) and writes its partial product, without the epilogue, to
+  // C + z * M * N, a scratch area that sgemm_sum_kernel adds up in slice order.
+  const int kbeg = blockIdx.z * kchunk;
+  K = min(K, kbeg + kchunk);
+  C += (size_t)blockIdx.z * M * N;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -103,9 +109,9 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const float* __restr
 
   TileMover<TA == 0> ma;   // A: k contiguous unless transposed
   TileMover<TB != 0> mb;   // B: k contiguous only when transposed
-  ma.load(A, lda, m0, 0, M, K, inside && kSgBK <= K, tid);
-  mb.load(B, ldb, n0, 0, N, K, inside && kSgBK <= K, tid);
-  for (int k0 = 0; k0 < K; k0 += kSgBK) {
+  ma.load(A, lda, m0, kbeg, M, K, inside && kbeg + kSgBK <= K, tid);
+  mb.load(B, ldb, n0, kbeg, N, K, inside && kbeg + kSgBK <= K, tid);
+  for (int k0 = kbeg; k0 < K; k0 += kSgBK) {
     __syncthreads();   // the previous slab has been consumed
     ma.store(As, tid);
     mb.store(Bs, tid);
@@ -150,21 +156,53 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const float* __restr
     }
 }
 
+// C[i] = (sum over slices of part[s][i]) * scale + offset, slices in ascending order.
+__global__ __launch_bounds__(256) void sgemm_sum_kernel(const float* __restrict__ part, float* __restrict__ C,
+                                                        size_t n, int S, float scale, float offset, int epi) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float a = part[i];
+  for (int s = 1; s < S; s++) a += part[(size_t)s * n + i];
+  C[i] = epi ? __fadd_rn(__fmul_rn(a, scale), offset) : a;
+}
+
 // Launches the matrix-pipe GEMM; the caller has checked the arguments.
 int launch_sgemm_mfma(const float* pa, int64_t lda, int ta, const float* pb, int64_t ldb, int tb, float* pc,
                       int M, int N, int K, float scale, float offset, int epi) {
-  const dim3 grid((unsigned)((N + kSgBN - 1) / kSgBN), (unsigned)((M + kSgBM - 1) / kSgBM));
+  const int64_t tiles = (int64_t)((N + kSgBN - 1) / kSgBN) * ((M + kSgBM - 1) / kSgBM);
+  // Too few tiles to fill the chip: split K over gridDim.z (at least 256 of K per slice) into
+  // scratch parts that are summed in a fixed order - deterministic, no atomics.
+  int S = 1;
+  if (tiles < ctx().cus) {
+    S = (int)((2 * (int64_t)ctx().cus + tiles - 1) / tiles);
+    if (S > 8) S = 8;
+    while (S > 1 && K / S < 256) S--;
+  }
+  int kchunk = K;
+  float* dst = pc;
+  if (S > 1) {
+    kchunk = ((K + S - 1) / S + kSgBK - 1) / kSgBK * kSgBK;
+    S = (K + kchunk - 1) / kchunk;
+    dst = S > 1 ? static_cast<float*>(scratch((size_t)S * M * N * sizeof(float))) : pc;
+    if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm: no scratch for %d K-splits", S);
+  }
+  const dim3 grid((unsigned)((N + kSgBN - 1) / kSgBN), (unsigned)((M + kSgBM - 1) / kSgBM), (unsigned)S);
   // 16-byte loads need aligned bases and row strides that keep every row aligned
   const int aligned = aligned16(pa) && aligned16(pb) && (lda % 4) == 0 && (ldb % 4) == 0;
   hipStream_t st = ctx().stream;
-#define TLHIP_SGEMM(TA_, TB_)                                                                        \
-  sgemm_mfma_kernel<TA_, TB_><<<grid, dim3(256), 0, st>>>(pa, lda, pb, ldb, pc, M, N, K, scale, offset, \
-                                                          epi, aligned)
+  const int kepi = S > 1 ? 0 : epi;   // the part sum applies the epilogue when K is split
+#define TLHIP_SGEMM(TA_, TB_)                                                                         \
+  sgemm_mfma_kernel<TA_, TB_><<<grid, dim3(256), 0, st>>>(pa, lda, pb, ldb, dst, M, N, K, scale, offset, \
+                                                          kepi, aligned, kchunk)
   if (!ta && !tb) TLHIP_SGEMM(0, 0);
   else if (!ta && tb) TLHIP_SGEMM(0, 1);
   else if (ta && !tb) TLHIP_SGEMM(1, 0);
   else TLHIP_SGEMM(1, 1);
 #undef TLHIP_SGEMM
+  if (S > 1) {
+    const size_t n = (size_t)M * N;
+    sgemm_sum_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(dst, pc, n, S, scale, offset, epi);
+  }
   return 0;
 }
 
