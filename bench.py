@@ -38,13 +38,21 @@ def q4_nbytes(N, K):
     return N * K // 2 + N * (K // 32) * 4
 
 
-def make_q4_host(orc, N, K, seed):
-    """Seeded N(0,0.02) weights quantised exactly as array::to_q4 does. Quantising
-    545 M weights on one core would take minutes, so a block of rows is quantised
-    and tiled along N: kernel time does not depend on the values."""
+def normal(n, seed, mean=0.0, std=1.0):
+    return (np.random.default_rng(seed).standard_normal(n, dtype=np.float32) * np.float32(std)
+            + np.float32(mean)).astype(np.float32)
+
+
+def make_q4_host(lib, N, K, seed):
+    """Seeded N(0,0.02) weight rows in the int4 group format (what array::to_q4 produces),
+    quantised by the library's own load-time converter on the device. A block of rows is
+    quantised and tiled along N: kernel time does not depend on the values."""
     rows = min(N, 2048)
-    w = orc.normal(K * rows, seed, 0.0, 0.02).reshape(K, rows)
-    blk = orc.to_q4(w)
+    src = lib.to_device(normal(rows * K, seed, 0.0, 0.02))
+    q4 = lib.empty_bytes(q4_nbytes(rows, K))
+    lib.quantize_q4(src, lib.T_F32, q4, rows, K)
+    blk = q4.numpy(np.uint8)
+    src.free(); q4.free()
     packed, scales = blk[:rows * K // 2], blk[rows * K // 2:]
     reps = -(-N // rows)
     out = np.empty(q4_nbytes(N, K), np.uint8)
@@ -53,19 +61,29 @@ def make_q4_host(orc, N, K, seed):
     return out
 
 
-def cpu_baseline(orc, refl, budget_s=25.0):
-    """The reference CPU path (x.dot(Wq) in use_cpu() mode: per-call widening to f32
+def cpu_baseline(guard, budget_s=25.0):
+    """The only leg that touches oracle/: it first checks the GPU result of the sweep's smallest
+    shape (`guard` = x, q4 buffer, N, K, y from the GPU) against the CPU checker, then times
+    the reference CPU path (x.dot(Wq) in use_cpu() mode: per-call widening to f32
     plus cpu::sgemm on ONE thread, array.h:1980-1984, cpu.h:436-438) on the sweep's own
-    shapes, smallest first: median of 3 calls after a warm-up for the four smaller ones,
-    one call for the LM head; a shape is skipped once the time budget is spent (the sample
+    shapes, smallest first: median of 3 calls (after a warm-up call for the four smaller
+    ones); a shape is skipped once the time budget is spent (the sample
     says which were timed). Falls back to the plain-C restatement when oracle/_ref was
     not built."""
     import ctypes as C
+    from oraclelib import oracle, ref
+    orc = oracle()
+    refl = ref()            # None when oracle/_ref was not built
+    gx, gbuf, gN, gK, got = guard
+    want = orc.gemv_q4(gx, gbuf, gN, gK)
+    if not np.all(np.abs(got - want) <= 1e-5 + 1e-4 * np.abs(want)):
+        print("bench.py: GPU result differs from the CPU oracle", file=sys.stderr)
+        sys.exit(3)
     total_bytes, total_s, timed = 0, 0.0, []
     t_start = time.time()
     for (N, K) in sorted(SHAPES, key=lambda s: s[0] * s[1]):
         big = N * K > 10 ** 8
-        est = 0.62 * N * K / 0.1e9 * (1.3 if big else 4.2)     # ~0.1 GB/s, calls incl. warm-up
+        est = 0.62 * N * K / 0.1e9 * (3.3 if big else 4.2)     # ~0.1 GB/s, calls incl. warm-up
         if time.time() - t_start + est > budget_s and timed:
             continue
         buf = orc.fill_q4(N, K, 77)
@@ -82,7 +100,7 @@ def cpu_baseline(orc, refl, budget_s=25.0):
         ts = []
         if not big:
             run()
-        for _ in range(1 if big else 3):
+        for _ in range(3):
             t = time.perf_counter()
             run()
             ts.append(time.perf_counter() - t)
@@ -93,9 +111,9 @@ def cpu_baseline(orc, refl, budget_s=25.0):
         timed.append("%dx%d" % (N, K))
     return {
         "value": round(total_bytes / total_s / 1e9, 4), "unit": "GB/s", "cores": 1,
-        "kind": "reference" if refl is not None else "port",
-        "sample": "int4 x.dot(Wq) at %s (%d of the 5 sweep shapes; median of 3 calls, one call for "
-                  "the LM head); the reference's dot at M=1 runs on one thread whatever the core "
+        "kind": "reference" if refl is not None else "port", "gpu_result_checked": "512x3584 allclose(1e-4, 1e-5)",
+        "sample": "int4 x.dot(Wq) at %s (%d of the 5 sweep shapes; median of 3 calls, after a warm-up "
+                  "call except for the LM head); the reference's dot at M=1 runs on one thread whatever the core "
                   "count" % (", ".join(timed), len(timed)),
         "ms": round(total_s * 1e3, 2), "cpu_seconds_spent": round(time.time() - t_start, 1),
         "host_cores_online": os.cpu_count(),
@@ -234,7 +252,7 @@ def decode_05b(lib, steps):
     return out
 
 
-def side_kernels(lib, orc):
+def side_kernels(lib):
     """The other bandwidth-bound kernels of the path at their BASELINE shapes: the bf16 GEMV in
     both layouts (configs[1] weights as bf16; [N,K] rows for the harness, [K,N] at the array
     seam) and decode attention (configs[2]: q[28,128], K/V[28,ctx,128] f32). Bytes counted the
@@ -262,7 +280,7 @@ def side_kernels(lib, orc):
         w.upload(host)
         for c in range(1, copies):
             lib._chk(lib.c.tlhip_memcpy_d2d_async(w.ptr + c * nb, w.ptr, nb))
-        x, y = lib.to_device(orc.normal(K, 5)), lib.empty(N)
+        x, y = lib.to_device(normal(K, 5)), lib.empty(N)
         for name, fn in (("gemv_bf16_row", lib.c.tlhip_gemv_bf16_row), ("gemv_bf16_kn", lib.c.tlhip_gemv_bf16)):
             ms = timed(lambda i: lib._chk(fn(x.ptr, w.ptr + (i % copies) * nb, y.ptr, N, K)), max(10, copies))
             out[name]["%dx%d" % (N, K)] = {"us": round(ms * 1e3, 2), "GB/s": round(nb / ms / 1e6, 1)}
@@ -290,12 +308,12 @@ def side_kernels(lib, orc):
         per = H * ctx * D
         copies = max(2, min(8, int(1.2e9 // (8 * per)) + 1))
         Ks, Vs = lib.empty(per * copies), lib.empty(per * copies)
-        blk = orc.normal(min(per, 1 << 22), 9)
+        blk = normal(min(per, 1 << 22), 9)
         for b in (Ks, Vs):
             for o in range(0, per * copies, len(blk)):
                 n = min(len(blk), per * copies - o)
                 lib._chk(lib.c.tlhip_memcpy_h2d(b.ptr + o * 4, blk.ctypes.data, n * 4))
-        q, o_ = lib.to_device(orc.normal(H * D, 10)), lib.empty(H * D)
+        q, o_ = lib.to_device(normal(H * D, 10)), lib.empty(H * D)
         scale = 1.0 / np.sqrt(128.0)
         ms = timed(lambda i: lib._chk(lib.c.tlhip_attn_decode(
             q.ptr, Ks.ptr + (i % copies) * per * 4, Vs.ptr + (i % copies) * per * 4, o_.ptr,
@@ -369,41 +387,6 @@ def prefill_7b(lib, rounds=3):
     }
 
 
-def reference_benches():
-    """Not the bench line: runs the REFERENCE's own benchmark programs (bench/cuda/speed/*.cpp,
-    compiled unmodified against this backend by `make -C oracle refprogs` where the reference tree
-    exists; the binaries travel, the sources do not) and prints what they print. The three that
-    load a model get a synthetic Qwen2.5-0.5B-shaped F16 GGUF (tests/ggufwriter.py): the shape the
-    reference's published RTX 3090 figures are quoted on (README.md:310-313)."""
-    import subprocess
-    import tempfile
-    import ggufwriter
-    progs = os.path.join(ROOT, "oracle", "_ref", "refprogs")
-    if not os.path.isdir(progs):
-        print("bench.py: oracle/_ref/refprogs is not built (make -C oracle refprogs, needs the reference tree)", file=sys.stderr)
-        sys.exit(2)
-    env = dict(os.environ, TENSORLIB_HIP_LIB=os.path.join(ROOT, "cpp-tensorlib_amd", "lib", "libtensorlib_hip.so"))
-    out = {}
-
-    def run(name, *args, limit=280):
-        print("== %s %s" % (name, " ".join(args[1:])), flush=True)
-        r = subprocess.run([os.path.join(progs, name)] + list(args), env=env, stdout=subprocess.PIPE,
-                           stderr=subprocess.STDOUT, timeout=limit)
-        text = r.stdout.decode(errors="replace")
-        print(text, flush=True)
-        out[" ".join([name] + [os.path.basename(a) for a in args])] = {"rc": r.returncode, "output": text}
-    for name in ("bench_q4_gemv", "bench_bf16_gemv", "bench_qwen_gemv", "bench_attn_decode", "bench_llm"):
-        run(name)
-    with tempfile.TemporaryDirectory() as d:
-        path = os.path.join(d, "qwen05b_synthetic_f16.gguf")
-        ggufwriter.qwen05b_synthetic(path)
-        run("bench_qwen_decode", path)
-        run("bench_qwen_decode", path, "bf16", "64", "all")
-        run("bench_qwen_prefill", path)
-        run("bench_qwen_ctx", path)
-    print(json.dumps({"reference_benches": out}))
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -418,12 +401,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the 7B-shape prompt-chunk leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch the plain 1 GiB copy kernel 3 times (scale for --pmc runs)")
-    ap.add_argument("--reference-benches", action="store_true",
-                    help="instead of the bench line: run the reference's own benchmark programs on this backend")
     a = ap.parse_args()
-    if a.reference_benches:
-        reference_benches()
-        return
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; every GPU box of this run has one. "
               "Run with --gpus 1 (DESIGN.md says how the path would shard).", file=sys.stderr)
@@ -431,8 +409,6 @@ def main():
 
     pkg = importlib.import_module("cpp-tensorlib_amd")
     lib = pkg.load()                      # raises when the HIP library or the GPU is missing
-    from oraclelib import oracle, ref
-    orc = oracle()
 
     # ---- device-resident inputs: a ring of weight copies per shape -----------------
     rings = []
@@ -440,25 +416,21 @@ def main():
         nb = q4_nbytes(N, K)
         stride = (nb + 255) // 256 * 256
         copies = max(2, int(RING_BYTES // nb) + 1)
-        host = make_q4_host(orc, N, K, 100 + si)
+        host = make_q4_host(lib, N, K, 100 + si)
         first = lib.empty_bytes(stride * copies)
         first.upload(host)
         for c in range(1, copies):
             lib._chk(lib.c.tlhip_memcpy_d2d_async(first.ptr + c * stride, first.ptr, nb))
-        x = lib.to_device(orc.normal(K, 200 + si))
+        x = lib.to_device(normal(K, 200 + si))
         y = lib.empty(N)
         rings.append(dict(N=N, K=K, nb=nb, stride=stride, copies=copies, buf=first, x=x, y=y, it=0,
                           host=host if N == 512 else None))
     lib.sync()
 
-    # correctness guard on the smallest shape against the CPU oracle (one call)
+    # the smallest shape's GPU result, kept for the CPU leg's check
     r0 = rings[1]
     lib.gemv_q4(r0["x"], r0["buf"], r0["y"], r0["N"], r0["K"])
-    want = orc.gemv_q4(r0["x"].numpy(), r0["host"], r0["N"], r0["K"])
-    got = r0["y"].numpy()
-    if not np.all(np.abs(got - want) <= 1e-5 + 1e-4 * np.abs(want)):
-        print("bench.py: GPU result differs from the CPU oracle", file=sys.stderr)
-        sys.exit(3)
+    guard = (r0["x"].numpy(), r0["host"], r0["N"], r0["K"], r0["y"].numpy())
 
     def one_step(ev=None):
         for r in rings:
@@ -534,7 +506,7 @@ def main():
     # by what the same counter reads for a plain 1 GiB copy kernel (x2.000 and x1.000 here)
     out["roofline"]["traffic"] = LMHEAD_HBM_BYTES_PER_LAUNCH
     if not a.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(orc, ref())
+        out["cpu_baseline"] = cpu_baseline(guard)
     if not a.no_decode:
         out["decode"] = decode_7b(lib, max(10, a.steps), eager=a.eager_decode)
         if "cpu_baseline" in out and "algorithmic_bytes" in out["decode"]:
@@ -547,7 +519,7 @@ def main():
         if not a.eager_decode:
             out["decode_05b"] = decode_05b(lib, max(20, a.steps))
     if not a.no_side:
-        out["side_kernels"] = side_kernels(lib, orc)
+        out["side_kernels"] = side_kernels(lib)
     if not a.no_prefill:
         out["prefill"] = prefill_7b(lib)
     print(json.dumps(out))
