@@ -96,6 +96,8 @@ SIGNATURES = {
     "tlhip_gemv_bf16_row_swiglu": (cint, [P, P, P, i64, i64]),
     "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
     "tlhip_gemv_bf16_row_rmsnorm": (cint, [P, P, P, P, P, P, i64, i64, f32]),
+    "tlhip_gemv_q4_rmsnorm_gateup": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
+    "tlhip_gemv_bf16_row_rmsnorm_gateup": (cint, [P, P, P, P, P, P, i64, i64, f32]),
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
     "tlhip_tune_gemv_cols": (cint, [cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
@@ -387,6 +389,16 @@ class TlHip:
         self._chk(self.c.tlhip_gemv_bf16_row_rmsnorm(
             x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
             xout.ptr if xout is not None else None, W.ptr, y.ptr, N, K, eps))
+
+    def gemv_q4_rmsnorm_gateup(self, x, delta, norm_w, xout, wq, act, N2, K, eps, group=32):
+        self._chk(self.c.tlhip_gemv_q4_rmsnorm_gateup(
+            x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
+            xout.ptr if xout is not None else None, wq.ptr, wq.ptr + N2 * K // 2, act.ptr, N2, K, group, eps))
+
+    def gemv_bf16_row_rmsnorm_gateup(self, x, delta, norm_w, xout, W, act, N2, K, eps):
+        self._chk(self.c.tlhip_gemv_bf16_row_rmsnorm_gateup(
+            x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
+            xout.ptr if xout is not None else None, W.ptr, act.ptr, N2, K, eps))
 
     def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0, lpr=0):
         self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw, lpr))

@@ -114,7 +114,11 @@ struct RowFrag {          // one (row tile, chunk) work item of a lane: R weight
 // Weight and scale addresses are formed as a uniform base plus a 32-bit byte
 // offset per lane (the launcher checks that the matrix is below 4 GiB), which is
 // the cheapest global addressing form: one 24-bit multiply-add per row.
-template <typename Fmt, int R>
+//
+// PAIR: the matrix is two stacked halves of N/2 rows (gate rows, then up rows) and the R
+// fragments are R/2 consecutive rows of the first half followed by the same rows of the
+// second; row0 counts rows of a half.
+template <typename Fmt, int R, bool PAIR = false>
 __device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __restrict__ W,
                                           const float* __restrict__ scales, int N, int upr,
                                           int row0, int u) {
@@ -123,7 +127,9 @@ __device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __res
     const char* sb = reinterpret_cast<const char*>(scales);
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      const uint32_t row = (uint32_t)min(row0 + r, N - 1);
+      const uint32_t row = PAIR ? (uint32_t)(min(row0 + (r % (R / 2 > 0 ? R / 2 : 1)), N / 2 - 1) +
+                                             (r >= R / 2 ? N / 2 : 0))
+                                : (uint32_t)min(row0 + r, N - 1);
       const uint32_t idx = __umul24(row, (uint32_t)upr) + (uint32_t)u;
       f.w[r] = load_stream16(reinterpret_cast<const uint4*>(wb + (idx << 4)));
       if (Fmt::kScaled)
@@ -180,7 +186,15 @@ __device__ __forceinline__ float wave_sum_rows(float (&a)[R], int lane) {
 //   kRmsnorm: s = in (+ delta); x = (s * 1/sqrt(mean(s*s) + eps)) * norm_w   (array.h:2429-2433);
 //             block 0 also writes s to xout (the residual stream), which therefore
 //             must not alias in or delta: other blocks still read them.
+// How a block leaves its results (EPI):
+//   kStore:  y[row] = dot.
+//   kGateUp: W is [gate rows | up rows] (N/2 each); a lane group owns R/2 gate rows and the
+//            matching up rows, and writes y[i] = (g*sigmoid(g))*u for i < N/2 - the gated
+//            activation in the GEMV that produces it, once per element, instead of in every
+//            block of the GEMV that consumes it.
 enum { kPlain = 0, kSwiglu = 1, kRmsnorm = 2 };
+enum { kStore = 0, kGateUp = 1 };
+__device__ __forceinline__ float gated(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 struct Producer {
   const float* delta;
   const float* norm_w;
@@ -194,7 +208,7 @@ struct Producer {
 // lanes idle in the 64-lane form (K = 3584 is 112 units: 12.5 % idle; K = 896 is
 // 28 units: 56 % idle); the 16-lane form wastes at most 15 units per row and
 // finishes a row sum inside one DPP row.
-template <typename Fmt, int R, int PRO, int LPR>
+template <typename Fmt, int R, int PRO, int LPR, int EPI = kStore>
 __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
     float* __restrict__ y, int N, int upr, int KW, int ntiles, const Producer pro) {
@@ -214,12 +228,16 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   const int groups = nw / KW;        // wavefront row groups per block tile
   const int rows_per_tile = groups * QN * R;
   const int wrow = (wn * QN + q) * R;  // this lane's first row inside a tile
+  constexpr bool kPair = EPI == kGateUp;
+  static_assert(!kPair || R >= 2, "a gate/up pair needs two rows per lane group");
+  // first row of work item (tile tt): a row of W, or with kPair a row of each half
+  const auto item_row = [&](int tt) { return kPair ? (tt * rows_per_tile + wrow) >> 1 : tt * rows_per_tile + wrow; };
 
   // The first work item's weights are requested before x is staged, so that the
   // HBM latency of the weights and the L2 latency of x overlap.
   int t = blockIdx.x, c = kw;
   RowFrag<Fmt, R> cur;
-  if (t < ntiles) load_frag<Fmt, R>(cur, W, scales, N, upr, t * rows_per_tile + wrow, c * LPR + li);
+  if (t < ntiles) load_frag<Fmt, R, kPair>(cur, W, scales, N, upr, item_row(t), c * LPR + li);
 
   {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
      // thread i owns float4 i; the J threads of a unit are adjacent lanes, so the
@@ -293,7 +311,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     int nc = c + KW, nt = t;
     if (nc >= chunks) { nc = kw; nt = t + gridDim.x; }
     if (nt < ntiles)
-      load_frag<Fmt, R>(nxt, W, scales, N, upr, nt * rows_per_tile + wrow, nc * LPR + li);
+      load_frag<Fmt, R, kPair>(nxt, W, scales, N, upr, item_row(nt), nc * LPR + li);
 
     const int u = c * LPR + li;
     if (u < upr) {
@@ -311,7 +329,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     }
 
     if (nt != t) {  // last chunk of tile t for this wavefront: reduce and store
-      const int row0 = t * rows_per_tile + wrow;
+      const int row0 = item_row(t);
       float v;
       int r;
       bool writer;
@@ -331,12 +349,24 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         writer = li < R;
       }
       if (KW == 1) {
-        if (writer && row0 + r < N) y[row0 + r] = v;
+        if constexpr (kPair) {
+          // the up row's total sits half a wavefront (64-lane form) or R/2 lanes (16-lane form) away
+          const float up = LPR == 64 ? __shfl_xor(v, 32, kWave) : __shfl_down(v, R / 2, kWave);
+          if (writer && r < R / 2 && row0 + r < N / 2) y[row0 + r] = gated(v, up);
+        } else {
+          if (writer && row0 + r < N) y[row0 + r] = v;
+        }
       } else {
         // every wavefront of the block passes these two barriers once per tile
         if (writer) red[(wrow / R * KW + kw) * R + r] = v;
         __syncthreads();
-        if (kw == 0 && li < R && row0 + li < N) {
+        if constexpr (kPair) {
+          float sum = 0.f;
+          if (kw == 0 && li < R)
+            for (int sidx = 0; sidx < KW; sidx++) sum += red[(wrow / R * KW + sidx) * R + li];
+          const float up = __shfl_down(sum, R / 2, kWave);
+          if (kw == 0 && li < R / 2 && row0 + li < N / 2) y[row0 + li] = gated(sum, up);
+        } else if (kw == 0 && li < R && row0 + li < N) {
           float sum = 0.f;
           for (int sidx = 0; sidx < KW; sidx++) sum += red[(wrow / R * KW + sidx) * R + li];
           y[row0 + li] = sum;
@@ -569,19 +599,22 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   return c;
 }
 
-template <typename Fmt, int PRO, int LPR>
+template <typename Fmt, int PRO, int LPR, int EPI>
 static auto pick_rows_fn(int R) -> void (*)(const float*, const uint4*, const float*, float*, int, int,
                                             int, int, const Producer) {
   switch (R) {
-    case 1: return gemv_rows_kernel<Fmt, 1, PRO, LPR>;
-    case 2: return gemv_rows_kernel<Fmt, 2, PRO, LPR>;
-    case 4: return gemv_rows_kernel<Fmt, 4, PRO, LPR>;
-    case 8: return gemv_rows_kernel<Fmt, 8, PRO, LPR>;
+    case 1:
+      if constexpr (EPI == kStore) return gemv_rows_kernel<Fmt, 1, PRO, LPR, EPI>;
+      else return nullptr;
+    case 2: return gemv_rows_kernel<Fmt, 2, PRO, LPR, EPI>;
+    case 4: return gemv_rows_kernel<Fmt, 4, PRO, LPR, EPI>;
+    case 8: return gemv_rows_kernel<Fmt, 8, PRO, LPR, EPI>;
     default: return nullptr;
   }
 }
 
-template <typename Fmt, int PRO = kPlain>
+// N counts the rows of W; with EPI = kGateUp, y has N / 2 entries.
+template <typename Fmt, int PRO = kPlain, int EPI = kStore>
 static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
                        int64_t K, int census_id, const RowTune tn = RowTune{0, 0, 0, 0, 0},
                        const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
@@ -594,13 +627,20 @@ static int launch_rows(const float* x, const void* W, const float* scales, float
   if (max_rows >= (1 << 24)) max_rows = (1 << 24) - 1;
   max_rows &= ~(int64_t)255;
   if (max_rows <= 0) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large");
+  if (EPI == kGateUp && N > max_rows) return fail(TLHIP_EUNSUPPORTED, "gemv: gate|up matrix too large for one launch");
   for (int64_t n0 = 0; n0 < N; n0 += max_rows) {
     const int64_t n = N - n0 < max_rows ? N - n0 : max_rows;
     RowCfg cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, tn);
+    if (EPI == kGateUp && cfg.R == 1) {   // a lane group needs a gate row and its up row
+      RowTune two = tn;
+      two.R = 2;
+      if (cfg.nw / cfg.KW >= 2 && cfg.nw > 4) two.nw = cfg.nw / 2;   // keeps the rows of a block tile
+      cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, two);
+    }
     if (cfg.lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large for the LDS-staged kernel");
     const int rows_per_tile = (cfg.nw / cfg.KW) * (64 / cfg.lpr) * cfg.R;
     const int ntiles = (int)((n + rows_per_tile - 1) / rows_per_tile);
-    auto fn = cfg.lpr == 16 ? pick_rows_fn<Fmt, PRO, 16>(cfg.R) : pick_rows_fn<Fmt, PRO, 64>(cfg.R);
+    auto fn = cfg.lpr == 16 ? pick_rows_fn<Fmt, PRO, 16, EPI>(cfg.R) : pick_rows_fn<Fmt, PRO, 64, EPI>(cfg.R);
     if (!fn) return fail(TLHIP_EINVAL, "rows per wavefront must be 1, 2, 4 or 8");
     if (cfg.lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
@@ -767,6 +807,36 @@ int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, 
                      static_cast<float*>(xout), eps};
   return launch_rows<FmtQ4, kRmsnorm>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
                                       static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c), pro);
+}
+
+int tlhip_gemv_q4_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
+                                 const void* qw, const void* scales, void* act, int64_t N2, int64_t K,
+                                 int64_t group, float eps) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(x, qw, act, N2, K, "tlhip_gemv_q4_rmsnorm_gateup")) return rc;
+  if (N2 % 2) return fail(TLHIP_EINVAL, "tlhip_gemv_q4_rmsnorm_gateup: odd row count %lld", (long long)N2);
+  if (int rc = check_fused_q4(qw, scales, K, group, K, "tlhip_gemv_q4_rmsnorm_gateup")) return rc;
+  if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_q4_rmsnorm_gateup")) return rc;
+  Context& c = ctx();
+  const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
+                     static_cast<float*>(xout), eps};
+  return launch_rows<FmtQ4, kRmsnorm, kGateUp>(static_cast<const float*>(x), qw,
+                                               static_cast<const float*>(scales), static_cast<float*>(act),
+                                               N2, K, TLHIP_C_GEMV_Q4, q4_tune(c), pro);
+}
+
+int tlhip_gemv_bf16_row_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
+                                       const void* W, void* act, int64_t n2, int64_t k, float eps) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(x, W, act, n2, k, "tlhip_gemv_bf16_row_rmsnorm_gateup")) return rc;
+  if (n2 % 2) return fail(TLHIP_EINVAL, "tlhip_gemv_bf16_row_rmsnorm_gateup: odd row count %lld", (long long)n2);
+  if (int rc = check_fused_bf16(W, k, "tlhip_gemv_bf16_row_rmsnorm_gateup")) return rc;
+  if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_bf16_row_rmsnorm_gateup")) return rc;
+  const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
+                     static_cast<float*>(xout), eps};
+  return launch_rows<FmtBf16, kRmsnorm, kGateUp>(static_cast<const float*>(x), W, nullptr,
+                                                 static_cast<float*>(act), n2, k, TLHIP_C_GEMV_BF16_ROW,
+                                                 RowTune{0, 0, 0, 0, 0}, pro);
 }
 
 int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n, int64_t k) {

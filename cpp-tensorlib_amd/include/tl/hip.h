@@ -139,6 +139,10 @@ struct api {
                          int64_t, int64_t, int64_t, float) = nullptr;
   int (*gemv_bf16_row_rmsnorm)(const void*, const void*, const void*, void*, const void*, void*,
                                int64_t, int64_t, float) = nullptr;
+  int (*gemv_q4_rmsnorm_gateup)(const void*, const void*, const void*, void*, const void*, const void*,
+                                void*, int64_t, int64_t, int64_t, float) = nullptr;
+  int (*gemv_bf16_row_rmsnorm_gateup)(const void*, const void*, const void*, void*, const void*, void*,
+                                      int64_t, int64_t, float) = nullptr;
 };
 
 struct context {
@@ -235,7 +239,9 @@ struct context {
               bind(f.gemv_q4_swiglu, "tlhip_gemv_q4_swiglu") &&
               bind(f.gemv_bf16_row_swiglu, "tlhip_gemv_bf16_row_swiglu") &&
               bind(f.gemv_q4_rmsnorm, "tlhip_gemv_q4_rmsnorm") &&
-              bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm");
+              bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm") &&
+              bind(f.gemv_q4_rmsnorm_gateup, "tlhip_gemv_q4_rmsnorm_gateup") &&
+              bind(f.gemv_bf16_row_rmsnorm_gateup, "tlhip_gemv_bf16_row_rmsnorm_gateup");
     if (!ok) return;
     if (f.abi_version() != 1) {
       why = "libtensorlib_hip.so has a different ABI version";
@@ -916,6 +922,34 @@ inline bool gemv_bf16_row_rmsnorm(void* x, void* delta, void* norm_w, void* xout
   if (xout) c.device_write_(xout);
   c.device_write_(y);
   return detail::done_(c, c.f.gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, B, y, n, k, eps));
+}
+// The same with W = [gate rows | up rows] (N2 / 2 each) and the gated activation as the
+// epilogue: act[i] = swiglu(gate_i, up_i), i < N2 / 2.
+inline bool gemv_q4_rmsnorm_gateup(void* x, void* delta, void* norm_w, void* xout, void* qw, void* scales,
+                                   void* act, int64_t N2, int64_t K, int64_t group, float eps) {
+  auto& c = context::get();
+  if (!c.ready || group != 32 || (K % 32) != 0 || (N2 % 2) != 0 || (xout && (xout == x || xout == delta)))
+    return false;
+  c.device_read_(x);
+  if (delta) c.device_read_(delta);
+  c.device_read_(norm_w);
+  c.device_read_(qw);
+  c.device_read_(scales);
+  if (xout) c.device_write_(xout);
+  c.device_write_(act);
+  return detail::done_(c, c.f.gemv_q4_rmsnorm_gateup(x, delta, norm_w, xout, qw, scales, act, N2, K, group, eps));
+}
+inline bool gemv_bf16_row_rmsnorm_gateup(void* x, void* delta, void* norm_w, void* xout, void* B, void* act,
+                                         int64_t n2, int64_t k, float eps) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0 || (n2 % 2) != 0 || (xout && (xout == x || xout == delta))) return false;
+  c.device_read_(x);
+  if (delta) c.device_read_(delta);
+  c.device_read_(norm_w);
+  c.device_read_(B);
+  if (xout) c.device_write_(xout);
+  c.device_write_(act);
+  return detail::done_(c, c.f.gemv_bf16_row_rmsnorm_gateup(x, delta, norm_w, xout, B, act, n2, k, eps));
 }
 
 // ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------

@@ -91,6 +91,16 @@ inline bool gemv_rmsnorm(const linear& L, void* x, void* delta, void* norm_w, vo
   return hip::gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, L.w, y, L.N, L.K, eps);
 }
 
+// L = [gate rows | up rows]; s = x (+ delta) -> xout ; act = swiglu(gate . n, up . n), n = rmsnorm(s, norm_w)
+inline bool gemv_rmsnorm_gateup(const linear& L, void* x, void* delta, void* norm_w, void* xout, void* act,
+                                float eps) {
+  if (L.fmt == wfmt::q4) {
+    void* scales = static_cast<char*>(L.w) + L.N * L.K / 2;
+    return hip::gemv_q4_rmsnorm_gateup(x, delta, norm_w, xout, L.w, scales, act, L.N, L.K, kQ4Group, eps);
+  }
+  return hip::gemv_bf16_row_rmsnorm_gateup(x, delta, norm_w, xout, L.w, act, L.N, L.K, eps);
+}
+
 struct layer {
   linear wqkv, wo, wgu, wd;          // fused [wq|wk|wv] and [wg|wu] (qm:188-199)
   void* bqkv = nullptr;                              // fused bias [q_dim + 2 kv_dim] (qm:196)
@@ -135,6 +145,7 @@ struct model {
   // GEMV that consumes them). false: the reference's call sequence, one launch per op.
   bool fused = true;
   bool fused_attn = true;   // within the fused path: q/k/v epilogue + append inside the attention launch
+  bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
 };
 
 namespace detail {
@@ -642,8 +653,13 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
         ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
       }
       ok &= gemv(L.wo, S.ab, S.hb);
-      ok &= gemv_rmsnorm(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.gub, d.eps);
-      ok &= gemv_swiglu(L.wd, S.gub, S.mdb);
+      if (M.gateup_epilogue) {
+        ok &= gemv_rmsnorm_gateup(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.mb, d.eps);
+        ok &= gemv(L.wd, S.mb, S.mdb);
+      } else {
+        ok &= gemv_rmsnorm(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.gub, d.eps);
+        ok &= gemv_swiglu(L.wd, S.gub, S.mdb);
+      }
       rin = S.res[1];
       din = S.mdb;
     }

@@ -289,6 +289,15 @@ int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, 
                           int64_t group, float eps);
 int tlhip_gemv_bf16_row_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
                                 const void* W, void* y, int64_t n, int64_t k, float eps);
+/* The same with the gated activation as the GEMV's epilogue: W = [gate rows | up rows], N2 / 2
+ * rows each (the fused [wg|wu] of qwen_model.h:194-199); act[i] = swiglu(gate_i, up_i) for
+ * i < N2 / 2, arithmetic of tlhip_swiglu. The activation is then formed once per element by the
+ * GEMV that produces it, and the down projection is a plain tlhip_gemv_*. */
+int tlhip_gemv_q4_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
+                                 const void* qw, const void* scales, void* act, int64_t N2, int64_t K,
+                                 int64_t group, float eps);
+int tlhip_gemv_bf16_row_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
+                                       const void* W, void* act, int64_t n2, int64_t k, float eps);
 
 /* ---- prefill ------------------------------------------------------------------ */
 /* C[M,N] = A[M,K] f32 . W[N,K]^T bf16, fp32 accumulate; K % 8 == 0.  cuda.h:787-841 */

@@ -25,16 +25,17 @@ def _near_tie(logits, rtol=1e-4, atol=1e-5):
     return (top2[1] - top2[0]) <= atol + rtol * abs(top2[1])
 
 
-@pytest.mark.parametrize("mode", ["fused", "fused_attn_apart", "plain"])
+@pytest.mark.parametrize("mode", ["fused", "fused_attn_apart", "fused_swiglu_in_down", "plain"])
 @pytest.mark.parametrize("dims,steps", [(SMALL, 40), (SMALL128, 270)])
 def test_decode_loop_matches_oracle(orc, dims, steps, mode):
     """mode: every fusion on (5 launches a layer), the q/k/v epilogue as a launch of its own,
-    or one launch per reference op."""
+    swiglu evaluated by the down GEMV instead of the gate|up GEMV, or one launch per reference op."""
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     om = orc.qwen_create(dims, seed=3, q4=True)
     g = qwen.QwenGPU.from_blobs(om)
     g.set_fused(mode != "plain")
-    g.set_fused_attn(mode == "fused")
+    g.set_fused_attn(mode != "fused_attn_apart")
+    g.set_gateup_epilogue(mode != "fused_swiglu_in_down")
     rng = np.random.default_rng(5)
     tok = int(rng.integers(0, dims["vocab"]))
     worst = 0.0

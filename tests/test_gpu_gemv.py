@@ -234,6 +234,56 @@ def test_gemv_rmsnorm_fused(lib, orc, fmt, N, K, with_delta, with_xout):
             b.free()
 
 
+@pytest.mark.parametrize("fmt", ["q4", "bf16"])
+@pytest.mark.parametrize("FF,K,with_delta", [(18944, 3584, True), (4864, 896, True), (4864, 896, False),
+                                             (33, 160, True), (7, 64, False), (1000, 18944, True),
+                                             (256 * 3, 3584, False)])
+def test_gemv_rmsnorm_gateup_epilogue(lib, orc, fmt, FF, K, with_delta):
+    """W = [gate rows | up rows]; act = swiglu(gate . n, up . n), n = rmsnorm(x + delta): the one
+    launch equals the oracle's rmsnorm_res, GEMV and swiglu (array.h:2429-2439) in sequence, and
+    the library's own two-launch form (GEMV, then tlhip_swiglu); xout is the exact fp32 sum.
+    Shapes: the 7B and 0.5B gate|up, ragged ones (odd FF, one tile), a long-K one whose launch
+    shape splits K over wavefronts, and a few rows per CU."""
+    print("case gemv_rmsnorm_gateup", fmt, FF, K, with_delta, flush=True)
+    eps, N2 = 1e-6, 2 * FF
+    x = orc.normal(K, 90 + FF, 0.0, 2.0)
+    delta = orc.normal(K, 91, 0.0, 0.5) if with_delta else np.zeros(K, np.float32)
+    nw = (1.0 + orc.normal(K, 92, 0.0, 0.1)).astype(np.float32)
+    s, h = orc.rmsnorm_res(x.reshape(1, K), delta.reshape(1, K), nw, eps)
+    dx, dn = lib.to_device(x), lib.to_device(nw)
+    dd = lib.to_device(delta) if with_delta else None
+    dxo = lib.to_device(np.full(K, np.nan, np.float32))
+    dact = lib.to_device(np.full(FF, np.nan, np.float32))
+    dgu, dact2 = lib.empty(N2), lib.empty(FF)
+    # weights with a spread that puts gate values on both sides of zero
+    if fmt == "q4":
+        buf = orc.to_q4(orc.normal(K * N2, 93, 0.0, 0.05).reshape(K, N2))
+        gu = orc.gemv_q4(h.reshape(K), buf, N2, K)
+        dw = lib.to_device(buf)
+        lib.gemv_q4_rmsnorm_gateup(dx, dd, dn, dxo, dw, dact, N2, K, eps)
+        lib.gemv_q4_rmsnorm(dx, dd, dn, None, dw, dgu, N2, K, eps)
+    else:
+        w = orc.to_bf16(orc.normal(N2 * K, 94, 0.0, 0.05).reshape(N2, K))
+        gu = orc.gemv_bf16_row(h.reshape(K), w)
+        dw = lib.to_device(w)
+        lib.gemv_bf16_row_rmsnorm_gateup(dx, dd, dn, dxo, dw, dact, N2, K, eps)
+        lib.gemv_bf16_row_rmsnorm(dx, dd, dn, None, dw, dgu, N2, K, eps)
+    lib.swiglu(dgu, dact2, FF)
+    want = orc.swiglu_fused(gu, FF).reshape(FF)
+    got, two = dact.numpy(), dact2.numpy()
+    assert not np.isnan(got).any()
+    # the GEMV bar (|dg| <= ATOL + RTOL |g|, same for u) carried through silu(g) * u, |silu'| <= 1.1
+    g, u = np.abs(gu[:FF]), np.abs(gu[FF:])
+    tol = ATOL * (1.1 * u + g + 1.0) + 2.1 * RTOL * g * u
+    assert np.all(np.abs(got - want) <= tol), maxrel(got, want)
+    assert np.all(np.abs(got - two) <= tol), maxrel(got, two)
+    assert np.array_equal(dxo.numpy(), s.reshape(K))
+    assert np.array_equal(dx.numpy(), x)
+    for b in (dx, dn, dw, dd, dxo, dact, dgu, dact2):
+        if b is not None:
+            b.free()
+
+
 def test_gemv_fused_rejects_aliasing_and_other_groups(lib, pkg):
     x, n, y, w = lib.empty(64), lib.empty(64), lib.empty(8), lib.empty_bytes(4096)
     with pytest.raises(pkg.TlHipError) as e:
@@ -245,6 +295,12 @@ def test_gemv_fused_rejects_aliasing_and_other_groups(lib, pkg):
     with pytest.raises(pkg.TlHipError) as e:
         lib.gemv_q4_swiglu(x, w, y, 8, 32, group=8)
     assert e.value.code == -3
+    with pytest.raises(pkg.TlHipError) as e:
+        lib.gemv_q4_rmsnorm_gateup(x, None, n, None, w, y, 7, 64, 1e-6)     # odd row count
+    assert e.value.code == -2
+    with pytest.raises(pkg.TlHipError) as e:
+        lib.gemv_q4_rmsnorm_gateup(x, None, n, x, w, y, 8, 64, 1e-6)        # xout aliases x
+    assert e.value.code == -2
 
 
 def test_gemv_q4_full_size_linearity(lib, orc):
