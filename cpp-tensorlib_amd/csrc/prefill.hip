@@ -11,7 +11,9 @@
 // the bf16 matrix rate (still ~5x the fp32 MFMA rate).
 //
 // Tiling: a block of 4 wavefronts (2x2) owns a (64*TM) x (64*TN) tile of C; each
-// wavefront TM x TN MFMA tiles of 32x32. K advances in slabs of 32 through LDS:
+// wavefront TM x TN MFMA tiles of 32x32 (2 x 4 for prompt chunks: an A fragment costs three
+// LDS reads, one per plane, so tiles are wide in N, where a fragment costs one).
+// K advances in slabs of 32 through LDS:
 // the A slab is split into its three bf16 planes while it is written to LDS, the
 // W slab is copied as is (rows XOR-swizzled against bank conflicts). Both operands are K-contiguous per lane (A is [M,K],
 // W is [N,K]), which is exactly the MFMA operand layout: one ds_read_b128 per
@@ -36,20 +38,23 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elemen
 
 // gridDim.y > 1 is split-K: block row y takes K range [y*kchunk, (y+1)*kchunk) and
 // writes its partial product to C + y*M*N (a scratch area); splitk_sum_kernel adds
-// the parts in a fixed order.
-template <int TM, int TN>
-__global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
+// the parts in a fixed order. ldc = row stride of C (N for a scratch part; the full
+// width when the launch covers a column range of a wider result).
+template <int TM, int TN, int WM = 2, int WN = 2>
+__global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
-                                                           int K, int kchunk) {
-  constexpr int BM = 64 * TM, BN = 64 * TN;
-  constexpr int A_LOADS = BM * kBK / 4 / 256;   // float4 per thread per slab
-  constexpr int B_LOADS = BN * kBK / 8 / 256;   // uint4 (8 bf16) per thread per slab
+                                                           int K, int kchunk, int ldc) {
+  constexpr int NT = 64 * WM * WN;              // threads: WM x WN wavefronts
+  constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
+  constexpr int A_LOADS = BM * kBK / 4 / NT;    // float4 per thread per slab
+  constexpr int B_LOADS = BN * kBK / 8 / NT;    // uint4 (8 bf16) per thread per slab
+  static_assert(A_LOADS >= 1 && B_LOADS >= 1 && BM * kBK / 4 % NT == 0 && BN * kBK / 8 % NT == 0, "tile vs threads");
   __shared__ __attribute__((aligned(16))) uint16_t As[3][BM * kBK];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * kBK];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   // Block order. Hardware deals consecutive block ids round-robin to the 8 XCDs,
   // each with a private L2. Give every XCD one contiguous run of tiles, M fastest,
   // so the blocks that share a weight tile run together on one L2 and W is
@@ -60,7 +65,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
   const int lid = xcd * q8 + min(xcd, r8) + within;
   const int m0 = (lid % mt) * BM, n0 = (lid / mt) * BN;
   const int kbeg = blockIdx.y * kchunk, kend = min(K, kbeg + kchunk);
-  C += (size_t)blockIdx.y * M * N;
+  C += (size_t)blockIdx.y * M * ldc;   // split parts are dense [M][N] (ldc == N there)
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -75,14 +80,14 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-      const int idx = tid + i * 256, row = idx >> 3, c4 = idx & 7;
+      const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
       const int gm = m0 + row, gk = k0 + c4 * 4;
       ra[i] = (gm < M && gk < kend) ? *reinterpret_cast<const float4*>(A + (size_t)gm * K + gk)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      const int idx = tid + i * 256, row = idx >> 2, c8 = idx & 3;
+      const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
       const int gn = n0 + row, gk = k0 + c8 * 8;
       rb[i] = (gn < N && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
                                  : make_uint4(0u, 0u, 0u, 0u);
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
   auto lstore = [&]() {
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
-      const int idx = tid + i * 256, row = idx >> 3, c4 = idx & 7;
+      const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
       uint32_t h[4], m[4], l[4];
       split3(ra[i].x, h[0], m[0], l[0]);
       split3(ra[i].y, h[1], m[1], l[1]);
@@ -113,7 +118,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
-      const int idx = tid + i * 256, row = idx >> 2, c8 = idx & 3;
+      const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
       *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8)]) = rb[i];
     }
   };
@@ -155,22 +160,25 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_nt_kernel(const float* __res
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (gm < M) C[(size_t)gm * N + gn] = acc[i][j][v];
+        if (gm < M) C[(size_t)gm * ldc + gn] = acc[i][j][v];
       }
     }
 }
 
-// C[i] = sum_s part[s][i], s in ascending order; n4 = M*N/4 float4s per part.
+// C[m][n] = sum_s part[s][m][n], s in ascending order. Parts are dense [M][n4 * 4]; C rows
+// are ldc4 float4s apart (the result may be a column range of a wider matrix).
 __global__ __launch_bounds__(256) void splitk_sum_kernel(const float4* __restrict__ part,
-                                                         float4* __restrict__ C, size_t n4, int S) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n4) return;
+                                                         float4* __restrict__ C, int M, int n4,
+                                                         int ldc4, int S) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)M * n4;
+  if (i >= total) return;
   float4 a = part[i];
   for (int sidx = 1; sidx < S; sidx++) {
-    const float4 b = part[(size_t)sidx * n4 + i];
+    const float4 b = part[sidx * total + i];
     a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
   }
-  C[i] = a;
+  const size_t m = i / n4;
+  C[m * ldc4 + (i - m * n4)] = a;
 }
 
 }  // namespace tlhip
@@ -192,45 +200,81 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
   const float* pa = static_cast<const float*>(A);
   const uint16_t* pw = static_cast<const uint16_t*>(W);
   float* pc = static_cast<float*>(C);
-  // Largest tile that still gives every CU about two blocks. When even 128x128
-  // tiles are too few (M of one prompt chunk against a narrow N), K is split over
-  // gridDim.y instead of shrinking the tile: small tiles re-read both operands
-  // through L2 far more often per MFMA.
-  auto blocks = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  const int64_t want = (int64_t)c.cus * 2;
-  int tm = 2, tn = 2, S = 1;
-  if (blocks(128, 128) < want) {
-    S = (int)((want + blocks(128, 128) - 1) / blocks(128, 128));
-    if (S > 8) S = 8;
-    while (S > 1 && K / S < 512) S--;
-    if ((M * N) % 4 != 0 || !aligned16(C)) S = 1;   // the part sum works on float4s
-    if (S == 1) {
-      if (blocks(64, 128) >= want) { tm = 1; tn = 2; }
-      else { tm = 1; tn = 1; }
+  // Tile variants {MFMA tiles per wavefront in M, in N}, 2 x 2 wavefronts each. The wide one
+  // (128 x 256 block tile, 64 x 128 per wavefront) needs fewest LDS reads per MFMA - the three
+  // A planes make LDS, not the matrix pipe, the first limit - and runs 2 blocks per CU.
+  // Work is shaped to fill those 2 * CUs block slots in whole rounds:
+  //   * fewer tiles than slots: K is split over gridDim.y so that tiles * S comes close to
+  //     the slots; parts go to scratch and are summed in a fixed order (no atomics);
+  //   * more tiles than slots: the columns that make whole rounds run with full K, the
+  //     remaining columns (less than one round of tiles) are split over K the same way.
+  auto cdiv = [](int64_t a, int64_t b) { return (a + b - 1) / b; };
+  const int64_t slots = (int64_t)c.cus * 2;
+  const bool can_split = (N % 4) == 0 && aligned16(C);   // the part sum works on float4s
+  struct Piece { int64_t n0, n; int S; int variant; };    // columns [n0, n0 + n)
+  Piece pieces[2];
+  int npieces = 0;
+  auto pick_S = [&](int64_t tiles) {   // K splits that bring `tiles` blocks up to the slots
+    if (!can_split || tiles >= slots) return 1;
+    int64_t S = (slots + tiles / 2) / tiles;
+    if (S > 16) S = 16;
+    while (S > 1 && K / S < 256) S--;
+    return (int)S;
+  };
+  if (M > 64) {
+    const int64_t tm = cdiv(M, 128), tn = cdiv(N, 256), tiles = tm * tn;
+    const int64_t cols_per_round = slots / tm;            // whole tile columns in one round
+    if (tiles <= slots || cols_per_round == 0 || !can_split) {
+      pieces[npieces++] = Piece{0, N, pick_S(tiles), 0};
+    } else {
+      const int64_t main_tn = tn / cols_per_round * cols_per_round;   // whole rounds
+      const int64_t n_main = main_tn * 256;
+      pieces[npieces++] = Piece{0, n_main, 1, 0};
+      if (n_main < N) pieces[npieces++] = Piece{n_main, N - n_main, pick_S(tm * (tn - main_tn)), 0};
     }
+  } else {
+    // short prompts: 64-row tiles; narrow ones when that is what fills the chip
+    const int64_t t128 = cdiv(N, 128), t64 = cdiv(N, 64);
+    if (t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
+    else pieces[npieces++] = Piece{0, N, pick_S(t64), 2};
   }
-  int kchunk = (int)K;
-  float* dst = pc;
-  if (S > 1) {
-    kchunk = (int)(((K + S - 1) / S + kBK - 1) / kBK * kBK);
-    S = (int)((K + kchunk - 1) / kchunk);
-    dst = static_cast<float*>(scratch((size_t)S * M * N * sizeof(float)));
-    if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
-  }
-  const int64_t nblk = ((N + 64 * tn - 1) / (64 * tn)) * ((M + 64 * tm - 1) / (64 * tm));
-  if (nblk > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
-  const dim3 grid((unsigned)nblk, (unsigned)S);
-#define TLHIP_GEMM(TM_, TN_)                                                                     \
-  gemm_bf16_nt_kernel<TM_, TN_><<<grid, dim3(256), 0, c.stream>>>(pa, pw, dst, (int)M, (int)N, \
-                                                                   (int)K, kchunk)
-  if (tm == 2) TLHIP_GEMM(2, 2);
-  else if (tn == 2) TLHIP_GEMM(1, 2);
-  else TLHIP_GEMM(1, 1);
+  for (int pi = 0; pi < npieces; pi++) {
+    const Piece& P = pieces[pi];
+    static const int kBm[3] = {128, 64, 64}, kBn[3] = {256, 128, 64};
+    const int bm = kBm[P.variant], bn = kBn[P.variant];
+    int S = P.S, kchunk = (int)K;
+    float* dst = pc + P.n0;
+    int ldc = (int)N;
+    if (S > 1) {
+      kchunk = (int)(cdiv(cdiv(K, S), kBK) * kBK);
+      S = (int)cdiv(K, kchunk);
+    }
+    if (S > 1) {
+      dst = static_cast<float*>(scratch((size_t)S * M * P.n * sizeof(float)));
+      if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
+      ldc = (int)P.n;
+    } else {
+      kchunk = (int)K;
+    }
+    const int64_t nblk = cdiv(M, bm) * cdiv(P.n, bn);
+    if (nblk > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
+    const dim3 grid((unsigned)nblk, (unsigned)S);
+    const uint16_t* wp = pw + (size_t)P.n0 * K;
+#define TLHIP_GEMM(TM_, TN_)                                                                        \
+  gemm_bf16_nt_kernel<TM_, TN_><<<grid, dim3(256), 0, c.stream>>>(pa, wp, dst, (int)M, (int)P.n, \
+                                                                   (int)K, kchunk, ldc)
+    switch (P.variant) {
+      case 0: TLHIP_GEMM(2, 4); break;
+      case 1: TLHIP_GEMM(1, 2); break;
+      default: TLHIP_GEMM(1, 1); break;
+    }
 #undef TLHIP_GEMM
-  if (S > 1) {
-    const size_t n4 = (size_t)M * N / 4;
-    splitk_sum_kernel<<<dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, c.stream>>>(
-        reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc), n4, S);
+    if (S > 1) {
+      const size_t total4 = (size_t)M * P.n / 4;
+      splitk_sum_kernel<<<dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, c.stream>>>(
+          reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + P.n0), (int)M, (int)(P.n / 4),
+          (int)(N / 4), S);
+    }
   }
   TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
 }

@@ -21,13 +21,14 @@ def _gemm(lib, A, Wb):
 
 
 @pytest.mark.parametrize("M,N,K", [
-    (512, 512, 3584),      # a prompt chunk against a kv-sized projection: 64x64 tiles
-    (512, 4608, 896),      # 64x128 tiles
-    (1024, 4864, 896),     # 128x128 tiles
+    (512, 512, 3584),      # a prompt chunk against a kv-sized projection: 8 wide tiles, K split 14 ways
+    (512, 4608, 896),      # 72 wide tiles, K split 3 ways
+    (1024, 4864, 896),     # 152 wide tiles, K split 3 ways
     (128, 1152, 896),      # 0.5B fused q|k|v
-    (33, 200, 40),         # ragged in M, N and K (K % 32 != 0)
+    (33, 200, 40),         # short prompt: 64-row tiles; ragged in M, N and K (K % 32 != 0)
+    (64, 4608, 896),       # short prompt, K split
     (1, 64, 8),            # smallest legal
-    (257, 129, 264),
+    (257, 129, 264),       # N % 4 != 0: no K split possible
 ])
 def test_gemm_bf16_nt_matches_oracle(lib, orc, M, N, K):
     """out[M,N] = A[M,K] . W[N,K]^T, W bf16 (cuda.h:786-840). Weights N(0,0.02) as in the
@@ -65,6 +66,21 @@ def test_gemm_bf16_nt_exact_cases(lib, orc):
     A = np.full((32, 8), np.float32(1.0) + np.float32(2.0 ** -23), np.float32)
     got = _gemm(lib, A, orc.to_bf16(np.ones((32, 8), np.float32)).reshape(32, 8))
     assert np.all(got == np.float32(8.0 * (1.0 + 2.0 ** -23)))
+
+
+def test_gemm_bf16_nt_whole_rounds_plus_split_tail(lib, orc):
+    """More tiles than the chip runs at once: the columns that make whole rounds of tiles run
+    with full K, the rest (here 9 tile columns, the last one ragged) is split over K into scratch
+    parts and summed into its column range of the result. Integer-valued operands make every
+    partial sum exact, so the result must equal the float64 product bit for bit wherever a
+    column lands."""
+    M, N, K = 640, 256 * 110 + 100, 1024
+    rng = np.random.default_rng(17)
+    A = rng.integers(-100, 100, (M, K)).astype(np.float32) + 0.5
+    Wf = rng.integers(-16, 16, (N, K)).astype(np.float32)
+    got = _gemm(lib, A, orc.to_bf16(Wf).reshape(N, K))
+    want = A.astype(np.float64) @ Wf.astype(np.float64).T
+    assert np.array_equal(got.astype(np.float64), want)
 
 
 def test_gemm_bf16_nt_row_equals_gemv(lib, orc):
