@@ -83,6 +83,23 @@ def test_gemm_bf16_nt_whole_rounds_plus_split_tail(lib, orc):
     assert np.array_equal(got.astype(np.float64), want)
 
 
+def test_gemm_bf16_nt_random_shapes_exact(lib, orc):
+    """Forty random shapes (every tile variant, K-split counts from 1 to 16, ragged edges in M, N
+    and K, N % 4 != 0 where K cannot be split) with integer-valued operands: each result must
+    equal the float64 product exactly, whatever the launch shape chosen for it."""
+    rng = np.random.default_rng(23)
+    for case in range(40):
+        M = int(rng.choice([1, 7, 33, 64, 65, 128, 200, 257, 512, 640]))
+        N = int(rng.integers(1, 1400)) if case % 3 else int(rng.integers(1, 350)) * 4
+        K = int(rng.integers(1, 260)) * 8
+        print("case gemm random", M, N, K, flush=True)
+        A = rng.integers(-60, 60, (M, K)).astype(np.float32) + 0.25
+        Wf = rng.integers(-12, 12, (N, K)).astype(np.float32)
+        got = _gemm(lib, A, orc.to_bf16(Wf).reshape(N, K))
+        want = A.astype(np.float64) @ Wf.astype(np.float64).T
+        assert np.array_equal(got.astype(np.float64), want), (M, N, K)
+
+
 def test_gemm_bf16_nt_row_equals_gemv(lib, orc):
     """Row m of the GEMM and the decode GEMV over the same [N,K] bf16 weights agree to
     summation-order noise."""
