@@ -250,11 +250,14 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     // the first two float4s a thread owns (all of them for rows up to 2 * blockDim * 4
     // floats) stay in registers between the two passes of the norm
     float4 kept0 = make_float4(0.f, 0.f, 0.f, 0.f), kept1 = kept0;
+    float4 keptw0 = kept0, keptw1 = kept0;   // their norm weights, requested ahead of the block sum
     if (PRO == kRmsnorm) {   // mean square of the row, summed in a fixed order
       float ss = 0.f;
       int it = 0;
       for (int i = tid; i < n4; i += blockDim.x, it++) {
         float4 v = x4[i];
+        if (it == 0) keptw0 = reinterpret_cast<const float4*>(pro.norm_w)[i];
+        if (it == 1) keptw1 = reinterpret_cast<const float4*>(pro.norm_w)[i];
         if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
         if (it == 0) kept0 = v;
         if (it == 1) kept1 = v;
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       if (PRO == kRmsnorm && live) {
         if (d4 && !have) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
         if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
-        const float4 w4 = reinterpret_cast<const float4*>(pro.norm_w)[i];
+        const float4 w4 = have ? (it2 == 0 ? keptw0 : keptw1) : reinterpret_cast<const float4*>(pro.norm_w)[i];
         v.x = (v.x * inv) * w4.x; v.y = (v.y * inv) * w4.y;
         v.z = (v.z * inv) * w4.z; v.w = (v.w * inv) * w4.w;
       }
