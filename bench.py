@@ -464,11 +464,15 @@ def main():
     e0, e1 = lib.event(), lib.event()
     for r in rings:
         n = max(10, min(r["copies"], 60))
-        lib.record(e0)
-        for i in range(n):
-            lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"], wq_off=((r["it"] + i) % r["copies"]) * r["stride"])
-        lib.record(e1)
-        ms = lib.elapsed_ms(e0, e1) / n
+        rounds = []
+        for _ in range(5):      # median of 5 rounds, the reference's discipline (bench_q4_gemv.cpp:106-119)
+            lib.record(e0)
+            for i in range(n):
+                lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"], wq_off=((r["it"] + i) % r["copies"]) * r["stride"])
+            lib.record(e1)
+            rounds.append(lib.elapsed_ms(e0, e1) / n)
+            r["it"] += n
+        ms = float(np.median(rounds))
         per_shape["%dx%d" % (r["N"], r["K"])] = {"us": round(ms * 1e3, 2),
                                                  "GB/s": round(r["nb"] / ms / 1e6, 1)}
     # dominant kernel: average launch duration over back-to-back launches of the LM-head
