@@ -565,6 +565,13 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
     if (rows_per_cu >= 128) { nw = 8; R = 4; KW = 1; }  // two 8-wave blocks per CU, 32-row tiles
     else if (rows_per_cu >= 64) { nw = 8; R = 4; KW = 2; }  // same blocks, 16-row tiles
     else if (rows_per_cu >= 32) { R = 2; KW = 1; }    // 32
+    else if (N > 16 * (int64_t)cus) {
+      // 17..31 rows per CU: 16-row tiles would leave a second, nearly empty round. Two blocks
+      // per CU, one row per wavefront, as many wavefronts as make the rows one round.
+      R = 1; KW = 1;
+      nw = (int)((N + 2 * (int64_t)cus - 1) / (2 * (int64_t)cus));
+      if (nw < 4) nw = 4;
+    }
     else if (rows_per_cu >= 8) { R = 2; KW = 2; }     // 16
     else { nw = 8; R = 1; KW = 2; }                   // 4
   } else {
