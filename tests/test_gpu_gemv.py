@@ -29,7 +29,8 @@ def _q4_case(lib, orc, N, K, seed, from_weights):
     return got, want
 
 
-@pytest.mark.parametrize("N,K", [(4864, 896), (3584, 3584), (512, 3584), (1024, 18944)])
+@pytest.mark.parametrize("N,K", [(4864, 896), (3584, 3584), (512, 3584), (1024, 18944),
+                                 (4608, 3584), (4097, 512), (8191, 256)])   # the last three: 17..31 rows per CU
 def test_gemv_q4_baseline_shapes(lib, orc, N, K):
     print("case gemv_q4", N, K, flush=True)
     got, want = _q4_case(lib, orc, N, K, 100 + N % 97, from_weights=(K != 896))
@@ -119,7 +120,7 @@ def test_gemv_q4_declines(lib, pkg):
 
 
 @pytest.mark.parametrize("N,K", [(3584, 3584), (512, 3584), (4864, 896), (40, 64), (1000, 520),
-                                 (9, 8), (151936 // 8, 896)])
+                                 (9, 8), (151936 // 8, 896), (4608, 3584), (7001, 1024)])
 def test_gemv_bf16_row(lib, orc, N, K):
     print("case gemv_bf16_row", N, K, flush=True)
     w = orc.to_bf16(orc.normal(N * K, 11 + N, 0.0, 0.02).reshape(N, K))
