@@ -100,6 +100,7 @@ SIGNATURES = {
     "tlhip_gemv_bf16_row_rmsnorm_gateup": (cint, [P, P, P, P, P, P, i64, i64, f32]),
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
     "tlhip_tune_gemv_cols": (cint, [cint]),
+    "tlhip_tune_attn_prefill": (cint, [cint]),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
 }
@@ -399,6 +400,9 @@ class TlHip:
         self._chk(self.c.tlhip_gemv_bf16_row_rmsnorm_gateup(
             x.ptr, delta.ptr if delta is not None else None, norm_w.ptr,
             xout.ptr if xout is not None else None, W.ptr, act.ptr, N2, K, eps))
+
+    def tune_attn_prefill(self, valu_kernel):
+        self._chk(self.c.tlhip_tune_attn_prefill(1 if valu_kernel else 0))
 
     def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0, lpr=0):
         self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw, lpr))

@@ -655,10 +655,19 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
 }
 
+// attn_prefill_mfma.hip
+template <int D, typename KT>
+int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
+                        int64_t kv_max, float scale, int pos0);
+
 template <int D, typename KT>
 static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
                           int T, int64_t kv_max, float scale, int pos0) {
   Context& c = tlhip::ctx();
+  if (!c.tune_prefill_valu) {
+    if (int rc = launch_prefill_mfma<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0)) return rc;
+    TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
+  }
   constexpr int G = 8;   // query positions per block
   const dim3 grid(Hq, 1, (T + 4 * G - 1) / (4 * G)), block(256);   // 4 wavefronts x G query rows
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,

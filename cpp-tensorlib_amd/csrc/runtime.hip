@@ -346,4 +346,10 @@ int tlhip_tune_gemv_cols(int max_k_splits) {
   return TLHIP_OK;
 }
 
+int tlhip_tune_attn_prefill(int valu_kernel) {
+  TLHIP_REQUIRE_READY();
+  ctx().tune_prefill_valu = valu_kernel != 0;
+  return 0;
+}
+
 }  // extern "C"

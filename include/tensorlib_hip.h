@@ -328,6 +328,10 @@ int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int wa
  * split, 0 = the built-in choice. The reference's diagnostic knob set_no_splitk (cuda.h:193-197,
  * 496-497), which its GEMV benchmark toggles. */
 int tlhip_tune_gemv_cols(int max_k_splits);
+/* Which kernel serves tlhip_attn_prefill: 0 = the matrix-pipe one (default), 1 = the VALU kernel
+ * that shares its code with decode attention. Same results within fp32 summation order; for A/B
+ * timing and tests. No reference counterpart. */
+int tlhip_tune_attn_prefill(int valu_kernel);
 
 #ifdef __cplusplus
 }
