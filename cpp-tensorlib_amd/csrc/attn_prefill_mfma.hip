@@ -33,20 +33,24 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_mov(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
-// max / sum over the 32 lanes of a half wavefront (lanes that share lane / 32); result in every lane
+// max / sum over the 32 lanes of a half wavefront (lanes that share lane / 32); result in every
+// lane. Four DPP steps finish a 16-lane row; v_permlane16_swap (gfx950) then hands each row of a
+// pair the other row's value: with both operands = v it returns (rows 0,0,2,2 ; rows 1,1,3,3).
 __device__ __forceinline__ float half_max(float v) {
   v = fmaxf(v, dpp_mov<0xB1>(v));    // quad_perm [1,0,3,2]
   v = fmaxf(v, dpp_mov<0x4E>(v));    // quad_perm [2,3,0,1]
   v = fmaxf(v, dpp_mov<0x141>(v));   // row_half_mirror
   v = fmaxf(v, dpp_mov<0x140>(v));   // row_mirror
-  return fmaxf(v, __shfl_xor(v, 16, 64));
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float half_sum(float v) {
   v += dpp_mov<0xB1>(v);
   v += dpp_mov<0x4E>(v);
   v += dpp_mov<0x141>(v);
   v += dpp_mov<0x140>(v);
-  return v + __shfl_xor(v, 16, 64);
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 __device__ __forceinline__ float4 load_kv4(const float* p) { return *reinterpret_cast<const float4*>(p); }
