@@ -5,11 +5,11 @@
 // v_mfma_f32_32x32x2_f32 multiplies f32 by f32 exactly and accumulates in fp32, so scores and
 // outputs differ from the reference's loops in summation order only.
 //
-// A block owns one query head and 32 consecutive query positions; its 4 wavefronts deal the
+// A block owns one query head and 32 consecutive query positions; its 8 wavefronts deal the
 // 32-key tiles of the causal range round-robin and each keeps a running (max, sum, output) state
 // for all 32 queries (online softmax), merged through LDS at the end. Per key tile a wavefront
 // issues 2 x D/2 MFMAs (Q.K^T, then P.V):
-//   * S[32 q x 32 k] : A = Q (held in registers for the whole block), B = the K tile from LDS;
+//   * S[32 q x 32 k] : A = the Q tile (in LDS, shared by the block), B = the K tile from LDS;
 //   * the score tile leaves the MFMA as one column (key) per lane and 16 rows (queries) per
 //     lane, so row maxima and sums are lane reductions over half a wavefront;
 //   * P goes through a 32 x 32 LDS tile to become the A operand of P.V; the output
@@ -19,10 +19,10 @@
 // makes a lane's four consecutive steps one 16-byte LDS read (Q and K, or P and V, use the
 // same order, and a sum does not care).
 //
-// K and V tiles are private to their wavefront (no block barriers inside the loop); the next
-// tile's global loads are in flight in registers while the current tile is multiplied. LDS per
-// wavefront: K 32 x (D+4), V 32 x D, P 32 x 36 floats - one block per CU, one wavefront per SIMD,
-// which is what a chain of 64-cycle MFMAs wants.
+// K, P and V tiles are private to their wavefront and take turns in ONE LDS region (no block
+// barriers inside the loop): K is dead once the scores exist, P once it sits in registers.
+// Eight wavefronts are two per SIMD: one's softmax (~750 VALU instructions a tile) and load
+// latency run under the other's 64-cycle MFMAs. One block per CU (9 regions of 32 x (D+4) floats).
 #include "common.hpp"
 
 namespace tlhip {
@@ -59,97 +59,81 @@ __device__ __forceinline__ float4 load_kv4(const uint16_t* p) {   // 4 bf16, wid
   return make_float4(bf16_lo(r.x), bf16_hi(r.x), bf16_lo(r.y), bf16_hi(r.y));
 }
 
+// LDS: the Q tile (shared by the block) and one 32 x (D+4) region per wavefront that holds the K
+// tile, then P, then the V tile.
 template <int D>
 struct PrefillLds {
-  static constexpr int KS = D + 4;                        // K row stride: 16-byte reads of 8 keys hit 32 banks
-  static constexpr int PS = 36;                           // P row stride
-  static constexpr int kWave = 32 * KS + 32 * D + 32 * PS;   // floats per wavefront
-  static constexpr size_t kBytes = (size_t)4 * kWave * sizeof(float);
+  static constexpr int KS = D + 4;
+  static constexpr int PS = 36;
+  static constexpr int kRegion = 32 * KS;                 // floats: Q, and one region per wavefront
+  static constexpr size_t kBytes = (size_t)9 * kRegion * sizeof(float);
 };
 
-// grid = (Hq, ceil(T / 32)); blockIdx.y = 0 is the LAST query tile (longest key range first).
 template <int D, typename KT>
-__global__ __launch_bounds__(256, 1) void attn_prefill_mfma_kernel(const float* __restrict__ q,
-                                                                   const KT* __restrict__ K,
-                                                                   const KT* __restrict__ V,
-                                                                   float* __restrict__ out, int group, int T,
-                                                                   int pos0, int64_t kv_stride, float scale) {
+__global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* __restrict__ q,
+                                                                    const KT* __restrict__ K,
+                                                                    const KT* __restrict__ V,
+                                                                    float* __restrict__ out, int group, int T,
+                                                                    int pos0, int64_t kv_stride, float scale) {
   using L = PrefillLds<D>;
   constexpr int KS = L::KS, PS = L::PS;
-  constexpr int kLoads = 32 * D / 4 / 64;                 // float4 per lane per tile (K, and again V)
+  constexpr int kLoads = 32 * D / 4 / 64;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l31 = lane & 31, hi = lane >> 5;
   const int h = blockIdx.x;
   const int nqt = (T + 31) >> 5;
-  const int p0 = (nqt - 1 - (int)blockIdx.y) * 32;        // first query position of the tile
+  const int p0 = (nqt - 1 - (int)blockIdx.y) * 32;
   const KT* Kh = K + (size_t)(h / group) * kv_stride;
   const KT* Vh = V + (size_t)(h / group) * kv_stride;
-  float* Kl = lds + wave * L::kWave;
-  float* Vl = Kl + 32 * KS;
-  float* Pl = Vl + 32 * D;
-
-  // keys some row of this tile may see: [0, kend)
+  float* Qs = lds;
+  float* R = lds + (1 + wave) * L::kRegion;
   const int kend = min(pos0 + p0 + 32, pos0 + T);
   const int nkt = (kend + 31) >> 5;
 
-  // Q fragments: qf[m] = Q[p0 + l31][8m + 4hi .. +3] (rows beyond T are clamped and never stored)
-  float4 qf[D / 8];
-  {
-    const float* qp = q + ((size_t)h * T + min(p0 + l31, T - 1)) * D + 4 * hi;
-#pragma unroll
-    for (int m = 0; m < D / 8; m++) qf[m] = *reinterpret_cast<const float4*>(qp + 8 * m);
+  for (int slot = tid; slot < 32 * D / 4; slot += 512) {   // Q tile -> LDS (rows beyond T clamped, never stored)
+    const int row = slot / (D / 4), c4 = slot % (D / 4);
+    *reinterpret_cast<float4*>(Qs + row * KS + 4 * c4) =
+        *reinterpret_cast<const float4*>(q + ((size_t)h * T + min(p0 + row, T - 1)) * D + 4 * c4);
   }
+  __syncthreads();
 
   f32x16 o[D / 32];
 #pragma unroll
   for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
     for (int v = 0; v < 16; v++) o[dt][v] = 0.f;
-  float mrow[16], lrow[16];   // running max / sum of row 8*(v/4) + 4*hi + v%4
+  float mrow[16], lrow[16];
 #pragma unroll
   for (int v = 0; v < 16; v++) { mrow[v] = -INFINITY; lrow[v] = 0.f; }
 
-  // this lane's float4 slots of a tile: slot = lane + 64 i -> key = slot / (D/4), column 4 * (slot % (D/4))
-  float4 kreg[kLoads], vreg[kLoads];
-  auto gload = [&](int k0) {
+  for (int kt = wave; kt < nkt; kt += 8) {
+    const int k0 = kt * 32;
+    float4 kreg[kLoads], vreg[kLoads];
 #pragma unroll
     for (int i = 0; i < kLoads; i++) {
       const int slot = lane + 64 * i, key = slot / (D / 4), c4 = slot % (D / 4);
-      const size_t off = (size_t)min(k0 + key, kend - 1) * D + 4 * c4;   // rows past the range are masked below
+      const size_t off = (size_t)min(k0 + key, kend - 1) * D + 4 * c4;
       kreg[i] = load_kv4(Kh + off);
       vreg[i] = load_kv4(Vh + off);
     }
-  };
-  auto lstore = [&]() {
 #pragma unroll
     for (int i = 0; i < kLoads; i++) {
       const int slot = lane + 64 * i, key = slot / (D / 4), c4 = slot % (D / 4);
-      *reinterpret_cast<float4*>(Kl + key * KS + 4 * c4) = kreg[i];
-      *reinterpret_cast<float4*>(Vl + key * D + 4 * c4) = vreg[i];
+      *reinterpret_cast<float4*>(R + key * KS + 4 * c4) = kreg[i];
     }
-  };
-
-  if (wave < nkt) gload(wave * 32);
-  for (int kt = wave; kt < nkt; kt += 4) {
-    const int k0 = kt * 32;
-    lstore();                                   // this tile, requested one iteration ago
-    if (kt + 4 < nkt) gload(k0 + 128);          // the next one, in flight during the MFMAs below
-
-    // ---- scores: S[q][k] = sum_d Q[q][d] K[k][d]
     f32x16 s;
 #pragma unroll
     for (int v = 0; v < 16; v++) s[v] = 0.f;
 #pragma unroll
     for (int m = 0; m < D / 8; m++) {
-      const float4 kf = *reinterpret_cast<const float4*>(Kl + l31 * KS + 8 * m + 4 * hi);
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[m].x, kf.x, s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[m].y, kf.y, s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[m].z, kf.z, s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[m].w, kf.w, s, 0, 0, 0);
+      const float4 qa = *reinterpret_cast<const float4*>(Qs + l31 * KS + 8 * m + 4 * hi);
+      const float4 kf = *reinterpret_cast<const float4*>(R + l31 * KS + 8 * m + 4 * hi);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.x, kf.x, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.y, kf.y, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.z, kf.z, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.w, kf.w, s, 0, 0, 0);
     }
-
-    // ---- online softmax; lane = key k0 + l31, value v = query row 8*(v/4) + 4*hi + v%4
     const int key = k0 + l31;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
@@ -157,25 +141,28 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_mfma_kernel(const float* 
       const bool seen = key <= pos0 + p0 + r && key < kend;
       const float sv = seen ? s[v] * scale : -INFINITY;
       const float mnew = fmaxf(mrow[v], half_max(sv));
-      const float mref = mnew == -INFINITY ? 0.f : mnew;   // a row with nothing seen yet
-      const float corr = __expf(mrow[v] - mref);           // 0 on the row's first tile
-      const float p = __expf(sv - mref);                   // 0 for masked keys
+      const float mref = mnew == -INFINITY ? 0.f : mnew;
+      const float corr = __expf(mrow[v] - mref);
+      const float p = __expf(sv - mref);
       lrow[v] = lrow[v] * corr + half_sum(p);
       mrow[v] = mnew;
 #pragma unroll
       for (int dt = 0; dt < D / 32; dt++) o[dt][v] *= corr;
-      Pl[r * PS + l31] = p;
+      R[r * PS + l31] = p;                      // the K tile is dead: P takes its place
     }
-
-    // ---- output: O[q][d] += sum_k P[q][k] V[k][d]
     float4 pf[4];
 #pragma unroll
-    for (int m = 0; m < 4; m++) pf[m] = *reinterpret_cast<const float4*>(Pl + l31 * PS + 8 * m + 4 * hi);
+    for (int m = 0; m < 4; m++) pf[m] = *reinterpret_cast<const float4*>(R + l31 * PS + 8 * m + 4 * hi);
+#pragma unroll
+    for (int i = 0; i < kLoads; i++) {          // P is in registers: V takes the region
+      const int slot = lane + 64 * i, vkey = slot / (D / 4), c4 = slot % (D / 4);
+      *reinterpret_cast<float4*>(R + vkey * D + 4 * c4) = vreg[i];
+    }
 #pragma unroll
     for (int dt = 0; dt < D / 32; dt++) {
 #pragma unroll
       for (int m = 0; m < 4; m++) {
-        const float* vp = Vl + (8 * m + 4 * hi) * D + dt * 32 + l31;
+        const float* vp = R + (8 * m + 4 * hi) * D + dt * 32 + l31;
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].x, vp[0], o[dt], 0, 0, 0);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].y, vp[D], o[dt], 0, 0, 0);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].z, vp[2 * D], o[dt], 0, 0, 0);
@@ -184,39 +171,37 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_mfma_kernel(const float* 
     }
   }
 
-  // ---- merge the four wavefronts' states. Each writes O [32][D], m [32], l [32] over its own
-  // K/V region (32 * (2D + 4) floats >= 32 * D + 64), then 8 threads finish one query row.
-  float* Ow = Kl;
-  float* Mw = Ow + 32 * D;
-  float* Lw = Mw + 32;
+  // merge: each wavefront leaves O [32][D], m [32], l [32] in its region; 16 threads finish a row
+  float* Mw = R + 32 * D;
 #pragma unroll
   for (int v = 0; v < 16; v++) {
     const int r = 8 * (v >> 2) + 4 * hi + (v & 3);
 #pragma unroll
-    for (int dt = 0; dt < D / 32; dt++) Ow[r * D + dt * 32 + l31] = o[dt][v];
-    if (l31 == 0) { Mw[r] = mrow[v]; Lw[r] = lrow[v]; }
+    for (int dt = 0; dt < D / 32; dt++) R[r * D + dt * 32 + l31] = o[dt][v];
+    if (l31 == 0) { Mw[r] = mrow[v]; Mw[32 + r] = lrow[v]; }
   }
   __syncthreads();
   {
-    const int row = tid >> 3, d0 = (tid & 7) * (D / 8);
-    float f[4], M = -INFINITY, Lsum = 0.f;
+    const int row = tid >> 4, d0 = (tid & 15) * (D / 16);
+    const float* base = lds + L::kRegion;
+    float f[8], M = -INFINITY, Lsum = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; w++) M = fmaxf(M, lds[w * L::kWave + 32 * D + row]);
+    for (int w = 0; w < 8; w++) M = fmaxf(M, base[w * L::kRegion + 32 * D + row]);
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
-      const float mw = lds[w * L::kWave + 32 * D + row];
+    for (int w = 0; w < 8; w++) {
+      const float mw = base[w * L::kRegion + 32 * D + row];
       f[w] = mw == -INFINITY ? 0.f : __expf(mw - M);
-      Lsum += f[w] * lds[w * L::kWave + 32 * D + 32 + row];
+      Lsum += f[w] * base[w * L::kRegion + 32 * D + 32 + row];
     }
     if (p0 + row < T) {
       const float inv = 1.0f / Lsum;
       float* op = out + ((size_t)h * T + p0 + row) * D + d0;
 #pragma unroll
-      for (int d = 0; d < D / 8; d += 4) {
+      for (int d = 0; d < D / 16; d += 4) {
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-          const float4 ow = *reinterpret_cast<const float4*>(lds + w * L::kWave + row * D + d0 + d);
+        for (int w = 0; w < 8; w++) {
+          const float4 ow = *reinterpret_cast<const float4*>(base + w * L::kRegion + row * D + d0 + d);
           a.x += f[w] * ow.x; a.y += f[w] * ow.y; a.z += f[w] * ow.z; a.w += f[w] * ow.w;
         }
         *reinterpret_cast<float4*>(op + d) = make_float4(a.x * inv, a.y * inv, a.z * inv, a.w * inv);
@@ -234,7 +219,7 @@ int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, in
   if ((size_t)lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  const dim3 grid((unsigned)Hq, (unsigned)((T + 31) / 32)), block(256);
+  const dim3 grid((unsigned)Hq, (unsigned)((T + 31) / 32)), block(512);
   hipLaunchKernelGGL(fn, grid, block, (size_t)lds, c.stream, q, K, V, out, Hq / Hkv, T, pos0, kv_max * (int64_t)D, scale);
   return 0;
 }
