@@ -85,15 +85,15 @@ __device__ __forceinline__ float4 rope4(float4 own, const float2* __restrict__ t
   const float4 t1 = *reinterpret_cast<const float4*>(table + j0 + 2);   // (c2, s2, c3, s3)
   float4 o;
   if (lo) {
-    o.x = __fsub_rn(__fmul_rn(a.x, t0.x), __fmul_rn(b.x, t0.y));
-    o.y = __fsub_rn(__fmul_rn(a.y, t0.z), __fmul_rn(b.y, t0.w));
-    o.z = __fsub_rn(__fmul_rn(a.z, t1.x), __fmul_rn(b.z, t1.y));
-    o.w = __fsub_rn(__fmul_rn(a.w, t1.z), __fmul_rn(b.w, t1.w));
+    o.x = sub_rn(mul_rn(a.x, t0.x), mul_rn(b.x, t0.y));
+    o.y = sub_rn(mul_rn(a.y, t0.z), mul_rn(b.y, t0.w));
+    o.z = sub_rn(mul_rn(a.z, t1.x), mul_rn(b.z, t1.y));
+    o.w = sub_rn(mul_rn(a.w, t1.z), mul_rn(b.w, t1.w));
   } else {
-    o.x = __fadd_rn(__fmul_rn(a.x, t0.y), __fmul_rn(b.x, t0.x));
-    o.y = __fadd_rn(__fmul_rn(a.y, t0.w), __fmul_rn(b.y, t0.z));
-    o.z = __fadd_rn(__fmul_rn(a.z, t1.y), __fmul_rn(b.z, t1.x));
-    o.w = __fadd_rn(__fmul_rn(a.w, t1.w), __fmul_rn(b.w, t1.z));
+    o.x = add_rn(mul_rn(a.x, t0.y), mul_rn(b.x, t0.x));
+    o.y = add_rn(mul_rn(a.y, t0.w), mul_rn(b.y, t0.z));
+    o.z = add_rn(mul_rn(a.z, t1.y), mul_rn(b.z, t1.x));
+    o.w = add_rn(mul_rn(a.w, t1.w), mul_rn(b.w, t1.z));
   }
   return o;
 }
@@ -658,16 +658,17 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
 // attn_prefill_mfma.hip
 template <int D, typename KT>
 int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
-                        int64_t kv_max, float scale, int pos0);
+                        int64_t kv_max, float scale, int pos0, int token_major);
 
 template <int D, typename KT>
 static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
-                          int T, int64_t kv_max, float scale, int pos0) {
+                          int T, int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = tlhip::ctx();
   if (!c.tune_prefill_valu) {
-    if (int rc = launch_prefill_mfma<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0)) return rc;
+    if (int rc = launch_prefill_mfma<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
     TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
   }
+  if (token_major) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill_tok: the VALU kernel writes head-major only");
   constexpr int G = 8;   // query positions per block
   const dim3 grid(Hq, 1, (T + 4 * G - 1) / (4 * G)), block(256);   // 4 wavefronts x G query rows
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
@@ -711,9 +712,9 @@ int tlhip_attn_decode(const void* q, const void* K, const void* V, void* out, in
                   : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale);
 }
 
-int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
-                       int64_t n_kv_heads, int64_t T, int64_t kv_max, int64_t D, float scale,
-                       int kv_bf16, int64_t pos0) {
+static int attn_prefill_entry(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                              int64_t n_kv_heads, int64_t T, int64_t kv_max, int64_t D, float scale,
+                              int kv_bf16, int64_t pos0, int token_major) {
   TLHIP_REQUIRE_READY();
   if (!q || !K || !V || !out) return fail(TLHIP_EINVAL, "tlhip_attn_prefill: null pointer");
   // the reference's gates (cuda.h:1171-1177)
@@ -732,13 +733,25 @@ int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out, i
   if (kv_bf16) {
     const uint16_t* pk = static_cast<const uint16_t*>(K);
     const uint16_t* pv = static_cast<const uint16_t*>(V);
-    return D == 128 ? launch_prefill<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0)
-                    : launch_prefill<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0);
+    return D == 128 ? launch_prefill<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0, token_major)
+                    : launch_prefill<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0, token_major);
   }
   const float* pk = static_cast<const float*>(K);
   const float* pv = static_cast<const float*>(V);
-  return D == 128 ? launch_prefill<128, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0)
-                  : launch_prefill<64, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0);
+  return D == 128 ? launch_prefill<128, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0, token_major)
+                  : launch_prefill<64, float>(pq, pk, pv, po, Hq, Hkv, t, kv_max, scale, p0, token_major);
+}
+
+int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                       int64_t n_kv_heads, int64_t T, int64_t kv_max, int64_t D, float scale,
+                       int kv_bf16, int64_t pos0) {
+  return attn_prefill_entry(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale, kv_bf16, pos0, 0);
+}
+
+int tlhip_attn_prefill_tok(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                           int64_t n_kv_heads, int64_t T, int64_t kv_max, int64_t D, float scale,
+                           int kv_bf16, int64_t pos0) {
+  return attn_prefill_entry(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale, kv_bf16, pos0, 1);
 }
 
 int64_t tlhip_attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t kv_max, int64_t D) {

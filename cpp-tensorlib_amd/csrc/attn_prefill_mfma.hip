@@ -74,7 +74,8 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
                                                                     const KT* __restrict__ K,
                                                                     const KT* __restrict__ V,
                                                                     float* __restrict__ out, int group, int T,
-                                                                    int pos0, int64_t kv_stride, float scale) {
+                                                                    int pos0, int64_t kv_stride, float scale,
+                                                                    int64_t o_head, int64_t o_row) {
   using L = PrefillLds<D>;
   constexpr int KS = L::KS, PS = L::PS;
   constexpr int kLoads = 32 * D / 4 / 64;
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
     }
     if (p0 + row < T) {
       const float inv = 1.0f / Lsum;
-      float* op = out + ((size_t)h * T + p0 + row) * D + d0;
+      float* op = out + (size_t)h * o_head + (size_t)(p0 + row) * o_row + d0;   // [Hq,T,D] or [T,Hq*D]
 #pragma unroll
       for (int d = 0; d < D / 16; d += 4) {
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
 
 template <int D, typename KT>
 int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
-                        int64_t kv_max, float scale, int pos0) {
+                        int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = ctx();
   auto fn = attn_prefill_mfma_kernel<D, KT>;
   const int lds = (int)PrefillLds<D>::kBytes;
@@ -220,13 +221,15 @@ int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, in
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
   const dim3 grid((unsigned)Hq, (unsigned)((T + 31) / 32)), block(512);
-  hipLaunchKernelGGL(fn, grid, block, (size_t)lds, c.stream, q, K, V, out, Hq / Hkv, T, pos0, kv_max * (int64_t)D, scale);
+  const int64_t o_head = token_major ? D : (int64_t)T * D, o_row = token_major ? (int64_t)Hq * D : D;
+  hipLaunchKernelGGL(fn, grid, block, (size_t)lds, c.stream, q, K, V, out, Hq / Hkv, T, pos0, kv_max * (int64_t)D, scale,
+                     o_head, o_row);
   return 0;
 }
 
-template int launch_prefill_mfma<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int);
-template int launch_prefill_mfma<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int);
-template int launch_prefill_mfma<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int);
-template int launch_prefill_mfma<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int);
+template int launch_prefill_mfma<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_mfma<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_mfma<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_mfma<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
 
 }  // namespace tlhip

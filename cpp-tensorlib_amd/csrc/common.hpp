@@ -70,6 +70,23 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // ---- device helpers ----------------------------------------------------------
 #if defined(__HIPCC__)
 
+// One rounding each, never contracted into an FMA with a neighbouring operation: the CPU path
+// multiplies and adds separately (its loops are compiled without FMA contraction). hipcc's
+// __fmul_rn / __fadd_rn are plain `*` / `+` and do NOT prevent contraction; these do, because
+// the operations are built in a scope where contraction is off and keep that property when inlined.
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);

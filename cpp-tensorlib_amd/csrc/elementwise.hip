@@ -28,7 +28,7 @@ __device__ __forceinline__ float un_op(float a) {
 // out = f(...)*scale + offset with separate multiply and add, like the CPU
 // loops (array.h:1879, 2223); identity epilogues leave the value untouched.
 __device__ __forceinline__ float epilogue(float v, float scale, float offset) {
-  return __fadd_rn(__fmul_rn(v, scale), offset);
+  return add_rn(mul_rn(v, scale), offset);
 }
 
 template <int OP>

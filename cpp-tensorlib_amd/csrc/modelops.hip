@@ -33,8 +33,8 @@ __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ x,
     x0 += bias[bi + j];
     x1 += bias[bi + j + half];
   }
-  out[bi + j] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
-  out[bi + j + half] = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+  out[bi + j] = sub_rn(mul_rn(x0, c), mul_rn(x1, s));
+  out[bi + j + half] = add_rn(mul_rn(x0, s), mul_rn(x1, c));
 }
 
 // ---- rmsnorm --------------------------------------------------------------------
@@ -296,8 +296,8 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(
     const float* bias = is_k ? (bk ? bk + (size_t)(r - Hq) * D : nullptr) : (bq ? bq + bi : nullptr);
     float x0 = qkv[bi + j], x1 = qkv[bi + j + half];
     if (bias) { x0 += bias[j]; x1 += bias[j + half]; }
-    const float o0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
-    const float o1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+    const float o0 = sub_rn(mul_rn(x0, c), mul_rn(x1, s));
+    const float o1 = add_rn(mul_rn(x0, s), mul_rn(x1, c));
     qkv[bi + j] = o0;
     qkv[bi + j + half] = o1;
     if (is_k) {
@@ -327,6 +327,93 @@ __global__ void rope_table_kernel(float2* __restrict__ table, int D, int64_t pos
   const double theta = pow((double)base, -2.0 * (double)j / (double)D);
   const double ang = (double)pos * theta;
   table[j] = make_float2((float)cos(ang), (float)sin(ang));
+}
+
+// table[t][j] = (cos, sin)((pos0 + t) * base^(-2j/D)), t < T: the angles of a prompt chunk, the
+// same for every layer and every head (rope_kernel forms each of them once per head and layer).
+__global__ __launch_bounds__(256) void rope_table_range_kernel(float2* __restrict__ table, int D,
+                                                               int64_t pos0, int T, float base) {
+  const int half = D >> 1;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * half) return;
+  const int t = i / half, j = i - t * half;
+  const double theta = pow((double)base, -2.0 * (double)j / (double)D);
+  const double ang = (double)(pos0 + t) * theta;
+  table[i] = make_float2((float)cos(ang), (float)sin(ang));
+}
+
+// ---- fused q/k/v epilogue of a prompt chunk --------------------------------------------------
+// One launch for what the chunk otherwise does in five (split_heads with bias, rope of q, rope
+// of k, and the two cache fills): qkv [T, (Hq + 2 Hkv) D] token-major from the projection GEMM;
+// q gets bias and rotation and lands head-major in qh [Hq, T, D]; k gets bias and rotation,
+// v its bias, and both go straight into cache rows pos0 .. pos0 + T. Same arithmetic as the
+// separate kernels (bias add, unfused multiplies, one add / sub), so results are bit-identical.
+// A thread owns 4 consecutive rotary pairs (j .. j+3 with j + D/2 ..) or 4 consecutive v values.
+template <typename KT>
+__device__ __forceinline__ void kv_store4(KT* p, const float4 v);
+template <> __device__ __forceinline__ void kv_store4<float>(float* p, const float4 v) {
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <> __device__ __forceinline__ void kv_store4<uint16_t>(uint16_t* p, const float4 v) {
+  const uint32_t lo = (uint32_t)f32_to_bf16_rne(v.x) | ((uint32_t)f32_to_bf16_rne(v.y) << 16);
+  const uint32_t hi = (uint32_t)f32_to_bf16_rne(v.z) | ((uint32_t)f32_to_bf16_rne(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+}
+
+template <typename KT>
+__global__ __launch_bounds__(256) void qkv_rope_fill_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ bq, const float* __restrict__ bk,
+    const float* __restrict__ bv, const float2* __restrict__ table, float* __restrict__ qh,
+    KT* __restrict__ Kc, KT* __restrict__ Vc, int T, int Hq, int Hkv, int D, int64_t pos0,
+    int64_t kv_max) {
+  const int half = D >> 1, q4 = half >> 2;            // float4 groups per half row
+  const int rot_per_t = (Hq + Hkv) * q4, v_per_t = Hkv * (D >> 2);
+  const int per_t = rot_per_t + v_per_t;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)T * per_t) return;
+  const int t = (int)(i / per_t), e = (int)(i - (int64_t)t * per_t);
+  const float* row = qkv + (size_t)t * (Hq + 2 * Hkv) * D;
+  if (e < rot_per_t) {
+    const int r = e / q4, j = (e - r * q4) * 4;       // r: head within [q heads | k heads]
+    const bool is_k = r >= Hq;
+    const float* bias = is_k ? (bk ? bk + (size_t)(r - Hq) * D : nullptr) : (bq ? bq + (size_t)r * D : nullptr);
+    float4 x0 = *reinterpret_cast<const float4*>(row + (size_t)r * D + j);
+    float4 x1 = *reinterpret_cast<const float4*>(row + (size_t)r * D + j + half);
+    if (bias) {
+      const float4 b0 = *reinterpret_cast<const float4*>(bias + j);
+      const float4 b1 = *reinterpret_cast<const float4*>(bias + j + half);
+      x0.x += b0.x; x0.y += b0.y; x0.z += b0.z; x0.w += b0.w;
+      x1.x += b1.x; x1.y += b1.y; x1.z += b1.z; x1.w += b1.w;
+    }
+    const float2* cs = table + (size_t)t * half + j;
+    const float2 c0 = cs[0], c1 = cs[1], c2 = cs[2], c3 = cs[3];
+    float4 o0, o1;
+    o0.x = sub_rn(mul_rn(x0.x, c0.x), mul_rn(x1.x, c0.y));
+    o1.x = add_rn(mul_rn(x0.x, c0.y), mul_rn(x1.x, c0.x));
+    o0.y = sub_rn(mul_rn(x0.y, c1.x), mul_rn(x1.y, c1.y));
+    o1.y = add_rn(mul_rn(x0.y, c1.y), mul_rn(x1.y, c1.x));
+    o0.z = sub_rn(mul_rn(x0.z, c2.x), mul_rn(x1.z, c2.y));
+    o1.z = add_rn(mul_rn(x0.z, c2.y), mul_rn(x1.z, c2.x));
+    o0.w = sub_rn(mul_rn(x0.w, c3.x), mul_rn(x1.w, c3.y));
+    o1.w = add_rn(mul_rn(x0.w, c3.y), mul_rn(x1.w, c3.x));
+    if (is_k) {
+      KT* dst = Kc + ((size_t)(r - Hq) * kv_max + pos0 + t) * D;
+      kv_store4<KT>(dst + j, o0);
+      kv_store4<KT>(dst + j + half, o1);
+    } else {
+      float* dst = qh + ((size_t)r * T + t) * D;
+      *reinterpret_cast<float4*>(dst + j) = o0;
+      *reinterpret_cast<float4*>(dst + j + half) = o1;
+    }
+  } else {
+    const int ev = e - rot_per_t, h = ev / (D >> 2), d = (ev - h * (D >> 2)) * 4;
+    float4 v = *reinterpret_cast<const float4*>(row + (size_t)(Hq + Hkv) * D + (size_t)h * D + d);
+    if (bv) {
+      const float4 b = *reinterpret_cast<const float4*>(bv + (size_t)h * D + d);
+      v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+    }
+    kv_store4<KT>(Vc + ((size_t)h * kv_max + pos0 + t) * D + d, v);
+  }
 }
 
 // ---- device-resident greedy loop --------------------------------------------------------
@@ -563,6 +650,42 @@ int tlhip_rope_table(void* table, int64_t D, int64_t pos, const void* d_pos, flo
   hipError_t e_ = hipGetLastError();
   if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
   return TLHIP_OK;
+}
+
+int tlhip_rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, float base) {
+  TLHIP_REQUIRE_READY();
+  if (!table || D <= 0 || (D & 1) || D > 65536 || T <= 0 || T > 65535 || pos0 < 0)
+    return fail(TLHIP_EINVAL, "tlhip_rope_table_range: bad arguments");
+  rope_table_range_kernel<<<dim3(blocks_for(T * (D / 2))), dim3(256), 0, ctx().stream>>>(
+      static_cast<float2*>(table), (int)D, pos0, (int)T, base);
+  hipError_t e_ = hipGetLastError();
+  if (e_ != hipSuccess) return hip_fail(e_, "kernel launch");
+  return TLHIP_OK;
+}
+
+int tlhip_qkv_rope_fill(const void* qkv, const void* bq, const void* bk, const void* bv, const void* table,
+                        void* qh, void* Kc, void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads,
+                        int64_t D, int64_t pos0, int64_t kv_max, int kv_bf16) {
+  TLHIP_REQUIRE_READY();
+  if (!qkv || !table || !qh || !Kc || !Vc) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_fill: null pointer");
+  if (T <= 0 || T > 65535 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads > 65535 || n_kv_heads > 65535)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_fill: bad shape");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_fill: head_dim must be 64 or 128");   // the cache ops' gate
+  if (pos0 < 0 || pos0 + T > kv_max) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_fill: need 0 <= pos0, pos0 + T <= kv_max");
+  if (!aligned16(qkv) || !aligned16(qh) || !aligned16(Kc) || !aligned16(Vc) || (bq && !aligned16(bq)) ||
+      (bk && !aligned16(bk)) || (bv && !aligned16(bv)) || !aligned16(table))
+    return fail(TLHIP_EINVAL, "tlhip_qkv_rope_fill: operands must be 16-byte aligned");
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads;
+  const int64_t total = T * ((int64_t)(Hq + Hkv) * (D / 8) + (int64_t)Hkv * (D / 4));
+#define TLHIP_FILL(KT_)                                                                              \
+  qkv_rope_fill_kernel<KT_><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(                \
+      static_cast<const float*>(qkv), static_cast<const float*>(bq), static_cast<const float*>(bk), \
+      static_cast<const float*>(bv), static_cast<const float2*>(table), static_cast<float*>(qh),    \
+      static_cast<KT_*>(Kc), static_cast<KT_*>(Vc), (int)T, Hq, Hkv, (int)D, pos0, kv_max)
+  if (kv_bf16) TLHIP_FILL(uint16_t);
+  else TLHIP_FILL(float);
+#undef TLHIP_FILL
+  TLHIP_CHECK_LAUNCH(TLHIP_C_KV_FILL);
 }
 
 int tlhip_qkv_rope_append_tab(void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,

@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const float* __restr
         if (gm < M) {
           const float r = acc[i][j][v];
           // separate multiply and add, like the CPU loops (array.h:1879, 2223)
-          C[(size_t)gm * N + gn] = epi ? __fadd_rn(__fmul_rn(r, scale), offset) : r;
+          C[(size_t)gm * N + gn] = epi ? add_rn(mul_rn(r, scale), offset) : r;
         }
       }
     }
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void sgemm_sum_kernel(const float* __restrict_
   if (i >= n) return;
   float a = part[i];
   for (int s = 1; s < S; s++) a += part[(size_t)s * n + i];
-  C[i] = epi ? __fadd_rn(__fmul_rn(a, scale), offset) : a;
+  C[i] = epi ? add_rn(mul_rn(a, scale), offset) : a;
 }
 
 // Launches the matrix-pipe GEMM; the caller has checked the arguments.

@@ -121,6 +121,11 @@ struct api {
   int (*qkv_rope_append_dpos)(void*, const void*, const void*, const void*, void*, void*, int64_t,
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
   int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
+  int (*rope_table_range)(void*, int64_t, int64_t, int64_t, float) = nullptr;
+  int (*qkv_rope_fill)(const void*, const void*, const void*, const void*, const void*, void*, void*, void*,
+                       int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int) = nullptr;
+  int (*attn_prefill_tok)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
+                          int64_t, int64_t, float, int, int64_t) = nullptr;
   int (*tune_gemv_cols)(int) = nullptr;
   int (*convert)(const void*, int, void*, int, int64_t) = nullptr;
   int (*convert_transpose)(const void*, int, void*, int, int64_t, int64_t, int64_t, int64_t) = nullptr;
@@ -230,6 +235,9 @@ struct context {
               bind(f.attn_decode_dpos, "tlhip_attn_decode_dpos") &&
               bind(f.qkv_rope_append_dpos, "tlhip_qkv_rope_append_dpos") &&
               bind(f.rope_table, "tlhip_rope_table") &&
+              bind(f.rope_table_range, "tlhip_rope_table_range") &&
+              bind(f.qkv_rope_fill, "tlhip_qkv_rope_fill") &&
+              bind(f.attn_prefill_tok, "tlhip_attn_prefill_tok") &&
               bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
               bind(f.attn_decode_qkv, "tlhip_attn_decode_qkv") &&
               bind(f.tune_gemv_cols, "tlhip_tune_gemv_cols") && bind(f.convert, "tlhip_convert") && bind(f.convert_transpose, "tlhip_convert_transpose") &&
@@ -783,6 +791,48 @@ inline bool qkv_rope_append_tab(void* qkv, void* bq, void* bk, void* bv, void* K
                                                   d_pos, kv_max, table, kv_bf16 ? 1 : 0));
 }
 
+// The same for a prompt chunk: rope_table_range writes the angles of positions pos0 .. pos0+T-1
+// once per chunk; qkv_rope_fill takes the raw token-major [T, (Hq + 2 Hkv) D] projection, adds the
+// biases, rotates q and k, writes q head-major into qh [Hq, T, D] and k, v into cache rows
+// pos0 .. pos0+T-1 (one launch for split_heads + 2 x rope + kv_fill; bit-identical to them).
+inline bool rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, float base) {
+  auto& c = context::get();
+  if (!c.ready || !table) return false;
+  c.device_write_(table);
+  return detail::done_(c, c.f.rope_table_range(table, D, pos0, T, base));
+}
+inline bool qkv_rope_fill(void* qkv, void* bq, void* bk, void* bv, void* table, void* qh, void* Kc,
+                          void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
+                          int64_t pos0, int64_t kv_max, bool kv_bf16 = false) {
+  auto& c = context::get();
+  if (!c.ready || !table || (D != 128 && D != 64) || pos0 < 0 || pos0 + T > kv_max) return false;
+  c.device_read_(qkv);
+  if (bq) c.device_read_(bq);
+  if (bk) c.device_read_(bk);
+  if (bv) c.device_read_(bv);
+  c.device_read_(table);
+  c.device_write_(qh);
+  c.device_write_(Kc);
+  c.device_write_(Vc);
+  return detail::done_(c, c.f.qkv_rope_fill(qkv, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads, n_kv_heads, D,
+                                            pos0, kv_max, kv_bf16 ? 1 : 0));
+}
+// attn_prefill with the result written token-major, [T, Hq*D] (no merge_heads afterwards).
+inline bool attn_prefill_tok(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
+                             int64_t T, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false,
+                             int64_t pos0 = 0) {
+  auto& c = context::get();
+  if (!c.ready || (D != 128 && D != 64)) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  if (T <= 0 || T > 65535) return false;
+  c.device_read_(q);
+  c.device_read_(K);
+  c.device_read_(V);
+  c.device_write_(out);
+  return detail::done_(c, c.f.attn_prefill_tok(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
+                                               kv_bf16 ? 1 : 0, pos0));
+}
+
 // Bias + rotation of the raw [q|k|v] projection, the cache append and the attention over
 // keys [0, pos] in one launch (plus the split merge). qkv itself is left untouched.
 inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc, void* out,
@@ -1089,6 +1139,17 @@ struct kv_cache {
     const int64_t p0 = pos;
     pos += T;
     return attn_prefill(q, K, V, out, n_q_heads, n_kv_heads, T, max_ctx, D, scale, kv_bf16, p0);
+  }
+  // The chunk form of attn_qkv: raw token-major projection in, token-major attention out;
+  // qh is [n_q_heads, T, D] scratch for the rotated queries.
+  bool prefill_qkv(void* qkv, void* bq, void* bk, void* bv, void* table, void* qh, void* out_tok, int64_t T,
+                   int64_t n_q_heads, float scale) {
+    if (T <= 0 || pos + T > max_ctx) return false;
+    if (!qkv_rope_fill(qkv, bq, bk, bv, table, qh, K, V, T, n_q_heads, n_kv_heads, D, pos, max_ctx, kv_bf16))
+      return false;
+    const int64_t p0 = pos;
+    pos += T;
+    return attn_prefill_tok(qh, K, V, out_tok, n_q_heads, n_kv_heads, T, max_ctx, D, scale, kv_bf16, p0);
   }
   void destroy() {
     if (K) release(K, 0, nullptr);

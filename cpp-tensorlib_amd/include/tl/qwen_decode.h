@@ -124,6 +124,7 @@ struct prefill_scratch {
   void *emb = nullptr, *h = nullptr, *h2 = nullptr, *qkv = nullptr, *qkvh = nullptr, *ah = nullptr,
        *at = nullptr, *gu = nullptr, *mb = nullptr, *md = nullptr;
   void* res[2] = {nullptr, nullptr};
+  void* rope = nullptr;         // (cos, sin)[T][head_dim/2] of the chunk being run
   float* emb_host = nullptr;
 };
 
@@ -145,6 +146,7 @@ struct model {
   // GEMV that consumes them). false: the reference's call sequence, one launch per op.
   bool fused = true;
   bool fused_attn = true;   // within the fused path: q/k/v epilogue + append inside the attention launch
+  bool fused_prefill = true;     // prompt chunks: one launch for split_heads + rope + kv_fill, attention writes token-major
   bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
 };
 
@@ -720,7 +722,7 @@ inline bool prefill_reserve(model& M, int64_t T) {
   if (P.T >= T) return true;
   const dims& d = M.d;
   auto A = [](int64_t n) { return hip::alloc_device(n * 4); };
-  for (void* b : {P.emb, P.h, P.h2, P.qkv, P.qkvh, P.ah, P.at, P.gu, P.mb, P.md, P.res[0], P.res[1]})
+  for (void* b : {P.emb, P.h, P.h2, P.qkv, P.qkvh, P.ah, P.at, P.gu, P.mb, P.md, P.res[0], P.res[1], P.rope})
     if (b) hip::release(b, 0, nullptr);
   P.emb = hip::alloc(T * d.hidden * 4, &P.emb_host);
   P.h = A(T * d.hidden);
@@ -734,8 +736,9 @@ inline bool prefill_reserve(model& M, int64_t T) {
   P.md = A(T * d.hidden);
   P.res[0] = A(T * d.hidden);
   P.res[1] = A(T * d.hidden);
+  P.rope = A(T * d.head_dim);
   const bool ok = P.emb && P.h && P.h2 && P.qkv && P.qkvh && P.ah && P.at && P.gu && P.mb && P.md &&
-                  P.res[0] && P.res[1];
+                  P.res[0] && P.res[1] && P.rope;
   P.T = ok ? T : 0;
   return ok;
 }
@@ -754,10 +757,17 @@ inline bool prefill_layers(model& M, int64_t T) {
   bool ok = true;
   void* x = P.emb;
   ok &= hip::rmsnorm(x, M.layers[0].an, P.h, E, d.eps, T);
+  const bool fused = M.fused_prefill;
+  if (fused) ok &= hip::rope_table_range(P.rope, HD, pos0, T, d.rope_base);   // once for all layers
   for (int64_t l = 0; l < d.n_layers; l++) {
     layer& L = M.layers[(size_t)l];
     void* ro = P.res[l & 1];
     ok &= hip::gemm_bf16_nt(P.h, L.wqkv.w, P.qkv, T, QKVN, E);
+    if (fused) {
+      // bias + rope + head-major q + cache rows in one launch; attention writes [T, Hq*D]
+      L.cache.pos = pos0;
+      ok &= L.cache.prefill_qkv(P.qkv, L.bq, L.bk, L.bv, P.rope, P.qkvh, P.at, T, d.n_q_heads, scale);
+    } else {
     // [T, q|k|v] -> head-major [Hq + 2 Hkv, T, D], bias added on the way
     ok &= hip::split_heads(P.qkv, L.bqkv, P.qkvh, T, QKVN, 0, d.n_q_heads + 2 * d.n_kv_heads, HD);
     void* kh = static_cast<char*>(P.qkvh) + QD * T * 4;
@@ -768,6 +778,7 @@ inline bool prefill_layers(model& M, int64_t T) {
     L.cache.pos = pos0;
     ok &= L.cache.prefill(P.qkvh, kh, vh, P.ah, T, d.n_q_heads, scale);
     ok &= hip::merge_heads(P.ah, P.at, T, d.n_q_heads, HD);
+    }
     ok &= hip::gemm_bf16_nt(P.at, L.wo.w, ro, T, E, QD);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, P.h2, E, d.eps, T);
     ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);

@@ -59,6 +59,7 @@ def _load():
             "tlq_set_fused": (None, [P, cint]),
             "tlq_set_fused_attn": (None, [P, cint]),
             "tlq_set_gateup_epilogue": (None, [P, cint]),
+            "tlq_set_fused_prefill": (None, [P, cint]),
             "tlq_greedy_init": (cint, [P, i64, i64]),
             "tlq_greedy_run": (i64, [P, i64]),
             "tlq_greedy_tokens": (cint, [P, i64, i64, P]),
@@ -317,6 +318,10 @@ class QwenGPU:
     def set_fused_attn(self, on):
         """Within the fused path: run the q/k/v epilogue inside the attention launch (default) or alone."""
         self.L.tlq_set_fused_attn(self.h, 1 if on else 0)
+
+    def set_fused_prefill(self, on):
+        """Prompt chunks: one launch for split_heads + rope + kv_fill and token-major attention output (default), or the reference's op sequence."""
+        self.L.tlq_set_fused_prefill(self.h, 1 if on else 0)
 
     def set_gateup_epilogue(self, on):
         """Within the fused path: swiglu as the epilogue of the gate|up GEMV (default) or as the producer of the down GEMV."""

@@ -220,6 +220,24 @@ int tlhip_qkv_rope_append_tab(void* qkv, const void* bq, const void* bk, const v
                               void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                               const void* d_pos, int64_t kv_max, const void* table, int kv_bf16);
 
+/* ---- q/k/v epilogue of a prompt chunk in one launch (no reference counterpart: the reference runs
+ * split_heads with bias, rope of q, rope of k and kv_fill as separate ops, qwen_model.h:367-382) --
+ * tlhip_rope_table_range: table[T][D/2] of float2 (cos, sin) at positions pos0 .. pos0 + T - 1, the
+ * fp64 expression of tlhip_rope; every layer and head of the chunk rotates by these.
+ * tlhip_qkv_rope_fill: qkv = the chunk's raw [T, (Hq + 2 Hkv) D] projection (token-major, left
+ * untouched); adds the biases (each may be NULL), rotates q and k by `table`; q lands head-major in
+ * qh [Hq, T, D], k and v go into cache rows pos0 .. pos0 + T - 1. Bit-identical to the separate
+ * ops. D in {64, 128}, like the cache ops. */
+int tlhip_rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, float base);
+int tlhip_qkv_rope_fill(const void* qkv, const void* bq, const void* bk, const void* bv, const void* table,
+                        void* qh, void* Kc, void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads,
+                        int64_t D, int64_t pos0, int64_t kv_max, int kv_bf16);
+/* tlhip_attn_prefill writing out token-major, [T, Hq*D] - what merge_heads (cuda.h:862-880) would
+ * make of the head-major result, so that launch is not needed. */
+int tlhip_attn_prefill_tok(const void* q, const void* K, const void* V, void* out,
+                           int64_t n_q_heads, int64_t n_kv_heads, int64_t T, int64_t kv_max,
+                           int64_t D, float scale, int kv_bf16, int64_t pos0);
+
 /* ---- decode attention with the step's prologue fused in (no reference counterpart: the
  * reference runs bias, rope, cache append and attention as separate ops, qwen_model.h:560-600) --
  * qkv = the step's raw [q (Hq*D) | k (Hkv*D) | v (Hkv*D)] projection, left untouched. Adds the

@@ -133,14 +133,18 @@ def test_bf16_decode_loop_matches_oracle(orc):
     g.close(); om.close()
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("dims,n_prompt,chunk", [(SMALL, 50, 32), (SMALL128, 130, 64), (SMALL, 40, 512)])
-def test_prefill_chunks_match_token_by_token_oracle(orc, dims, n_prompt, chunk):
+def test_prefill_chunks_match_token_by_token_oracle(orc, dims, n_prompt, chunk, fused):
     """A prompt consumed in chunks through the MFMA GEMM + causal prefill attention
     (bench/cuda/qwen_model.h:357-401) gives the logits of feeding the same tokens one at a
-    time to the oracle, and leaves caches from which decode continues identically."""
+    time to the oracle, and leaves caches from which decode continues identically. fused: the
+    chunk's q/k/v epilogue in one launch and token-major attention output, or the reference's
+    op sequence (split_heads, rope x2, kv_fill, attention, merge_heads)."""
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     om = orc.qwen_create(dims, seed=8, q4=False)
     g = qwen.QwenGPU.from_blobs(om, fmt="bf16")
+    g.set_fused_prefill(fused)
     rng = np.random.default_rng(9)
     prompt = rng.integers(0, dims["vocab"], n_prompt)
     for pos, tok in enumerate(prompt):

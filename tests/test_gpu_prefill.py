@@ -205,6 +205,63 @@ def test_attn_prefill_bf16_cache(lib, orc, D, valu):
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
+@pytest.mark.parametrize("kv_bf16", [False, True])
+@pytest.mark.parametrize("D,Hq,Hkv,T,pos0", [(128, 28, 4, 64, 0), (64, 14, 2, 100, 7), (128, 4, 2, 1, 300), (64, 3, 1, 5, 2)])
+def test_qkv_rope_fill_equals_the_separate_ops(lib, orc, D, Hq, Hkv, T, pos0, kv_bf16):
+    """tlhip_rope_table_range + tlhip_qkv_rope_fill against split_heads (with bias) + rope(q) +
+    rope(k) + kv_fill: rotated queries and both caches bit for bit (f32 and bf16 caches), cache rows
+    outside [pos0, pos0 + T) untouched."""
+    print("case qkv_rope_fill", D, Hq, Hkv, T, pos0, kv_bf16, flush=True)
+    base, kv_max = 1e6, pos0 + T + 3
+    qd, kvd = Hq * D, Hkv * D
+    ld = qd + 2 * kvd
+    qkv = orc.normal(T * ld, 61).reshape(T, ld)
+    bias = orc.normal(ld, 62, 0.0, 0.1)
+    cdt = np.uint16 if kv_bf16 else np.float32
+    fill = np.full(Hkv * kv_max * D, 0x7fc0 if kv_bf16 else np.nan, cdt)
+    dqkv, db = lib.to_device(qkv), lib.to_device(bias)
+    # the separate ops
+    dh = lib.empty((Hq + 2 * Hkv, T, D))
+    lib.split_heads(dqkv, db, dh, T, ld, 0, Hq + 2 * Hkv, D)
+    lib.rope(dh, dh, Hq * T, T, D, pos0, base)
+    c = lib.c
+    kh, vh = dh.ptr + qd * T * 4, dh.ptr + (qd + kvd) * T * 4
+    lib._chk(c.tlhip_rope(kh, kh, Hkv * T, T, D, pos0, base, None))
+    K1, V1 = lib.to_device(fill), lib.to_device(fill)
+    lib._chk(c.tlhip_kv_fill(K1.ptr, V1.ptr, kh, vh, T, kv_max, Hkv, D, int(kv_bf16), pos0))
+    want_q = dh.numpy().reshape(-1)[:qd * T]
+    # the fused launch
+    tab, qh = lib.empty(T * D), lib.to_device(np.full(qd * T, np.nan, np.float32))
+    K2, V2 = lib.to_device(fill), lib.to_device(fill)
+    lib.rope_table_range(tab, D, pos0, T, base)
+    lib._chk(c.tlhip_qkv_rope_fill(dqkv.ptr, db.ptr, db.ptr + qd * 4, db.ptr + (qd + kvd) * 4, tab.ptr, qh.ptr,
+                                   K2.ptr, V2.ptr, T, Hq, Hkv, D, pos0, kv_max, int(kv_bf16)))
+    assert np.array_equal(qh.numpy(), want_q)
+    assert np.array_equal(K2.numpy(cdt).view(np.uint16 if kv_bf16 else np.uint32),
+                          K1.numpy(cdt).view(np.uint16 if kv_bf16 else np.uint32))
+    assert np.array_equal(V2.numpy(cdt).view(np.uint16 if kv_bf16 else np.uint32),
+                          V1.numpy(cdt).view(np.uint16 if kv_bf16 else np.uint32))
+    assert np.array_equal(dqkv.numpy().reshape(T, ld), qkv)        # the projection is left untouched
+    for b in (dqkv, db, dh, K1, V1, K2, V2, tab, qh):
+        b.free()
+
+
+def test_attn_prefill_tok_is_the_merged_layout(lib, orc):
+    """tlhip_attn_prefill_tok writes [T, Hq*D]: exactly merge_heads of tlhip_attn_prefill's result."""
+    D, Hq, Hkv, T, pos0 = 128, 6, 2, 75, 11
+    kv_max = pos0 + T
+    q = orc.normal(Hq * T * D, 71).reshape(Hq, T, D)
+    K = orc.normal(Hkv * kv_max * D, 72).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 73).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    head_major = _prefill(lib, q, K, V, scale, pos0)
+    dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((T, Hq * D))
+    lib.attn_prefill_tok(dq, dk, dv, do, Hq, Hkv, T, kv_max, D, scale, False, pos0)
+    assert np.array_equal(do.numpy(), head_major.transpose(1, 0, 2).reshape(T, Hq * D))
+    for b in (dq, dk, dv, do):
+        b.free()
+
+
 def test_prefill_chunk_pipeline(lib, orc):
     """The attention half of a prompt chunk as the reference harness runs it
     (bench/cuda/qwen_model.h:357-383): fused q|k|v GEMM -> split_heads (+bias) -> rope at pos0
