@@ -87,15 +87,49 @@ __device__ __forceinline__ float sub_rn(float a, float b) {
   return a - b;
 }
 
+// Cross-lane exchanges without the LDS crossbar (gfx950).
+//   swap32(x, y): lanes 0-31 get (x.lo, x.hi), lanes 32-63 get (y.lo, y.hi) as (first, second):
+//   v_permlane32_swap trades x's upper half with y's lower half.
+//   swap16(x, y): the same per pair of 16-lane rows (v_permlane16_swap).
+// With x == y == v, first + second is v[l] + v[l ^ 32] (resp. ^ 16) in every lane.
+struct LanePair { float first, second; };
+__device__ __forceinline__ LanePair swap32(float x, float y) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+  return LanePair{__uint_as_float(r[0]), __uint_as_float(r[1])};
+}
+__device__ __forceinline__ LanePair swap16(float x, float y) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+  return LanePair{__uint_as_float(r[0]), __uint_as_float(r[1])};
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_read(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Butterfly over the wavefront: the pairings of xor 32, 16, 8, 4, 2, 1 in that order (row_ror n
+// reads the xor-n partner's value once the values have period 2n within a row), so the sums
+// are those of the shuffle form bit for bit.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  LanePair p = swap32(v, v);
+  v = p.first + p.second;
+  p = swap16(v, v);
+  v = p.first + p.second;
+  v += dpp_read<0x128>(v);   // row_ror:8
+  v += dpp_read<0x124>(v);   // row_ror:4
+  v += dpp_read<0x122>(v);   // row_ror:2
+  v += dpp_read<0x121>(v);   // row_ror:1
   return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+  LanePair p = swap32(v, v);
+  v = fmaxf(p.first, p.second);
+  p = swap16(v, v);
+  v = fmaxf(p.first, p.second);
+  v = fmaxf(v, dpp_read<0x128>(v));
+  v = fmaxf(v, dpp_read<0x124>(v));
+  v = fmaxf(v, dpp_read<0x122>(v));
+  v = fmaxf(v, dpp_read<0x121>(v));
   return v;
 }
 

@@ -152,12 +152,22 @@ __device__ __forceinline__ float dpp_add_f32(float v) {
 // group on DPP. Returns, in every lane, the total of row (lane * R) >> 6.
 template <int N, int M, int R>
 __device__ __forceinline__ void halve_rows(float (&a)[R], int lane) {  // N live values -> N/2
-  const bool up = (lane & M) != 0;
+  if constexpr (M == 32 || M == 16) {
+    // one v_permlane swap hands the lower lanes both halves' a[i] and the upper lanes both
+    // halves' a[i + N/2]: the same two operands the shuffle form adds
 #pragma unroll
-  for (int i = 0; i < N / 2; i++) {
-    const float keep = up ? a[i + N / 2] : a[i];
-    const float send = up ? a[i] : a[i + N / 2];
-    a[i] = keep + __shfl_xor(send, M, kWave);
+    for (int i = 0; i < N / 2; i++) {
+      const LanePair p = M == 32 ? swap32(a[i], a[i + N / 2]) : swap16(a[i], a[i + N / 2]);
+      a[i] = p.first + p.second;
+    }
+  } else {
+    const bool up = (lane & M) != 0;
+#pragma unroll
+    for (int i = 0; i < N / 2; i++) {
+      const float keep = up ? a[i + N / 2] : a[i];
+      const float send = up ? a[i] : a[i + N / 2];
+      a[i] = keep + __shfl_xor(send, M, kWave);
+    }
   }
 }
 
@@ -169,8 +179,8 @@ __device__ __forceinline__ float wave_sum_rows(float (&a)[R], int lane) {
   if constexpr (R == 2) { halve_rows<2, 32>(a, lane); }
   float v = a[0];
   // lanes that differ only in bits below the last halving mask share a row
-  if (R <= 1) v += __shfl_xor(v, 32, kWave);
-  if (R <= 2) v += __shfl_xor(v, 16, kWave);
+  if (R <= 1) { const LanePair p = swap32(v, v); v = p.first + p.second; }
+  if (R <= 2) { const LanePair p = swap16(v, v); v = p.first + p.second; }
   v = dpp_add_f32<0xB1>(v);                 // quad_perm [1,0,3,2]
   v = dpp_add_f32<0x4E>(v);                 // quad_perm [2,3,0,1]
   v = dpp_add_f32<0x141>(v);                // row_half_mirror: the two quads of 8 lanes
