@@ -404,12 +404,17 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     l[g] = wave_sum(l[g]);
 #pragma unroll
     for (int v = 0; v < NV; v++) {
-#pragma unroll
-      for (int msk = 16; msk < 64; msk <<= 1) {
-        acc[g][v].x += __shfl_xor(acc[g][v].x, msk, kWave);
-        acc[g][v].y += __shfl_xor(acc[g][v].y, msk, kWave);
-        acc[g][v].z += __shfl_xor(acc[g][v].z, msk, kWave);
-        acc[g][v].w += __shfl_xor(acc[g][v].w, msk, kWave);
+      {   // + the value 16 lanes away, then + the value 32 lanes away
+        const auto both = [](float a) {
+          LanePair p = swap16(a, a);
+          a = p.first + p.second;
+          p = swap32(a, a);
+          return p.first + p.second;
+        };
+        acc[g][v].x = both(acc[g][v].x);
+        acc[g][v].y = both(acc[g][v].y);
+        acc[g][v].z = both(acc[g][v].z);
+        acc[g][v].w = both(acc[g][v].w);
       }
       if constexpr (PRE) {   // this wavefront's rows are complete: normalise and store
         if (slot == 0 && g < ng) {

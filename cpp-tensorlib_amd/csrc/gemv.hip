@@ -305,8 +305,14 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       if (live) xs[((u / LPR) * J + j) * LPR + (u & (LPR - 1))] = Fmt::stage(v);
       if (Fmt::kScaled) {
         float sx = (v.x + v.y) + (v.z + v.w);
+        if constexpr (J == 8) {   // the unit's 8 adjacent lanes, on DPP: quads, then the other quad of the 8
+          sx = dpp_add_f32<0xB1>(sx);
+          sx = dpp_add_f32<0x4E>(sx);
+          sx = dpp_add_f32<0x141>(sx);
+        } else {
 #pragma unroll
-        for (int msk = J / 2; msk >= 1; msk >>= 1) sx += __shfl_xor(sx, msk, kWave);
+          for (int msk = J / 2; msk >= 1; msk >>= 1) sx += __shfl_xor(sx, msk, kWave);
+        }
         if (live && j == 0) xsum[u] = -8.0f * sx;  // sum_k (nib_k-8) x_k = sum nib_k x_k - 8 sum x_k
       }
     }
@@ -364,7 +370,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       if (KW == 1) {
         if constexpr (kPair) {
           // the up row's total sits half a wavefront (64-lane form) or R/2 lanes (16-lane form) away
-          const float up = LPR == 64 ? __shfl_xor(v, 32, kWave) : __shfl_down(v, R / 2, kWave);
+          const float up = LPR == 64 ? swap32(v, v).second : __shfl_down(v, R / 2, kWave);   // .second: the upper half's value in the lower lanes
           if (writer && r < R / 2 && row0 + r < N / 2) y[row0 + r] = gated(v, up);
         } else {
           if (writer && row0 + r < N) y[row0 + r] = v;
