@@ -74,6 +74,8 @@ SIGNATURES = {
     "tlhip_argmax": (cint, [P, i64, C.POINTER(i64)]),
     "tlhip_argmax_async": (cint, [P, i64, P]),
     "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
+    "tlhip_gemm_bf16_nt_parts": (cint, [P, P, P, i64, i64, i64, i64, P]),
+    "tlhip_rmsnorm_res_parts": (cint, [P, P, i64, P, P, P, i64, f32, i64]),
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
     "tlhip_qkv_rope_append": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
@@ -296,6 +298,16 @@ class TlHip:
 
     def gemm_bf16_nt(self, A, W, out, M, N, K):
         self._chk(self.c.tlhip_gemm_bf16_nt(A.ptr, W.ptr, out.ptr, M, N, K))
+
+    def gemm_bf16_nt_parts(self, A, W, parts, M, N, K):
+        """The product as its K-split parts in `parts`; returns how many there are."""
+        n = C.c_int(0)
+        self._chk(self.c.tlhip_gemm_bf16_nt_parts(A.ptr, W.ptr, parts.ptr, parts.nbytes, M, N, K, C.byref(n)))
+        return n.value
+
+    def rmsnorm_res_parts(self, x, parts, n_parts, w, xout, hout, n, eps, rows=1):
+        self._chk(self.c.tlhip_rmsnorm_res_parts(x.ptr, parts.ptr, n_parts, w.ptr, xout.ptr, hout.ptr,
+                                                 n, eps, rows))
 
     def split_heads(self, src, bias, dst, T, ld, off, H, D):
         self._chk(self.c.tlhip_split_heads(src.ptr, bias.ptr if bias is not None else None, dst.ptr,

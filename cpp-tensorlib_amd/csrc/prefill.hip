@@ -187,8 +187,13 @@ using namespace tlhip;
 
 extern "C" {
 
-int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K) {
+// parts != nullptr: the K-split parts are the result - C is then `parts`, [S][M][N], no part sum is
+// launched and *S_out says how many there are (1: the plain product); one piece, so that the
+// layout is uniform.
+static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K,
+                             size_t parts_bytes, int* S_out) {
   TLHIP_REQUIRE_READY();
+  const bool want_parts = S_out != nullptr;
   if (!A || !W || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt: null pointer");
   // the reference's gate: K a multiple of 8
   if ((K % 8) != 0 || M <= 0 || N <= 0 || K <= 0)
@@ -219,12 +224,14 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
     int64_t S = (slots + tiles / 2) / tiles;
     if (S > 16) S = 16;
     while (S > 1 && K / S < 256) S--;
+    if (want_parts)   // the caller's buffer bounds the parts
+      while (S > 1 && (size_t)S * M * N * sizeof(float) > parts_bytes) S--;
     return (int)S;
   };
   if (M > 64) {
     const int64_t tm = cdiv(M, 128), tn = cdiv(N, 256), tiles = tm * tn;
     const int64_t cols_per_round = slots / tm;            // whole tile columns in one round
-    if (tiles <= slots || cols_per_round == 0 || !can_split) {
+    if (tiles <= slots || cols_per_round == 0 || !can_split || want_parts) {
       pieces[npieces++] = Piece{0, N, pick_S(tiles), 0};
     } else {
       const int64_t main_tn = tn / cols_per_round * cols_per_round;   // whole rounds
@@ -249,7 +256,10 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
       kchunk = (int)(cdiv(cdiv(K, S), kBK) * kBK);
       S = (int)cdiv(K, kchunk);
     }
-    if (S > 1) {
+    if (want_parts) {
+      *S_out = S;             // one piece: dst is the caller's parts, [S][M][N]
+      if (S == 1) kchunk = (int)K;
+    } else if (S > 1) {
       dst = static_cast<float*>(scratch((size_t)S * M * P.n * sizeof(float)));
       if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
       ldc = (int)P.n;
@@ -269,7 +279,7 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
       default: TLHIP_GEMM(1, 1); break;
     }
 #undef TLHIP_GEMM
-    if (S > 1) {
+    if (S > 1 && !want_parts) {
       const size_t total4 = (size_t)M * P.n / 4;
       splitk_sum_kernel<<<dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, c.stream>>>(
           reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + P.n0), (int)M, (int)(P.n / 4),
@@ -277,6 +287,20 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
     }
   }
   TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
+}
+
+int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K) {
+  return gemm_bf16_nt_impl(A, W, C, M, N, K, 0, nullptr);
+}
+
+int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t parts_bytes, int64_t M,
+                             int64_t N, int64_t K, int* n_parts) {
+  if (!n_parts) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: null n_parts");
+  if (M > 0 && N > 0 && parts_bytes < (int64_t)(M * N * sizeof(float)))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: the buffer must hold at least one [M, N] part");
+  if (parts && !aligned16(parts)) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: parts must be 16-byte aligned");
+  *n_parts = 0;
+  return gemm_bf16_nt_impl(A, W, parts, M, N, K, (size_t)parts_bytes, n_parts);
 }
 
 }  // extern "C"

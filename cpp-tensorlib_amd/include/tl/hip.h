@@ -106,6 +106,10 @@ struct api {
   int (*argmax)(const void*, int64_t, int64_t*) = nullptr;
   int (*argmax_async)(const void*, int64_t, void*) = nullptr;
   int (*gemm_bf16_nt)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemm_bf16_nt_parts)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
+                            int*) = nullptr;
+  int (*rmsnorm_res_parts)(const void*, const void*, int64_t, const void*, void*, void*, int64_t, float,
+                           int64_t) = nullptr;
   int (*split_heads)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
                      int64_t) = nullptr;
   int (*merge_heads)(const void*, void*, int64_t, int64_t, int64_t) = nullptr;
@@ -227,6 +231,8 @@ struct context {
               bind(f.swiglu, "tlhip_swiglu") && bind(f.argmax, "tlhip_argmax") &&
               bind(f.argmax_async, "tlhip_argmax_async") &&
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
+              bind(f.gemm_bf16_nt_parts, "tlhip_gemm_bf16_nt_parts") &&
+              bind(f.rmsnorm_res_parts, "tlhip_rmsnorm_res_parts") &&
               bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
               bind(f.qkv_rope_append, "tlhip_qkv_rope_append") &&
               bind(f.rope_dpos, "tlhip_rope_dpos") && bind(f.incr_u32, "tlhip_incr_u32") &&
@@ -553,6 +559,17 @@ inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int6
   return detail::done_(c, c.f.gemm_bf16_nt(a, B, out, m, n, k));
 }
 
+// The product left as its K-split parts ([*n_parts][m][n] in `parts`), for rmsnorm_res_parts.
+inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_bytes, int64_t m, int64_t n,
+                               int64_t k, int* n_parts) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(parts);
+  return detail::done_(c, c.f.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
+}
+
 inline bool attn_decode(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
                         int64_t ctx, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false) {
   auto& c = context::get();
@@ -633,6 +650,19 @@ inline bool rmsnorm_res(void* x, void* delta, void* w, void* xout, void* hout, i
   c.device_write_(xout);
   c.device_write_(hout);
   return detail::done_(c, c.f.rmsnorm_res(x, delta, w, xout, hout, n, eps, rows));
+}
+
+// rmsnorm_res with delta = parts[0] + ... + parts[n_parts-1], rows * n floats apart.
+inline bool rmsnorm_res_parts(void* x, void* parts, int64_t n_parts, void* w, void* xout, void* hout,
+                              int64_t n, float eps, int64_t rows = 1) {
+  auto& c = context::get();
+  if (!c.ready || n <= 0 || rows <= 0 || n_parts <= 0) return false;
+  c.device_read_(x);
+  c.device_read_(parts);
+  c.device_read_(w);
+  c.device_write_(xout);
+  c.device_write_(hout);
+  return detail::done_(c, c.f.rmsnorm_res_parts(x, parts, n_parts, w, xout, hout, n, eps, rows));
 }
 
 inline bool swiglu(void* gu, void* out, int64_t ff, int64_t rows = 1) {

@@ -125,6 +125,8 @@ struct prefill_scratch {
        *at = nullptr, *gu = nullptr, *mb = nullptr, *md = nullptr;
   void* res[2] = {nullptr, nullptr};
   void* rope = nullptr;         // (cos, sin)[T][head_dim/2] of the chunk being run
+  void* parts = nullptr;        // K-split parts of the o-proj / down products, read by the residual norm
+  int64_t parts_bytes = 0;
   float* emb_host = nullptr;
 };
 
@@ -722,7 +724,7 @@ inline bool prefill_reserve(model& M, int64_t T) {
   if (P.T >= T) return true;
   const dims& d = M.d;
   auto A = [](int64_t n) { return hip::alloc_device(n * 4); };
-  for (void* b : {P.emb, P.h, P.h2, P.qkv, P.qkvh, P.ah, P.at, P.gu, P.mb, P.md, P.res[0], P.res[1], P.rope})
+  for (void* b : {P.emb, P.h, P.h2, P.qkv, P.qkvh, P.ah, P.at, P.gu, P.mb, P.md, P.res[0], P.res[1], P.rope, P.parts})
     if (b) hip::release(b, 0, nullptr);
   P.emb = hip::alloc(T * d.hidden * 4, &P.emb_host);
   P.h = A(T * d.hidden);
@@ -737,8 +739,10 @@ inline bool prefill_reserve(model& M, int64_t T) {
   P.res[0] = A(T * d.hidden);
   P.res[1] = A(T * d.hidden);
   P.rope = A(T * d.head_dim);
+  P.parts_bytes = 16 * T * d.hidden * 4;   // the GEMM splits K at most 16 ways
+  P.parts = hip::alloc_device(P.parts_bytes);
   const bool ok = P.emb && P.h && P.h2 && P.qkv && P.qkvh && P.ah && P.at && P.gu && P.mb && P.md &&
-                  P.res[0] && P.res[1] && P.rope;
+                  P.res[0] && P.res[1] && P.rope && P.parts;
   P.T = ok ? T : 0;
   return ok;
 }
@@ -779,13 +783,24 @@ inline bool prefill_layers(model& M, int64_t T) {
     ok &= L.cache.prefill(P.qkvh, kh, vh, P.ah, T, d.n_q_heads, scale);
     ok &= hip::merge_heads(P.ah, P.at, T, d.n_q_heads, HD);
     }
+    void* nextw = (l + 1 < d.n_layers) ? M.layers[(size_t)l + 1].an : M.onorm;
+    if (fused) {
+      // o-proj and down leave their K-split parts; the residual norm adds them up as it reads
+      int np = 0;
+      ok &= hip::gemm_bf16_nt_parts(P.at, L.wo.w, P.parts, P.parts_bytes, T, E, QD, &np);
+      ok = ok && hip::rmsnorm_res_parts(x, P.parts, np, L.fn, ro, P.h2, E, d.eps, T);
+      ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);
+      ok &= hip::swiglu(P.gu, P.mb, d.ff, T);
+      ok &= hip::gemm_bf16_nt_parts(P.mb, L.wd.w, P.parts, P.parts_bytes, T, E, d.ff, &np);
+      ok = ok && hip::rmsnorm_res_parts(ro, P.parts, np, nextw, ro, P.h, E, d.eps, T);
+    } else {
     ok &= hip::gemm_bf16_nt(P.at, L.wo.w, ro, T, E, QD);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, P.h2, E, d.eps, T);
     ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);
     ok &= hip::swiglu(P.gu, P.mb, d.ff, T);
     ok &= hip::gemm_bf16_nt(P.mb, L.wd.w, P.md, T, E, d.ff);
-    void* nextw = (l + 1 < d.n_layers) ? M.layers[(size_t)l + 1].an : M.onorm;
     ok &= hip::rmsnorm_res(ro, P.md, nextw, ro, P.h, E, d.eps, T);
+    }
     x = ro;
   }
   return ok;

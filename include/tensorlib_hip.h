@@ -170,6 +170,10 @@ int tlhip_rmsnorm(const void* x, const void* w, void* out, int64_t n, float eps,
 /* xout = x + delta; hout = rmsnorm(xout)*w.  xout may alias x.  cuda.h:1229-1252 */
 int tlhip_rmsnorm_res(const void* x, const void* delta, const void* w, void* xout, void* hout,
                       int64_t n, float eps, int64_t rows);
+/* tlhip_rmsnorm_res with delta = parts[0] + ... + parts[S-1] (ascending, each [rows][n], rows*n
+ * floats apart): the K-split parts of tlhip_gemm_bf16_nt_parts. xout must not be the parts. */
+int tlhip_rmsnorm_res_parts(const void* x, const void* parts, int64_t S, const void* w, void* xout,
+                            void* hout, int64_t n, float eps, int64_t rows);
 /* out[rows,ff] = silu(gu[:, :ff]) * gu[:, ff:], gu [rows,2*ff].  cuda.h:1304-1319 */
 int tlhip_swiglu(const void* gu, void* out, int64_t ff, int64_t rows);
 /* index of the maximum of in[0..n), ties to the smallest index; blocks until the
@@ -320,6 +324,13 @@ int tlhip_gemv_bf16_row_rmsnorm_gateup(const void* x, const void* delta, const v
 /* ---- prefill ------------------------------------------------------------------ */
 /* C[M,N] = A[M,K] f32 . W[N,K]^T bf16, fp32 accumulate; K % 8 == 0.  cuda.h:787-841 */
 int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K);
+/* The same product left as its K-split parts: parts = [*n_parts][M][N] f32, dense, in a buffer
+ * of the caller's (parts_bytes >= M*N*4; it also bounds the split), no part-sum launch. The
+ * product is parts[0] + parts[1] + ... in that order - exactly what tlhip_gemm_bf16_nt stores
+ * when it splits - and tlhip_rmsnorm_res_parts forms it while it reads. For the products whose
+ * consumer is the residual norm (o-proj and down, qwen_model.h:383, 390: dot then add). */
+int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t parts_bytes, int64_t M,
+                             int64_t N, int64_t K, int* n_parts);
 /* [T,ld] token-major (+ optional bias [H*D]) -> [H,T,D]; `off` selects a column
  * block of a fused projection.  cuda.h:846-864 */
 int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, int64_t ld,

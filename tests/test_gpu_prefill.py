@@ -100,6 +100,69 @@ def test_gemm_bf16_nt_random_shapes_exact(lib, orc):
         assert np.array_equal(got.astype(np.float64), want), (M, N, K)
 
 
+@pytest.mark.parametrize("M,N,K,room", [
+    (512, 3584, 3584, 16),    # o-proj of the 7B shape: 56 tiles, 9 parts
+    (512, 3584, 18944, 16),   # down
+    (512, 3584, 3584, 4),     # the caller's buffer holds 4 parts: the split stops there
+    (512, 3584, 3584, 1),     # room for the product only: one part
+    (200, 896, 4864, 16),     # 0.5B down, ragged M
+    (33, 896, 896, 16),       # short prompt: 64-row tiles
+    (257, 130, 264, 16),      # N % 4 != 0: never split
+])
+def test_gemm_parts_then_residual_norm_is_gemm_then_residual_norm(lib, orc, M, N, K, room):
+    """The product left as its K-split parts and summed by the residual norm while it reads them
+    is, bit for bit, the product summed by the GEMM's own part-sum launch and then normalised:
+    same parts, same order of addition (when the caller's buffer has room for the split the plain
+    GEMM picks - 16 parts always is). Checked on the residual stream and on the normalised rows."""
+    print("case gemm parts", M, N, K, room, flush=True)
+    A = orc.normal(M * K, 41).reshape(M, K)
+    Wb = orc.to_bf16(orc.normal(N * K, 42, std=0.02)).reshape(N, K)
+    res = orc.normal(M * N, 43).reshape(M, N)
+    nw = orc.normal(N, 44) + 1.0
+    da, dw, dres, dnw = (lib.to_device(a) for a in (A, Wb, res, nw))
+    dc, x1, h1, x2, h2 = (lib.empty((M, N)) for _ in range(5))
+    parts = lib.empty((room, M, N))
+    lib.gemm_bf16_nt(da, dw, dc, M, N, K)
+    lib.rmsnorm_res(dc, dres, dnw, x1, h1, N, 1e-6, M)
+    n = lib.gemm_bf16_nt_parts(da, dw, parts, M, N, K)
+    assert 1 <= n <= room
+    if room == 16 and N % 4 == 0 and M * N < 4 * 512 * 3584:
+        assert n > 1          # these shapes do split: the test is not vacuous
+    if N % 4 != 0:
+        assert n == 1
+    lib.rmsnorm_res_parts(dres, parts, n, dnw, x2, h2, N, 1e-6, M)
+    if room == 16:            # room for the split the plain GEMM picks: the same parts
+        assert np.array_equal(x1.numpy(), x2.numpy())
+        assert np.array_equal(h1.numpy(), h2.numpy())
+    else:                     # fewer, longer parts: the same product to summation-order noise
+        assert allclose(x2.numpy(), x1.numpy(), RTOL, ATOL)
+        assert allclose(h2.numpy(), h1.numpy(), RTOL, ATOL)
+    x1n, h1n = x2.numpy(), h2.numpy()
+    # and the parts do add up to the product the oracle computes
+    p = parts.numpy()[:n].astype(np.float64).sum(axis=0)
+    want = orc.gemm_bf16_nt(A[:8], Wb)
+    assert allclose(p[:8].astype(np.float32), want, RTOL, ATOL)
+    # in place on the residual stream, as the model's second norm of a layer does
+    lib.rmsnorm_res_parts(dres, parts, n, dnw, dres, h2, N, 1e-6, M)
+    assert np.array_equal(dres.numpy(), x1n) and np.array_equal(h2.numpy(), h1n)
+    for b in (da, dw, dres, dnw, dc, x1, h1, x2, h2, parts):
+        b.free()
+
+
+def test_gemm_parts_rejects(lib):
+    a, w = lib.empty((64, 64)), lib.empty((64, 32))
+    small = lib.empty(16)
+    with pytest.raises(RuntimeError):
+        lib.gemm_bf16_nt_parts(a, w, small, 64, 64, 64)          # no room for one [M, N] part
+    x = lib.empty((64, 64))
+    with pytest.raises(RuntimeError):
+        lib.rmsnorm_res_parts(a, x, 0, w, small, small, 64, 1e-6, 64)   # S = 0
+    with pytest.raises(RuntimeError):
+        lib.rmsnorm_res_parts(a, x, 1, w, x, small, 64, 1e-6, 64)       # xout is the parts
+    for b in (a, w, small, x):
+        b.free()
+
+
 def test_gemm_bf16_nt_row_equals_gemv(lib, orc):
     """Row m of the GEMM and the decode GEMV over the same [N,K] bf16 weights agree to
     summation-order noise."""
