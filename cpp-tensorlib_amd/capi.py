@@ -74,6 +74,7 @@ SIGNATURES = {
     "tlhip_argmax": (cint, [P, i64, C.POINTER(i64)]),
     "tlhip_argmax_async": (cint, [P, i64, P]),
     "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
+    "tlhip_gemm_bf16_nt_swiglu": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_parts": (cint, [P, P, P, i64, i64, i64, i64, P]),
     "tlhip_rmsnorm_res_parts": (cint, [P, P, i64, P, P, P, i64, f32, i64]),
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
@@ -298,6 +299,9 @@ class TlHip:
 
     def gemm_bf16_nt(self, A, W, out, M, N, K):
         self._chk(self.c.tlhip_gemm_bf16_nt(A.ptr, W.ptr, out.ptr, M, N, K))
+
+    def gemm_bf16_nt_swiglu(self, A, W, act, M, ff, K):
+        self._chk(self.c.tlhip_gemm_bf16_nt_swiglu(A.ptr, W.ptr, act.ptr, M, ff, K))
 
     def gemm_bf16_nt_parts(self, A, W, parts, M, N, K):
         """The product as its K-split parts in `parts`; returns how many there are."""

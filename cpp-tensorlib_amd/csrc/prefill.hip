@@ -40,11 +40,21 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elemen
 // writes its partial product to C + y*M*N (a scratch area); splitk_sum_kernel adds
 // the parts in a fixed order. ldc = row stride of C (N for a scratch part; the full
 // width when the launch covers a column range of a wider result).
-template <int TM, int TN, int WM = 2, int WN = 2>
+//
+// GU = true: W is a fused [gate rows | up rows] matrix ([2*ff, K], qwen_model.h:194-199) and the
+// result is the gated activation act[m][f] = swiglu(A.gate_f, A.up_f), never the two products.
+// Each wavefront's 32*TN tile columns are then 16*TN gate features followed by the SAME features'
+// up rows (`ff` rows further down in W), so a lane holds both accumulators of a feature
+// (MFMA tile j and j + TN/2) and the epilogue gates in registers. N counts features, n0 still
+// counts tile columns (two per feature). Under split-K the raw parts are stored in that tile
+// column order ([M][tiles * BN]) and splitk_sum_swiglu_kernel gates after the sum.
+template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false>
 __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
-                                                           int K, int kchunk, int ldc) {
+                                                           int K, int kchunk, int ldc, int ff) {
+  static_assert(!GU || TN % 2 == 0, "gate and up accumulators of a feature must share a lane");
+  constexpr int WT = 32 * TN, HW = WT / 2;      // a wavefront's tile columns; GU: gate half, up half
   constexpr int NT = 64 * WM * WN;              // threads: WM x WN wavefronts
   constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
   constexpr int A_LOADS = BM * kBK / 4 / NT;    // float4 per thread per slab
@@ -88,9 +98,16 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
-      const int gn = n0 + row, gk = k0 + c8 * 8;
-      rb[i] = (gn < N && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
-                                 : make_uint4(0u, 0u, 0u, 0u);
+      const int gk = k0 + c8 * 8;
+      int gn = n0 + row;
+      bool in = gn < N;
+      if (GU) {
+        const int j = row % WT, f = (n0 >> 1) + (row / WT) * HW + j % HW;
+        in = f < N;
+        gn = f + (j >= HW ? ff : 0);
+      }
+      rb[i] = (in && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
+                                : make_uint4(0u, 0u, 0u, 0u);
     }
   };
   auto split3 = [](float a, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
@@ -151,12 +168,29 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
   }
 
   // acc[v] of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32x32 tile
+  if (GU && gridDim.y == 1) {
+    // act = (g * sigmoid(g)) * u, the arithmetic of swiglu_kernel (array.h:2435-2439)
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN / 2; j++) {
+        const int f = (n0 >> 1) + wn * HW + j * 32 + (lane & 31);
+        if (f >= N) continue;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const float g = acc[i][j][v], sg = 1.0f / (1.0f + expf(-g));
+          if (gm < M) C[(size_t)gm * ldc + f] = (g * sg) * acc[i][j + TN / 2][v];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       const int gn = n0 + wn * 32 * TN + j * 32 + (lane & 31);
-      if (gn >= N) continue;
+      if (!GU && gn >= N) continue;   // GU parts are whole tiles wide
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
@@ -181,17 +215,45 @@ __global__ __launch_bounds__(256) void splitk_sum_kernel(const float4* __restric
   C[m * ldc4 + (i - m * n4)] = a;
 }
 
+// The same for the parts of a GU launch: out[m][f] = swiglu(sum_s gate part, sum_s up part). Parts are
+// [M][nv] in tile column order: per wavefront strip of 2 * HW columns, HW gate features then their
+// up values. pf4 = features / 4 of this piece, ldc4 = row stride of out in float4s.
+__global__ __launch_bounds__(256) void splitk_sum_swiglu_kernel(const float4* __restrict__ part,
+                                                                float4* __restrict__ out, int M, int pf4,
+                                                                int nv4, int ldc4, int S, int hw4) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)M * pf4) return;
+  const size_t m = i / pf4;
+  const int f4 = (int)(i - m * pf4);
+  const size_t gi = m * nv4 + (size_t)(f4 / hw4) * 2 * hw4 + f4 % hw4, total = (size_t)M * nv4;
+  float4 g = part[gi], u = part[gi + hw4];
+  for (int sidx = 1; sidx < S; sidx++) {
+    const float4 a = part[sidx * total + gi], b = part[sidx * total + gi + hw4];
+    g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+    u.x += b.x; u.y += b.y; u.z += b.z; u.w += b.w;
+  }
+  float4 o;
+  o.x = (g.x * (1.0f / (1.0f + expf(-g.x)))) * u.x;
+  o.y = (g.y * (1.0f / (1.0f + expf(-g.y)))) * u.y;
+  o.z = (g.z * (1.0f / (1.0f + expf(-g.z)))) * u.z;
+  o.w = (g.w * (1.0f / (1.0f + expf(-g.w)))) * u.w;
+  out[m * ldc4 + f4] = o;
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;
 
 extern "C" {
 
-// parts != nullptr: the K-split parts are the result - C is then `parts`, [S][M][N], no part sum is
-// launched and *S_out says how many there are (1: the plain product); one piece, so that the
-// layout is uniform.
+// Three forms of one launcher.
+//   plain: C[M][N] is the product.
+//   parts (S_out != nullptr): the K-split parts are the result - C is then the caller's buffer,
+//     [S][M][N], no part sum is launched and *S_out says how many there are (1: the plain
+//     product); one piece, so that the layout is uniform.
+//   gu: W = [gate rows | up rows], N = features (rows of each), C[M][N] = the gated activation.
 static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K,
-                             size_t parts_bytes, int* S_out) {
+                             size_t parts_bytes, int* S_out, bool gu) {
   TLHIP_REQUIRE_READY();
   const bool want_parts = S_out != nullptr;
   if (!A || !W || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt: null pointer");
@@ -213,10 +275,13 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
   //     the slots; parts go to scratch and are summed in a fixed order (no atomics);
   //   * more tiles than slots: the columns that make whole rounds run with full K, the
   //     remaining columns (less than one round of tiles) are split over K the same way.
+  // gu: a tile column of bn is bn / 2 features wide (gate and up of each), so all widths below
+  // are in units of N - columns, or features.
   auto cdiv = [](int64_t a, int64_t b) { return (a + b - 1) / b; };
   const int64_t slots = (int64_t)c.cus * 2;
+  const int per = gu ? 2 : 1;                             // tile columns per unit of N
   const bool can_split = (N % 4) == 0 && aligned16(C);   // the part sum works on float4s
-  struct Piece { int64_t n0, n; int S; int variant; };    // columns [n0, n0 + n)
+  struct Piece { int64_t n0, n; int S; int variant; };    // columns (features) [n0, n0 + n)
   Piece pieces[2];
   int npieces = 0;
   auto pick_S = [&](int64_t tiles) {   // K splits that bring `tiles` blocks up to the slots
@@ -229,26 +294,30 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
     return (int)S;
   };
   if (M > 64) {
-    const int64_t tm = cdiv(M, 128), tn = cdiv(N, 256), tiles = tm * tn;
+    const int64_t w = 256 / per;
+    const int64_t tm = cdiv(M, 128), tn = cdiv(N, w), tiles = tm * tn;
     const int64_t cols_per_round = slots / tm;            // whole tile columns in one round
     if (tiles <= slots || cols_per_round == 0 || !can_split || want_parts) {
       pieces[npieces++] = Piece{0, N, pick_S(tiles), 0};
     } else {
       const int64_t main_tn = tn / cols_per_round * cols_per_round;   // whole rounds
-      const int64_t n_main = main_tn * 256;
+      const int64_t n_main = main_tn * w;
       pieces[npieces++] = Piece{0, n_main, 1, 0};
       if (n_main < N) pieces[npieces++] = Piece{n_main, N - n_main, pick_S(tm * (tn - main_tn)), 0};
     }
   } else {
-    // short prompts: 64-row tiles; narrow ones when that is what fills the chip
-    const int64_t t128 = cdiv(N, 128), t64 = cdiv(N, 64);
-    if (t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
+    // short prompts: 64-row tiles; narrow ones when that is what fills the chip (a gated
+    // tile needs two MFMA tiles per wavefront in N, so the narrow one is not for gu)
+    const int64_t t128 = cdiv(N, 128 / per), t64 = cdiv(N, 64 / per);
+    if (gu || t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
     else pieces[npieces++] = Piece{0, N, pick_S(t64), 2};
   }
   for (int pi = 0; pi < npieces; pi++) {
     const Piece& P = pieces[pi];
     static const int kBm[3] = {128, 64, 64}, kBn[3] = {256, 128, 64};
     const int bm = kBm[P.variant], bn = kBn[P.variant];
+    const int64_t tcols = cdiv(P.n, bn / per);            // tile columns of this piece
+    const int64_t part_w = gu ? tcols * bn : P.n;         // row width of a K-split part
     int S = P.S, kchunk = (int)K;
     float* dst = pc + P.n0;
     int ldc = (int)N;
@@ -260,37 +329,50 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
       *S_out = S;             // one piece: dst is the caller's parts, [S][M][N]
       if (S == 1) kchunk = (int)K;
     } else if (S > 1) {
-      dst = static_cast<float*>(scratch((size_t)S * M * P.n * sizeof(float)));
+      dst = static_cast<float*>(scratch((size_t)S * M * part_w * sizeof(float)));
       if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
-      ldc = (int)P.n;
+      ldc = (int)part_w;
     } else {
       kchunk = (int)K;
     }
-    const int64_t nblk = cdiv(M, bm) * cdiv(P.n, bn);
-    if (nblk > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
+    const int64_t nblk = cdiv(M, bm) * tcols;
+    if (nblk > 0x7fffffff || part_w > 0x7fffffff)
+      return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
     const dim3 grid((unsigned)nblk, (unsigned)S);
     const uint16_t* wp = pw + (size_t)P.n0 * K;
-#define TLHIP_GEMM(TM_, TN_)                                                                        \
-  gemm_bf16_nt_kernel<TM_, TN_><<<grid, dim3(256), 0, c.stream>>>(pa, wp, dst, (int)M, (int)P.n, \
-                                                                   (int)K, kchunk, ldc)
-    switch (P.variant) {
-      case 0: TLHIP_GEMM(2, 4); break;
-      case 1: TLHIP_GEMM(1, 2); break;
-      default: TLHIP_GEMM(1, 1); break;
+#define TLHIP_GEMM(TM_, TN_, GU_)                                                              \
+  gemm_bf16_nt_kernel<TM_, TN_, 2, 2, GU_><<<grid, dim3(256), 0, c.stream>>>(                  \
+      pa, wp, dst, (int)M, (int)P.n, (int)K, kchunk, ldc, (int)N)
+    switch (P.variant + (gu ? 3 : 0)) {
+      case 0: TLHIP_GEMM(2, 4, false); break;
+      case 1: TLHIP_GEMM(1, 2, false); break;
+      case 2: TLHIP_GEMM(1, 1, false); break;
+      case 3: TLHIP_GEMM(2, 4, true); break;
+      default: TLHIP_GEMM(1, 2, true); break;
     }
 #undef TLHIP_GEMM
     if (S > 1 && !want_parts) {
       const size_t total4 = (size_t)M * P.n / 4;
-      splitk_sum_kernel<<<dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, c.stream>>>(
-          reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + P.n0), (int)M, (int)(P.n / 4),
-          (int)(N / 4), S);
+      const dim3 sgrid((unsigned)((total4 + 255) / 256));
+      if (gu)
+        splitk_sum_swiglu_kernel<<<sgrid, dim3(256), 0, c.stream>>>(
+            reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + P.n0), (int)M,
+            (int)(P.n / 4), (int)(part_w / 4), (int)(N / 4), S, bn / 4 / 4);
+      else
+        splitk_sum_kernel<<<sgrid, dim3(256), 0, c.stream>>>(
+            reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + P.n0), (int)M,
+            (int)(P.n / 4), (int)(N / 4), S);
     }
   }
   TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
 }
 
 int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K) {
-  return gemm_bf16_nt_impl(A, W, C, M, N, K, 0, nullptr);
+  return gemm_bf16_nt_impl(A, W, C, M, N, K, 0, nullptr, false);
+}
+
+int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M, int64_t ff, int64_t K) {
+  return gemm_bf16_nt_impl(A, W, act, M, ff, K, 0, nullptr, true);
 }
 
 int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t parts_bytes, int64_t M,
@@ -300,7 +382,7 @@ int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t 
     return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: the buffer must hold at least one [M, N] part");
   if (parts && !aligned16(parts)) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: parts must be 16-byte aligned");
   *n_parts = 0;
-  return gemm_bf16_nt_impl(A, W, parts, M, N, K, (size_t)parts_bytes, n_parts);
+  return gemm_bf16_nt_impl(A, W, parts, M, N, K, (size_t)parts_bytes, n_parts, false);
 }
 
 }  // extern "C"

@@ -106,6 +106,7 @@ struct api {
   int (*argmax)(const void*, int64_t, int64_t*) = nullptr;
   int (*argmax_async)(const void*, int64_t, void*) = nullptr;
   int (*gemm_bf16_nt)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemm_bf16_nt_swiglu)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*gemm_bf16_nt_parts)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
                             int*) = nullptr;
   int (*rmsnorm_res_parts)(const void*, const void*, int64_t, const void*, void*, void*, int64_t, float,
@@ -232,6 +233,7 @@ struct context {
               bind(f.argmax_async, "tlhip_argmax_async") &&
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.gemm_bf16_nt_parts, "tlhip_gemm_bf16_nt_parts") &&
+              bind(f.gemm_bf16_nt_swiglu, "tlhip_gemm_bf16_nt_swiglu") &&
               bind(f.rmsnorm_res_parts, "tlhip_rmsnorm_res_parts") &&
               bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
               bind(f.qkv_rope_append, "tlhip_qkv_rope_append") &&
@@ -557,6 +559,17 @@ inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int6
   c.device_read_(B);
   c.device_write_(out);
   return detail::done_(c, c.f.gemm_bf16_nt(a, B, out, m, n, k));
+}
+
+// act[m, ff] = swiglu(a . gate^T, a . up^T) for B = [gate rows | up rows] ([2*ff, k] bf16):
+// gemm_bf16_nt + swiglu in one launch.
+inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t ff, int64_t k) {
+  auto& c = context::get();
+  if (!c.ready || (k % 8) != 0 || m <= 0 || ff <= 0) return false;
+  c.device_read_(a);
+  c.device_read_(B);
+  c.device_write_(act);
+  return detail::done_(c, c.f.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
 }
 
 // The product left as its K-split parts ([*n_parts][m][n] in `parts`), for rmsnorm_res_parts.

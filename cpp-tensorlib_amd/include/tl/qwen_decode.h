@@ -789,8 +789,7 @@ inline bool prefill_layers(model& M, int64_t T) {
       int np = 0;
       ok &= hip::gemm_bf16_nt_parts(P.at, L.wo.w, P.parts, P.parts_bytes, T, E, QD, &np);
       ok = ok && hip::rmsnorm_res_parts(x, P.parts, np, L.fn, ro, P.h2, E, d.eps, T);
-      ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);
-      ok &= hip::swiglu(P.gu, P.mb, d.ff, T);
+      ok &= hip::gemm_bf16_nt_swiglu(P.h2, L.wgu.w, P.mb, T, d.ff, E);   // the gate as the epilogue
       ok &= hip::gemm_bf16_nt_parts(P.mb, L.wd.w, P.parts, P.parts_bytes, T, E, d.ff, &np);
       ok = ok && hip::rmsnorm_res_parts(ro, P.parts, np, nextw, ro, P.h, E, d.eps, T);
     } else {

@@ -328,9 +328,16 @@ int tlhip_gemm_bf16_nt(const void* A, const void* W, void* C, int64_t M, int64_t
  * of the caller's (parts_bytes >= M*N*4; it also bounds the split), no part-sum launch. The
  * product is parts[0] + parts[1] + ... in that order - exactly what tlhip_gemm_bf16_nt stores
  * when it splits - and tlhip_rmsnorm_res_parts forms it while it reads. For the products whose
- * consumer is the residual norm (o-proj and down, qwen_model.h:383, 390: dot then add). */
+ * consumer is the residual norm (o-proj and down, qwen_model.h:382-383, 386-388). */
 int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t parts_bytes, int64_t M,
                              int64_t N, int64_t K, int* n_parts);
+/* The gate|up product of a prompt chunk with the gated activation as its epilogue:
+ * W = [gate rows | up rows], [2*ff, K] bf16 (the fused [wg|wu] of qwen_model.h:194-199),
+ * act[M, ff] = swiglu(A . gate^T, A . up^T) with tlhip_swiglu's arithmetic - the two launches of
+ * qwen_model.h:384-385 in one; the [M, 2*ff] products are never written. Same products as
+ * tlhip_gemm_bf16_nt on the same W; where K is split, it is split for other columns than there,
+ * so the two agree to fp32 summation order, not bit for bit. */
+int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M, int64_t ff, int64_t K);
 /* [T,ld] token-major (+ optional bias [H*D]) -> [H,T,D]; `off` selects a column
  * block of a fused projection.  cuda.h:846-864 */
 int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, int64_t ld,

@@ -149,6 +149,67 @@ def test_gemm_parts_then_residual_norm_is_gemm_then_residual_norm(lib, orc, M, N
         b.free()
 
 
+@pytest.mark.parametrize("M,ff,K", [
+    (512, 18944, 3584),    # 7B chunk: 128 whole-round tile columns + 20 split over K
+    (512, 4864, 896),      # 0.5B chunk: 152 tiles, split over K
+    (200, 1000, 264),      # ragged in M and in the last tile's features
+    (64, 4864, 896),       # short prompt: 64-row tiles
+    (7, 36, 40),           # less than one tile
+    (130, 130, 64),        # ff % 4 != 0: never split
+])
+def test_gemm_swiglu_epilogue(lib, orc, M, ff, K):
+    """act = swiglu(A . Wg^T, A . Wu^T) from one launch over the fused [gate rows | up rows] matrix:
+    against the oracle's product and gate, and against this library's gemm_bf16_nt followed by
+    swiglu (the same products; the K split may fall on other columns, hence not bit for bit)."""
+    print("case gemm swiglu", M, ff, K, flush=True)
+    A = orc.normal(M * K, 51).reshape(M, K)
+    Wb = orc.to_bf16(orc.normal(2 * ff * K, 52, std=0.05)).reshape(2 * ff, K)
+    da, dw = lib.to_device(A), lib.to_device(Wb)
+    act, gu, act2 = lib.empty((M, ff)), lib.empty((M, 2 * ff)), lib.empty((M, ff))
+    lib.gemm_bf16_nt_swiglu(da, dw, act, M, ff, K)
+    lib.gemm_bf16_nt(da, dw, gu, M, 2 * ff, K)
+    lib.swiglu(gu, act2, ff, M)
+    got, two = act.numpy(), act2.numpy()
+
+    def within(got, want, prod):
+        # the GEMM's tolerance on each product, carried through act = (g * sigmoid(g)) * u:
+        # |d act| <= |u| * 1.1 * |dg| + |g * sigmoid(g)| * |du|   (|d(g * sigmoid(g)) / dg| < 1.1)
+        g, u = prod[:, :ff].astype(np.float64), prod[:, ff:].astype(np.float64)
+        dg, du = RTOL * np.abs(g) + ATOL, RTOL * np.abs(u) + ATOL
+        tol = 1.1 * np.abs(u) * dg + np.abs(g / (1.0 + np.exp(-g))) * du + ATOL
+        return bool(np.all(np.abs(got.astype(np.float64) - want) <= tol))
+
+    assert within(got, two, gu.numpy()), maxrel(got, two)
+    rows = [0, M // 2, M - 1]
+    p = orc.gemm_bf16_nt(A[rows], Wb)
+    want = orc.swiglu_fused(np.ascontiguousarray(p), ff)
+    assert within(got[rows], want, p), maxrel(got[rows], want)
+    assert maxrel(got, two) < 1e-4
+    for b in (da, dw, act, gu, act2):
+        b.free()
+
+
+def test_gemm_swiglu_exact_cases(lib, orc):
+    """What the layout fixes without an oracle. A gate product of exactly 0 gives act = 0 * 0.5 * up
+    = 0 whatever up is, and a gate product large enough that sigmoid rounds to 1 gives act = g * up
+    exactly; with a one-hot A row both products are weight entries, so every (row, feature) pair
+    must land where its gate AND its up row say - a feature gated with another feature's up
+    value, or stored under another feature's index, fails."""
+    M, ff, K = 96, 320, 64
+    rng = np.random.default_rng(9)
+    Wg = rng.integers(20, 40, (ff, K)).astype(np.float32)           # sigmoid(g >= 20) == 1 in f32
+    Wu = rng.integers(-64, 64, (ff, K)).astype(np.float32)
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), np.arange(M) % K] = 1.0
+    Wb = orc.to_bf16(np.concatenate([Wg, Wu])).reshape(2 * ff, K)
+    da, dw, act = lib.to_device(A), lib.to_device(Wb), lib.empty((M, ff))
+    lib.gemm_bf16_nt_swiglu(da, dw, act, M, ff, K)
+    cols = np.arange(M) % K
+    assert np.array_equal(act.numpy(), (Wg[:, cols] * Wu[:, cols]).T)
+    for b in (da, dw, act):
+        b.free()
+
+
 def test_gemm_parts_rejects(lib):
     a, w = lib.empty((64, 64)), lib.empty((64, 32))
     small = lib.empty(16)
