@@ -89,6 +89,7 @@ SIGNATURES = {
     "tlhip_rope_table": (cint, [P, i64, i64, P, f32]),
     "tlhip_rope_table_range": (cint, [P, i64, i64, i64, f32]),
     "tlhip_qkv_rope_fill": (cint, [P, P, P, P, P, P, P, P, i64, i64, i64, i64, i64, i64, cint]),
+    "tlhip_qkv_rope_fill_parts": (cint, [P, i64, P, P, P, P, P, P, P, i64, i64, i64, i64, i64, i64, cint]),
     "tlhip_attn_prefill_tok": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint, i64]),
     "tlhip_qkv_rope_append_tab": (cint, [P, P, P, P, P, P, i64, i64, i64, i64, P, i64, P, cint]),
     "tlhip_convert": (cint, [P, cint, P, cint, i64]),
@@ -423,10 +424,13 @@ class TlHip:
     def rope_table_range(self, table, D, pos0, T, base):
         self._chk(self.c.tlhip_rope_table_range(table.ptr, D, pos0, T, base))
 
-    def qkv_rope_fill(self, qkv, bq, bk, bv, table, qh, Kc, Vc, T, Hq, Hkv, D, pos0, kv_max, kv_bf16=False):
+    def qkv_rope_fill(self, qkv, bq, bk, bv, table, qh, Kc, Vc, T, Hq, Hkv, D, pos0, kv_max, kv_bf16=False,
+                      n_parts=1):
+        """n_parts > 1: qkv holds the projection's K-split parts, [n_parts][T][(Hq + 2 Hkv) D]."""
         opt = lambda b: b.ptr if b is not None else None
-        self._chk(self.c.tlhip_qkv_rope_fill(qkv.ptr, opt(bq), opt(bk), opt(bv), table.ptr, qh.ptr, Kc.ptr, Vc.ptr,
-                                             T, Hq, Hkv, D, pos0, kv_max, 1 if kv_bf16 else 0))
+        self._chk(self.c.tlhip_qkv_rope_fill_parts(qkv.ptr, n_parts, opt(bq), opt(bk), opt(bv), table.ptr,
+                                                   qh.ptr, Kc.ptr, Vc.ptr, T, Hq, Hkv, D, pos0, kv_max,
+                                                   1 if kv_bf16 else 0))
 
     def attn_prefill_tok(self, q, K, V, out, Hq, Hkv, T, kv_max, D, scale, kv_bf16=False, pos0=0):
         self._chk(self.c.tlhip_attn_prefill_tok(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, T, kv_max, D, scale,

@@ -390,7 +390,17 @@ __global__ __launch_bounds__(256) void qkv_rope_fill_kernel(
     const float* __restrict__ qkv, const float* __restrict__ bq, const float* __restrict__ bk,
     const float* __restrict__ bv, const float2* __restrict__ table, float* __restrict__ qh,
     KT* __restrict__ Kc, KT* __restrict__ Vc, int T, int Hq, int Hkv, int D, int64_t pos0,
-    int64_t kv_max) {
+    int64_t kv_max, int S, size_t part_stride) {
+  // S > 1: qkv is the S K-split parts of the projection, part_stride floats apart, added up in
+  // ascending order as the part-sum launch would have
+  auto ld4 = [&](const float* p) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    for (int sidx = 1; sidx < S; sidx++) {
+      const float4 b = *reinterpret_cast<const float4*>(p + sidx * part_stride);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    return a;
+  };
   const int half = D >> 1, q4 = half >> 2;            // float4 groups per half row
   const int rot_per_t = (Hq + Hkv) * q4, v_per_t = Hkv * (D >> 2);
   const int per_t = rot_per_t + v_per_t;
@@ -402,8 +412,8 @@ __global__ __launch_bounds__(256) void qkv_rope_fill_kernel(
     const int r = e / q4, j = (e - r * q4) * 4;       // r: head within [q heads | k heads]
     const bool is_k = r >= Hq;
     const float* bias = is_k ? (bk ? bk + (size_t)(r - Hq) * D : nullptr) : (bq ? bq + (size_t)r * D : nullptr);
-    float4 x0 = *reinterpret_cast<const float4*>(row + (size_t)r * D + j);
-    float4 x1 = *reinterpret_cast<const float4*>(row + (size_t)r * D + j + half);
+    float4 x0 = ld4(row + (size_t)r * D + j);
+    float4 x1 = ld4(row + (size_t)r * D + j + half);
     if (bias) {
       const float4 b0 = *reinterpret_cast<const float4*>(bias + j);
       const float4 b1 = *reinterpret_cast<const float4*>(bias + j + half);
@@ -432,7 +442,7 @@ __global__ __launch_bounds__(256) void qkv_rope_fill_kernel(
     }
   } else {
     const int ev = e - rot_per_t, h = ev / (D >> 2), d = (ev - h * (D >> 2)) * 4;
-    float4 v = *reinterpret_cast<const float4*>(row + (size_t)(Hq + Hkv) * D + (size_t)h * D + d);
+    float4 v = ld4(row + (size_t)(Hq + Hkv) * D + (size_t)h * D + d);
     if (bv) {
       const float4 b = *reinterpret_cast<const float4*>(bv + (size_t)h * D + d);
       v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
@@ -706,7 +716,16 @@ int tlhip_rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, floa
 int tlhip_qkv_rope_fill(const void* qkv, const void* bq, const void* bk, const void* bv, const void* table,
                         void* qh, void* Kc, void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads,
                         int64_t D, int64_t pos0, int64_t kv_max, int kv_bf16) {
+  return tlhip_qkv_rope_fill_parts(qkv, 1, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads, n_kv_heads, D, pos0,
+                                   kv_max, kv_bf16);
+}
+
+int tlhip_qkv_rope_fill_parts(const void* qkv, int64_t n_parts, const void* bq, const void* bk,
+                              const void* bv, const void* table, void* qh, void* Kc, void* Vc, int64_t T,
+                              int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos0,
+                              int64_t kv_max, int kv_bf16) {
   TLHIP_REQUIRE_READY();
+  if (n_parts <= 0 || n_parts > 64) return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_fill: need 1 <= n_parts <= 64");
   if (!qkv || !table || !qh || !Kc || !Vc) return fail(TLHIP_EINVAL, "tlhip_qkv_rope_fill: null pointer");
   if (T <= 0 || T > 65535 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads > 65535 || n_kv_heads > 65535)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_qkv_rope_fill: bad shape");
@@ -721,7 +740,8 @@ int tlhip_qkv_rope_fill(const void* qkv, const void* bq, const void* bk, const v
   qkv_rope_fill_kernel<KT_><<<dim3(blocks_for(total)), dim3(256), 0, ctx().stream>>>(                \
       static_cast<const float*>(qkv), static_cast<const float*>(bq), static_cast<const float*>(bk), \
       static_cast<const float*>(bv), static_cast<const float2*>(table), static_cast<float*>(qh),    \
-      static_cast<KT_*>(Kc), static_cast<KT_*>(Vc), (int)T, Hq, Hkv, (int)D, pos0, kv_max)
+      static_cast<KT_*>(Kc), static_cast<KT_*>(Vc), (int)T, Hq, Hkv, (int)D, pos0, kv_max,        \
+      (int)n_parts, (size_t)(T * (Hq + 2 * Hkv) * D))
   if (kv_bf16) TLHIP_FILL(uint16_t);
   else TLHIP_FILL(float);
 #undef TLHIP_FILL

@@ -127,6 +127,8 @@ struct api {
                               int64_t, int64_t, const void*, int64_t, float, int) = nullptr;
   int (*rope_table)(void*, int64_t, int64_t, const void*, float) = nullptr;
   int (*rope_table_range)(void*, int64_t, int64_t, int64_t, float) = nullptr;
+  int (*qkv_rope_fill_parts)(const void*, int64_t, const void*, const void*, const void*, const void*, void*,
+                             void*, void*, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int) = nullptr;
   int (*qkv_rope_fill)(const void*, const void*, const void*, const void*, const void*, void*, void*, void*,
                        int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int) = nullptr;
   int (*attn_prefill_tok)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
@@ -245,6 +247,7 @@ struct context {
               bind(f.rope_table, "tlhip_rope_table") &&
               bind(f.rope_table_range, "tlhip_rope_table_range") &&
               bind(f.qkv_rope_fill, "tlhip_qkv_rope_fill") &&
+              bind(f.qkv_rope_fill_parts, "tlhip_qkv_rope_fill_parts") &&
               bind(f.attn_prefill_tok, "tlhip_attn_prefill_tok") &&
               bind(f.qkv_rope_append_tab, "tlhip_qkv_rope_append_tab") &&
               bind(f.attn_decode_qkv, "tlhip_attn_decode_qkv") &&
@@ -844,11 +847,12 @@ inline bool rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, fl
   c.device_write_(table);
   return detail::done_(c, c.f.rope_table_range(table, D, pos0, T, base));
 }
+// n_parts > 1: qkv is the projection's K-split parts (gemm_bf16_nt_parts), summed as they are read.
 inline bool qkv_rope_fill(void* qkv, void* bq, void* bk, void* bv, void* table, void* qh, void* Kc,
                           void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
-                          int64_t pos0, int64_t kv_max, bool kv_bf16 = false) {
+                          int64_t pos0, int64_t kv_max, bool kv_bf16 = false, int64_t n_parts = 1) {
   auto& c = context::get();
-  if (!c.ready || !table || (D != 128 && D != 64) || pos0 < 0 || pos0 + T > kv_max) return false;
+  if (!c.ready || !table || (D != 128 && D != 64) || pos0 < 0 || pos0 + T > kv_max || n_parts <= 0) return false;
   c.device_read_(qkv);
   if (bq) c.device_read_(bq);
   if (bk) c.device_read_(bk);
@@ -857,8 +861,8 @@ inline bool qkv_rope_fill(void* qkv, void* bq, void* bk, void* bv, void* table, 
   c.device_write_(qh);
   c.device_write_(Kc);
   c.device_write_(Vc);
-  return detail::done_(c, c.f.qkv_rope_fill(qkv, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads, n_kv_heads, D,
-                                            pos0, kv_max, kv_bf16 ? 1 : 0));
+  return detail::done_(c, c.f.qkv_rope_fill_parts(qkv, n_parts, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads,
+                                                  n_kv_heads, D, pos0, kv_max, kv_bf16 ? 1 : 0));
 }
 // attn_prefill with the result written token-major, [T, Hq*D] (no merge_heads afterwards).
 inline bool attn_prefill_tok(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
@@ -1185,10 +1189,12 @@ struct kv_cache {
   }
   // The chunk form of attn_qkv: raw token-major projection in, token-major attention out;
   // qh is [n_q_heads, T, D] scratch for the rotated queries.
+  // qkv_parts > 1: qkv holds the projection's K-split parts.
   bool prefill_qkv(void* qkv, void* bq, void* bk, void* bv, void* table, void* qh, void* out_tok, int64_t T,
-                   int64_t n_q_heads, float scale) {
+                   int64_t n_q_heads, float scale, int64_t qkv_parts = 1) {
     if (T <= 0 || pos + T > max_ctx) return false;
-    if (!qkv_rope_fill(qkv, bq, bk, bv, table, qh, K, V, T, n_q_heads, n_kv_heads, D, pos, max_ctx, kv_bf16))
+    if (!qkv_rope_fill(qkv, bq, bk, bv, table, qh, K, V, T, n_q_heads, n_kv_heads, D, pos, max_ctx, kv_bf16,
+                       qkv_parts))
       return false;
     const int64_t p0 = pos;
     pos += T;

@@ -739,7 +739,7 @@ inline bool prefill_reserve(model& M, int64_t T) {
   P.res[0] = A(T * d.hidden);
   P.res[1] = A(T * d.hidden);
   P.rope = A(T * d.head_dim);
-  P.parts_bytes = 16 * T * d.hidden * 4;   // the GEMM splits K at most 16 ways
+  P.parts_bytes = 16 * T * std::max(d.hidden, d.qkv_dim()) * 4;   // the GEMM splits K at most 16 ways
   P.parts = hip::alloc_device(P.parts_bytes);
   const bool ok = P.emb && P.h && P.h2 && P.qkv && P.qkvh && P.ah && P.at && P.gu && P.mb && P.md &&
                   P.res[0] && P.res[1] && P.rope && P.parts;
@@ -766,12 +766,15 @@ inline bool prefill_layers(model& M, int64_t T) {
   for (int64_t l = 0; l < d.n_layers; l++) {
     layer& L = M.layers[(size_t)l];
     void* ro = P.res[l & 1];
-    ok &= hip::gemm_bf16_nt(P.h, L.wqkv.w, P.qkv, T, QKVN, E);
     if (fused) {
-      // bias + rope + head-major q + cache rows in one launch; attention writes [T, Hq*D]
+      // the projection's K-split parts are added up by the launch that does bias + rope +
+      // head-major q + cache rows; attention writes [T, Hq*D]
+      int np = 0;
+      ok &= hip::gemm_bf16_nt_parts(P.h, L.wqkv.w, P.parts, P.parts_bytes, T, QKVN, E, &np);
       L.cache.pos = pos0;
-      ok &= L.cache.prefill_qkv(P.qkv, L.bq, L.bk, L.bv, P.rope, P.qkvh, P.at, T, d.n_q_heads, scale);
+      ok = ok && L.cache.prefill_qkv(P.parts, L.bq, L.bk, L.bv, P.rope, P.qkvh, P.at, T, d.n_q_heads, scale, np);
     } else {
+    ok &= hip::gemm_bf16_nt(P.h, L.wqkv.w, P.qkv, T, QKVN, E);
     // [T, q|k|v] -> head-major [Hq + 2 Hkv, T, D], bias added on the way
     ok &= hip::split_heads(P.qkv, L.bqkv, P.qkvh, T, QKVN, 0, d.n_q_heads + 2 * d.n_kv_heads, HD);
     void* kh = static_cast<char*>(P.qkvh) + QD * T * 4;

@@ -236,6 +236,12 @@ int tlhip_rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, floa
 int tlhip_qkv_rope_fill(const void* qkv, const void* bq, const void* bk, const void* bv, const void* table,
                         void* qh, void* Kc, void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads,
                         int64_t D, int64_t pos0, int64_t kv_max, int kv_bf16);
+/* The same with qkv = the n_parts K-split parts of the projection (tlhip_gemm_bf16_nt_parts:
+ * [n_parts][T][(Hq + 2 Hkv) D]), added up in ascending order as they are read. */
+int tlhip_qkv_rope_fill_parts(const void* qkv, int64_t n_parts, const void* bq, const void* bk,
+                              const void* bv, const void* table, void* qh, void* Kc, void* Vc, int64_t T,
+                              int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos0,
+                              int64_t kv_max, int kv_bf16);
 /* tlhip_attn_prefill writing out token-major, [T, Hq*D] - what merge_heads (cuda.h:862-880) would
  * make of the head-major result, so that launch is not needed. */
 int tlhip_attn_prefill_tok(const void* q, const void* K, const void* V, void* out,

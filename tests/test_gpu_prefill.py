@@ -370,6 +370,41 @@ def test_qkv_rope_fill_equals_the_separate_ops(lib, orc, D, Hq, Hkv, T, pos0, kv
         b.free()
 
 
+@pytest.mark.parametrize("kv_bf16", [False, True])
+@pytest.mark.parametrize("D,Hq,Hkv,T,pos0,S", [(128, 28, 4, 64, 0, 7), (64, 14, 2, 100, 7, 2), (64, 3, 1, 5, 2, 16)])
+def test_qkv_rope_fill_from_k_split_parts(lib, orc, D, Hq, Hkv, T, pos0, S, kv_bf16):
+    """tlhip_qkv_rope_fill_parts on S parts equals tlhip_qkv_rope_fill on their sum, taken in
+    ascending order in fp32 (what the GEMM's part-sum launch stores): queries and caches bit for bit."""
+    print("case qkv_rope_fill_parts", D, Hq, Hkv, T, pos0, S, kv_bf16, flush=True)
+    base, kv_max = 1e6, pos0 + T + 1
+    qd, kvd = Hq * D, Hkv * D
+    ld = qd + 2 * kvd
+    parts = orc.normal(S * T * ld, 81).reshape(S, T, ld)
+    total = parts[0].copy()
+    for sidx in range(1, S):
+        total = total + parts[sidx]            # fp32, one rounding per part, ascending
+    bias = orc.normal(ld, 82, 0.0, 0.1)
+    cdt = np.uint16 if kv_bf16 else np.float32
+    bits = np.uint16 if kv_bf16 else np.uint32
+    fill = np.zeros(Hkv * kv_max * D, cdt)
+    db, tab = lib.to_device(bias), lib.empty(T * D)
+    lib.rope_table_range(tab, D, pos0, T, base)
+    view = lambda off: type("View", (), {"ptr": db.ptr + off * 4})()
+    bq, bk, bv = db, view(qd), view(qd + kvd)
+    out = []
+    for src, n in ((total, 1), (parts, S)):
+        dsrc, qh = lib.to_device(src), lib.empty(qd * T)
+        Kc, Vc = lib.to_device(fill), lib.to_device(fill)
+        lib.qkv_rope_fill(dsrc, bq, bk, bv, tab, qh, Kc, Vc, T, Hq, Hkv, D, pos0, kv_max, kv_bf16, n_parts=n)
+        out.append((qh.numpy().view(np.uint32), Kc.numpy(cdt).view(bits), Vc.numpy(cdt).view(bits)))
+        for b in (dsrc, qh, Kc, Vc):
+            b.free()
+    for a, b in zip(*out):
+        assert np.array_equal(a, b)
+    db.free()
+    tab.free()
+
+
 def test_attn_prefill_tok_is_the_merged_layout(lib, orc):
     """tlhip_attn_prefill_tok writes [T, Hq*D]: exactly merge_heads of tlhip_attn_prefill's result."""
     D, Hq, Hkv, T, pos0 = 128, 6, 2, 75, 11
