@@ -74,6 +74,9 @@ SIGNATURES = {
     "tlhip_argmax": (cint, [P, i64, C.POINTER(i64)]),
     "tlhip_argmax_async": (cint, [P, i64, P]),
     "tlhip_gemm_bf16_nt": (cint, [P, P, P, i64, i64, i64]),
+    "tlhip_gemm_q4_nt": (cint, [P, P, P, P, i64, i64, i64, i64]),
+    "tlhip_gemm_q4_nt_parts": (cint, [P, P, P, P, i64, i64, i64, i64, i64, P]),
+    "tlhip_gemm_q4_nt_swiglu": (cint, [P, P, P, P, i64, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_swiglu": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_parts": (cint, [P, P, P, i64, i64, i64, i64, P]),
     "tlhip_rmsnorm_res_parts": (cint, [P, P, i64, P, P, P, i64, f32, i64]),
@@ -300,6 +303,19 @@ class TlHip:
 
     def gemm_bf16_nt(self, A, W, out, M, N, K):
         self._chk(self.c.tlhip_gemm_bf16_nt(A.ptr, W.ptr, out.ptr, M, N, K))
+
+    def gemm_q4_nt(self, A, q4, out, M, N, K):
+        """q4: the one-buffer int4 weight (packed nibbles, then scales) that gemv_q4 takes."""
+        self._chk(self.c.tlhip_gemm_q4_nt(A.ptr, q4.ptr, q4.ptr + N * K // 2, out.ptr, M, N, K, 32))
+
+    def gemm_q4_nt_swiglu(self, A, q4, act, M, ff, K):
+        self._chk(self.c.tlhip_gemm_q4_nt_swiglu(A.ptr, q4.ptr, q4.ptr + 2 * ff * K // 2, act.ptr, M, ff, K, 32))
+
+    def gemm_q4_nt_parts(self, A, q4, parts, M, N, K):
+        n = C.c_int(0)
+        self._chk(self.c.tlhip_gemm_q4_nt_parts(A.ptr, q4.ptr, q4.ptr + N * K // 2, parts.ptr, parts.nbytes,
+                                                M, N, K, 32, C.byref(n)))
+        return n.value
 
     def gemm_bf16_nt_swiglu(self, A, W, act, M, ff, K):
         self._chk(self.c.tlhip_gemm_bf16_nt_swiglu(A.ptr, W.ptr, act.ptr, M, ff, K))

@@ -48,12 +48,21 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elemen
 // (MFMA tile j and j + TN/2) and the epilogue gates in registers. N counts features, n0 still
 // counts tile columns (two per feature). Under split-K the raw parts are stored in that tile
 // column order ([M][tiles * BN]) and splitk_sum_swiglu_kernel gates after the sum.
-template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false>
+//
+// Q4 = true: W is the int4 weight of the decode path - packed nibbles [rows][K/2] (even k in the
+// low nibble, value = nibble - 8) with f32 scales [rows][K/32] (types.h:25-31). A slab of 32 k is
+// exactly one scale group: the nibbles go to LDS as the bf16 integers they stand for (exact), the
+// slab's MFMAs run into a second set of accumulators that starts at zero, and
+// acc += group sum * scale closes the slab - sum over groups of scale * (a . q), the decode GEMV's
+// arithmetic on the matrix pipe. Two accumulator sets fit for 64-column wavefront tiles (TN = 2).
+template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false, bool Q4 = false>
 __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
-                                                           int K, int kchunk, int ldc, int ff) {
+                                                           int K, int kchunk, int ldc, int ff,
+                                                           const float* __restrict__ scales) {
   static_assert(!GU || TN % 2 == 0, "gate and up accumulators of a feature must share a lane");
+  static_assert(!Q4 || (32 * TN * WN == 128 && 64 * WM * WN == 256), "int4 slab copy: two threads per tile column");
   constexpr int WT = 32 * TN, HW = WT / 2;      // a wavefront's tile columns; GU: gate half, up half
   constexpr int NT = 64 * WM * WN;              // threads: WM x WN wavefronts
   constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
@@ -86,7 +95,17 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
   float4 ra[A_LOADS];
-  uint4 rb[B_LOADS];
+  uint4 rb[Q4 ? 1 : B_LOADS];
+  uint2 rq = make_uint2(0u, 0u);      // Q4: 16 nibbles of one tile column
+  float sc[TN], sc_next[TN];          // Q4: this lane's scale per MFMA tile column, this slab / next
+  // W row of tile column `col` of this block (-1: past the edge)
+  auto wrow = [&](int col) {
+    if (GU) {
+      const int j = col % WT, f = (n0 >> 1) + (col / WT) * HW + j % HW;
+      return f < N ? f + (j >= HW ? ff : 0) : -1;
+    }
+    return n0 + col < N ? n0 + col : -1;
+  };
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
@@ -95,20 +114,38 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       ra[i] = (gm < M && gk < kend) ? *reinterpret_cast<const float4*>(A + (size_t)gm * K + gk)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+    if (Q4) {
+      // thread t: tile column t / 2, nibbles of k0 + 16 * (t % 2) .. + 15 (8 bytes)
+      const int gn = wrow(tid >> 1), gk = k0 + (tid & 1) * 16;
+      rq = (gn >= 0 && gk < kend)
+               ? *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(W) + ((size_t)gn * K + gk) / 2)
+               : make_uint2(0x88888888u, 0x88888888u);   // nibble 8 = weight 0
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int gn2 = wrow(wn * WT + j * 32 + (lane & 31));
+        sc_next[j] = (gn2 >= 0 && k0 < kend) ? scales[(size_t)gn2 * (K >> 5) + (k0 >> 5)] : 0.f;
+      }
+    } else {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
-      const int gk = k0 + c8 * 8;
-      int gn = n0 + row;
-      bool in = gn < N;
-      if (GU) {
-        const int j = row % WT, f = (n0 >> 1) + (row / WT) * HW + j % HW;
-        in = f < N;
-        gn = f + (j >= HW ? ff : 0);
-      }
-      rb[i] = (in && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
-                                : make_uint4(0u, 0u, 0u, 0u);
+      const int gk = k0 + c8 * 8, gn = wrow(row);
+      rb[i] = (gn >= 0 && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
+                                     : make_uint4(0u, 0u, 0u, 0u);
     }
+    }
+  };
+  // 4 bytes = 8 nibbles -> 8 bf16 (k ascending): float(nibble) - 8 is an integer in [-8, 7], exact in bf16
+  auto nib8 = [](uint32_t w) {
+    const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;   // even k, odd k
+    uint4 o;
+    uint32_t* po = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      const float e = (float)((lo >> (8 * b)) & 0xffu) - 8.0f, d = (float)((hi >> (8 * b)) & 0xffu) - 8.0f;
+      po[b] = (__float_as_uint(e) >> 16) | (__float_as_uint(d) & 0xffff0000u);
+    }
+    return o;
   };
   auto split3 = [](float a, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
     const uint32_t h = __float_as_uint(a) & 0xffff0000u;
@@ -133,10 +170,18 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       *reinterpret_cast<uint2*>(&As[1][o]) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
       *reinterpret_cast<uint2*>(&As[2][o]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
     }
+    if (Q4) {
+      const int row = tid >> 1, c8 = (tid & 1) * 2;
+      *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8)]) = nib8(rq.x);
+      *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + 1)]) = nib8(rq.y);
+#pragma unroll
+      for (int j = 0; j < TN; j++) sc[j] = sc_next[j];
+    } else {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
       *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8)]) = rb[i];
+    }
     }
   };
 
@@ -146,6 +191,15 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     lstore();
     __syncthreads();
     if (k0 + kBK < kend) gload(k0 + kBK);
+    f32x16 grp[Q4 ? TM : 1][Q4 ? TN : 1];   // Q4: this slab's (= this scale group's) sums
+    if (Q4) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) grp[i][j][v] = 0.f;
+    }
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ks++) {
       const int kc = ks * 2 + (lane >> 5);   // 16-byte chunk of the slab this lane multiplies
@@ -160,10 +214,20 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
         for (int p = 0; p < 3; p++) {
           const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
 #pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; j++) {
+            if (Q4) grp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], grp[i][j], 0, 0, 0);
+            else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
+          }
         }
       }
+    }
+    if (Q4) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[i][j][v] = fmaf(grp[i][j][v], sc[j], acc[i][j][v]);
     }
   }
 
@@ -252,11 +316,16 @@ extern "C" {
 //     [S][M][N], no part sum is launched and *S_out says how many there are (1: the plain
 //     product); one piece, so that the layout is uniform.
 //   gu: W = [gate rows | up rows], N = features (rows of each), C[M][N] = the gated activation.
+//   scales != nullptr: W is an int4 weight (packed nibbles [rows][K/2], scales [rows][K/32]); any of
+//     the three forms above.
 static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K,
-                             size_t parts_bytes, int* S_out, bool gu) {
+                             size_t parts_bytes, int* S_out, bool gu, const void* scales = nullptr) {
   TLHIP_REQUIRE_READY();
   const bool want_parts = S_out != nullptr;
+  const bool q4 = scales != nullptr;
   if (!A || !W || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt: null pointer");
+  if (q4 && ((K % 32) != 0 || !aligned16(scales)))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_q4_nt: need K %% 32 == 0 (one scale per 32 weights) and aligned scales");
   // the reference's gate: K a multiple of 8
   if ((K % 8) != 0 || M <= 0 || N <= 0 || K <= 0)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: need K %% 8 == 0 and positive M, N, K");
@@ -294,27 +363,29 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
     return (int)S;
   };
   if (M > 64) {
-    const int64_t w = 256 / per;
+    // int4: two accumulator sets per wavefront, so 64 x 64 wavefront tiles (128 x 128 per block)
+    const int64_t w = (q4 ? 128 : 256) / per;
+    const int wide = q4 ? 3 : 0;
     const int64_t tm = cdiv(M, 128), tn = cdiv(N, w), tiles = tm * tn;
     const int64_t cols_per_round = slots / tm;            // whole tile columns in one round
     if (tiles <= slots || cols_per_round == 0 || !can_split || want_parts) {
-      pieces[npieces++] = Piece{0, N, pick_S(tiles), 0};
+      pieces[npieces++] = Piece{0, N, pick_S(tiles), wide};
     } else {
       const int64_t main_tn = tn / cols_per_round * cols_per_round;   // whole rounds
       const int64_t n_main = main_tn * w;
-      pieces[npieces++] = Piece{0, n_main, 1, 0};
-      if (n_main < N) pieces[npieces++] = Piece{n_main, N - n_main, pick_S(tm * (tn - main_tn)), 0};
+      pieces[npieces++] = Piece{0, n_main, 1, wide};
+      if (n_main < N) pieces[npieces++] = Piece{n_main, N - n_main, pick_S(tm * (tn - main_tn)), wide};
     }
   } else {
     // short prompts: 64-row tiles; narrow ones when that is what fills the chip (a gated
     // tile needs two MFMA tiles per wavefront in N, so the narrow one is not for gu)
     const int64_t t128 = cdiv(N, 128 / per), t64 = cdiv(N, 64 / per);
-    if (gu || t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
+    if (gu || q4 || t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
     else pieces[npieces++] = Piece{0, N, pick_S(t64), 2};
   }
   for (int pi = 0; pi < npieces; pi++) {
     const Piece& P = pieces[pi];
-    static const int kBm[3] = {128, 64, 64}, kBn[3] = {256, 128, 64};
+    static const int kBm[4] = {128, 64, 64, 128}, kBn[4] = {256, 128, 64, 128};
     const int bm = kBm[P.variant], bn = kBn[P.variant];
     const int64_t tcols = cdiv(P.n, bn / per);            // tile columns of this piece
     const int64_t part_w = gu ? tcols * bn : P.n;         // row width of a K-split part
@@ -339,16 +410,24 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
     if (nblk > 0x7fffffff || part_w > 0x7fffffff)
       return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: too many tiles for one grid");
     const dim3 grid((unsigned)nblk, (unsigned)S);
-    const uint16_t* wp = pw + (size_t)P.n0 * K;
-#define TLHIP_GEMM(TM_, TN_, GU_)                                                              \
-  gemm_bf16_nt_kernel<TM_, TN_, 2, 2, GU_><<<grid, dim3(256), 0, c.stream>>>(                  \
-      pa, wp, dst, (int)M, (int)P.n, (int)K, kchunk, ldc, (int)N)
-    switch (P.variant + (gu ? 3 : 0)) {
-      case 0: TLHIP_GEMM(2, 4, false); break;
-      case 1: TLHIP_GEMM(1, 2, false); break;
-      case 2: TLHIP_GEMM(1, 1, false); break;
-      case 3: TLHIP_GEMM(2, 4, true); break;
-      default: TLHIP_GEMM(1, 2, true); break;
+    // first row of the piece: bf16 rows are K elements, int4 rows K / 2 bytes + K / 32 scales
+    const uint16_t* wp = q4 ? reinterpret_cast<const uint16_t*>(static_cast<const uint8_t*>(W) + (size_t)P.n0 * K / 2)
+                            : pw + (size_t)P.n0 * K;
+    const float* sp = q4 ? static_cast<const float*>(scales) + (size_t)P.n0 * (K / 32) : nullptr;
+#define TLHIP_GEMM(TM_, TN_, GU_, Q4_)                                                         \
+  gemm_bf16_nt_kernel<TM_, TN_, 2, 2, GU_, Q4_><<<grid, dim3(256), 0, c.stream>>>(             \
+      pa, wp, dst, (int)M, (int)P.n, (int)K, kchunk, ldc, (int)N, sp)
+    switch (P.variant + (gu ? 4 : 0) + (q4 ? 8 : 0)) {
+      case 0: TLHIP_GEMM(2, 4, false, false); break;
+      case 1: TLHIP_GEMM(1, 2, false, false); break;
+      case 2: TLHIP_GEMM(1, 1, false, false); break;
+      case 4: TLHIP_GEMM(2, 4, true, false); break;
+      case 5: TLHIP_GEMM(1, 2, true, false); break;
+      case 9: TLHIP_GEMM(1, 2, false, true); break;
+      case 11: TLHIP_GEMM(2, 2, false, true); break;
+      case 13: TLHIP_GEMM(1, 2, true, true); break;
+      case 15: TLHIP_GEMM(2, 2, true, true); break;
+      default: return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: no kernel for this plan");
     }
 #undef TLHIP_GEMM
     if (S > 1 && !want_parts) {
@@ -375,14 +454,46 @@ int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M
   return gemm_bf16_nt_impl(A, W, act, M, ff, K, 0, nullptr, true);
 }
 
+static int gemm_parts_entry(const void* A, const void* W, const void* scales, void* parts,
+                            int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int* n_parts) {
+  if (!n_parts) return fail(TLHIP_EINVAL, "tlhip_gemm_*_nt_parts: null n_parts");
+  if (M > 0 && N > 0 && parts_bytes < (int64_t)(M * N * sizeof(float)))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_*_nt_parts: the buffer must hold at least one [M, N] part");
+  if (parts && !aligned16(parts)) return fail(TLHIP_EINVAL, "tlhip_gemm_*_nt_parts: parts must be 16-byte aligned");
+  *n_parts = 0;
+  return gemm_bf16_nt_impl(A, W, parts, M, N, K, (size_t)parts_bytes, n_parts, false, scales);
+}
+
 int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t parts_bytes, int64_t M,
                              int64_t N, int64_t K, int* n_parts) {
-  if (!n_parts) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: null n_parts");
-  if (M > 0 && N > 0 && parts_bytes < (int64_t)(M * N * sizeof(float)))
-    return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: the buffer must hold at least one [M, N] part");
-  if (parts && !aligned16(parts)) return fail(TLHIP_EINVAL, "tlhip_gemm_bf16_nt_parts: parts must be 16-byte aligned");
-  *n_parts = 0;
-  return gemm_bf16_nt_impl(A, W, parts, M, N, K, (size_t)parts_bytes, n_parts, false);
+  return gemm_parts_entry(A, W, nullptr, parts, parts_bytes, M, N, K, n_parts);
+}
+
+// ---- the same three forms over an int4 weight (no reference counterpart: the reference feeds
+// prompts to an int4 model token by token, qwen_model.h:419) ----
+static int q4_gate(const void* scales, int64_t group) {
+  if (!scales) return fail(TLHIP_EINVAL, "tlhip_gemm_q4_nt: null scales");
+  if (group != 32) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_q4_nt: group must be 32");   // types.h:30
+  return TLHIP_OK;
+}
+
+int tlhip_gemm_q4_nt(const void* A, const void* qw, const void* scales, void* C, int64_t M, int64_t N,
+                     int64_t K, int64_t group) {
+  if (int rc = q4_gate(scales, group)) return rc;
+  return gemm_bf16_nt_impl(A, qw, C, M, N, K, 0, nullptr, false, scales);
+}
+
+int tlhip_gemm_q4_nt_swiglu(const void* A, const void* qw, const void* scales, void* act, int64_t M,
+                            int64_t ff, int64_t K, int64_t group) {
+  if (int rc = q4_gate(scales, group)) return rc;
+  return gemm_bf16_nt_impl(A, qw, act, M, ff, K, 0, nullptr, true, scales);
+}
+
+int tlhip_gemm_q4_nt_parts(const void* A, const void* qw, const void* scales, void* parts,
+                           int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int64_t group,
+                           int* n_parts) {
+  if (int rc = q4_gate(scales, group)) return rc;
+  return gemm_parts_entry(A, qw, scales, parts, parts_bytes, M, N, K, n_parts);
 }
 
 }  // extern "C"

@@ -106,6 +106,11 @@ struct api {
   int (*argmax)(const void*, int64_t, int64_t*) = nullptr;
   int (*argmax_async)(const void*, int64_t, void*) = nullptr;
   int (*gemm_bf16_nt)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemm_q4_nt)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemm_q4_nt_parts)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
+                          int64_t, int*) = nullptr;
+  int (*gemm_q4_nt_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
+                           int64_t) = nullptr;
   int (*gemm_bf16_nt_swiglu)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*gemm_bf16_nt_parts)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
                             int*) = nullptr;
@@ -236,6 +241,8 @@ struct context {
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.gemm_bf16_nt_parts, "tlhip_gemm_bf16_nt_parts") &&
               bind(f.gemm_bf16_nt_swiglu, "tlhip_gemm_bf16_nt_swiglu") &&
+              bind(f.gemm_q4_nt, "tlhip_gemm_q4_nt") && bind(f.gemm_q4_nt_parts, "tlhip_gemm_q4_nt_parts") &&
+              bind(f.gemm_q4_nt_swiglu, "tlhip_gemm_q4_nt_swiglu") &&
               bind(f.rmsnorm_res_parts, "tlhip_rmsnorm_res_parts") &&
               bind(f.split_heads, "tlhip_split_heads") && bind(f.merge_heads, "tlhip_merge_heads") &&
               bind(f.qkv_rope_append, "tlhip_qkv_rope_append") &&
@@ -573,6 +580,36 @@ inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t 
   c.device_read_(B);
   c.device_write_(act);
   return detail::done_(c, c.f.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
+}
+
+// The prompt-chunk products over an int4 weight (packed nibbles + scales, group 32), M rows at a
+// time on the matrix pipe; plain, gated and parts forms like the bf16 ones.
+inline bool gemm_q4_nt(void* a, void* qw, void* scales, void* out, int64_t m, int64_t n, int64_t k,
+                       int64_t group = 32) {
+  auto& c = context::get();
+  if (!c.ready || (k % 32) != 0 || m <= 0 || n <= 0) return false;
+  c.device_read_(a);
+  c.device_read_(qw);
+  c.device_write_(out);
+  return detail::done_(c, c.f.gemm_q4_nt(a, qw, scales, out, m, n, k, group));
+}
+inline bool gemm_q4_nt_swiglu(void* a, void* qw, void* scales, void* act, int64_t m, int64_t ff, int64_t k,
+                              int64_t group = 32) {
+  auto& c = context::get();
+  if (!c.ready || (k % 32) != 0 || m <= 0 || ff <= 0) return false;
+  c.device_read_(a);
+  c.device_read_(qw);
+  c.device_write_(act);
+  return detail::done_(c, c.f.gemm_q4_nt_swiglu(a, qw, scales, act, m, ff, k, group));
+}
+inline bool gemm_q4_nt_parts(void* a, void* qw, void* scales, void* parts, int64_t parts_bytes, int64_t m,
+                             int64_t n, int64_t k, int* n_parts, int64_t group = 32) {
+  auto& c = context::get();
+  if (!c.ready || (k % 32) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
+  c.device_read_(a);
+  c.device_read_(qw);
+  c.device_write_(parts);
+  return detail::done_(c, c.f.gemm_q4_nt_parts(a, qw, scales, parts, parts_bytes, m, n, k, group, n_parts));
 }
 
 // The product left as its K-split parts ([*n_parts][m][n] in `parts`), for rmsnorm_res_parts.

@@ -73,6 +73,27 @@ inline bool gemv(const linear& L, void* a, void* y) {
   return hip::gemv_bf16_row(a, L.w, y, L.N, L.K);
 }
 
+// Prompt-chunk products, T rows at a time: out[T, N] = a[T, K] . W^T for either weight format
+// (bf16 rows or int4); `_parts` leaves the K-split parts for the launch that consumes them,
+// `_swiglu` takes the fused [gate | up] weight and writes the gated activation [T, N / 2].
+inline bool gemm(const linear& L, void* a, void* out, int64_t T) {
+  if (L.fmt == wfmt::q4)
+    return hip::gemm_q4_nt(a, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, out, T, L.N, L.K, kQ4Group);
+  return hip::gemm_bf16_nt(a, L.w, out, T, L.N, L.K);
+}
+inline bool gemm_parts(const linear& L, void* a, void* parts, int64_t parts_bytes, int64_t T, int* n_parts) {
+  if (L.fmt == wfmt::q4)
+    return hip::gemm_q4_nt_parts(a, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, parts, parts_bytes, T, L.N,
+                                 L.K, n_parts, kQ4Group);
+  return hip::gemm_bf16_nt_parts(a, L.w, parts, parts_bytes, T, L.N, L.K, n_parts);
+}
+inline bool gemm_swiglu(const linear& L, void* a, void* act, int64_t T) {
+  if (L.fmt == wfmt::q4)
+    return hip::gemm_q4_nt_swiglu(a, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, act, T, L.N / 2, L.K,
+                                  kQ4Group);
+  return hip::gemm_bf16_nt_swiglu(a, L.w, act, T, L.N / 2, L.K);
+}
+
 // y = W . swiglu(gu)
 inline bool gemv_swiglu(const linear& L, void* gu, void* y) {
   if (L.fmt == wfmt::q4) {
@@ -753,8 +774,8 @@ inline bool prefill_layers(model& M, int64_t T) {
   const dims& d = M.d;
   prefill_scratch& P = M.ps;
   if (T <= 0 || T > P.T) return false;
-  for (const layer& L : M.layers)
-    if (L.wqkv.fmt != wfmt::bf16_row) return false;  // the MFMA GEMM reads bf16 rows only
+  for (const layer& L : M.layers)   // the MFMA GEMM reads bf16 rows or int4, not [K,N] bf16
+    if (L.wqkv.fmt != wfmt::bf16_row && L.wqkv.fmt != wfmt::q4) return false;
   const float scale = 1.0f / std::sqrt((float)d.head_dim);
   const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim(), QKVN = d.qkv_dim(), HD = d.head_dim;
   const int64_t pos0 = M.layers[0].cache.pos;
@@ -770,11 +791,11 @@ inline bool prefill_layers(model& M, int64_t T) {
       // the projection's K-split parts are added up by the launch that does bias + rope +
       // head-major q + cache rows; attention writes [T, Hq*D]
       int np = 0;
-      ok &= hip::gemm_bf16_nt_parts(P.h, L.wqkv.w, P.parts, P.parts_bytes, T, QKVN, E, &np);
+      ok &= gemm_parts(L.wqkv, P.h, P.parts, P.parts_bytes, T, &np);
       L.cache.pos = pos0;
       ok = ok && L.cache.prefill_qkv(P.parts, L.bq, L.bk, L.bv, P.rope, P.qkvh, P.at, T, d.n_q_heads, scale, np);
     } else {
-    ok &= hip::gemm_bf16_nt(P.h, L.wqkv.w, P.qkv, T, QKVN, E);
+    ok &= gemm(L.wqkv, P.h, P.qkv, T);
     // [T, q|k|v] -> head-major [Hq + 2 Hkv, T, D], bias added on the way
     ok &= hip::split_heads(P.qkv, L.bqkv, P.qkvh, T, QKVN, 0, d.n_q_heads + 2 * d.n_kv_heads, HD);
     void* kh = static_cast<char*>(P.qkvh) + QD * T * 4;
@@ -790,17 +811,17 @@ inline bool prefill_layers(model& M, int64_t T) {
     if (fused) {
       // o-proj and down leave their K-split parts; the residual norm adds them up as it reads
       int np = 0;
-      ok &= hip::gemm_bf16_nt_parts(P.at, L.wo.w, P.parts, P.parts_bytes, T, E, QD, &np);
+      ok &= gemm_parts(L.wo, P.at, P.parts, P.parts_bytes, T, &np);
       ok = ok && hip::rmsnorm_res_parts(x, P.parts, np, L.fn, ro, P.h2, E, d.eps, T);
-      ok &= hip::gemm_bf16_nt_swiglu(P.h2, L.wgu.w, P.mb, T, d.ff, E);   // the gate as the epilogue
-      ok &= hip::gemm_bf16_nt_parts(P.mb, L.wd.w, P.parts, P.parts_bytes, T, E, d.ff, &np);
+      ok &= gemm_swiglu(L.wgu, P.h2, P.mb, T);   // the gate as the epilogue
+      ok &= gemm_parts(L.wd, P.mb, P.parts, P.parts_bytes, T, &np);
       ok = ok && hip::rmsnorm_res_parts(ro, P.parts, np, nextw, ro, P.h, E, d.eps, T);
     } else {
-    ok &= hip::gemm_bf16_nt(P.at, L.wo.w, ro, T, E, QD);
+    ok &= gemm(L.wo, P.at, ro, T);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, P.h2, E, d.eps, T);
-    ok &= hip::gemm_bf16_nt(P.h2, L.wgu.w, P.gu, T, 2 * d.ff, E);
+    ok &= gemm(L.wgu, P.h2, P.gu, T);
     ok &= hip::swiglu(P.gu, P.mb, d.ff, T);
-    ok &= hip::gemm_bf16_nt(P.mb, L.wd.w, P.md, T, E, d.ff);
+    ok &= gemm(L.wd, P.mb, P.md, T);
     ok &= hip::rmsnorm_res(ro, P.md, nextw, ro, P.h, E, d.eps, T);
     }
     x = ro;

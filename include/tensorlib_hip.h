@@ -344,6 +344,19 @@ int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t 
  * tlhip_gemm_bf16_nt on the same W; where K is split, it is split for other columns than there,
  * so the two agree to fp32 summation order, not bit for bit. */
 int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M, int64_t ff, int64_t K);
+/* The three prompt-chunk products over an int4 weight (qw = packed nibbles [N][K/2], scales
+ * [N][K/32], group 32 - the operand of tlhip_gemv_q4): C = A . dequant(W)^T formed as
+ * sum over groups of scale * (A . q) with exact products on the matrix pipe, fp32 sums - the decode
+ * GEMV's arithmetic, M rows at a time. No reference counterpart: the reference feeds prompts to
+ * an int4 model one token at a time (qwen_model.h:419 gates its batched prefill on bf16 weights);
+ * parity is against tlhip_gemv_q4 / the CPU path row by row. */
+int tlhip_gemm_q4_nt(const void* A, const void* qw, const void* scales, void* C, int64_t M, int64_t N,
+                     int64_t K, int64_t group);
+int tlhip_gemm_q4_nt_parts(const void* A, const void* qw, const void* scales, void* parts,
+                           int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int64_t group,
+                           int* n_parts);
+int tlhip_gemm_q4_nt_swiglu(const void* A, const void* qw, const void* scales, void* act, int64_t M,
+                            int64_t ff, int64_t K, int64_t group);
 /* [T,ld] token-major (+ optional bias [H*D]) -> [H,T,D]; `off` selects a column
  * block of a fused projection.  cuda.h:846-864 */
 int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, int64_t ld,

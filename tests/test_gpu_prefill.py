@@ -210,6 +210,82 @@ def test_gemm_swiglu_exact_cases(lib, orc):
         b.free()
 
 
+@pytest.mark.parametrize("M,N,K", [
+    (512, 3584, 3584),     # 7B o-proj: 128 x 128 tiles, K split
+    (512, 1152, 896),      # 0.5B q|k|v
+    (300, 4864, 896),      # ragged M
+    (64, 896, 4864),       # short prompt (64-row tiles), long K
+    (5, 130, 64),          # less than one tile, N % 4 != 0: never split
+    (130, 520, 32),        # one scale group
+])
+def test_gemm_q4_nt_matches_oracle_and_the_decode_gemv(lib, orc, M, N, K):
+    """C = A . dequant(Wq)^T over the int4 weight of the decode path: every row against the CPU
+    path's int4 dot (array.h:1980-1984) and against this library's decode GEMV on the same buffer."""
+    print("case gemm_q4_nt", M, N, K, flush=True)
+    A = orc.normal(M * K, 91).reshape(M, K)
+    buf = orc.fill_q4(N, K, 92) if K > 64 else orc.to_q4(orc.normal(K * N, 92, 0.0, 0.02).reshape(K, N))
+    da, dw, dc, dy = lib.to_device(A), lib.to_device(buf), lib.empty((M, N)), lib.empty(N)
+    lib.gemm_q4_nt(da, dw, dc, M, N, K)
+    got = dc.numpy()
+    for m in sorted({0, M // 3, M - 1}):
+        want = orc.gemv_q4(A[m], buf, N, K)
+        assert allclose(got[m], want, RTOL, ATOL), (m, maxrel(got[m], want))
+        dx = lib.to_device(A[m])
+        lib.gemv_q4(dx, dw, dy, N, K)
+        assert allclose(got[m], dy.numpy(), RTOL, ATOL), (m, maxrel(got[m], dy.numpy()))
+        dx.free()
+    # the K-split parts add up to the product
+    parts = lib.empty((16, M, N))
+    n = lib.gemm_q4_nt_parts(da, dw, parts, M, N, K)
+    assert 1 <= n <= 16
+    total = parts.numpy()[:n].astype(np.float64).sum(axis=0).astype(np.float32)
+    assert allclose(total, got, RTOL, ATOL), maxrel(total, got)
+    for b in (da, dw, dc, dy, parts):
+        b.free()
+
+
+def test_gemm_q4_nt_exact_cases(lib, orc):
+    """What the arithmetic fixes without an oracle: integer-valued activations, every nibble value
+    and power-of-two scales make each group sum and each scaled sum exact, so the result must equal
+    the float64 value of sum_g scale_g * (a . (nibble - 8)) bit for bit - a wrong nibble order,
+    a scale taken from the neighbouring group or row, or a transposed tile fails."""
+    M, N, K = 130, 200, 128
+    rng = np.random.default_rng(31)
+    A = rng.integers(-300, 300, (M, K)).astype(np.float32) + 0.5
+    q = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    scales = (2.0 ** rng.integers(-6, 2, (N, K // 32))).astype(np.float32)
+    packed = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)         # even k in the low nibble
+    buf = np.concatenate([packed.reshape(-1), scales.reshape(-1).view(np.uint8)])
+    da, dw, dc = lib.to_device(A), lib.to_device(buf), lib.empty((M, N))
+    lib.gemm_q4_nt(da, dw, dc, M, N, K)
+    w = (q.astype(np.float64) - 8.0) * np.repeat(scales.astype(np.float64), 32, axis=1)
+    want = A.astype(np.float64) @ w.T
+    assert np.array_equal(dc.numpy().astype(np.float64), want)
+    for b in (da, dw, dc):
+        b.free()
+
+
+@pytest.mark.parametrize("M,ff,K", [(512, 4864, 896), (200, 1000, 64), (64, 4864, 896), (512, 18944, 3584)])
+def test_gemm_q4_nt_swiglu_epilogue(lib, orc, M, ff, K):
+    """The gated activation from one launch over the fused int4 [gate rows | up rows] weight against
+    gemm_q4_nt followed by swiglu, with the GEMM's tolerance carried through the gate."""
+    print("case gemm_q4 swiglu", M, ff, K, flush=True)
+    A = orc.normal(M * K, 95).reshape(M, K)
+    buf = orc.fill_q4(2 * ff, K, 96)
+    da, dw = lib.to_device(A), lib.to_device(buf)
+    act, gu, act2 = lib.empty((M, ff)), lib.empty((M, 2 * ff)), lib.empty((M, ff))
+    lib.gemm_q4_nt_swiglu(da, dw, act, M, ff, K)
+    lib.gemm_q4_nt(da, dw, gu, M, 2 * ff, K)
+    lib.swiglu(gu, act2, ff, M)
+    got, two, prod = act.numpy().astype(np.float64), act2.numpy(), gu.numpy()
+    g, u = prod[:, :ff].astype(np.float64), prod[:, ff:].astype(np.float64)
+    dg, du = RTOL * np.abs(g) + ATOL, RTOL * np.abs(u) + ATOL
+    tol = 1.1 * np.abs(u) * dg + np.abs(g / (1.0 + np.exp(-g))) * du + ATOL
+    assert np.all(np.abs(got - two) <= tol), maxrel(got, two)
+    for b in (da, dw, act, gu, act2):
+        b.free()
+
+
 def test_gemm_parts_rejects(lib):
     a, w = lib.empty((64, 64)), lib.empty((64, 32))
     small = lib.empty(16)
