@@ -355,7 +355,7 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
   int npieces = 0;
   auto pick_S = [&](int64_t tiles) {   // K splits that bring `tiles` blocks up to the slots
     if (!can_split || tiles >= slots) return 1;
-    int64_t S = (slots + tiles / 2) / tiles;
+    int64_t S = slots / tiles;   // never past the slots: a few blocks left for a second round double the launch
     if (S > 16) S = 16;
     while (S > 1 && K / S < 256) S--;
     if (want_parts)   // the caller's buffer bounds the parts
