@@ -54,7 +54,9 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elemen
 // exactly one scale group: the nibbles go to LDS as the bf16 integers they stand for (exact), the
 // slab's MFMAs run into a second set of accumulators that starts at zero, and
 // acc += group sum * scale closes the slab - sum over groups of scale * (a . q), the decode GEMV's
-// arithmetic on the matrix pipe. Two accumulator sets fit for 64-column wavefront tiles (TN = 2).
+// arithmetic on the matrix pipe. The second set holds one row block of MFMA tiles at a time; with
+// it, 64-column wavefront tiles (TN = 2) fit the registers, 128-column ones spill (and then run
+// at half the speed).
 template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false, bool Q4 = false>
 __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
@@ -62,7 +64,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
                                                            int K, int kchunk, int ldc, int ff,
                                                            const float* __restrict__ scales) {
   static_assert(!GU || TN % 2 == 0, "gate and up accumulators of a feature must share a lane");
-  static_assert(!Q4 || (32 * TN * WN == 128 && 64 * WM * WN == 256), "int4 slab copy: two threads per tile column");
+  static_assert(!Q4 || ((32 * TN * WN == 128 || 32 * TN * WN == 256) && 64 * WM * WN == 256),
+                "int4 slab copy: one or two threads per tile column");
+  constexpr int TPC = Q4 ? 256 / (32 * TN * WN) : 1;   // Q4: threads per tile column of the slab copy
   constexpr int WT = 32 * TN, HW = WT / 2;      // a wavefront's tile columns; GU: gate half, up half
   constexpr int NT = 64 * WM * WN;              // threads: WM x WN wavefronts
   constexpr int BM = 32 * TM * WM, BN = 32 * TN * WN;
@@ -96,7 +100,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 
   float4 ra[A_LOADS];
   uint4 rb[Q4 ? 1 : B_LOADS];
-  uint2 rq = make_uint2(0u, 0u);      // Q4: 16 nibbles of one tile column
+  uint32_t rq[4 / TPC] = {};          // Q4: 32 / TPC nibbles of one tile column
   float sc[TN], sc_next[TN];          // Q4: this lane's scale per MFMA tile column, this slab / next
   // W row of tile column `col` of this block (-1: past the edge)
   auto wrow = [&](int col) {
@@ -115,11 +119,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     if (Q4) {
-      // thread t: tile column t / 2, nibbles of k0 + 16 * (t % 2) .. + 15 (8 bytes)
-      const int gn = wrow(tid >> 1), gk = k0 + (tid & 1) * 16;
-      rq = (gn >= 0 && gk < kend)
-               ? *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(W) + ((size_t)gn * K + gk) / 2)
-               : make_uint2(0x88888888u, 0x88888888u);   // nibble 8 = weight 0
+      // thread t: tile column t / TPC, nibbles of k0 + (32 / TPC) * (t % TPC) .. (16 / TPC bytes)
+      const int gn = wrow(tid / TPC), gk = k0 + (tid % TPC) * (32 / TPC);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(W) + ((size_t)max(gn, 0) * K + gk) / 2);
+      const bool in = gn >= 0 && gk < kend;
+#pragma unroll
+      for (int u = 0; u < 4 / TPC; u++) rq[u] = in ? src[u] : 0x88888888u;   // nibble 8 = weight 0
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const int gn2 = wrow(wn * WT + j * 32 + (lane & 31));
@@ -171,9 +176,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       *reinterpret_cast<uint2*>(&As[2][o]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
     }
     if (Q4) {
-      const int row = tid >> 1, c8 = (tid & 1) * 2;
-      *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8)]) = nib8(rq.x);
-      *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + 1)]) = nib8(rq.y);
+      const int row = tid / TPC, c8 = (tid % TPC) * (4 / TPC);
+#pragma unroll
+      for (int u = 0; u < 4 / TPC; u++) *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + u)]) = nib8(rq[u]);
 #pragma unroll
       for (int j = 0; j < TN; j++) sc[j] = sc_next[j];
     } else {
@@ -191,14 +196,38 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     lstore();
     __syncthreads();
     if (k0 + kBK < kend) gload(k0 + kBK);
-    f32x16 grp[Q4 ? TM : 1][Q4 ? TN : 1];   // Q4: this slab's (= this scale group's) sums
     if (Q4) {
+      // one row block of MFMA tiles at a time: its sums over this slab (= this scale group) in a
+      // second accumulator set that starts at zero, then acc += sums * scale
 #pragma unroll
-      for (int i = 0; i < TM; i++)
+      for (int i = 0; i < TM; i++) {
+        f32x16 grp[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++)
 #pragma unroll
-          for (int v = 0; v < 16; v++) grp[i][j][v] = 0.f;
+          for (int v = 0; v < 16; v++) grp[j][v] = 0.f;
+        const int row = wm * 32 * TM + i * 32 + (lane & 31);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ks++) {
+          const int kc = ks * 2 + (lane >> 5);
+          bf16x8 bfrag[TN];
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            bfrag[j] = *reinterpret_cast<const bf16x8*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
+#pragma unroll
+          for (int p = 0; p < 3; p++) {
+            const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+              grp[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], grp[j], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[i][j][v] = fmaf(grp[j][v], sc[j], acc[i][j][v]);
+      }
+      continue;
     }
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ks++) {
@@ -214,20 +243,10 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
         for (int p = 0; p < 3; p++) {
           const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
 #pragma unroll
-          for (int j = 0; j < TN; j++) {
-            if (Q4) grp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], grp[i][j], 0, 0, 0);
-            else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
-          }
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
         }
       }
-    }
-    if (Q4) {
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) acc[i][j][v] = fmaf(grp[i][j][v], sc[j], acc[i][j][v]);
     }
   }
 
