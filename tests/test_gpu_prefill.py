@@ -1,5 +1,7 @@
 """GPU parity: the prefill pair (MFMA GEMM against bf16 weights, causal attention over a
 cache) through the C ABI vs the CPU oracle."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -283,6 +285,25 @@ def test_gemm_q4_nt_swiglu_epilogue(lib, orc, M, ff, K):
     tol = 1.1 * np.abs(u) * dg + np.abs(g / (1.0 + np.exp(-g))) * du + ATOL
     assert np.all(np.abs(got - two) <= tol), maxrel(got, two)
     for b in (da, dw, act, gu, act2):
+        b.free()
+
+
+def test_gemm_q4_nt_rejects(lib):
+    """The int4 GEMM refuses what its kernel does not cover instead of computing something else:
+    a scale group other than 32, K that is not whole groups, missing scales."""
+    a, w, c_ = lib.empty((8, 64)), lib.empty_bytes(64 * 64), lib.empty((8, 64))
+    n = C.c_int(0)
+    with pytest.raises(RuntimeError):
+        lib._chk(lib.c.tlhip_gemm_q4_nt(a.ptr, w.ptr, w.ptr + 2048, c_.ptr, 8, 64, 64, 64))      # group 64
+    with pytest.raises(RuntimeError):
+        lib._chk(lib.c.tlhip_gemm_q4_nt(a.ptr, w.ptr, w.ptr + 2048, c_.ptr, 8, 64, 48, 32))      # K % 32 != 0
+    with pytest.raises(RuntimeError):
+        lib._chk(lib.c.tlhip_gemm_q4_nt(a.ptr, w.ptr, None, c_.ptr, 8, 64, 64, 32))              # no scales
+    with pytest.raises(RuntimeError):
+        lib._chk(lib.c.tlhip_gemm_q4_nt_parts(a.ptr, w.ptr, w.ptr + 2048, c_.ptr, 16, 8, 64, 64, 32, C.byref(n)))  # no room
+    with pytest.raises(RuntimeError):
+        lib._chk(lib.c.tlhip_gemm_q4_nt_swiglu(a.ptr, w.ptr, w.ptr + 2048, c_.ptr, 8, 32, 64, 16))  # group 16
+    for b in (a, w, c_):
         b.free()
 
 
