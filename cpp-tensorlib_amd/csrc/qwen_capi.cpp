@@ -190,6 +190,29 @@ int tlq_fill_cache_random(void* hv, int64_t upto, uint32_t seed) {
   return qwen::fill_cache_random(static_cast<handle*>(hv)->M, upto, seed) ? 0 : -1;
 }
 
+// Overwrite a layer's f32 K and V caches with host arrays [n_kv_heads, max_ctx, head_dim] and set
+// every cache's position: a step or a chunk can then start deep in a context whose rows the caller
+// chose.
+int tlq_cache_upload(void* hv, int64_t layer, const float* K, const float* V, int64_t pos) {
+  auto* h = static_cast<handle*>(hv);
+  if (layer < 0 || layer >= (int64_t)h->M.layers.size()) return -1;
+  hip::kv_cache& c = h->M.layers[(size_t)layer].cache;
+  if (c.kv_bf16) return -1;
+  const int64_t bytes = c.n_kv_heads * c.max_ctx * c.D * 4;
+  hip::flush();
+  if (!hip::upload_raw(c.K, K, bytes) || !hip::upload_raw(c.V, V, bytes)) return -1;
+  qwen::set_cache_pos(h->M, pos);
+  return 0;
+}
+
+// The last chunk's final-norm rows [T, hidden] (what the lm_head would read), copied to out.
+int tlq_prefill_hidden(void* hv, float* out, int64_t T) {
+  auto* h = static_cast<handle*>(hv);
+  if (T <= 0 || T > h->M.ps.T) return -1;
+  hip::flush();
+  return hip::download_raw(out, h->M.ps.h, T * h->M.d.hidden * 4) ? 0 : -1;
+}
+
 // Greedy step; logits_out (may be NULL) receives the [vocab] logits.
 int64_t tlq_step(void* hv, int64_t token, int64_t pos, float* logits_out) {
   auto* h = static_cast<handle*>(hv);

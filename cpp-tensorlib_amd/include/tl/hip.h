@@ -444,6 +444,14 @@ inline bool upload_raw(void* dst_dev, const void* src_host, int64_t bytes) {
   return bytes == 0 || c.f.memcpy_h2d(dst_dev, src_host, (size_t)bytes) == 0;
 }
 
+// Blocking D2H from a device address (which may lie inside a managed buffer) into any host
+// memory; ordered after the launches queued so far.
+inline bool download_raw(void* dst_host, const void* src_dev, int64_t bytes) {
+  auto& c = context::get();
+  if (!c.ready || !dst_host || !src_dev || bytes < 0) return false;
+  return bytes == 0 || c.f.memcpy_d2h(dst_host, src_dev, (size_t)bytes) == 0;
+}
+
 inline void upload_u32(void* native, unsigned val) {
   auto& c = context::get();
   if (!c.ready || !native) return;

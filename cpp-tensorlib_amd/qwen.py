@@ -51,6 +51,8 @@ def _load():
             "tlq_prefill_layers": (cint, [P, i64, i64]),
             "tlq_set_cache_pos": (None, [P, i64]),
             "tlq_fill_cache_random": (cint, [P, i64, u32]),
+            "tlq_cache_upload": (cint, [P, i64, P, P, i64]),
+            "tlq_prefill_hidden": (cint, [P, P, i64]),
             "tlq_step": (i64, [P, i64, i64, P]),
             "tlq_run_layers": (cint, [P, i64, i64]),
             "tlq_argmax": (i64, [P]),
@@ -244,6 +246,22 @@ class QwenGPU:
     def fill_cache_random(self, upto, seed=2):
         if self.L.tlq_fill_cache_random(self.h, upto, seed) != 0:
             raise RuntimeError("tlq_fill_cache_random failed")
+
+    def cache_upload(self, layer, K, V, pos):
+        """Overwrite a layer's f32 caches with [n_kv_heads, max_ctx, head_dim] arrays; every
+        cache's position becomes pos."""
+        K, V = np.ascontiguousarray(K, np.float32), np.ascontiguousarray(V, np.float32)
+        want = self.d.n_kv_heads * self.d.max_ctx * self.d.head_dim
+        assert K.size == want and V.size == want
+        if self.L.tlq_cache_upload(self.h, layer, _p(K), _p(V), pos) != 0:
+            raise RuntimeError("cache_upload failed")
+
+    def prefill_hidden(self, T):
+        """Final-norm rows [T, hidden] of the last chunk run."""
+        out = np.empty((T, self.d.hidden), np.float32)
+        if self.L.tlq_prefill_hidden(self.h, _p(out), T) != 0:
+            raise RuntimeError("prefill_hidden: no chunk of that length was run")
+        return out
 
     def step(self, token, pos, want_logits=False):
         logits = np.empty(self.d.vocab, np.float32) if want_logits else None

@@ -9,8 +9,10 @@
 #include "oracle.h"
 
 #include <math.h>
+#include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
 /* ------------------------------------------------------------------------ */
 /* seeded inputs                                                             */
@@ -640,29 +642,72 @@ static float* vec_normal(int64_t n, uint32_t seed, float mean, float std) {
   return v;
 }
 
+/* Weight generation is a set of independent seeded streams (one per matrix), so it is
+ * spread over a few threads; every value is what the serial order produces. */
+typedef struct {
+  orc_lin* lin;         /* a linear weight ... */
+  int64_t K, N;
+  uint16_t* embed;      /* ... or the bf16 embedding table of n values */
+  int64_t n;
+  uint32_t seed;
+  int q4;
+} gen_task;
+
+typedef struct {
+  gen_task* tasks;
+  int n_tasks;
+  int next;
+  pthread_mutex_t mu;
+} gen_queue;
+
+static void* gen_worker(void* qv) {
+  gen_queue* q = (gen_queue*)qv;
+  for (;;) {
+    pthread_mutex_lock(&q->mu);
+    int i = q->next < q->n_tasks ? q->next++ : -1;
+    pthread_mutex_unlock(&q->mu);
+    if (i < 0) return NULL;
+    gen_task* t = &q->tasks[i];
+    if (t->lin) {
+      lin_init(t->lin, t->K, t->N, t->seed, t->q4);
+    } else {
+      float* emb = vec_normal(t->n, t->seed, 0.0f, 0.02f);
+      orc_to_bf16(emb, t->embed, t->n);
+      free(emb);
+    }
+  }
+}
+
+static int by_size_desc(const void* a, const void* b) {
+  const gen_task *x = (const gen_task*)a, *y = (const gen_task*)b;
+  int64_t sx = x->lin ? x->K * x->N : x->n, sy = y->lin ? y->K * y->N : y->n;
+  return sx < sy ? 1 : sx > sy ? -1 : 0;
+}
+
 orc_qwen* orc_qwen_create(const orc_qwen_dims* d, uint32_t seed, int q4) {
   orc_qwen* m = (orc_qwen*)calloc(1, sizeof(orc_qwen));
   m->d = *d;
   m->q4 = q4;
   const int64_t E = d->hidden, QD = d->n_q_heads * d->head_dim,
                 KD = d->n_kv_heads * d->head_dim;
-  float* emb = vec_normal(d->vocab * E, seed * 1000u + 1u, 0.0f, 0.02f);
+  gen_task* tasks = (gen_task*)calloc((size_t)(2 + 7 * d->n_layers), sizeof(gen_task));
+  int nt = 0;
+#define LIN(ptr, k, n, sd) do { gen_task t = {(ptr), (k), (n), NULL, 0, (sd), q4}; tasks[nt++] = t; } while (0)
   m->embed = (uint16_t*)malloc((size_t)(d->vocab * E) * 2);
-  orc_to_bf16(emb, m->embed, d->vocab * E);
-  free(emb);
+  { gen_task t = {NULL, 0, 0, m->embed, d->vocab * E, seed * 1000u + 1u, q4}; tasks[nt++] = t; }
   m->onorm = vec_normal(E, seed * 1000u + 2u, 1.0f, 0.02f);
-  lin_init(&m->outw, E, d->vocab, seed * 1000u + 3u, q4);
+  LIN(&m->outw, E, d->vocab, seed * 1000u + 3u);
   m->layers = (orc_layer*)calloc((size_t)d->n_layers, sizeof(orc_layer));
   for (int64_t l = 0; l < d->n_layers; l++) {
     orc_layer* L = &m->layers[l];
     uint32_t b = seed * 1000u + 100u + (uint32_t)l * 20u;
-    lin_init(&L->wq, E, QD, b + 1, q4);
-    lin_init(&L->wk, E, KD, b + 2, q4);
-    lin_init(&L->wv, E, KD, b + 3, q4);
-    lin_init(&L->wo, QD, E, b + 4, q4);
-    lin_init(&L->wg, E, d->ff, b + 5, q4);
-    lin_init(&L->wu, E, d->ff, b + 6, q4);
-    lin_init(&L->wd, d->ff, E, b + 7, q4);
+    LIN(&L->wq, E, QD, b + 1);
+    LIN(&L->wk, E, KD, b + 2);
+    LIN(&L->wv, E, KD, b + 3);
+    LIN(&L->wo, QD, E, b + 4);
+    LIN(&L->wg, E, d->ff, b + 5);
+    LIN(&L->wu, E, d->ff, b + 6);
+    LIN(&L->wd, d->ff, E, b + 7);
     L->bq = vec_normal(QD, b + 8, 0.0f, 0.02f);
     L->bk = vec_normal(KD, b + 9, 0.0f, 0.02f);
     L->bv = vec_normal(KD, b + 10, 0.0f, 0.02f);
@@ -671,7 +716,27 @@ orc_qwen* orc_qwen_create(const orc_qwen_dims* d, uint32_t seed, int q4) {
     L->Kc = (float*)calloc((size_t)(d->n_kv_heads * d->max_ctx * d->head_dim), sizeof(float));
     L->Vc = (float*)calloc((size_t)(d->n_kv_heads * d->max_ctx * d->head_dim), sizeof(float));
   }
+#undef LIN
+  qsort(tasks, (size_t)nt, sizeof(gen_task), by_size_desc);   /* largest first */
+  gen_queue q = {tasks, nt, 0, PTHREAD_MUTEX_INITIALIZER};
+  long cpus = sysconf(_SC_NPROCESSORS_ONLN);
+  int n_thr = (int)(cpus < 1 ? 1 : cpus > 8 ? 8 : cpus);
+  if (n_thr > nt) n_thr = nt;
+  pthread_t thr[8];
+  int started = 0;
+  for (int i = 1; i < n_thr; i++)
+    if (pthread_create(&thr[started], NULL, gen_worker, &q) == 0) started++;
+  gen_worker(&q);
+  for (int i = 0; i < started; i++) pthread_join(thr[i], NULL);
+  free(tasks);
   return m;
+}
+
+/* The host K (which = 0) or V (which = 1) cache of a layer, [n_kv_heads, max_ctx, head_dim]:
+ * lets a test start a step deep in a context from seeded cache rows. */
+float* orc_qwen_cache(orc_qwen* m, int64_t layer, int which) {
+  if (layer < 0 || layer >= m->d.n_layers) return NULL;
+  return which ? m->layers[layer].Vc : m->layers[layer].Kc;
 }
 
 void orc_qwen_destroy(orc_qwen* m) {

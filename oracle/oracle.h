@@ -143,6 +143,8 @@ int64_t   orc_qwen_step(orc_qwen* m, int64_t token, int64_t pos, float* logits);
 /* accessors so the GPU harness can upload the very same weight bytes */
 int       orc_qwen_set(orc_qwen* m, int64_t layer, const char* name, const float* data);
 const void*  orc_qwen_weight(const orc_qwen* m, int64_t layer, const char* name, int64_t* bytes);
+/* host K (which = 0) / V (which = 1) cache of a layer, [n_kv_heads, max_ctx, head_dim] */
+float*    orc_qwen_cache(orc_qwen* m, int64_t layer, int which);
 
 #ifdef __cplusplus
 }

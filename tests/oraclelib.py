@@ -91,6 +91,7 @@ class Oracle:
             "orc_qwen_step": (i64, [P, i64, i64, P]),
             "orc_qwen_weight": (P, [P, i64, C.c_char_p, C.POINTER(i64)]),
             "orc_qwen_set": (cint, [P, i64, C.c_char_p, P]),
+            "orc_qwen_cache": (P, [P, i64, cint]),
             "orc_f16_widen": (None, [P, P, i64]),
         }
         for name, (res, args) in sig.items():
@@ -323,6 +324,17 @@ class OracleQwen:
         logits = np.empty(self.d.vocab, np.float32)
         tok = self.orc.lib.orc_qwen_step(self.h, token, pos, _ptr(logits))
         return int(tok), logits
+
+    def cache(self, layer):
+        """The host K and V caches of a layer as writable [n_kv_heads, max_ctx, head_dim] views."""
+        d = self.d
+        n = d.n_kv_heads * d.max_ctx * d.head_dim
+        out = []
+        for which in (0, 1):
+            p = self.orc.lib.orc_qwen_cache(self.h, layer, which)
+            buf = (C.c_float * n).from_address(p)
+            out.append(np.frombuffer(buf, np.float32).reshape(d.n_kv_heads, d.max_ctx, d.head_dim))
+        return out
 
     def set(self, layer, name, data):
         """Replace a weight: linear layers as f32 in the logical [K,N] layout (stored in the model's

@@ -368,6 +368,7 @@ def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, valu=False):
     (128, 28, 4, 64, 0), (64, 14, 2, 100, 0), (128, 4, 2, 7, 0), (128, 8, 8, 33, 300),
     (64, 6, 2, 257, 19), (128, 2, 1, 1, 0), (128, 2, 1, 1, 77), (64, 4, 4, 130, 513),
     (128, 7, 1, 512, 0), (64, 2, 2, 512, 0), (128, 2, 1, 200, 1000), (128, 1, 1, 31, 32), (64, 3, 1, 32, 31),
+    (128, 7, 1, 512, 3584), (128, 4, 4, 256, 7680),      # deep in a context: > 120 key tiles per wavefront
 ])
 def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, valu):
     """Causal prefill over a cache: query p at absolute position pos0+p sees keys
