@@ -64,6 +64,7 @@ SIGNATURES = {
     "tlhip_gemv_bf16_row": (cint, [P, P, P, i64, i64]),
     "tlhip_gemv_q4": (cint, [P, P, P, P, i64, i64, i64]),
     "tlhip_attn_decode": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
+    "tlhip_attn_decode_static": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint]),
     "tlhip_attn_prefill": (cint, [P, P, P, P, i64, i64, i64, i64, i64, f32, cint, i64]),
     "tlhip_kv_append": (cint, [P, P, P, P, i64, i64, i64, i64, cint]),
     "tlhip_kv_fill": (cint, [P, P, P, P, i64, i64, i64, i64, cint, i64]),
@@ -270,6 +271,10 @@ class TlHip:
     def attn_decode(self, q, K, V, out, Hq, Hkv, ctx, kv_max, D, scale, kv_bf16=False):
         self._chk(self.c.tlhip_attn_decode(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, ctx, kv_max, D,
                                            scale, int(kv_bf16)))
+
+    def attn_decode_static(self, q, K, V, out, Hq, Hkv, ctx, kv_max, D, scale, kv_bf16=False):
+        self._chk(self.c.tlhip_attn_decode_static(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, ctx, kv_max, D,
+                                                  scale, 1 if kv_bf16 else 0))
 
     def attn_prefill(self, q, K, V, out, Hq, Hkv, T, kv_max, D, scale, kv_bf16=False, pos0=0):
         self._chk(self.c.tlhip_attn_prefill(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, T, kv_max, D,

@@ -622,9 +622,10 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     const size_t hs = (size_t)Hq * S;
     const size_t need = attn_partials_floats(Hq, S, D) * sizeof(float);
     float* base;
-    if (dpos) {
+    if (dpos || partials) {   // a buffer the caller named: never the library's growable scratch
       if (!partials || partials_bytes < need)
-        return fail(TLHIP_EINVAL, "tlhip_attn_decode_dpos: partials buffer of %zu bytes needed", need);
+        return fail(TLHIP_EINVAL, "attention: %zu bytes of split partials needed, the buffer given holds %zu",
+                    need, partials_bytes);
       base = partials;
     } else {
       base = static_cast<float*>(scratch(need));
@@ -682,11 +683,73 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
 }
 
+// ---- memory of the entry point that allocates nothing -------------------------------------
+// tlhip_attn_decode_static keeps its split partials in this array instead of the library's
+// growable scratch. Each GPU holds its own copy at its own address; host code never uses the
+// array's name as an address, only the pointer hipGetSymbolAddress returned for that device.
+namespace fixed {
+constexpr size_t kBytes = size_t(1) << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kBytes];
+static void* dev_ptr[kMaxDevices] = {};   // per device: where that device's copy lives
+}  // namespace fixed
+
+// Resolves the array's address on `device`, which must be the current one. Called by tlhip_init.
+int attn_static_setup(int device) {
+  if (device < 0 || device >= fixed::kMaxDevices) return fail(TLHIP_EINVAL, "device %d out of range", device);
+  if (fixed::dev_ptr[device]) return TLHIP_OK;
+  void* p = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(fixed::scratch));
+  if (e != hipSuccess || !p) return hip_fail(e, "hipGetSymbolAddress");
+  fixed::dev_ptr[device] = p;
+  return TLHIP_OK;
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;
 
 extern "C" {
+
+int tlhip_attn_decode_static(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
+                             int64_t n_kv_heads, int64_t ctx_len, int64_t kv_max, int64_t D, float scale,
+                             int kv_bf16) {
+  Context& c = ctx();
+  if (!c.ready)   // tlhip_init allocates (stream, result slots); this entry point may not
+    return fail(TLHIP_ERUNTIME, "tlhip_attn_decode_static: call tlhip_init first");
+  void* fixed_ptr = c.device >= 0 && c.device < fixed::kMaxDevices ? fixed::dev_ptr[c.device] : nullptr;
+  if (!fixed_ptr) return fail(TLHIP_ERUNTIME, "tlhip_attn_decode_static: fixed buffer not resolved on device %d", c.device);
+  if (!q || !K || !V || !out) return fail(TLHIP_EINVAL, "tlhip_attn_decode_static: null pointer");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_static: head_dim must be 64 or 128");
+  if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_static: Hq must be a positive multiple of Hkv");
+  if (ctx_len <= 0 || ctx_len > kv_max) return fail(TLHIP_EINVAL, "tlhip_attn_decode_static: need 0 < ctx <= kv_max");
+  if (ctx_len > 0x3fffffff || n_kv_heads > 65535 || n_q_heads > 0x7fffffff || kv_max * D > ((int64_t)1 << 40))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_static: shape too large");
+  if (!aligned16(q) || !aligned16(K) || !aligned16(V) || !aligned16(out))
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_static: operands must be 16-byte aligned");
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads, cx = (int)ctx_len;
+  // the same launch plan as tlhip_attn_decode; its split partials must fit the fixed array
+  const AttnPlan p = plan_attn(Hkv, Hq / Hkv, cx, c.cus, false);
+  const size_t need = p.S > 1 ? attn_partials_floats(Hq, p.S, (int)D) * sizeof(float) : 0;
+  if (need > fixed::kBytes)
+    return fail(TLHIP_EUNSUPPORTED,
+                "tlhip_attn_decode_static: this shape splits the context %d ways and needs %zu bytes of "
+                "partials; the fixed buffer holds %zu (use tlhip_attn_decode)", p.S, need, fixed::kBytes);
+  const float* pq = static_cast<const float*>(q);
+  float* po = static_cast<float*>(out);
+  float* part = static_cast<float*>(fixed_ptr);
+  if (kv_bf16) {
+    const uint16_t* pk = static_cast<const uint16_t*>(K);
+    const uint16_t* pv = static_cast<const uint16_t*>(V);
+    return D == 128 ? launch_attn<128, uint16_t>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, nullptr, part, fixed::kBytes)
+                    : launch_attn<64, uint16_t>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, nullptr, part, fixed::kBytes);
+  }
+  const float* pk = static_cast<const float*>(K);
+  const float* pv = static_cast<const float*>(V);
+  return D == 128 ? launch_attn<128, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, nullptr, part, fixed::kBytes)
+                  : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, nullptr, part, fixed::kBytes);
+}
 
 int tlhip_attn_decode(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,
                       int64_t n_kv_heads, int64_t ctx_len, int64_t kv_max, int64_t D, float scale,

@@ -43,6 +43,7 @@ Context& ctx();
 int fail(int code, const char* fmt, ...);   // records the message, returns code
 int hip_fail(hipError_t e, const char* what);
 void* scratch(size_t bytes);                // nullptr on allocation failure
+int attn_static_setup(int device);          // attn.hip: address of the allocation-free entry point's array
 
 inline const char* at(const void* base, int64_t byte_off) {
   return static_cast<const char*>(base) + byte_off;

@@ -115,6 +115,7 @@ int tlhip_init(int device) {
   if ((e = hipMalloc((void**)&c.argmax_dev, 256)) != hipSuccess) return hip_fail(e, "hipMalloc");
   if ((e = hipHostMalloc((void**)&c.argmax_host, 256, hipHostMallocDefault)) != hipSuccess)
     return hip_fail(e, "hipHostMalloc");
+  if (int rc = attn_static_setup(device)) return rc;
   c.device = device;
   c.cus = prop.multiProcessorCount;
   c.lds_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;

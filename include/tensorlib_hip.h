@@ -147,6 +147,18 @@ int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, in
 int tlhip_attn_decode(const void* q, const void* K, const void* V, void* out,
                       int64_t n_q_heads, int64_t n_kv_heads, int64_t ctx, int64_t kv_max,
                       int64_t D, float scale, int kv_bf16);
+/* tlhip_attn_decode for callers that cannot allocate device memory (code under hipGraph
+ * capture, serving loops and harnesses that forbid hipMalloc). No counterpart in the reference.
+ * Same arguments, same launch plan and bit-identical results; the split partials live in a
+ * 1 MiB array that is part of the library's code object (one copy per GPU, held until the process
+ * ends) instead of the library's growable scratch, and the call itself allocates and frees
+ * nothing. Needs a prior tlhip_init (which does allocate). A shape whose partials exceed 1 MiB
+ * (Hq * splits * (D + 2) * 4 bytes; the BASELINE shapes need at most 466 KB) is refused with
+ * TLHIP_EUNSUPPORTED. Every call on a GPU shares that GPU's array: calls that overlap on one
+ * GPU race. Nothing in the array has to start at zero (each call writes every partial it reads). */
+int tlhip_attn_decode_static(const void* q, const void* K, const void* V, void* out,
+                             int64_t n_q_heads, int64_t n_kv_heads, int64_t ctx, int64_t kv_max,
+                             int64_t D, float scale, int kv_bf16);
 /* causal prefill: q,out [Hq,T,D]; query p is at position pos0+p and sees keys
  * [0,pos0+p].  cuda.h:1166-1201 */
 int tlhip_attn_prefill(const void* q, const void* K, const void* V, void* out,
