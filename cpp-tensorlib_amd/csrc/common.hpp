@@ -71,6 +71,21 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // ---- device helpers ----------------------------------------------------------
 #if defined(__HIPCC__)
 
+// Phase timestamps for kernel tuning. Off in the library build; a single-translation-unit
+// build with TLHIP_TRACE defined makes lane 0 of every wavefront record the shader clock at
+// the marks, into g_trace[block][wave][slot].
+#ifdef TLHIP_TRACE
+constexpr int kTraceSlots = 8, kTraceWaves = 16, kTraceBlocks = 1024;
+static __device__ unsigned long long g_trace[kTraceBlocks * kTraceWaves * kTraceSlots];
+__device__ __forceinline__ void trace_mark(int slot) {
+  if ((threadIdx.x & 63) == 0 && blockIdx.x < kTraceBlocks)
+    g_trace[(blockIdx.x * kTraceWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = __builtin_readcyclecounter();
+}
+#define TLHIP_MARK(slot) ::tlhip::trace_mark(slot)
+#else
+#define TLHIP_MARK(slot)
+#endif
+
 // One rounding each, never contracted into an FMA with a neighbouring operation: the CPU path
 // multiplies and adds separately (its loops are compiled without FMA contraction). hipcc's
 // __fmul_rn / __fadd_rn are plain `*` / `+` and do NOT prevent contraction; these do, because

@@ -18,85 +18,9 @@
 //     partials go to scratch and are summed in a fixed order by a second
 //     kernel.
 #include "common.hpp"
+#include "gemv_shared.hpp"
 
 namespace tlhip {
-
-// ---------------------------------------------------------------------------
-// weight formats for the row kernel
-// ---------------------------------------------------------------------------
-
-// 16-byte streaming load: weights are read exactly once per GEMV, so they are
-// marked non-temporal and do not displace x and the scales in the caches.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 load_stream16(const uint4* p) {
-  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
-}
-
-// int4: a byte of a packed row holds k even in its low nibble and k+1 in its
-// high nibble. Instead of isolating the high nibble, the kernel converts the
-// WHOLE byte (lo + 16*hi) and the masked low nibble, and folds the difference
-// into the activations when they are staged:
-//     lo*x_e + hi*x_o  =  lo*(x_e - x_o/16) + (lo + 16*hi)*(x_o/16)
-// so a 32-bit word of 8 weights costs one v_and, eight v_cvt_f32_ubyteN and
-// eight FMAs. The "-8" of the offset-binary nibbles becomes -8*sum(x) per
-// group, also formed once at staging.
-__device__ __forceinline__ uint32_t low_nibbles(uint32_t v) {
-  uint32_t r;  // opaque to the optimiser so the byte converts below stay byte converts
-  asm("v_and_b32 %0, 0x0f0f0f0f, %1" : "=v"(r) : "v"(v));
-  return r;
-}
-__device__ __forceinline__ float byte0(uint32_t v) { return (float)(v & 0xffu); }
-__device__ __forceinline__ float byte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
-__device__ __forceinline__ float byte2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
-__device__ __forceinline__ float byte3(uint32_t v) { return (float)(v >> 24); }
-
-struct FmtQ4 {
-  static constexpr int E = 32;  // weights per 16-byte unit == one scale group
-  static constexpr bool kScaled = true;
-  // staged form of (x_even, x_odd, x_even, x_odd)
-  static __device__ __forceinline__ float4 stage(const float4 v) {
-    const float o0 = v.y * 0.0625f, o1 = v.w * 0.0625f;
-    return make_float4(v.x - o0, o0, v.z - o1, o1);
-  }
-  // sum_k nib_k * x_k over the unit, x in staged form
-  static __device__ __forceinline__ float dot(const uint4 w, const float4 (&x)[8]) {
-    const uint32_t d[4] = {w.x, w.y, w.z, w.w};
-    float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const uint32_t full = d[i], lo = low_nibbles(full);
-      const float4 xa = x[2 * i], xb = x[2 * i + 1];
-      a0 = fmaf(byte0(lo), xa.x, a0);
-      a1 = fmaf(byte0(full), xa.y, a1);
-      a0 = fmaf(byte1(lo), xa.z, a0);
-      a1 = fmaf(byte1(full), xa.w, a1);
-      a0 = fmaf(byte2(lo), xb.x, a0);
-      a1 = fmaf(byte2(full), xb.y, a1);
-      a0 = fmaf(byte3(lo), xb.z, a0);
-      a1 = fmaf(byte3(full), xb.w, a1);
-    }
-    return a0 + a1;
-  }
-};
-
-struct FmtBf16 {
-  static constexpr int E = 8;
-  static constexpr bool kScaled = false;
-  static __device__ __forceinline__ float4 stage(const float4 v) { return v; }
-  static __device__ __forceinline__ float dot(const uint4 w, const float4 (&x)[2]) {
-    float a0 = 0.f, a1 = 0.f;
-    a0 = fmaf(bf16_lo(w.x), x[0].x, a0);
-    a1 = fmaf(bf16_hi(w.x), x[0].y, a1);
-    a0 = fmaf(bf16_lo(w.y), x[0].z, a0);
-    a1 = fmaf(bf16_hi(w.y), x[0].w, a1);
-    a0 = fmaf(bf16_lo(w.z), x[1].x, a0);
-    a1 = fmaf(bf16_hi(w.z), x[1].y, a1);
-    a0 = fmaf(bf16_lo(w.w), x[1].z, a0);
-    a1 = fmaf(bf16_hi(w.w), x[1].w, a1);
-    return a0 + a1;
-  }
-};
 
 // ---------------------------------------------------------------------------
 // row kernel
@@ -122,95 +46,23 @@ template <typename Fmt, int R, bool PAIR = false>
 __device__ __forceinline__ void load_frag(RowFrag<Fmt, R>& f, const uint4* __restrict__ W,
                                           const float* __restrict__ scales, int N, int upr,
                                           int row0, int u) {
-  if (u < upr) {
-    const char* wb = reinterpret_cast<const char*>(W);
-    const char* sb = reinterpret_cast<const char*>(scales);
+  // Branch-free: a lane past the end of the row re-reads the row's last unit (its result is
+  // never used). Loads under a condition would make the compiler's wait counters
+  // conservative - every wait would also cover the loads issued after the ones it needs.
+  u = min(u, upr - 1);
+  const char* wb = reinterpret_cast<const char*>(W);
+  const char* sb = reinterpret_cast<const char*>(scales);
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      const uint32_t row = PAIR ? (uint32_t)(min(row0 + (r % (R / 2 > 0 ? R / 2 : 1)), N / 2 - 1) +
-                                             (r >= R / 2 ? N / 2 : 0))
-                                : (uint32_t)min(row0 + r, N - 1);
-      const uint32_t idx = __umul24(row, (uint32_t)upr) + (uint32_t)u;
-      f.w[r] = load_stream16(reinterpret_cast<const uint4*>(wb + (idx << 4)));
-      if (Fmt::kScaled)
-        f.sc[r] = __builtin_nontemporal_load(reinterpret_cast<const float*>(sb + (idx << 2)));
-    }
+  for (int r = 0; r < R; r++) {
+    const uint32_t row = PAIR ? (uint32_t)(min(row0 + (r % (R / 2 > 0 ? R / 2 : 1)), N / 2 - 1) +
+                                           (r >= R / 2 ? N / 2 : 0))
+                              : (uint32_t)min(row0 + r, N - 1);
+    const uint32_t idx = __umul24(row, (uint32_t)upr) + (uint32_t)u;
+    f.w[r] = load_stream16(reinterpret_cast<const uint4*>(wb + (idx << 4)));
+    if (Fmt::kScaled)
+      f.sc[r] = __builtin_nontemporal_load(reinterpret_cast<const float*>(sb + (idx << 2)));
   }
 }
-
-// ---- 16-lane sum on DPP: every lane of a DPP row ends up with the row's total ----
-template <int CTRL>
-__device__ __forceinline__ float dpp_add_f32(float v) {
-  const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
-  return v + __int_as_float(t);
-}
-
-// Sum R per-lane partials over the wavefront at once. Halving steps trade
-// values for lanes (lane bit m clear keeps the lower half of the values and
-// receives the partner's contribution to them), so R values cost R-1 exchanges
-// instead of 6R; what is left is one value per lane, finished inside its lane
-// group on DPP. Returns, in every lane, the total of row (lane * R) >> 6.
-template <int N, int M, int R>
-__device__ __forceinline__ void halve_rows(float (&a)[R], int lane) {  // N live values -> N/2
-  if constexpr (M == 32 || M == 16) {
-    // one v_permlane swap hands the lower lanes both halves' a[i] and the upper lanes both
-    // halves' a[i + N/2]: the same two operands the shuffle form adds
-#pragma unroll
-    for (int i = 0; i < N / 2; i++) {
-      const LanePair p = M == 32 ? swap32(a[i], a[i + N / 2]) : swap16(a[i], a[i + N / 2]);
-      a[i] = p.first + p.second;
-    }
-  } else {
-    const bool up = (lane & M) != 0;
-#pragma unroll
-    for (int i = 0; i < N / 2; i++) {
-      const float keep = up ? a[i + N / 2] : a[i];
-      const float send = up ? a[i] : a[i + N / 2];
-      a[i] = keep + __shfl_xor(send, M, kWave);
-    }
-  }
-}
-
-template <int R>
-__device__ __forceinline__ float wave_sum_rows(float (&a)[R], int lane) {
-  static_assert(R == 1 || R == 2 || R == 4 || R == 8, "rows per wavefront");
-  if constexpr (R == 8) { halve_rows<8, 32>(a, lane); halve_rows<4, 16>(a, lane); halve_rows<2, 8>(a, lane); }
-  if constexpr (R == 4) { halve_rows<4, 32>(a, lane); halve_rows<2, 16>(a, lane); }
-  if constexpr (R == 2) { halve_rows<2, 32>(a, lane); }
-  float v = a[0];
-  // lanes that differ only in bits below the last halving mask share a row
-  if (R <= 1) { const LanePair p = swap32(v, v); v = p.first + p.second; }
-  if (R <= 2) { const LanePair p = swap16(v, v); v = p.first + p.second; }
-  v = dpp_add_f32<0xB1>(v);                 // quad_perm [1,0,3,2]
-  v = dpp_add_f32<0x4E>(v);                 // quad_perm [2,3,0,1]
-  v = dpp_add_f32<0x141>(v);                // row_half_mirror: the two quads of 8 lanes
-  if (R <= 4) v = dpp_add_f32<0x140>(v);    // row_mirror: the two halves of 16 lanes
-  return v;
-}
-
-// How a block obtains the activation vector while it stages it. Folding the
-// producer of x into the GEMV removes a launch and a round trip through memory;
-// every block recomputes the (tiny) producer redundantly.
-//   kPlain:   x is read as is.
-//   kSwiglu:  x[k] = (g*sigmoid(g))*u with g = in[k], u = in[K + k]   (array.h:2435-2439)
-//   kRmsnorm: s = in (+ delta); x = (s * 1/sqrt(mean(s*s) + eps)) * norm_w   (array.h:2429-2433);
-//             block 0 also writes s to xout (the residual stream), which therefore
-//             must not alias in or delta: other blocks still read them.
-// How a block leaves its results (EPI):
-//   kStore:  y[row] = dot.
-//   kGateUp: W is [gate rows | up rows] (N/2 each); a lane group owns R/2 gate rows and the
-//            matching up rows, and writes y[i] = (g*sigmoid(g))*u for i < N/2 - the gated
-//            activation in the GEMV that produces it, once per element, instead of in every
-//            block of the GEMV that consumes it.
-enum { kPlain = 0, kSwiglu = 1, kRmsnorm = 2 };
-enum { kStore = 0, kGateUp = 1 };
-__device__ __forceinline__ float gated(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
-struct Producer {
-  const float* delta;
-  const float* norm_w;
-  float* xout;
-  float eps;
-};
 
 // LPR = lanes that share a weight row: 64 (a row segment of 64 units per
 // wavefront step) or 16 (the wavefront works on 4 row groups at once, 16 units
@@ -220,12 +72,15 @@ struct Producer {
 // finishes a row sum inside one DPP row.
 template <typename Fmt, int R, int PRO, int LPR, int EPI = kStore>
 __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
-    const float* __restrict__ x, const uint4* __restrict__ W, const float* __restrict__ scales,
+    const float* x, const uint4* __restrict__ W, const float* __restrict__ scales,
     float* __restrict__ y, int N, int upr, int KW, int ntiles, const Producer pro) {
   constexpr int J = Fmt::E / 4;
   constexpr int QN = 64 / LPR;       // row groups a wavefront works on at once
   extern __shared__ float4 smem4[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // wavefront-uniform, and known to be: the loop over work items then runs on scalar
+  // branches, which also keeps the compiler's wait counters exact
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & (LPR - 1), q = lane / LPR;
   const int nw = blockDim.x >> 6;
   const int chunks = (upr + LPR - 1) / LPR;
@@ -243,34 +98,72 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   // first row of work item (tile tt): a row of W, or with kPair a row of each half
   const auto item_row = [&](int tt) { return kPair ? (tt * rows_per_tile + wrow) >> 1 : tt * rows_per_tile + wrow; };
 
-  // The first work item's weights are requested before x is staged, so that the
-  // HBM latency of the weights and the L2 latency of x overlap.
-  int t = blockIdx.x, c = kw;
-  RowFrag<Fmt, R> cur;
-  if (t < ntiles) load_frag<Fmt, R, kPair>(cur, W, scales, N, upr, item_row(t), c * LPR + li);
+  // Requests go out in this order: the activations (and what their producer reads) first, then
+  // the first work item's weights. A wavefront's loads return in order, so x requested after
+  // the weights would keep the staging pass waiting for them.
+  TLHIP_MARK(0);
+  const float4* x4 = reinterpret_cast<const float4*>(x);
+  const int n4 = upr * J;
+  const float4* d4 = reinterpret_cast<const float4*>(pro.delta);
+  constexpr int PL = 2;   // float4s a thread requests up front (all of x up to 8 * threads floats)
+  float4 px[PL], pa[PL], pn[PL];
+  {
+    const float4* aux4 = PRO == kSwiglu ? x4 + n4 : (d4 ? d4 : x4);   // up half, or delta (x when none: ignored)
+#pragma unroll
+    for (int k = 0; k < PL; k++) {
+      const int i = min(tid + k * (int)blockDim.x, n4 - 1);
+      px[k] = x4[i];
+      if (PRO != kPlain) pa[k] = aux4[i];
+      if (PRO == kRmsnorm) pn[k] = reinterpret_cast<const float4*>(pro.norm_w)[i];
+    }
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  // This wavefront's work items, numbered i = 0, 1, ...: item i is chunk kw + (i % cpw) * KW of
+  // the block's tile number i / cpw. Two items are kept in flight (NS).
+  constexpr int NS = 2;
+  // chunks per tile for this wavefront; one (idle) when KW exceeds the chunk count, so that
+  // the wavefront still meets the block's barriers at every tile end
+  const int cpw = max((chunks - kw + KW - 1) / KW, 1);
+  const int my_tiles = (int)blockIdx.x < ntiles ? (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+  const int n_items = my_tiles * cpw;
+  const auto load_item = [&](RowFrag<Fmt, R>& f, int i) {
+    const int ti = i / cpw, ci = i - ti * cpw;
+    const int tt = min((int)blockIdx.x + ti * (int)gridDim.x, ntiles - 1);
+    load_frag<Fmt, R, kPair>(f, W, scales, N, upr, item_row(tt), (kw + ci * KW) * LPR + li);
+  };
+  RowFrag<Fmt, R> frag[NS];
+  load_item(frag[0], 0);
+  TLHIP_MARK(1);
 
   {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
      // thread i owns float4 i; the J threads of a unit are adjacent lanes, so the
      // unit's sum(x) is a J-lane shuffle reduction (J is 8 or 2, both divide 64).
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    const int n4 = upr * J;
     const int n4_padded = (n4 + 63) & ~63;   // whole wavefronts take part in the shuffles
-    const float4* d4 = reinterpret_cast<const float4*>(pro.delta);
+    // float4 number k of this thread before the norm: x (+ delta), or swiglu(gate, up);
+    // nv receives its norm weights. The first PL come from the registers requested above.
+    const auto raw = [&](int k, int i, float4& nv) -> float4 {
+      float4 v, aux;
+      bool have = false;
+#pragma unroll
+      for (int kk = 0; kk < PL; kk++)
+        if (k == kk) { v = px[kk]; aux = pa[kk]; nv = pn[kk]; have = true; }
+      if (!have) {
+        v = x4[i];
+        if (PRO == kSwiglu) aux = x4[n4 + i];
+        if (PRO == kRmsnorm) { nv = reinterpret_cast<const float4*>(pro.norm_w)[i]; if (d4) aux = d4[i]; }
+      }
+      if (PRO == kRmsnorm && d4) { v.x += aux.x; v.y += aux.y; v.z += aux.z; v.w += aux.w; }
+      if (PRO == kSwiglu) { v.x = gated(v.x, aux.x); v.y = gated(v.y, aux.y); v.z = gated(v.z, aux.z); v.w = gated(v.w, aux.w); }
+      return v;
+    };
     float inv = 0.f;
-    // the first two float4s a thread owns (all of them for rows up to 2 * blockDim * 4
-    // floats) stay in registers between the two passes of the norm
-    float4 kept0 = make_float4(0.f, 0.f, 0.f, 0.f), kept1 = kept0;
-    float4 keptw0 = kept0, keptw1 = kept0;   // their norm weights, requested ahead of the block sum
     if (PRO == kRmsnorm) {   // mean square of the row, summed in a fixed order
       float ss = 0.f;
-      int it = 0;
-      for (int i = tid; i < n4; i += blockDim.x, it++) {
-        float4 v = x4[i];
-        if (it == 0) keptw0 = reinterpret_cast<const float4*>(pro.norm_w)[i];
-        if (it == 1) keptw1 = reinterpret_cast<const float4*>(pro.norm_w)[i];
-        if (d4) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
-        if (it == 0) kept0 = v;
-        if (it == 1) kept1 = v;
+      int k = 0;
+      for (int i = tid; i < n4; i += blockDim.x, k++) {
+        float4 nv;
+        const float4 v = raw(k, i, nv);
         ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
       }
       ss = wave_sum(ss);
@@ -281,25 +174,18 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       inv = 1.0f / sqrtf(tot * (1.0f / (float)(n4 * 4)) + pro.eps);
       // red is reused only after the barrier that ends the staging pass
     }
-    int it2 = 0;
-    for (int i = tid; i < n4_padded; i += blockDim.x, it2++) {
+    int k2 = 0;
+    for (int i = tid; i < n4_padded; i += blockDim.x, k2++) {
       const bool live = i < n4;
-      const bool have = PRO == kRmsnorm && it2 < 2;   // already summed with delta, in registers
-      float4 v = have ? (it2 == 0 ? kept0 : kept1)
-                      : live ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-      if (PRO == kSwiglu && live) {
-        const float4 up = x4[n4 + i];
-        v.x = (v.x * (1.0f / (1.0f + expf(-v.x)))) * up.x;
-        v.y = (v.y * (1.0f / (1.0f + expf(-v.y)))) * up.y;
-        v.z = (v.z * (1.0f / (1.0f + expf(-v.z)))) * up.z;
-        v.w = (v.w * (1.0f / (1.0f + expf(-v.w)))) * up.w;
-      }
-      if (PRO == kRmsnorm && live) {
-        if (d4 && !have) { const float4 d = d4[i]; v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w; }
-        if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
-        const float4 w4 = have ? (it2 == 0 ? keptw0 : keptw1) : reinterpret_cast<const float4*>(pro.norm_w)[i];
-        v.x = (v.x * inv) * w4.x; v.y = (v.y * inv) * w4.y;
-        v.z = (v.z * inv) * w4.z; v.w = (v.w * inv) * w4.w;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (live) {
+        float4 nv;
+        v = raw(k2, i, nv);
+        if (PRO == kRmsnorm) {
+          if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
+          v.x = (v.x * inv) * nv.x; v.y = (v.y * inv) * nv.y;
+          v.z = (v.z * inv) * nv.z; v.w = (v.w * inv) * nv.w;
+        }
       }
       const int u = i / J, j = i - u * J;
       if (live) xs[((u / LPR) * J + j) * LPR + (u & (LPR - 1))] = Fmt::stage(v);
@@ -318,20 +204,17 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     }
   }
   __syncthreads();
+  TLHIP_MARK(2);
 
   float acc[R];
 #pragma unroll
   for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-  // Software pipeline over this wavefront's (tile, chunk) items: the next item's
-  // loads are in flight while the current one is unpacked and accumulated. The
-  // two fragments swap roles every step (no register copies).
-  auto step = [&](const RowFrag<Fmt, R>& cur, RowFrag<Fmt, R>& nxt) -> bool {
-    int nc = c + KW, nt = t;
-    if (nc >= chunks) { nc = kw; nt = t + gridDim.x; }
-    if (nt < ntiles)
-      load_frag<Fmt, R, kPair>(nxt, W, scales, N, upr, item_row(nt), nc * LPR + li);
-
+  // Software pipeline over the items: NS fragments in flight, each requested again right after
+  // it has been consumed. Loads are branch-free in the steady-state loop, so the waits of a
+  // compute cover exactly its own fragment.
+  int t = 0, c = 0, nt = 0;   // the item being computed: tile, chunk; nt != t at a tile's last chunk
+  const auto compute = [&](const RowFrag<Fmt, R>& cur) {   // item (t, c); nt != t ends its tile
     const int u = c * LPR + li;
     if (u < upr) {
       float4 xv[J];
@@ -395,15 +278,39 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
 #pragma unroll
       for (int r2 = 0; r2 < R; r2++) acc[r2] = 0.f;
     }
-    t = nt;
-    c = nc;
-    return t < ntiles;
   };
-  RowFrag<Fmt, R> other;
-  if (t < ntiles) {
-    while (step(cur, other) && step(other, cur)) {
+  const auto compute_item = [&](const RowFrag<Fmt, R>& f, int i) {
+    const int ti = i / cpw, ci = i - ti * cpw;
+    t = (int)blockIdx.x + ti * (int)gridDim.x;
+    c = kw + ci * KW;
+    nt = ci == cpw - 1 ? -1 : t;
+    compute(f);
+  };
+  if (n_items >= NS) {
+#pragma unroll
+    for (int k = 1; k < NS; k++) load_item(frag[k], k);
+    int it = 0;
+    for (; it + 2 * NS <= n_items; it += NS) {
+#pragma unroll
+      for (int k = 0; k < NS; k++) {
+        compute_item(frag[k], it + k);
+        load_item(frag[k], it + k + NS);
+      }
     }
+    TLHIP_MARK(3);
+    for (; it < n_items; it += NS) {
+#pragma unroll
+      for (int k = 0; k < NS; k++) {
+        if (it + k < n_items) {
+          compute_item(frag[k], it + k);
+          if (it + k + NS < n_items) load_item(frag[k], it + k + NS);
+        }
+      }
+    }
+  } else if (n_items == 1) {   // a single item: nothing more to request
+    compute_item(frag[0], 0);
   }
+  TLHIP_MARK(4);
 }
 
 // Generic int4 kernel for group sizes other than 32 (group % 8 == 0): one
@@ -558,15 +465,15 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(const float* __re
 struct RowCfg { int R, KW, nw, lpr, blocks; size_t lds; };
 struct RowTune { int R, KW, bpc, nw, lpr; };
 
-// Launch shape for the row kernel, from sweeps on MI355X:
-//  * lanes per row: 16 when the 64-lane form would leave a large part of the
-//    lanes without a unit (K = 896 is 28 units per row), else 64;
-//  * big matrices: two 8-wavefront blocks per CU, 4 rows per wavefront;
-//    otherwise one fat block per CU (16 wavefronts) so x is staged once per CU;
-//  * rows per block tile grow with the rows a CU owns (the x fragment held in
-//    VGPRs is reused for every row a lane group owns);
-//  * K is split over KW wavefronts of a block only when rows alone cannot give
-//    every CU a tile.
+// Launch shape for the row kernel, from sweeps on MI355X. With two work items in flight per
+// wavefront the memory pipe saturates at 8 to 16 wavefronts per CU, and HBM runs best when the
+// blocks that are active at one time cover a narrow band of the matrix, so the shapes below are
+// smaller than occupancy alone would suggest:
+//  * lanes per row: 16 when the 64-lane form would leave a large part of the lanes without
+//    a unit (K = 896 is 28 units per row), else 64;
+//  * many rows per CU: whole rows per wavefront (KW = 1), 2 to 4 rows in flight per lane group;
+//  * few rows per CU: K is split over KW wavefronts of a block so that every CU still has a
+//    tile, one chunk per wavefront where the chunks allow it.
 static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, const RowTune& tn) {
   RowCfg c{};
   const double waste64 = (double)((upr + 63) / 64 * 64) / upr, waste16 = (double)((upr + 15) / 16 * 16) / upr;
@@ -576,26 +483,24 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   const int chunks = (upr + lpr - 1) / lpr;
   const size_t xbytes = (size_t)chunks * lpr * E * 4 + (size_t)chunks * lpr * 4;
   const int64_t rows_per_cu = N / cus;
-  int nw = 16, R, KW;
+  int nw, R, KW, want_bpc;
   if (lpr == 64) {
-    if (rows_per_cu >= 128) { nw = 8; R = 4; KW = 1; }  // two 8-wave blocks per CU, 32-row tiles
-    else if (rows_per_cu >= 64) { nw = 8; R = 4; KW = 2; }  // same blocks, 16-row tiles
-    else if (rows_per_cu >= 32) { R = 2; KW = 1; }    // 32
-    else if (N > 16 * (int64_t)cus) {
-      // 17..31 rows per CU: 16-row tiles would leave a second, nearly empty round. Two blocks
-      // per CU, one row per wavefront, as many wavefronts as make the rows one round.
-      R = 1; KW = 1;
-      nw = (int)((N + 2 * (int64_t)cus - 1) / (2 * (int64_t)cus));
-      if (nw < 4) nw = 4;
+    if (rows_per_cu >= 512) { nw = 16; R = 4; KW = 2; want_bpc = 1; }        // LM head
+    else if (rows_per_cu >= 128) { nw = 8; R = 4; KW = 1; want_bpc = 1; }    // 7B gate|up
+    else if (rows_per_cu >= 32) { nw = 8; R = 2; KW = 1; want_bpc = 2; }     // 7B up-projection alone
+    else if (rows_per_cu >= 17) { nw = 8; R = 2; KW = 2; want_bpc = 2; }     // 7B q|k|v
+    else if (rows_per_cu >= 8) {
+      if (chunks <= 3) { nw = 8; R = 4; KW = 2; want_bpc = 2; }              // 7B o-projection
+      else { nw = 16; R = 1; KW = 2; want_bpc = 1; }                         // 7B down-projection (K = 18944)
+    } else {                                                                 // a few rows per CU
+      KW = chunks < 3 ? chunks : 3;
+      nw = 2 * KW; R = 2; want_bpc = 2;
     }
-    else if (rows_per_cu >= 8) { R = 2; KW = 2; }     // 16
-    else { nw = 8; R = 1; KW = 2; }                   // 4
   } else {
-    if (rows_per_cu >= 256) { R = 2; KW = 1; }        // 128 rows per block tile
-    else if (rows_per_cu >= 64) { R = 1; KW = 1; }    // 64
-    else if (rows_per_cu >= 16) { R = 1; KW = 2; }    // 32
-    else if (rows_per_cu >= 8) { R = 1; KW = 4; }     // 16
-    else { nw = 8; R = 1; KW = 4; }                   // 8
+    if (rows_per_cu >= 256) { nw = 8; R = 1; KW = 1; want_bpc = 2; }         // 0.5B LM head
+    else if (rows_per_cu >= 32) { nw = 4; R = 1; KW = 2; want_bpc = 4; }     // 0.5B gate|up
+    else if (rows_per_cu >= 8) { nw = 8; R = 1; KW = 2; want_bpc = 2; }
+    else { nw = 4; R = 1; KW = 1; want_bpc = 4; }
   }
   while (KW > chunks) {  // not enough K to split that far: more row groups instead
     KW /= 2;
@@ -606,9 +511,10 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   if (tn.KW > 0) KW = tn.KW;
   if (R >= 8 && nw > 8) nw = 8;  // the 8-row variant is built for <= 512 threads
   if (KW > nw) KW = nw;
+  if (nw % KW) nw -= nw % KW;    // whole row groups only (an override may ask for anything)
   int bpc = (int)((size_t)lds_per_cu / (xbytes + 4096));
   const int max_by_waves = 32 / nw > 0 ? 32 / nw : 1;
-  const int want_bpc = nw >= 16 ? 1 : nw == 8 ? 2 : 4;
+  if (tn.nw > 0) want_bpc = nw >= 16 ? 1 : nw == 8 ? 2 : 4;   // an overridden block size: the old default
   if (bpc > max_by_waves) bpc = max_by_waves;
   if (bpc > want_bpc) bpc = want_bpc;
   if (bpc < 1) bpc = 1;
@@ -716,6 +622,13 @@ static RowTune q4_tune(const Context& c) {
   return RowTune{c.tune_q4_rows, c.tune_q4_kw, c.tune_q4_bpc, c.tune_q4_nw, c.tune_q4_lpr};
 }
 
+// int4, group 32, through the row kernel.
+template <int PRO, int EPI>
+static int launch_q4(const float* x, const void* W, const float* scales, float* y, int64_t N, int64_t K,
+                     const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
+  return launch_rows<FmtQ4, PRO, EPI>(x, W, scales, y, N, K, TLHIP_C_GEMV_Q4, q4_tune(ctx()), pro);
+}
+
 static int check_gemv_args(const void* a, const void* B, const void* y, int64_t n, int64_t k,
                            const char* who) {
   if (!a || !B || !y) return fail(TLHIP_EINVAL, "%s: null pointer", who);
@@ -743,8 +656,8 @@ int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, in
   Context& c = ctx();
   const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
   if (group == 32 && aligned16(qw) && xbytes + 2048 <= (size_t)c.lds_per_cu)
-    return launch_rows<FmtQ4>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
-                              static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c));
+    return launch_q4<kPlain, kStore>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
+                                     static_cast<float*>(y), N, K);
   hipLaunchKernelGGL(gemv_q4_generic_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, c.stream,
                      static_cast<const float*>(a), static_cast<const uint32_t*>(qw),
                      static_cast<const float*>(scales), static_cast<float*>(y), (int)N, (int)K,
@@ -816,9 +729,8 @@ int tlhip_gemv_q4_swiglu(const void* gu, const void* qw, const void* scales, voi
   TLHIP_REQUIRE_READY();
   if (int rc = check_gemv_args(gu, qw, y, N, K, "tlhip_gemv_q4_swiglu")) return rc;
   if (int rc = check_fused_q4(qw, scales, K, group, 2 * K, "tlhip_gemv_q4_swiglu")) return rc;
-  Context& c = ctx();
-  return launch_rows<FmtQ4, kSwiglu>(static_cast<const float*>(gu), qw, static_cast<const float*>(scales),
-                                     static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c));
+  return launch_q4<kSwiglu, kStore>(static_cast<const float*>(gu), qw, static_cast<const float*>(scales),
+                                    static_cast<float*>(y), N, K);
 }
 
 int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,
@@ -828,11 +740,10 @@ int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, 
   if (int rc = check_gemv_args(x, qw, y, N, K, "tlhip_gemv_q4_rmsnorm")) return rc;
   if (int rc = check_fused_q4(qw, scales, K, group, K, "tlhip_gemv_q4_rmsnorm")) return rc;
   if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_q4_rmsnorm")) return rc;
-  Context& c = ctx();
   const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
                      static_cast<float*>(xout), eps};
-  return launch_rows<FmtQ4, kRmsnorm>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
-                                      static_cast<float*>(y), N, K, TLHIP_C_GEMV_Q4, q4_tune(c), pro);
+  return launch_q4<kRmsnorm, kStore>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
+                                     static_cast<float*>(y), N, K, pro);
 }
 
 int tlhip_gemv_q4_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
@@ -843,12 +754,10 @@ int tlhip_gemv_q4_rmsnorm_gateup(const void* x, const void* delta, const void* n
   if (N2 % 2) return fail(TLHIP_EINVAL, "tlhip_gemv_q4_rmsnorm_gateup: odd row count %lld", (long long)N2);
   if (int rc = check_fused_q4(qw, scales, K, group, K, "tlhip_gemv_q4_rmsnorm_gateup")) return rc;
   if (int rc = check_norm_args(x, delta, norm_w, xout, "tlhip_gemv_q4_rmsnorm_gateup")) return rc;
-  Context& c = ctx();
   const Producer pro{static_cast<const float*>(delta), static_cast<const float*>(norm_w),
                      static_cast<float*>(xout), eps};
-  return launch_rows<FmtQ4, kRmsnorm, kGateUp>(static_cast<const float*>(x), qw,
-                                               static_cast<const float*>(scales), static_cast<float*>(act),
-                                               N2, K, TLHIP_C_GEMV_Q4, q4_tune(c), pro);
+  return launch_q4<kRmsnorm, kGateUp>(static_cast<const float*>(x), qw, static_cast<const float*>(scales),
+                                      static_cast<float*>(act), N2, K, pro);
 }
 
 int tlhip_gemv_bf16_row_rmsnorm_gateup(const void* x, const void* delta, const void* norm_w, void* xout,
