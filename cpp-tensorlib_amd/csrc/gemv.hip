@@ -27,7 +27,7 @@ namespace tlhip {
 // ---------------------------------------------------------------------------
 // W: [N][upr] 16-byte units. scales: [N][upr] f32 (int4 only).
 // Block = nw wavefronts arranged as (nw/KW row groups) x (KW K-splits).
-// LDS: x as float4 xs[(chunk*J + j)*64 + lane], J = E/4, so that lane l's j-th
+// LDS: x as float4 xs[(chunk*J + j)*XS + lane], J = E/4, XS = LPR + a few (see the kernel), so that lane l's j-th
 // fragment of chunk c is one conflict-free ds_read_b128; then KW*rows floats.
 template <typename Fmt, int R>
 struct RowFrag {          // one (row tile, chunk) work item of a lane: R weight units in flight
@@ -84,8 +84,12 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   const int li = lane & (LPR - 1), q = lane / LPR;
   const int nw = blockDim.x >> 6;
   const int chunks = (upr + LPR - 1) / LPR;
+  // Row stride of the staged x: LPR float4s plus padding chosen so that the staging writes
+  // spread over all banks as well (the J threads of a unit write J rows at the same column:
+  // with a stride of exactly LPR float4s they would all hit one group of four banks).
+  constexpr int XS = LPR + (J == 8 ? 2 : 8);
   float4* xs = smem4;
-  float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * LPR);  // [chunks*LPR], int4 only
+  float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * XS);  // [chunks*LPR], int4 only
   float* red = xsum + (Fmt::kScaled ? chunks * LPR : 0);
 
   const int kw = wave % KW;          // which K split this wavefront takes
@@ -105,7 +109,9 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   const float4* x4 = reinterpret_cast<const float4*>(x);
   const int n4 = upr * J;
   const float4* d4 = reinterpret_cast<const float4*>(pro.delta);
-  constexpr int PL = 2;   // float4s a thread requests up front (all of x up to 8 * threads floats)
+  // float4s a thread requests up front: all of x up to 20 floats per thread (K = 18944 on 1024
+  // threads), 8 per thread in the norm form, whose vector is the hidden size (registers)
+  constexpr int PL = PRO == kRmsnorm ? 2 : 5;
   float4 px[PL], pa[PL], pn[PL];
   {
     const float4* aux4 = PRO == kSwiglu ? x4 + n4 : (d4 ? d4 : x4);   // up half, or delta (x when none: ignored)
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         }
       }
       const int u = i / J, j = i - u * J;
-      if (live) xs[((u / LPR) * J + j) * LPR + (u & (LPR - 1))] = Fmt::stage(v);
+      if (live) xs[((u / LPR) * J + j) * XS + (u & (LPR - 1))] = Fmt::stage(v);
       if (Fmt::kScaled) {
         float sx = (v.x + v.y) + (v.z + v.w);
         if constexpr (J == 8) {   // the unit's 8 adjacent lanes, on DPP: quads, then the other quad of the 8
@@ -219,7 +225,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     if (u < upr) {
       float4 xv[J];
 #pragma unroll
-      for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * LPR + li];
+      for (int j = 0; j < J; j++) xv[j] = xs[(c * J + j) * XS + li];
       if (Fmt::kScaled) {
         const float bias = xsum[u];
 #pragma unroll
@@ -298,14 +304,17 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       }
     }
     TLHIP_MARK(3);
-    for (; it < n_items; it += NS) {
-#pragma unroll
-      for (int k = 0; k < NS; k++) {
-        if (it + k < n_items) {
-          compute_item(frag[k], it + k);
-          if (it + k + NS < n_items) load_item(frag[k], it + k + NS);
-        }
-      }
+    // two or three items left, two of them in flight; each case is straight-line code so that
+    // its waits stay exact
+    static_assert(NS == 2, "the tail below is written for two fragments");
+    if (n_items - it == 2) {
+      compute_item(frag[0], it);
+      compute_item(frag[1], it + 1);
+    } else {
+      compute_item(frag[0], it);
+      load_item(frag[0], it + 2);
+      compute_item(frag[1], it + 1);
+      compute_item(frag[0], it + 2);
     }
   } else if (n_items == 1) {   // a single item: nothing more to request
     compute_item(frag[0], 0);
@@ -481,7 +490,8 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   if (tn.lpr == 16 || tn.lpr == 64) lpr = tn.lpr;
   const int qn = 64 / lpr;
   const int chunks = (upr + lpr - 1) / lpr;
-  const size_t xbytes = (size_t)chunks * lpr * E * 4 + (size_t)chunks * lpr * 4;
+  const int xs_stride = lpr + (E == 32 ? 2 : 8);   // float4s per staged row, as in the kernel
+  const size_t xbytes = (size_t)chunks * (E / 4) * xs_stride * 16 + (size_t)chunks * lpr * 4;
   const int64_t rows_per_cu = N / cus;
   int nw, R, KW, want_bpc;
   if (lpr == 64) {
@@ -654,7 +664,7 @@ int tlhip_gemv_q4(const void* a, const void* qw, const void* scales, void* y, in
   if (group <= 0 || (K % group) != 0 || (group % 8) != 0)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_q4: need group>0, K%%group==0, group%%8==0");
   Context& c = ctx();
-  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
+  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 66 * 32 * 4;
   if (group == 32 && aligned16(qw) && xbytes + 2048 <= (size_t)c.lds_per_cu)
     return launch_q4<kPlain, kStore>(static_cast<const float*>(a), qw, static_cast<const float*>(scales),
                                      static_cast<float*>(y), N, K);
@@ -670,7 +680,7 @@ int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_
   if (int rc = check_gemv_args(a, W, y, n, k, "tlhip_gemv_bf16_row")) return rc;
   if ((k % 8) != 0) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K %% 8 != 0");  // cuda.h:772
   if (!aligned16(W)) return fail(TLHIP_EINVAL, "tlhip_gemv_bf16_row: weight pointer not 16-byte aligned");
-  const size_t xbytes = (size_t)((k / 8 + 63) / 64) * 64 * 8 * 4;
+  const size_t xbytes = (size_t)((k / 8 + 63) / 64) * 72 * 8 * 4;
   if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K too large for the LDS-staged kernel");
   return launch_rows<FmtBf16>(static_cast<const float*>(a), W, nullptr, static_cast<float*>(y), n, k,
@@ -698,7 +708,7 @@ static int check_fused_q4(const void* qw, const void* scales, int64_t K, int64_t
   if (!scales) return fail(TLHIP_EINVAL, "%s: null scales", who);
   if (group != 32 || (K % 32) != 0 || !aligned16(qw))
     return fail(TLHIP_EUNSUPPORTED, "%s: fused form needs group 32, K %% 32 == 0, aligned weights", who);
-  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 64 * 32 * 4;
+  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 66 * 32 * 4;
   if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
     return fail(TLHIP_EUNSUPPORTED, "%s: K too large for the LDS-staged kernel", who);
   (void)in_floats;
@@ -708,7 +718,7 @@ static int check_fused_q4(const void* qw, const void* scales, int64_t K, int64_t
 static int check_fused_bf16(const void* W, int64_t K, const char* who) {
   if ((K % 8) != 0 || !aligned16(W))
     return fail(TLHIP_EUNSUPPORTED, "%s: need K %% 8 == 0 and aligned weights", who);
-  const size_t xbytes = (size_t)((K / 8 + 63) / 64) * 64 * 8 * 4;
+  const size_t xbytes = (size_t)((K / 8 + 63) / 64) * 72 * 8 * 4;
   if (xbytes + 2048 > (size_t)ctx().lds_per_cu)
     return fail(TLHIP_EUNSUPPORTED, "%s: K too large for the LDS-staged kernel", who);
   return 0;
