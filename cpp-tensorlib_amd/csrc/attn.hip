@@ -97,6 +97,27 @@ __device__ __forceinline__ float4 rope4(float4 own, const float2* __restrict__ t
   }
   return o;
 }
+// The same with the four (cos, sin) pairs of elements d0 .. d0+3 already in registers.
+template <int D>
+__device__ __forceinline__ float4 rope4_tab(float4 own, const float4 t0, const float4 t1, int d0) {
+  const bool lo = d0 < D / 2;
+  const float4 oth = make_float4(dpp_ror8(own.x), dpp_ror8(own.y), dpp_ror8(own.z), dpp_ror8(own.w));
+  const float4 a = lo ? own : oth;   // x0: elements j
+  const float4 b = lo ? oth : own;   // x1: elements j + half
+  float4 o;
+  if (lo) {
+    o.x = sub_rn(mul_rn(a.x, t0.x), mul_rn(b.x, t0.y));
+    o.y = sub_rn(mul_rn(a.y, t0.z), mul_rn(b.y, t0.w));
+    o.z = sub_rn(mul_rn(a.z, t1.x), mul_rn(b.z, t1.y));
+    o.w = sub_rn(mul_rn(a.w, t1.z), mul_rn(b.w, t1.w));
+  } else {
+    o.x = add_rn(mul_rn(a.x, t0.y), mul_rn(b.x, t0.x));
+    o.y = add_rn(mul_rn(a.y, t0.w), mul_rn(b.y, t0.z));
+    o.z = add_rn(mul_rn(a.z, t1.y), mul_rn(b.z, t1.x));
+    o.w = add_rn(mul_rn(a.w, t1.w), mul_rn(b.w, t1.z));
+  }
+  return o;
+}
 // x[d0..d0+4) + bias[d0..d0+4) (bias may be nullptr)
 __device__ __forceinline__ float4 load_biased4(const float* __restrict__ x, const float* __restrict__ bias, int d0) {
   float4 a = *reinterpret_cast<const float4*>(x + d0);
@@ -135,7 +156,8 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     const float* __restrict__ q, const KT* __restrict__ K, const KT* __restrict__ V,
     float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
     float* __restrict__ part_acc, int group, int ctx, int64_t kv_stride, int chunk, int TK,
-    float scale, int S, int T, int pos0, const uint32_t* __restrict__ dpos, QkvFuse fz, int kv_rows) {
+    float scale, int S, int T, int pos0, const uint32_t* __restrict__ dpos, QkvFuse fz, int kv_rows,
+    int n_kv_heads, int n_head_groups) {
   constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
   constexpr int NV = EPL / 4;        // float4 loads per lane per key
   constexpr int UNR = 4;             // key steps in flight per lane
@@ -152,23 +174,23 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int slot = lane >> 4, c = lane & 15;     // DPP row = key slot, c = position in the row
-  const int split = blockIdx.y;
-  float4 kpre[UNR][NV], vpre[UNR][NV];
-  if constexpr (kPre) {
-    const size_t hoff = (size_t)blockIdx.x * kv_stride;
-    const int kb0 = chunk ? split * chunk + wave * TK : (split * nw + wave) * TK;
-#pragma unroll
-    for (int u = 0; u < UNR; u++) {
-      const int key = min(kb0 + u * 4 + slot, kv_rows - 1);
-#pragma unroll
-      for (int v = 0; v < NV; v++) {
-        kpre[u][v] = KvLoad<KT>::ld(K + hoff + (size_t)key * D + c * EPL + v * 4);
-        vpre[u][v] = KvLoad<KT>::ld(V + hoff + (size_t)key * D + c * EPL + v * 4);
-      }
-    }
+  // Decode launches a 1-D grid and deals (kv head, split, head group) from the block number so
+  // that the head groups of one (kv head, split) - which read the same K/V rows - run on the
+  // same XCD back to back: workgroups go to the 8 XCDs round-robin by number, each XCD has an L2
+  // of its own, and the second reader of a tile then finds it there instead of in HBM.
+  // Block b runs on XCD b % 8 as that XCD's workgroup number b / 8; the XCD's sequence is
+  // (pair, head group) with the head group fastest. Blocks past the last pair exit.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if constexpr (!PRE) {
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    bz = seq % n_head_groups;
+    const int pair = (seq / n_head_groups) * 8 + xcd;
+    if (pair >= n_kv_heads * S) return;          // (uniform for the block; no barrier was passed)
+    bx = pair % n_kv_heads;
+    by = pair / n_kv_heads;
   }
-  // (the query rows first: nothing about them depends on the position, and with the
-  // position on the device its load should not stand in front of theirs)
+  const int split = by;
+  TLHIP_MARK(0);
   int kvh, g0, ng, k_begin, k_end;
   size_t row0;                                   // index of row g = 0 in q / out, in rows of D
   if constexpr (PRE) {
@@ -185,8 +207,8 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     k_end = pos0 + g0 + ng;                      // the last row's limit
     TK = k_end >= 64 ? 64 : k_end >= 32 ? 32 : 16;
   } else {
-    kvh = blockIdx.x;
-    g0 = blockIdx.z * G;
+    kvh = bx;
+    g0 = bz * G;
     ng = min(G, group - g0);
     row0 = (size_t)kvh * group + g0;
     k_begin = k_end = 0;                         // set below, once the position is known
@@ -196,20 +218,108 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
   const KT* Vh = V + (size_t)kvh * kv_stride;
   const int steps = TK >> 2;                     // load steps per tile
 
+  // ---- requests. A CU accepts roughly one vector memory instruction per 10 ns while misses are
+  // outstanding, so at decode sizes the number of load instructions is what the first microseconds
+  // cost. Decode: the block's G query rows (with bias) and the rotary table are fetched ONCE per
+  // block - one float4 per thread of the first wavefronts - and reach the other wavefronts
+  // through LDS; then every wavefront requests the first K and V rows of its first tile.
+  // Prefill (PRE): every wavefront has query rows of its own and loads them itself.
+  __shared__ float qs[PRE ? 1 : G][PRE ? 4 : D];   // decode: the block's query rows, bias added, not yet rotated
+  __shared__ float tabs[PRE ? 4 : D];              // decode, QKV: (cos, sin) pairs of the step
+  float4 qraw[PRE ? G : 1][NV];
+  float4 q_own = make_float4(0.f, 0.f, 0.f, 0.f), q_bias = q_own, t_own = q_own;
+  constexpr int QT = G * (D / 4);                  // float4s of the block's query rows
+  const int tq = threadIdx.x;
+  if constexpr (PRE) {
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      const size_t r = (row0 + (size_t)min(g, ng - 1)) * D;
+#pragma unroll
+      for (int v = 0; v < NV; v++) qraw[g][v] = *reinterpret_cast<const float4*>(q + r + c * EPL + v * 4);
+    }
+  } else {
+    if (tq < QT) {
+      const int gq = tq / (D / 4), dq = (tq - gq * (D / 4)) * 4;
+      const size_t r = (row0 + (size_t)min(gq, ng - 1)) * D;
+      q_own = *reinterpret_cast<const float4*>(q + r + dq);
+      if constexpr (QKV) {
+        const float* bsrc = fz.bq ? fz.bq : q;   // without a bias: any mapped address, the values are not used
+        q_bias = *reinterpret_cast<const float4*>(bsrc + r + dq);
+      }
+    } else if (QKV && tq < QT + D / 4) {
+      t_own = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(fz.table) + (tq - QT) * 4);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);   // (the scheduler may not move the K/V requests ahead of these)
+  float4 kpre[UNR][NV], vpre[UNR][NV];
+  if constexpr (kPre) {
+    const size_t hoff = (size_t)bx * kv_stride;
+    const int kb0 = chunk ? split * chunk + wave * TK : (split * nw + wave) * TK;
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      const int key = min(kb0 + u * 4 + slot, kv_rows - 1);
+#pragma unroll
+      for (int v = 0; v < NV; v++) {
+        kpre[u][v] = KvLoad<KT>::ld(K + hoff + (size_t)key * D + c * EPL + v * 4);
+        vpre[u][v] = KvLoad<KT>::ld(V + hoff + (size_t)key * D + c * EPL + v * 4);
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  TLHIP_MARK(7);
   float4 qv[G][NV];
+  if constexpr (PRE) {
 #pragma unroll
-  for (int g = 0; g < G; g++)
+    for (int g = 0; g < G; g++)
 #pragma unroll
-    for (int v = 0; v < NV; v++)
-      if constexpr (QKV)
-        // (rows g >= ng rotate zeros: the DPP exchange needs every lane of the row)
-        qv[g][v] = rope4<D>(g < ng ? load_biased4(q + (row0 + g) * D,
-                                                  fz.bq ? fz.bq + (row0 + g) * D : nullptr, c * EPL + v * 4)
-                                   : make_float4(0.f, 0.f, 0.f, 0.f),
-                            fz.table, c * EPL + v * 4);
-      else
-        qv[g][v] = g < ng ? *reinterpret_cast<const float4*>(q + (row0 + g) * D + c * EPL + v * 4)
-                          : make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int v = 0; v < NV; v++) qv[g][v] = g < ng ? qraw[g][v] : make_float4(0.f, 0.f, 0.f, 0.f);
+  } else {
+    if (tq < QT) {
+      const int gq = tq / (D / 4), dq = (tq - gq * (D / 4)) * 4;
+      if constexpr (QKV) {
+        if (fz.bq) { q_own.x += q_bias.x; q_own.y += q_bias.y; q_own.z += q_bias.z; q_own.w += q_bias.w; }
+      }
+      if (gq >= ng) q_own = make_float4(0.f, 0.f, 0.f, 0.f);
+      *reinterpret_cast<float4*>(&qs[gq][dq]) = q_own;
+    } else if (QKV && tq < QT + D / 4) {
+      *reinterpret_cast<float4*>(&tabs[(tq - QT) * 4]) = t_own;
+    }
+    // blocks of one or two wavefronts (short contexts) have fewer threads than there are float4s
+    for (int t2 = tq + (int)blockDim.x; t2 < QT + (QKV ? D / 4 : 0); t2 += (int)blockDim.x) {
+      if (t2 < QT) {
+        const int gq = t2 / (D / 4), dq = (t2 - gq * (D / 4)) * 4;
+        const size_t r = (row0 + (size_t)min(gq, ng - 1)) * D;
+        float4 a = *reinterpret_cast<const float4*>(q + r + dq);
+        if constexpr (QKV) {
+          if (fz.bq) {
+            const float4 b4 = *reinterpret_cast<const float4*>(fz.bq + r + dq);
+            a.x += b4.x; a.y += b4.y; a.z += b4.z; a.w += b4.w;
+          }
+        }
+        if (gq >= ng) a = make_float4(0.f, 0.f, 0.f, 0.f);
+        *reinterpret_cast<float4*>(&qs[gq][dq]) = a;
+      } else {
+        *reinterpret_cast<float4*>(&tabs[(t2 - QT) * 4]) =
+            *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(fz.table) + (t2 - QT) * 4);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+      for (int v = 0; v < NV; v++) {
+        const int d0 = c * EPL + v * 4;
+        const float4 own = *reinterpret_cast<const float4*>(&qs[g][d0]);
+        if constexpr (QKV) {
+          const int j0 = d0 < D / 2 ? d0 : d0 - D / 2;
+          const float4 t0 = *reinterpret_cast<const float4*>(&tabs[2 * j0]);       // (c0, s0, c1, s1)
+          const float4 t1 = *reinterpret_cast<const float4*>(&tabs[2 * j0 + 4]);   // (c2, s2, c3, s3)
+          qv[g][v] = rope4_tab<D>(own, t0, t1, d0);
+        } else {
+          qv[g][v] = own;
+        }
+      }
+  }
   // Position kept on the device (captured decode loops): the grid was planned for
   // the cache capacity, the live context is *dpos + 1. Splits past it find no keys
   // and write neutral partials (m = -inf, l = 0, acc = 0).
@@ -233,6 +343,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     k_begin = split * chunk;
     k_end = chunk ? min(ctx, k_begin + chunk) : ctx;
   }
+  TLHIP_MARK(1);
   float m[G], l[G];
   float4 acc[G][NV];
 #pragma unroll
@@ -247,12 +358,12 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
   // (its loads travel with the query's, so it costs that wavefront arithmetic only)
   if constexpr (QKV) {
     if (split == 0 && wave == 0 && has_new) {
-      const int Hkv = gridDim.x, Hq = Hkv * group;
+      const int Hkv = n_kv_heads, Hq = Hkv * group;
       const float* kraw = q + (size_t)(Hq + kvh) * D;
       const float* vraw = q + (size_t)(Hq + Hkv + kvh) * D;
       KT* krow = static_cast<KT*>(fz.Kw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
       KT* vrow = static_cast<KT*>(fz.Vw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
-      const bool store = blockIdx.z == 0 && slot == 0;
+      const bool store = bz == 0 && slot == 0;
       float4 kn[NV], vn[NV];
 #pragma unroll
       for (int v = 0; v < NV; v++) {
@@ -286,6 +397,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     }
   }
 
+  TLHIP_MARK(2);
   const int kb_first = PRE ? 0 : chunk ? k_begin + wave * TK : (split * nw + wave) * TK;
   const int kb_step = PRE ? TK : chunk ? nw * TK : S * nw * TK;
   for (int kb = kb_first; kb < k_end; kb += kb_step) {
@@ -398,6 +510,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     wave_lds_sync();  // pbuf is rewritten by the next tile
   }
 
+  TLHIP_MARK(3);
   // ---- wave totals: sum l over lanes, acc over the four key slots --------------------------
 #pragma unroll
   for (int g = 0; g < G; g++) {
@@ -430,7 +543,9 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     if (!PRE && lane == 0) { st_m[wave][g] = m[g]; st_l[wave][g] = l[g]; }
   }
   if constexpr (PRE) return;
+  TLHIP_MARK(4);
   __syncthreads();
+  TLHIP_MARK(5);
 
   // ---- block merge (fixed wave order) and store ---------------------------------------------
   for (int e = threadIdx.x; e < ng * D; e += blockDim.x) {
@@ -453,6 +568,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
       if (d == 0) { part_m[ps] = M; part_l[ps] = L; }
     }
   }
+  TLHIP_MARK(6);
 }
 
 // grid = Hq, block = 1024: merge the S split partials of one head. The threads are D
@@ -636,18 +752,19 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
     pacc = pl + hs;
   }
   if (S > 65535) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode: context too long");
-  const dim3 grid(Hkv, S, p.gz), block(p.nw * 64);
+  const int pairs8 = (Hkv * S + 7) / 8 * 8;       // (kv head, split) pairs, padded to whole rounds of the 8 XCDs
+  const dim3 grid(pairs8 * p.gz), block(p.nw * 64);
   const int64_t kv_stride = kv_max * D;
   const QkvFuse fz = fuse ? *fuse : QkvFuse{};
 #define TLHIP_ATTN(GG)                                                                            \
   if (fuse)                                                                                       \
     hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false, true>), grid, block, 0, c.stream, q, \
                        K, V, out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, S,   \
-                       1, 0, dpos, fz, (int)kv_max);                                              \
+                       1, 0, dpos, fz, (int)kv_max, Hkv, p.gz);                                   \
   else                                                                                            \
     hipLaunchKernelGGL((attn_decode_kernel<D, GG, KT, false>), grid, block, 0, c.stream, q, K, V, \
                        out, pm, pl, pacc, group, ctx, kv_stride, p.chunk, p.TK, scale, p.S, 1, 0, \
-                       dpos, fz, (int)kv_max)
+                       dpos, fz, (int)kv_max, Hkv, p.gz)
   switch (p.G) {
     case 1: TLHIP_ATTN(1); break;
     case 2: TLHIP_ATTN(2); break;
@@ -679,7 +796,7 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
   const dim3 grid(Hq, 1, (T + 4 * G - 1) / (4 * G)), block(256);   // 4 wavefronts x G query rows
   hipLaunchKernelGGL((attn_decode_kernel<D, G, KT, true>), grid, block, 0, c.stream, q, K, V, out,
                      (float*)nullptr, (float*)nullptr, (float*)nullptr, Hq / Hkv, pos0 + T,
-                     kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr, QkvFuse{}, (int)kv_max);
+                     kv_max * D, 0, 64, scale, 1, T, pos0, (const uint32_t*)nullptr, QkvFuse{}, (int)kv_max, 0, 1);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
 }
 

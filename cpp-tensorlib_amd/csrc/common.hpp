@@ -78,8 +78,9 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 constexpr int kTraceSlots = 8, kTraceWaves = 16, kTraceBlocks = 1024;
 static __device__ unsigned long long g_trace[kTraceBlocks * kTraceWaves * kTraceSlots];
 __device__ __forceinline__ void trace_mark(int slot) {
-  if ((threadIdx.x & 63) == 0 && blockIdx.x < kTraceBlocks)
-    g_trace[(blockIdx.x * kTraceWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = __builtin_readcyclecounter();
+  const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  if ((threadIdx.x & 63) == 0 && b < kTraceBlocks)
+    g_trace[(b * kTraceWaves + (threadIdx.x >> 6)) * kTraceSlots + slot] = __builtin_readcyclecounter();
 }
 #define TLHIP_MARK(slot) ::tlhip::trace_mark(slot)
 #else
