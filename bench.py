@@ -61,25 +61,46 @@ def make_q4_host(lib, N, K, seed):
     return out
 
 
-def cpu_baseline(guard, budget_s=25.0):
-    """The only leg that touches oracle/: it first checks the GPU result of the sweep's smallest
-    shape (`guard` = x, q4 buffer, N, K, y from the GPU) against the CPU checker, then times
-    the reference CPU path (x.dot(Wq) in use_cpu() mode: per-call widening to f32
-    plus cpu::sgemm on ONE thread, array.h:1980-1984, cpu.h:436-438) on the sweep's own
-    shapes, smallest first: median of 3 calls (after a warm-up call for the four smaller
-    ones); a shape is skipped once the time budget is spent (the sample
-    says which were timed). Falls back to the plain-C restatement when oracle/_ref was
-    not built."""
+def cpu_baseline(guards, budget_s=25.0):
+    """The only leg that touches oracle/. It first checks the GPU result of EVERY sweep shape
+    (`guards` = x, q4 buffer, N, K, y from the GPU; rows [::stride] of the big ones, whose rows
+    are independent) against the CPU checker, then times the reference CPU path (x.dot(Wq) in
+    use_cpu() mode: per-call widening to f32 plus cpu::sgemm on ONE thread, array.h:1980-1984,
+    cpu.h:436-438) on the sweep's own shapes, smallest first: median of 3 calls (after a
+    warm-up call for the four smaller ones); a shape is skipped once the time budget is spent
+    (the sample says which were timed). Then the other ops of a decode step at the 7B shape -
+    attn_decode over 28 heads at ctx 4096, rope, rmsnorm, swiglu - are timed the same way and
+    summed per layer the way the reference's bench_llm.cpp:167-176 sums per-op times into ms per
+    token. Falls back to the plain-C restatement when oracle/_ref was not built."""
     import ctypes as C
     from oraclelib import oracle, ref
     orc = oracle()
     refl = ref()            # None when oracle/_ref was not built
-    gx, gbuf, gN, gK, got = guard
-    want = orc.gemv_q4(gx, gbuf, gN, gK)
-    if not np.all(np.abs(got - want) <= 1e-5 + 1e-4 * np.abs(want)):
-        print("bench.py: GPU result differs from the CPU oracle", file=sys.stderr)
-        sys.exit(3)
-    total_bytes, total_s, timed = 0, 0.0, []
+    checked = []
+    for (gx, gbuf, gN, gK, got) in guards:
+        st = 1 if gN <= 4096 else 97
+        packed = gbuf[:gN * gK // 2].reshape(gN, gK // 2)[::st]
+        scales = gbuf[gN * gK // 2:].reshape(gN, gK // 32 * 4)[::st]
+        sub = np.concatenate([packed.ravel(), scales.ravel()])
+        want = orc.gemv_q4(gx, sub, packed.shape[0], gK)
+        if not np.all(np.abs(got[::st] - want) <= 1e-5 + 1e-4 * np.abs(want)):
+            print("bench.py: GPU result of %dx%d differs from the CPU oracle" % (gN, gK), file=sys.stderr)
+            sys.exit(3)
+        checked.append("%dx%d%s" % (gN, gK, "" if st == 1 else " rows[::%d]" % st))
+    P = C.c_void_p
+    ptr = lambda a: a.ctypes.data_as(P)
+
+    def med3(run, warm=True):
+        if warm:
+            run()
+        ts = []
+        for _ in range(3):
+            t = time.perf_counter()
+            run()
+            ts.append(time.perf_counter() - t)
+        return float(np.median(ts))
+
+    total_bytes, total_s, timed, per_shape_s = 0, 0.0, [], {}
     t_start = time.time()
     for (N, K) in sorted(SHAPES, key=lambda s: s[0] * s[1]):
         big = N * K > 10 ** 8
@@ -90,34 +111,89 @@ def cpu_baseline(guard, budget_s=25.0):
         x = orc.normal(K, 78)
         y = np.empty(N, np.float32)
         if refl is not None:
-            h = refl.lib.tlref_gemv_q4_prepare(x.ctypes.data_as(C.c_void_p), buf.ctypes.data_as(C.c_void_p), N, K)
-            run = lambda: refl.lib.tlref_gemv_run(h, y.ctypes.data_as(C.c_void_p))
+            h = refl.lib.tlref_gemv_q4_prepare(ptr(x), ptr(buf), N, K)
+            run = lambda: refl.lib.tlref_gemv_run(h, ptr(y))
         else:
             ws = np.empty(K * N, np.float32)
-            run = lambda: orc.lib.orc_gemv_q4(x.ctypes.data_as(C.c_void_p), buf.ctypes.data_as(C.c_void_p),
-                                              y.ctypes.data_as(C.c_void_p), N, K, 1.0, 0.0,
-                                              ws.ctypes.data_as(C.c_void_p))
-        ts = []
-        if not big:
-            run()
-        for _ in range(3):
-            t = time.perf_counter()
-            run()
-            ts.append(time.perf_counter() - t)
+            run = lambda: orc.lib.orc_gemv_q4(ptr(x), ptr(buf), ptr(y), N, K, 1.0, 0.0, ptr(ws))
+        sec = med3(run, warm=not big)
         if refl is not None:
             refl.lib.tlref_gemv_free(h)
         total_bytes += q4_nbytes(N, K)
-        total_s += float(np.median(ts))
+        total_s += sec
+        per_shape_s["%dx%d" % (N, K)] = sec
         timed.append("%dx%d" % (N, K))
-    return {
+    out = {
         "value": round(total_bytes / total_s / 1e9, 4), "unit": "GB/s", "cores": 1,
-        "kind": "reference" if refl is not None else "port", "gpu_result_checked": "512x3584 allclose(1e-4, 1e-5)",
+        "kind": "reference" if refl is not None else "port",
+        "gpu_result_checked": "allclose(1e-4, 1e-5) at " + ", ".join(checked),
         "sample": "int4 x.dot(Wq) at %s (%d of the 5 sweep shapes; median of 3 calls, after a warm-up "
                   "call except for the LM head); the reference's dot at M=1 runs on one thread whatever the core "
                   "count" % (", ".join(timed), len(timed)),
-        "ms": round(total_s * 1e3, 2), "cpu_seconds_spent": round(time.time() - t_start, 1),
-        "host_cores_online": os.cpu_count(),
+        "ms": round(total_s * 1e3, 2), "host_cores_online": os.cpu_count(),
     }
+    # ---- the other ops of a 7B-shape decode step at ctx 4096, one thread like the dots
+    if len(timed) == len(SHAPES):
+        L, E, HQ, HKV, D, FF, ctx = 28, 3584, 28, 4, 128, 18944, 4096
+        impl = refl if refl is not None else orc
+        q = orc.normal(HQ * D, 81).reshape(HQ, D)
+        # the array op has no GQA (array.h:1380-1381: one K/V head per query head)
+        Kc = np.tile(orc.normal(HKV * ctx * D, 82).reshape(HKV, 1, ctx, D), (1, HQ // HKV, 1, 1)).reshape(HQ, ctx, D)
+        Vc = np.tile(orc.normal(HKV * ctx * D, 83).reshape(HKV, 1, ctx, D), (1, HQ // HKV, 1, 1)).reshape(HQ, ctx, D)
+        scale = float(1.0 / np.sqrt(128.0))
+        t_attn = med3(lambda: impl.attn_decode(q, Kc, Vc, scale), warm=False)
+        qk = orc.normal((HQ + HKV) * D, 84).reshape(HQ + HKV, D)
+        t_rope = med3(lambda: impl.rope(qk, 4095, 1e6))
+        xr, wn = orc.normal(E, 85).reshape(1, E), orc.normal(E, 86, 1.0, 0.02)
+        t_norm = med3(lambda: impl.rmsnorm(xr, wn, 1e-6))
+        g_, u_ = orc.normal(FF, 87), orc.normal(FF, 88)
+        t_swiglu = med3(lambda: impl.swiglu(g_, u_))
+        ps = per_shape_s
+        # per layer: wq, wo (3584x3584), wk, wv (512x3584), wg, wu (18944x3584), wd (3584x18944)
+        dots = 2 * ps["3584x3584"] + 2 * ps["512x3584"] + 2 * ps["18944x3584"] + ps["3584x18944"]
+        layer = dots + t_attn + t_rope + 2 * t_norm + t_swiglu
+        token = L * layer + t_norm + ps["152064x3584"]
+        out["decode_7b_ctx4096"] = {
+            "kind": "summed per-op, measured (bench_llm.cpp:167-176)",
+            "ms_per_token": round(token * 1e3, 1), "tok_s": round(1.0 / token, 5),
+            "per_layer_ms": {"int4 dots": round(dots * 1e3, 2), "attn_decode 28 heads x ctx 4096": round(t_attn * 1e3, 2),
+                             "rope q+k": round(t_rope * 1e3, 4), "rmsnorm x2": round(2 * t_norm * 1e3, 4),
+                             "swiglu": round(t_swiglu * 1e3, 4)},
+            "lm_head_ms": round(ps["152064x3584"] * 1e3, 1),
+            "left_out": "bias adds, residual adds, cache append, embedding gather, argmax (microseconds)"}
+    out["cpu_seconds_spent"] = round(time.time() - t_start, 1)
+    return out
+
+
+def decode_guard(lib):
+    """One decode step at the 7B layer shape against the CPU oracle before anything is timed: a
+    one-layer model with the 7B dimensions (hidden 3584, 28/4 heads of 128, MLP 18944; a small
+    vocabulary - the LM-head shape is checked by the sweep's guard) built from the oracle's
+    seeded weights, caches of 4352 rows seeded up to row 4095 on both sides, one fused step at
+    position 4095 eagerly and one from a recorded graph with the position on the device. Bar: the
+    reference's own for a decode loop, logits maxrel < 2e-3 (check_llm_decode.cpp:268-276)."""
+    from oraclelib import QWEN_7B, maxrel, oracle
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    orc = oracle()
+    om = orc.qwen_create(dict(QWEN_7B, n_layers=1, vocab=4096), seed=9, q4=True)
+    g = qwen.QwenGPU.from_blobs(om)
+    d, pos = om.d, 4095
+    Kc, Vc = om.cache(0)
+    n = d.n_kv_heads * pos * d.head_dim
+    Kc[:, :pos, :] = orc.normal(n, 901).reshape(d.n_kv_heads, pos, d.head_dim)
+    Vc[:, :pos, :] = orc.normal(n, 902).reshape(d.n_kv_heads, pos, d.head_dim)
+    g.cache_upload(0, Kc, Vc, pos)
+    want_tok, want = om.step(1234, pos)
+    _, eager = g.step(1234, pos, want_logits=True)
+    ok = g.decoder_init(1234, pos)
+    _, replay = g.decoder_step(1234, want_logits=True)
+    worst = max(maxrel(eager, want), maxrel(replay, want))
+    g.close(); om.close()
+    if not (worst < 2e-3):
+        print("bench.py: 7B-shape decode step differs from the CPU oracle (maxrel %.2e)" % worst, file=sys.stderr)
+        sys.exit(3)
+    return {"what": "one-layer 7B-dims model, step at position 4095, eager and recorded graph, vs the CPU oracle",
+            "logits_maxrel": float("%.3g" % worst), "bar": 2e-3, "graph_captured": bool(ok)}
 
 
 def decode_7b(lib, steps, eager=False):
@@ -441,13 +517,16 @@ def main():
         x = lib.to_device(normal(K, 200 + si))
         y = lib.empty(N)
         rings.append(dict(N=N, K=K, nb=nb, stride=stride, copies=copies, buf=first, x=x, y=y, it=0,
-                          host=host if N == 512 else None))
+                          host=None if a.no_cpu else host))
     lib.sync()
 
-    # the smallest shape's GPU result, kept for the CPU leg's check
-    r0 = rings[1]
-    lib.gemv_q4(r0["x"], r0["buf"], r0["y"], r0["N"], r0["K"])
-    guard = (r0["x"].numpy(), r0["host"], r0["N"], r0["K"], r0["y"].numpy())
+    # every shape's GPU result (through the last copy of its ring), kept for the CPU leg's check
+    guards = []
+    if not a.no_cpu:
+        for r in rings:
+            lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"], wq_off=(r["copies"] - 1) * r["stride"])
+            guards.append((r["x"].numpy(), r["host"], r["N"], r["K"], r["y"].numpy()))
+            r["host"] = None
 
     def one_step(ev=None):
         for r in rings:
@@ -526,17 +605,23 @@ def main():
     # HBM bytes per LM-head launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
     # by what the same counter reads for a plain 1 GiB copy kernel (x2.000 and x1.000 here)
     out["roofline"]["traffic"] = LMHEAD_HBM_BYTES_PER_LAUNCH
+    out["roofline"]["traffic_source"] = ("profiles/gemv_q4_lmhead_hbm_traffic.md (rocprofv3 --pmc runs of this "
+                                         "command; a constant of the kernel, not measured by this run)")
     if not a.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(guard)
+        out["cpu_baseline"] = cpu_baseline(guards)
     if not a.no_decode:
+        guard7b = None if a.no_cpu else decode_guard(lib)
         out["decode"] = decode_7b(lib, max(10, a.steps), eager=a.eager_decode)
-        if "cpu_baseline" in out and "algorithmic_bytes" in out["decode"]:
-            # reference CPU tok/s implied by its int4 GEMV rate on the same weight bytes
-            cpu_gbs = out["cpu_baseline"]["value"]
+        if guard7b is not None:
+            out["decode"]["checked_against_oracle"] = guard7b
+        cpu_dec = out.get("cpu_baseline", {}).get("decode_7b_ctx4096")
+        if cpu_dec is not None:
+            # the reference's CPU kernels on this box's host cores (one thread: its M=1 dot and its
+            # attention are single-threaded), per-op times summed into ms per token
             d = out["decode"]
-            cpu_ms = d["algorithmic_bytes"] / (cpu_gbs * 1e9) * 1e3
-            d["cpu_reference_ms_per_token_est"] = round(cpu_ms, 1)
-            d["speedup_vs_cpu_reference_est"] = round(cpu_ms / d["ms_per_token"], 1)
+            d["cpu_reference_ms_per_token"] = cpu_dec["ms_per_token"]
+            d["cpu_reference_kind"] = cpu_dec["kind"]
+            d["speedup_vs_cpu_reference"] = round(cpu_dec["ms_per_token"] / d["ms_per_token"], 1)
         if not a.eager_decode:
             out["decode_05b"] = decode_05b(lib, max(20, a.steps))
     if not a.no_side:
