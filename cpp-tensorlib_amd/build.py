@@ -73,7 +73,6 @@ def build(force=False, verbose=True):
 
 
 QWEN_LIB = os.path.join(LIBDIR, "libtl_qwen.so")
-SEAM_CHECK = os.path.join(LIBDIR, "tl_seam_check")
 
 
 def build_host(force=False, verbose=True):
@@ -85,14 +84,6 @@ def build_host(force=False, verbose=True):
     if force or _stale(QWEN_LIB, deps):
         cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra", "-I", inc, src,
                "-o", QWEN_LIB, "-ldl"]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        subprocess.check_call(cmd)
-    # tl_seam_check: a program that drives the backend header the way the reference's
-    # evaluator drives a backend; the GPU tests run it
-    chk_src = os.path.join(CSRC, "seam_check.cpp")
-    if force or _stale(SEAM_CHECK, deps + [chk_src]):
-        cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-I", inc, chk_src, "-o", SEAM_CHECK, "-ldl"]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)

@@ -112,6 +112,7 @@ SIGNATURES = {
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
     "tlhip_tune_gemv_cols": (cint, [cint]),
     "tlhip_tune_attn_prefill": (cint, [cint]),
+    "tlhip_tune_reset": (cint, []),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
 }
@@ -459,6 +460,9 @@ class TlHip:
 
     def tune_attn_prefill(self, valu_kernel):
         self._chk(self.c.tlhip_tune_attn_prefill(1 if valu_kernel else 0))
+
+    def tune_reset(self):
+        self._chk(self.c.tlhip_tune_reset())
 
     def tune_gemv_q4(self, rows=0, kw=0, bpc=0, nw=0, lpr=0):
         self._chk(self.c.tlhip_tune_gemv_q4(rows, kw, bpc, nw, lpr))

@@ -225,7 +225,7 @@ int64_t tlq_step(void* hv, int64_t token, int64_t pos, float* logits_out) {
 // Enqueue one step's launches without the argmax and without any sync.
 int tlq_run_layers(void* hv, int64_t token, int64_t pos) {
   auto* h = static_cast<handle*>(hv);
-  qwen::stage_embed(h->M, token);
+  if (!qwen::stage_embed(h->M, token)) return -1;
   return qwen::run_layers(h->M, h->M.s.embedb, pos) ? 0 : -1;
 }
 
@@ -237,7 +237,7 @@ int64_t tlq_argmax(void* hv) {
 
 int tlq_capture(void* hv, int64_t token, int64_t pos) {
   auto* h = static_cast<handle*>(hv);
-  qwen::stage_embed(h->M, token);
+  if (!qwen::stage_embed(h->M, token)) return -1;
   return h->cap.capture(h->M, pos) ? 0 : -1;
 }
 // A decode loop on one recorded graph with the position on the device.

@@ -1,5 +1,6 @@
 // Library state, memory, stream, graph capture, events and the dispatch census.
 #include "common.hpp"
+#include "../../include/tensorlib_hip_bench.h"
 
 #include <cstring>
 #include <string>
@@ -333,12 +334,27 @@ int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks) {
 
 int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
                        int lanes_per_row) {
+  const bool rows_ok = rows_per_wave == 0 || rows_per_wave == 1 || rows_per_wave == 2 ||
+                       rows_per_wave == 4 || rows_per_wave == 8;
+  const bool lpr_ok = lanes_per_row == 0 || lanes_per_row == 16 || lanes_per_row == 64;
+  if (!rows_ok || !lpr_ok || k_waves < 0 || k_waves > 16 || waves_per_block < 0 || waves_per_block > 16 ||
+      blocks_per_cu < 0 || blocks_per_cu > 8)
+    return fail(TLHIP_EINVAL, "tlhip_tune_gemv_q4: rows_per_wave in {1,2,4,8}, k_waves and waves_per_block "
+                              "in [1,16], blocks_per_cu in [1,8], lanes_per_row in {16,64}; 0 = built-in");
   Context& c = ctx();
   c.tune_q4_rows = rows_per_wave;
   c.tune_q4_kw = k_waves;
   c.tune_q4_bpc = blocks_per_cu;
   c.tune_q4_nw = waves_per_block;
   c.tune_q4_lpr = lanes_per_row;
+  return TLHIP_OK;
+}
+
+int tlhip_tune_reset(void) {
+  Context& c = ctx();
+  c.tune_q4_rows = c.tune_q4_kw = c.tune_q4_bpc = c.tune_q4_nw = c.tune_q4_lpr = 0;
+  c.tune_cols_max_splits = 0;
+  c.tune_prefill_valu = 0;
   return TLHIP_OK;
 }
 

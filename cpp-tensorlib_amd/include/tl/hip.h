@@ -14,9 +14,9 @@
 // Unlike cuda.h, which dlopens the driver and loads an embedded PTX blob, this
 // header dlopens ONE shared object, libtensorlib_hip.so, that holds the gfx950
 // code objects and a plain C ABI (include/tensorlib_hip.h). What stays here is
-// the host policy the reference keeps in its backend header: the host/device
-// mirror with HOST/DEVICE/BOTH dirty state, the size-keyed buffer pool, the
-// `pending` flag, and turning every refusal of the library into the seam's
+// the host policy the reference keeps in its backend header: a ledger of buffers
+// with a device half and a pinned host half and a note of which one is current,
+// reuse of idle buffers by size, the `pending` flag, and turning every refusal of the library into the seam's
 // "declined" (`false` / nullptr) so the evaluator takes its CPU path. No
 // exception and no error code crosses the seam.
 //
@@ -162,6 +162,56 @@ struct api {
                                       int64_t, int64_t, float) = nullptr;
 };
 
+// ---- buffer ledger ----------------------------------------------------------------
+// A buffer handed to tensorlib's storage is an extent: device bytes at `base` (the handle
+// storage keeps) and, unless it is device-only, a pinned host half of the same size (the
+// `contents` pointer storage keeps). `live` names the half that holds the current bytes.
+struct extent {
+  enum class side : unsigned char { staging, device, either };
+  char* base = nullptr;
+  float* staging = nullptr;
+  size_t size = 0;
+  side live = side::staging;
+};
+
+// The extents in use, ordered by base address so that an address INSIDE one (q4 scales at
+// base + N*K/2, one projection of a fused weight) resolves to it, and the idle ones, filed by
+// exact size. Idle extents are reused, never returned to the driver: the evaluator allocates
+// the same few sizes over and over (the policy of cuda.h:211-216).
+class ledger {
+  std::map<uintptr_t, extent> in_use_;
+  std::unordered_map<size_t, std::vector<extent>> idle_;
+
+ public:
+  extent* containing(const void* p) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    auto after = in_use_.upper_bound(a);
+    if (!a || after == in_use_.begin()) return nullptr;
+    extent& e = std::prev(after)->second;
+    return a - reinterpret_cast<uintptr_t>(e.base) < e.size ? &e : nullptr;
+  }
+  extent* at_base(uintptr_t base) {
+    auto it = in_use_.find(base);
+    return it == in_use_.end() ? nullptr : &it->second;
+  }
+  bool reuse(size_t size, extent& out) {
+    auto it = idle_.find(size);
+    if (it == idle_.end() || it->second.empty()) return false;
+    out = it->second.back();
+    it->second.pop_back();
+    return true;
+  }
+  void enter(const extent& e) { in_use_[reinterpret_cast<uintptr_t>(e.base)] = e; }
+  bool leave(const void* base, extent& out) {
+    auto it = in_use_.find(reinterpret_cast<uintptr_t>(base));
+    if (it == in_use_.end()) return false;
+    out = it->second;
+    in_use_.erase(it);
+    return true;
+  }
+  void park(const extent& e) { idle_[e.size].push_back(e); }
+};
+
 struct context {
   void* lib = nullptr;
   api f;
@@ -175,20 +225,7 @@ struct context {
   std::unordered_map<void*, std::vector<uintptr_t>> graph_writes;
   std::string why;  // why the backend is unavailable (diagnostics only)
 
-  // Host/device mirror per allocation, keyed by the device pointer (== the
-  // `native` handle storage keeps). Ordered, so that a pointer INTO an
-  // allocation (q4 scales at native + N*K/2, a slice of a fused projection)
-  // finds its owner too.
-  enum loc { HOST, DEVICE, BOTH };
-  struct mirror {
-    float* host = nullptr;
-    char* dev = nullptr;
-    size_t bytes = 0;
-    loc where = HOST;
-  };
-  std::map<uintptr_t, mirror> mirrors;
-  // size-keyed free list; buffers are recycled, never freed (cuda.h:211-216)
-  std::unordered_map<size_t, std::vector<std::pair<char*, float*>>> pool;
+  ledger buffers;   // every extent handed out, and the idle ones waiting for reuse
 
   static context& get() {
     static auto* c = new context();  // leaked: outlives every storage deleter
@@ -280,35 +317,52 @@ struct context {
     ready = true;
   }
 
-  // the allocation containing p, or nullptr
-  mirror* mirror_(const void* p) {
-    if (!p || mirrors.empty()) return nullptr;
-    auto it = mirrors.upper_bound(reinterpret_cast<uintptr_t>(p));
-    if (it == mirrors.begin()) return nullptr;
-    --it;
-    mirror& m = it->second;
-    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
-    return (a >= it->first && a < it->first + m.bytes) ? &m : nullptr;
+  // ---- keeping the two halves of an extent coherent ---------------------------------
+  // The device half is about to be read by a launch: bring it up to date.
+  void refresh_device(const void* p) {
+    extent* e = buffers.containing(p);
+    if (e && e->live == extent::side::staging) push(*e, e->size);
   }
-  // A kernel is about to READ this buffer: make the device copy current.
-  void device_read_(const void* native) {
-    mirror* m = mirror_(native);
-    if (m && m->where == HOST) {
-      f.memcpy_h2d(m->dev, m->host, m->bytes);  // blocking, stream-ordered
-      m->where = BOTH;
-    }
+  // The device half is about to be written by a launch (at p, possibly inside the extent).
+  // A launch that starts past the extent's base may leave the bytes before it untouched, so a
+  // staging-live extent is pushed whole first. Recorded while a graph capture is open.
+  void claim_device(void* p) {
+    extent* e = buffers.containing(p);
+    if (!e) return;
+    if (e->live == extent::side::staging && static_cast<char*>(p) != e->base) push(*e, e->size);
+    e->live = extent::side::device;
+    if (capturing) capture_writes.push_back(reinterpret_cast<uintptr_t>(e->base));
   }
-  // A kernel is about to WRITE this buffer: it becomes the live copy. A write
-  // into part of a buffer whose live copy is on the host uploads first, so the
-  // untouched part is not lost.
-  void device_write_(void* native) {
-    mirror* m = mirror_(native);
-    if (!m) return;
-    if (m->where == HOST && reinterpret_cast<char*>(native) != m->dev) {
-      f.memcpy_h2d(m->dev, m->host, m->bytes);
-    }
-    m->where = DEVICE;
-    if (capturing) capture_writes.push_back(reinterpret_cast<uintptr_t>(m->dev));
+  // staging -> device, blocking and ordered after the queued launches
+  void push(extent& e, size_t n) {
+    f.memcpy_h2d(e.base, e.staging, n < e.size ? n : e.size);
+    e.live = extent::side::either;
+  }
+  // device -> staging
+  void pull(extent& e) {
+    f.memcpy_d2h(e.staging, e.base, e.size);
+    e.live = extent::side::either;
+  }
+};
+
+// One submission to the library. The caller names what the call reads and writes - stale device
+// halves are refreshed, written extents become device-live - and hands the library's return
+// code to sent(), which also notes that work is now queued.
+class launch {
+  context& c_;
+
+ public:
+  const api& lib;
+  const bool ok;   // false: no library or no device, the caller declines
+  launch() : c_(context::get()), lib(c_.f), ok(c_.ready) {}
+  template <class... P>
+  void reads(P... p) { (c_.refresh_device(p), ...); }
+  template <class... P>
+  void writes(P... p) { (c_.claim_device(p), ...); }
+  bool sent(int rc) {
+    if (rc != 0) return false;   // declined or failed: the caller falls back
+    c_.pending = true;
+    return true;
   }
 };
 
@@ -344,96 +398,85 @@ inline std::vector<uint64_t> census() {
   return v;
 }
 
-// ---- memory (cuda.h:553-637) ---------------------------------------------------
+// ---- memory: the storage hooks of the seam (cuda.h:553-637) ----------------------------
+// A buffer of `bytes` bytes: returns the device handle, *contents gets the host half.
+// The host half starts as the live one (storage fills it before any launch).
 inline void* alloc(int64_t bytes, float** contents) {
   auto& c = context::get();
   if (!c.ready) return nullptr;
-  const size_t nb = bytes > 0 ? (size_t)bytes : 4;
-  char* dev = nullptr;
-  float* host = nullptr;
-  auto it = c.pool.find(nb);
-  if (it != c.pool.end() && !it->second.empty()) {
-    dev = it->second.back().first;
-    host = it->second.back().second;
-    it->second.pop_back();
-  } else {
-    void* d = nullptr;
-    if (c.f.malloc_(&d, nb) != 0) return nullptr;
-    void* h = nullptr;
-    if (c.f.host_alloc(&h, nb) != 0) {  // pinned: H2D/D2H run at full PCIe rate
+  extent e;
+  e.size = bytes > 0 ? static_cast<size_t>(bytes) : 4;
+  if (!c.buffers.reuse(e.size, e)) {
+    void *d = nullptr, *h = nullptr;
+    if (c.f.malloc_(&d, e.size) != 0) return nullptr;
+    if (c.f.host_alloc(&h, e.size) != 0) {   // pinned, so both copy directions run at the link rate
       c.f.free_(d);
       return nullptr;
     }
-    dev = static_cast<char*>(d);
-    host = static_cast<float*>(h);
+    e.base = static_cast<char*>(d);
+    e.staging = static_cast<float*>(h);
   }
-  c.mirrors[reinterpret_cast<uintptr_t>(dev)] = context::mirror{host, dev, nb, context::HOST};
-  if (contents) *contents = host;
-  return dev;
+  e.live = extent::side::staging;
+  c.buffers.enter(e);
+  if (contents) *contents = e.staging;
+  return e.base;
 }
 
-// A buffer that only ever lives on the device (weights written by device
-// copies, KV caches): no host half, so nothing is pinned for it and
-// sync_to_host has nothing to bring back.
+// A buffer that never visits the host (weights written by device copies, KV caches): no
+// host half is pinned for it and sync_to_host leaves it alone.
 inline void* alloc_device(int64_t bytes) {
   auto& c = context::get();
   if (!c.ready) return nullptr;
-  const size_t nb = bytes > 0 ? (size_t)bytes : 4;
+  extent e;
+  e.size = bytes > 0 ? static_cast<size_t>(bytes) : 4;
   void* d = nullptr;
-  if (c.f.malloc_(&d, nb) != 0) return nullptr;
-  c.mirrors[reinterpret_cast<uintptr_t>(d)] =
-      context::mirror{nullptr, static_cast<char*>(d), nb, context::DEVICE};
+  if (c.f.malloc_(&d, e.size) != 0) return nullptr;
+  e.base = static_cast<char*>(d);
+  e.live = extent::side::device;
+  c.buffers.enter(e);
   return d;
 }
 
 // Stream-ordered device-to-device copy between two managed buffers.
 inline bool copy_d2d(void* dst, const void* src, int64_t bytes) {
-  auto& c = context::get();
-  if (!c.ready || !dst || !src || bytes < 0) return false;
-  c.device_read_(src);
-  c.device_write_(dst);
-  if (c.f.memcpy_d2d_async(dst, src, (size_t)bytes) != 0) return false;
-  c.pending = true;
-  return true;
+  launch L;
+  if (!L.ok || !dst || !src || bytes < 0) return false;
+  L.reads(src);
+  L.writes(dst);
+  return L.sent(L.lib.memcpy_d2d_async(dst, src, (size_t)bytes));
 }
 
 inline void release(void* buf, int64_t, float*) {
   auto& c = context::get();
   if (!c.ready || !buf) return;
-  auto it = c.mirrors.find(reinterpret_cast<uintptr_t>(buf));
-  if (it == c.mirrors.end()) return;
-  // a kernel still in flight may be using the buffer; recycle only after the drain
+  if (!c.buffers.at_base(reinterpret_cast<uintptr_t>(buf))) return;
+  // a queued launch may still use the buffer: it may change hands only after the drain
   if (c.pending && !c.capturing) flush();
-  if (it->second.host) c.pool[it->second.bytes].push_back({it->second.dev, it->second.host});
-  else c.f.free_(it->second.dev);  // device-only buffers are not pooled
-  c.mirrors.erase(it);
+  extent e;
+  c.buffers.leave(buf, e);
+  if (e.staging) c.buffers.park(e);
+  else c.f.free_(e.base);   // device-only extents are not kept for reuse
 }
 
+// The host is about to read (for_write: and then modify) the buffer through its host half.
 inline void sync_to_host(void* native, bool for_write) {
   auto& c = context::get();
-  if (!c.ready || !native) return;
-  context::mirror* m = c.mirror_(native);
-  if (!m) return;
+  extent* e = c.ready ? c.buffers.containing(native) : nullptr;
+  if (!e) return;
   if (c.pending) flush();
-  if (!m->host) return;  // device-only buffer
-  if (m->where == context::DEVICE) {
-    c.f.memcpy_d2h(m->host, m->dev, m->bytes);
-    m->where = context::BOTH;
-  }
-  if (for_write) m->where = context::HOST;
+  if (!e->staging) return;
+  if (e->live == extent::side::device) c.pull(*e);
+  if (for_write) e->live = extent::side::staging;
 }
 
-// Blocking H2D of the buffer's first n floats (cuda.h:553-568).
+// Blocking copy of n floats from src into the buffer, both halves (cuda.h:553-568).
 inline void upload(void* native, const float* src, int64_t n) {
   auto& c = context::get();
-  if (!c.ready || !native) return;
-  context::mirror* m = c.mirror_(native);
-  if (!m || !m->host) return;
-  size_t bytes = (size_t)n * sizeof(float);
-  if (bytes > m->bytes) bytes = m->bytes;
-  if (src != m->host) std::memcpy(m->host, src, bytes);
-  c.f.memcpy_h2d(m->dev, m->host, bytes);
-  m->where = context::BOTH;
+  extent* e = c.ready ? c.buffers.containing(native) : nullptr;
+  if (!e || !e->staging) return;
+  const size_t nb = std::min(static_cast<size_t>(n) * sizeof(float), e->size);
+  if (src != e->staging) std::memcpy(e->staging, src, nb);
+  c.push(*e, nb);
 }
 
 // Blocking H2D from any host memory (pageable or a file mapping) to a device address, which
@@ -452,286 +495,248 @@ inline bool download_raw(void* dst_host, const void* src_dev, int64_t bytes) {
   return bytes == 0 || c.f.memcpy_d2h(dst_host, src_dev, (size_t)bytes) == 0;
 }
 
+// A 4-byte device scalar (a position, a token id) set from the host.
 inline void upload_u32(void* native, unsigned val) {
   auto& c = context::get();
-  if (!c.ready || !native) return;
-  context::mirror* m = c.mirror_(native);
-  if (!m || !m->host || m->bytes < 4) return;
-  std::memcpy(m->host, &val, 4);
-  c.f.memcpy_h2d(m->dev, m->host, 4);
-  m->where = context::BOTH;
+  extent* e = c.ready ? c.buffers.containing(native) : nullptr;
+  if (!e || !e->staging || e->size < sizeof val) return;
+  std::memcpy(e->staging, &val, sizeof val);
+  c.push(*e, sizeof val);
 }
-
-namespace detail {
-inline bool done_(context& c, int rc) {
-  if (rc != 0) return false;  // declined or failed: the caller falls back
-  c.pending = true;
-  return true;
-}
-}  // namespace detail
 
 // ---- the seam ------------------------------------------------------------------
 inline bool binary(kop op, void* a, int64_t ao, void* b, int64_t bo, void* out, int64_t oo,
                    int64_t n, float scale, float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_read_(b);
-  c.device_write_(out);
-  return detail::done_(c, c.f.binary(static_cast<int>(op), a, ao, b, bo, out, oo, n, scale, offset));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a, b);
+  L.writes(out);
+  return L.sent(L.lib.binary(static_cast<int>(op), a, ao, b, bo, out, oo, n, scale, offset));
 }
 
 inline bool binary_bcast(kop op, void* a, int64_t ao, int64_t ars, int64_t acs, void* b, int64_t bo,
                          int64_t brs, int64_t bcs, void* out, int64_t oo, int64_t m, int64_t n,
                          float scale, float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_read_(b);
-  c.device_write_(out);
-  return detail::done_(c, c.f.binary_bcast(static_cast<int>(op), a, ao, ars, acs, b, bo, brs, bcs,
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a, b);
+  L.writes(out);
+  return L.sent(L.lib.binary_bcast(static_cast<int>(op), a, ao, ars, acs, b, bo, brs, bcs,
                                            out, oo, m, n, scale, offset));
 }
 
 inline bool unary(kop op, void* a, int64_t ao, void* out, int64_t oo, int64_t n, float scale,
                   float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_write_(out);
-  return detail::done_(c, c.f.unary(static_cast<int>(op), a, ao, out, oo, n, scale, offset));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a);
+  L.writes(out);
+  return L.sent(L.lib.unary(static_cast<int>(op), a, ao, out, oo, n, scale, offset));
 }
 
 // 1/x with an affine epilogue: an op the reference's seam lacks (its `recip`
 // node always runs on the CPU, array.h:2064-2066); offered so a host layer that
 // knows about it can keep array::rmsnorm on the device.
 inline bool recip(void* a, int64_t ao, void* out, int64_t oo, int64_t n, float scale, float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_write_(out);
-  return detail::done_(c, c.f.unary(64 /* TLHIP_RECIP */, a, ao, out, oo, n, scale, offset));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a);
+  L.writes(out);
+  return L.sent(L.lib.unary(64 /* TLHIP_RECIP */, a, ao, out, oo, n, scale, offset));
 }
 
 inline bool gemm(void* a, int64_t ao, int64_t lda, bool ta, void* b, int64_t bo, int64_t ldb, bool tb,
                  void* out, int64_t oo, int64_t m, int64_t n, int64_t k, float scale, float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_read_(b);
-  c.device_write_(out);
-  return detail::done_(c, c.f.gemm(a, ao, lda, ta ? 1 : 0, b, bo, ldb, tb ? 1 : 0, out, oo, m, n, k,
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a, b);
+  L.writes(out);
+  return L.sent(L.lib.gemm(a, ao, lda, ta ? 1 : 0, b, bo, ldb, tb ? 1 : 0, out, oo, m, n, k,
                                    scale, offset));
 }
 
 inline bool row_op(kop op, void* in, int64_t io, void* out, int64_t oo, int64_t rows, int64_t cols,
                    float scale, float offset) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(in);
-  c.device_write_(out);
-  return detail::done_(c, c.f.row_op(static_cast<int>(op), in, io, out, oo, rows, cols, scale, offset));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(in);
+  L.writes(out);
+  return L.sent(L.lib.row_op(static_cast<int>(op), in, io, out, oo, rows, cols, scale, offset));
 }
 
 inline bool gemv_f32(void* a, void* B, void* y, int64_t n, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_f32(a, B, y, n, k));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a, B);
+  L.writes(y);
+  return L.sent(L.lib.gemv_f32(a, B, y, n, k));
 }
 
 inline bool gemv_bf16(void* a, void* B, void* y, int64_t n, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_bf16(a, B, y, n, k));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(a, B);
+  L.writes(y);
+  return L.sent(L.lib.gemv_bf16(a, B, y, n, k));
 }
 
 inline bool gemv_bf16_row(void* a, void* B, void* y, int64_t n, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_bf16_row(a, B, y, n, k));
+  launch L;
+  if (!L.ok || (k % 8) != 0) return false;
+  L.reads(a, B);
+  L.writes(y);
+  return L.sent(L.lib.gemv_bf16_row(a, B, y, n, k));
 }
 
 inline bool gemv_q4(void* a, void* qw, void* scales, void* y, int64_t N, int64_t K, int64_t group) {
-  auto& c = context::get();
-  if (!c.ready || group <= 0 || (K % group) != 0 || (group % 8) != 0) return false;
-  c.device_read_(a);
-  c.device_read_(qw);
-  c.device_read_(scales);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_q4(a, qw, scales, y, N, K, group));
+  launch L;
+  if (!L.ok || group <= 0 || (K % group) != 0 || (group % 8) != 0) return false;
+  L.reads(a, qw, scales);
+  L.writes(y);
+  return L.sent(L.lib.gemv_q4(a, qw, scales, y, N, K, group));
 }
 
 inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0 || m <= 0 || n <= 0) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(out);
-  return detail::done_(c, c.f.gemm_bf16_nt(a, B, out, m, n, k));
+  launch L;
+  if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0) return false;
+  L.reads(a, B);
+  L.writes(out);
+  return L.sent(L.lib.gemm_bf16_nt(a, B, out, m, n, k));
 }
 
 // act[m, ff] = swiglu(a . gate^T, a . up^T) for B = [gate rows | up rows] ([2*ff, k] bf16):
 // gemm_bf16_nt + swiglu in one launch.
 inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t ff, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0 || m <= 0 || ff <= 0) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(act);
-  return detail::done_(c, c.f.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
+  launch L;
+  if (!L.ok || (k % 8) != 0 || m <= 0 || ff <= 0) return false;
+  L.reads(a, B);
+  L.writes(act);
+  return L.sent(L.lib.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
 }
 
 // The prompt-chunk products over an int4 weight (packed nibbles + scales, group 32), M rows at a
 // time on the matrix pipe; plain, gated and parts forms like the bf16 ones.
 inline bool gemm_q4_nt(void* a, void* qw, void* scales, void* out, int64_t m, int64_t n, int64_t k,
                        int64_t group = 32) {
-  auto& c = context::get();
-  if (!c.ready || (k % 32) != 0 || m <= 0 || n <= 0) return false;
-  c.device_read_(a);
-  c.device_read_(qw);
-  c.device_write_(out);
-  return detail::done_(c, c.f.gemm_q4_nt(a, qw, scales, out, m, n, k, group));
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0) return false;
+  L.reads(a, qw);
+  L.writes(out);
+  return L.sent(L.lib.gemm_q4_nt(a, qw, scales, out, m, n, k, group));
 }
 inline bool gemm_q4_nt_swiglu(void* a, void* qw, void* scales, void* act, int64_t m, int64_t ff, int64_t k,
                               int64_t group = 32) {
-  auto& c = context::get();
-  if (!c.ready || (k % 32) != 0 || m <= 0 || ff <= 0) return false;
-  c.device_read_(a);
-  c.device_read_(qw);
-  c.device_write_(act);
-  return detail::done_(c, c.f.gemm_q4_nt_swiglu(a, qw, scales, act, m, ff, k, group));
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || ff <= 0) return false;
+  L.reads(a, qw);
+  L.writes(act);
+  return L.sent(L.lib.gemm_q4_nt_swiglu(a, qw, scales, act, m, ff, k, group));
 }
 inline bool gemm_q4_nt_parts(void* a, void* qw, void* scales, void* parts, int64_t parts_bytes, int64_t m,
                              int64_t n, int64_t k, int* n_parts, int64_t group = 32) {
-  auto& c = context::get();
-  if (!c.ready || (k % 32) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
-  c.device_read_(a);
-  c.device_read_(qw);
-  c.device_write_(parts);
-  return detail::done_(c, c.f.gemm_q4_nt_parts(a, qw, scales, parts, parts_bytes, m, n, k, group, n_parts));
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
+  L.reads(a, qw);
+  L.writes(parts);
+  return L.sent(L.lib.gemm_q4_nt_parts(a, qw, scales, parts, parts_bytes, m, n, k, group, n_parts));
 }
 
 // The product left as its K-split parts ([*n_parts][m][n] in `parts`), for rmsnorm_res_parts.
 inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_bytes, int64_t m, int64_t n,
                                int64_t k, int* n_parts) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
-  c.device_read_(a);
-  c.device_read_(B);
-  c.device_write_(parts);
-  return detail::done_(c, c.f.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
+  launch L;
+  if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
+  L.reads(a, B);
+  L.writes(parts);
+  return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
 }
 
 inline bool attn_decode(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
                         int64_t ctx, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64)) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64)) return false;
   if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
-  c.device_read_(q);
-  c.device_read_(K);
-  c.device_read_(V);
-  c.device_write_(out);
-  return detail::done_(c, c.f.attn_decode(q, K, V, out, n_q_heads, n_kv_heads, ctx, kv_max, D, scale,
+  L.reads(q, K, V);
+  L.writes(out);
+  return L.sent(L.lib.attn_decode(q, K, V, out, n_q_heads, n_kv_heads, ctx, kv_max, D, scale,
                                           kv_bf16 ? 1 : 0));
 }
 
 inline bool attn_prefill(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
                          int64_t T, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false,
                          int64_t pos0 = 0) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64)) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64)) return false;
   if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
   if (T <= 0 || T > 65535) return false;
-  c.device_read_(q);
-  c.device_read_(K);
-  c.device_read_(V);
-  c.device_write_(out);
-  return detail::done_(c, c.f.attn_prefill(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
+  L.reads(q, K, V);
+  L.writes(out);
+  return L.sent(L.lib.attn_prefill(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
                                            kv_bf16 ? 1 : 0, pos0));
 }
 
 inline bool kv_append(void* Kc, void* Vc, void* k_new, void* v_new, int64_t pos, int64_t kv_max,
                       int64_t n_kv_heads, int64_t D, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64)) return false;
-  c.device_read_(k_new);
-  c.device_read_(v_new);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.kv_append(Kc, Vc, k_new, v_new, pos, kv_max, n_kv_heads, D,
+  launch L;
+  if (!L.ok || (D != 128 && D != 64)) return false;
+  L.reads(k_new, v_new);
+  L.writes(Kc, Vc);
+  return L.sent(L.lib.kv_append(Kc, Vc, k_new, v_new, pos, kv_max, n_kv_heads, D,
                                         kv_bf16 ? 1 : 0));
 }
 
 inline bool kv_fill(void* Kc, void* Vc, void* K, void* V, int64_t T, int64_t kv_max,
                     int64_t n_kv_heads, int64_t D, bool kv_bf16 = false, int64_t pos0 = 0) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64)) return false;
-  c.device_read_(K);
-  c.device_read_(V);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.kv_fill(Kc, Vc, K, V, T, kv_max, n_kv_heads, D, kv_bf16 ? 1 : 0, pos0));
+  launch L;
+  if (!L.ok || (D != 128 && D != 64)) return false;
+  L.reads(K, V);
+  L.writes(Kc, Vc);
+  return L.sent(L.lib.kv_fill(Kc, Vc, K, V, T, kv_max, n_kv_heads, D, kv_bf16 ? 1 : 0, pos0));
 }
 
 inline bool rope(void* x, void* out, int64_t rows, int64_t T, int64_t D, int64_t pos, float base,
                  void* bias = nullptr) {
-  auto& c = context::get();
-  if (!c.ready || D <= 0 || (D & 1)) return false;
-  c.device_read_(x);
-  if (bias) c.device_read_(bias);
-  c.device_write_(out);
-  return detail::done_(c, c.f.rope(x, out, rows, T, D, pos, base, bias));
+  launch L;
+  if (!L.ok || D <= 0 || (D & 1)) return false;
+  L.reads(x);
+  if (bias) L.reads(bias);
+  L.writes(out);
+  return L.sent(L.lib.rope(x, out, rows, T, D, pos, base, bias));
 }
 
 inline bool rmsnorm(void* x, void* w, void* out, int64_t n, float eps, int64_t rows = 1) {
-  auto& c = context::get();
-  if (!c.ready || n <= 0 || rows <= 0) return false;
-  c.device_read_(x);
-  c.device_read_(w);
-  c.device_write_(out);
-  return detail::done_(c, c.f.rmsnorm(x, w, out, n, eps, rows));
+  launch L;
+  if (!L.ok || n <= 0 || rows <= 0) return false;
+  L.reads(x, w);
+  L.writes(out);
+  return L.sent(L.lib.rmsnorm(x, w, out, n, eps, rows));
 }
 
 inline bool rmsnorm_res(void* x, void* delta, void* w, void* xout, void* hout, int64_t n, float eps,
                         int64_t rows = 1) {
-  auto& c = context::get();
-  if (!c.ready || n <= 0 || rows <= 0) return false;
-  c.device_read_(x);
-  c.device_read_(delta);
-  c.device_read_(w);
-  c.device_write_(xout);
-  c.device_write_(hout);
-  return detail::done_(c, c.f.rmsnorm_res(x, delta, w, xout, hout, n, eps, rows));
+  launch L;
+  if (!L.ok || n <= 0 || rows <= 0) return false;
+  L.reads(x, delta, w);
+  L.writes(xout, hout);
+  return L.sent(L.lib.rmsnorm_res(x, delta, w, xout, hout, n, eps, rows));
 }
 
 // rmsnorm_res with delta = parts[0] + ... + parts[n_parts-1], rows * n floats apart.
 inline bool rmsnorm_res_parts(void* x, void* parts, int64_t n_parts, void* w, void* xout, void* hout,
                               int64_t n, float eps, int64_t rows = 1) {
-  auto& c = context::get();
-  if (!c.ready || n <= 0 || rows <= 0 || n_parts <= 0) return false;
-  c.device_read_(x);
-  c.device_read_(parts);
-  c.device_read_(w);
-  c.device_write_(xout);
-  c.device_write_(hout);
-  return detail::done_(c, c.f.rmsnorm_res_parts(x, parts, n_parts, w, xout, hout, n, eps, rows));
+  launch L;
+  if (!L.ok || n <= 0 || rows <= 0 || n_parts <= 0) return false;
+  L.reads(x, parts, w);
+  L.writes(xout, hout);
+  return L.sent(L.lib.rmsnorm_res_parts(x, parts, n_parts, w, xout, hout, n, eps, rows));
 }
 
 inline bool swiglu(void* gu, void* out, int64_t ff, int64_t rows = 1) {
-  auto& c = context::get();
-  if (!c.ready || ff <= 0 || rows <= 0) return false;
-  c.device_read_(gu);
-  c.device_write_(out);
-  return detail::done_(c, c.f.swiglu(gu, out, ff, rows));
+  launch L;
+  if (!L.ok || ff <= 0 || rows <= 0) return false;
+  L.reads(gu);
+  L.writes(out);
+  return L.sent(L.lib.swiglu(gu, out, ff, rows));
 }
 
 // Greedy token: reduces on the device, copies 4 bytes back; the one blocking
@@ -739,7 +744,7 @@ inline bool swiglu(void* gu, void* out, int64_t ff, int64_t rows = 1) {
 inline bool argmax(void* in, int64_t n, int64_t* out_idx) {
   auto& c = context::get();
   if (!c.ready || !in || n <= 0 || !out_idx) return false;
-  c.device_read_(in);
+  c.refresh_device(in);
   if (c.f.argmax(in, n, out_idx) != 0) return false;
   c.pending = false;  // the library drained the stream to deliver the index
   return true;
@@ -747,20 +752,20 @@ inline bool argmax(void* in, int64_t n, int64_t* out_idx) {
 
 inline bool split_heads(void* src, void* bias, void* dst, int64_t T, int64_t ld, int64_t off,
                         int64_t H, int64_t D) {
-  auto& c = context::get();
-  if (!c.ready || T <= 0 || H <= 0 || D <= 0) return false;
-  c.device_read_(src);
-  if (bias) c.device_read_(bias);
-  c.device_write_(dst);
-  return detail::done_(c, c.f.split_heads(src, bias, dst, T, ld, off, H, D));
+  launch L;
+  if (!L.ok || T <= 0 || H <= 0 || D <= 0) return false;
+  L.reads(src);
+  if (bias) L.reads(bias);
+  L.writes(dst);
+  return L.sent(L.lib.split_heads(src, bias, dst, T, ld, off, H, D));
 }
 
 inline bool merge_heads(void* src, void* dst, int64_t T, int64_t H, int64_t D) {
-  auto& c = context::get();
-  if (!c.ready || T <= 0 || H <= 0 || D <= 0) return false;
-  c.device_read_(src);
-  c.device_write_(dst);
-  return detail::done_(c, c.f.merge_heads(src, dst, T, H, D));
+  launch L;
+  if (!L.ok || T <= 0 || H <= 0 || D <= 0) return false;
+  L.reads(src);
+  L.writes(dst);
+  return L.sent(L.lib.merge_heads(src, dst, T, H, D));
 }
 
 // One launch for the q/k/v epilogue of a decode step: rope(q,+bq), rope(k,+bk),
@@ -769,16 +774,14 @@ inline bool merge_heads(void* src, void* dst, int64_t T, int64_t H, int64_t D) {
 inline bool qkv_rope_append(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
                             int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                             int64_t kv_max, float base, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || pos < 0 || pos >= kv_max) return false;
-  c.device_read_(qkv);
-  if (bq) c.device_read_(bq);
-  if (bk) c.device_read_(bk);
-  if (bv) c.device_read_(bv);
-  c.device_write_(qkv);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.qkv_rope_append(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || pos < 0 || pos >= kv_max) return false;
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  L.writes(qkv, Kc, Vc);
+  return L.sent(L.lib.qkv_rope_append(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
                                               kv_max, base, kv_bf16 ? 1 : 0));
 }
 
@@ -788,31 +791,28 @@ inline bool qkv_rope_append(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
 // serves every token of a decode loop.
 inline bool rope_dpos(void* x, void* out, int64_t rows, int64_t T, int64_t D, void* d_pos, float base,
                       void* bias = nullptr) {
-  auto& c = context::get();
-  if (!c.ready || D <= 0 || (D & 1) || !d_pos) return false;
-  c.device_read_(x);
-  if (bias) c.device_read_(bias);
-  c.device_read_(d_pos);
-  c.device_write_(out);
-  return detail::done_(c, c.f.rope_dpos(x, out, rows, T, D, d_pos, base, bias));
+  launch L;
+  if (!L.ok || D <= 0 || (D & 1) || !d_pos) return false;
+  L.reads(x);
+  if (bias) L.reads(bias);
+  L.reads(d_pos);
+  L.writes(out);
+  return L.sent(L.lib.rope_dpos(x, out, rows, T, D, d_pos, base, bias));
 }
 inline bool incr_u32(void* d_pos) {
-  auto& c = context::get();
-  if (!c.ready || !d_pos) return false;
-  c.device_read_(d_pos);
-  c.device_write_(d_pos);
-  return detail::done_(c, c.f.incr_u32(d_pos));
+  launch L;
+  if (!L.ok || !d_pos) return false;
+  L.reads(d_pos);
+  L.writes(d_pos);
+  return L.sent(L.lib.incr_u32(d_pos));
 }
 inline bool kv_append_dpos(void* Kc, void* Vc, void* k_new, void* v_new, void* d_pos, int64_t kv_max,
                            int64_t n_kv_heads, int64_t D, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || !d_pos) return false;
-  c.device_read_(k_new);
-  c.device_read_(v_new);
-  c.device_read_(d_pos);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.kv_append_dpos(Kc, Vc, k_new, v_new, d_pos, kv_max, n_kv_heads, D,
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !d_pos) return false;
+  L.reads(k_new, v_new, d_pos);
+  L.writes(Kc, Vc);
+  return L.sent(L.lib.kv_append_dpos(Kc, Vc, k_new, v_new, d_pos, kv_max, n_kv_heads, D,
                                              kv_bf16 ? 1 : 0));
 }
 // Bytes of the caller-owned split-partials buffer attn_decode_dpos needs for a cache.
@@ -823,32 +823,26 @@ inline int64_t attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_
 inline bool attn_decode_dpos(void* q, void* K, void* V, void* out, int64_t n_q_heads,
                              int64_t n_kv_heads, void* d_pos, int64_t kv_max, int64_t D, float scale,
                              void* partials, int64_t partials_bytes, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || !partials || !d_pos) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !partials || !d_pos) return false;
   if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
-  c.device_read_(q);
-  c.device_read_(K);
-  c.device_read_(V);
-  c.device_read_(d_pos);
-  c.device_write_(out);
-  c.device_write_(partials);
-  return detail::done_(c, c.f.attn_decode_dpos(q, K, V, out, n_q_heads, n_kv_heads, d_pos, kv_max, D,
+  L.reads(q, K, V, d_pos);
+  L.writes(out, partials);
+  return L.sent(L.lib.attn_decode_dpos(q, K, V, out, n_q_heads, n_kv_heads, d_pos, kv_max, D,
                                                scale, kv_bf16 ? 1 : 0, partials, partials_bytes));
 }
 inline bool qkv_rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
                                  int64_t n_q_heads, int64_t n_kv_heads, int64_t D, void* d_pos,
                                  int64_t kv_max, float base, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || !d_pos) return false;
-  c.device_read_(qkv);
-  if (bq) c.device_read_(bq);
-  if (bk) c.device_read_(bk);
-  if (bv) c.device_read_(bv);
-  c.device_read_(d_pos);
-  c.device_write_(qkv);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.qkv_rope_append_dpos(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D,
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !d_pos) return false;
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  L.reads(d_pos);
+  L.writes(qkv, Kc, Vc);
+  return L.sent(L.lib.qkv_rope_append_dpos(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D,
                                                    d_pos, kv_max, base, kv_bf16 ? 1 : 0));
 }
 
@@ -857,28 +851,26 @@ inline bool qkv_rope_append_dpos(void* qkv, void* bq, void* bk, void* bv, void* 
 // for position pos (or *d_pos) once, qkv_rope_append_tab reads them instead of
 // evaluating fp64 pow/cos/sin per layer. Bit-identical to qkv_rope_append.
 inline bool rope_table(void* table, int64_t D, int64_t pos, void* d_pos, float base) {
-  auto& c = context::get();
-  if (!c.ready || !table) return false;
-  if (d_pos) c.device_read_(d_pos);
-  c.device_write_(table);
-  return detail::done_(c, c.f.rope_table(table, D, pos, d_pos, base));
+  launch L;
+  if (!L.ok || !table) return false;
+  if (d_pos) L.reads(d_pos);
+  L.writes(table);
+  return L.sent(L.lib.rope_table(table, D, pos, d_pos, base));
 }
 inline bool qkv_rope_append_tab(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc,
                                 int64_t n_q_heads, int64_t n_kv_heads, int64_t D, int64_t pos,
                                 void* d_pos, int64_t kv_max, void* table, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || !table) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !table) return false;
   if (!d_pos && (pos < 0 || pos >= kv_max)) return false;
-  c.device_read_(qkv);
-  if (bq) c.device_read_(bq);
-  if (bk) c.device_read_(bk);
-  if (bv) c.device_read_(bv);
-  if (d_pos) c.device_read_(d_pos);
-  c.device_read_(table);
-  c.device_write_(qkv);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.qkv_rope_append_tab(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  if (d_pos) L.reads(d_pos);
+  L.reads(table);
+  L.writes(qkv, Kc, Vc);
+  return L.sent(L.lib.qkv_rope_append_tab(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, D, pos,
                                                   d_pos, kv_max, table, kv_bf16 ? 1 : 0));
 }
 
@@ -887,41 +879,37 @@ inline bool qkv_rope_append_tab(void* qkv, void* bq, void* bk, void* bv, void* K
 // biases, rotates q and k, writes q head-major into qh [Hq, T, D] and k, v into cache rows
 // pos0 .. pos0+T-1 (one launch for split_heads + 2 x rope + kv_fill; bit-identical to them).
 inline bool rope_table_range(void* table, int64_t D, int64_t pos0, int64_t T, float base) {
-  auto& c = context::get();
-  if (!c.ready || !table) return false;
-  c.device_write_(table);
-  return detail::done_(c, c.f.rope_table_range(table, D, pos0, T, base));
+  launch L;
+  if (!L.ok || !table) return false;
+  L.writes(table);
+  return L.sent(L.lib.rope_table_range(table, D, pos0, T, base));
 }
 // n_parts > 1: qkv is the projection's K-split parts (gemm_bf16_nt_parts), summed as they are read.
 inline bool qkv_rope_fill(void* qkv, void* bq, void* bk, void* bv, void* table, void* qh, void* Kc,
                           void* Vc, int64_t T, int64_t n_q_heads, int64_t n_kv_heads, int64_t D,
                           int64_t pos0, int64_t kv_max, bool kv_bf16 = false, int64_t n_parts = 1) {
-  auto& c = context::get();
-  if (!c.ready || !table || (D != 128 && D != 64) || pos0 < 0 || pos0 + T > kv_max || n_parts <= 0) return false;
-  c.device_read_(qkv);
-  if (bq) c.device_read_(bq);
-  if (bk) c.device_read_(bk);
-  if (bv) c.device_read_(bv);
-  c.device_read_(table);
-  c.device_write_(qh);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  return detail::done_(c, c.f.qkv_rope_fill_parts(qkv, n_parts, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads,
+  launch L;
+  if (!L.ok || !table || (D != 128 && D != 64) || pos0 < 0 || pos0 + T > kv_max || n_parts <= 0) return false;
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  L.reads(table);
+  L.writes(qh, Kc, Vc);
+  return L.sent(L.lib.qkv_rope_fill_parts(qkv, n_parts, bq, bk, bv, table, qh, Kc, Vc, T, n_q_heads,
                                                   n_kv_heads, D, pos0, kv_max, kv_bf16 ? 1 : 0));
 }
 // attn_prefill with the result written token-major, [T, Hq*D] (no merge_heads afterwards).
 inline bool attn_prefill_tok(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
                              int64_t T, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false,
                              int64_t pos0 = 0) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64)) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64)) return false;
   if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
   if (T <= 0 || T > 65535) return false;
-  c.device_read_(q);
-  c.device_read_(K);
-  c.device_read_(V);
-  c.device_write_(out);
-  return detail::done_(c, c.f.attn_prefill_tok(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
+  L.reads(q, K, V);
+  L.writes(out);
+  return L.sent(L.lib.attn_prefill_tok(q, K, V, out, n_q_heads, n_kv_heads, T, kv_max, D, scale,
                                                kv_bf16 ? 1 : 0, pos0));
 }
 
@@ -931,21 +919,19 @@ inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
                             int64_t n_q_heads, int64_t n_kv_heads, int64_t pos, void* d_pos,
                             int64_t kv_max, int64_t D, float scale, void* table, void* partials,
                             int64_t partials_bytes, bool kv_bf16 = false) {
-  auto& c = context::get();
-  if (!c.ready || (D != 128 && D != 64) || !table) return false;
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !table) return false;
   if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
   if (d_pos ? !partials : (pos < 0 || pos >= kv_max)) return false;
-  c.device_read_(qkv);
-  if (bq) c.device_read_(bq);
-  if (bk) c.device_read_(bk);
-  if (bv) c.device_read_(bv);
-  if (d_pos) c.device_read_(d_pos);
-  c.device_read_(table);
-  c.device_write_(Kc);
-  c.device_write_(Vc);
-  c.device_write_(out);
-  if (partials) c.device_write_(partials);
-  return detail::done_(c, c.f.attn_decode_qkv(qkv, bq, bk, bv, Kc, Vc, out, n_q_heads, n_kv_heads, pos,
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  if (d_pos) L.reads(d_pos);
+  L.reads(table);
+  L.writes(Kc, Vc, out);
+  if (partials) L.writes(partials);
+  return L.sent(L.lib.attn_decode_qkv(qkv, bq, bk, bv, Kc, Vc, out, n_q_heads, n_kv_heads, pos,
                                               d_pos, kv_max, D, scale, table, kv_bf16 ? 1 : 0, partials,
                                               partials_bytes));
 }
@@ -955,36 +941,35 @@ inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
 enum class elem : int { f32 = 0, f16 = 1, bf16 = 2 };
 // dst[i] = narrow(widen(src[i])): file rows [out, in] into bf16 (or f32) rows [N, K].
 inline bool convert(void* src, elem st, void* dst, elem dt, int64_t n) {
-  auto& c = context::get();
-  if (!c.ready || !src || !dst || n <= 0) return false;
-  c.device_read_(src);
-  c.device_write_(dst);
-  return detail::done_(c, c.f.convert(src, (int)st, dst, (int)dt, n));
+  launch L;
+  if (!L.ok || !src || !dst || n <= 0) return false;
+  L.reads(src);
+  L.writes(dst);
+  return L.sent(L.lib.convert(src, (int)st, dst, (int)dt, n));
 }
 // file rows [out = rows, in = cols] into the seam's [K, N] layout at columns [col_base, col_base + rows)
 inline bool convert_transpose(void* src, elem st, void* dst, elem dt, int64_t rows, int64_t cols,
                               int64_t ld_dst, int64_t col_base) {
-  auto& c = context::get();
-  if (!c.ready || !src || !dst) return false;
-  c.device_read_(src);
-  c.device_write_(dst);
-  return detail::done_(c, c.f.convert_transpose(src, (int)st, dst, (int)dt, rows, cols, ld_dst, col_base));
+  launch L;
+  if (!L.ok || !src || !dst) return false;
+  L.reads(src);
+  L.writes(dst);
+  return L.sent(L.lib.convert_transpose(src, (int)st, dst, (int)dt, rows, cols, ld_dst, col_base));
 }
 // array::to_q4 of the widened rows, written into the packed and scale sections given
 inline bool quantize_q4(void* src, elem st, void* packed, void* scales, int64_t rows, int64_t K) {
-  auto& c = context::get();
-  if (!c.ready || !src || !packed || !scales) return false;
-  c.device_read_(src);
-  c.device_write_(packed);
-  return detail::done_(c, c.f.quantize_q4(src, (int)st, packed, scales, rows, K, kQ4Group));
+  launch L;
+  if (!L.ok || !src || !packed || !scales) return false;
+  L.reads(src);
+  L.writes(packed);
+  return L.sent(L.lib.quantize_q4(src, (int)st, packed, scales, rows, K, kQ4Group));
 }
 inline bool embed_gather_f16(void* table, void* d_token, void* out, int64_t hidden, int64_t vocab) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(table);
-  c.device_read_(d_token);
-  c.device_write_(out);
-  return detail::done_(c, c.f.embed_gather_f16(table, d_token, out, hidden, vocab));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(table, d_token);
+  L.writes(out);
+  return L.sent(L.lib.embed_gather_f16(table, d_token, out, hidden, vocab));
 }
 
 // ---- device-resident greedy loop -----------------------------------------------------------
@@ -992,28 +977,26 @@ inline bool embed_gather_f16(void* table, void* d_token, void* out, int64_t hidd
 // int32, what argmax_async wrote) is gathered on the device, and the step's tail
 // appends the token to a device history and advances the position.
 inline bool embed_gather_bf16(void* table, void* d_token, void* out, int64_t hidden, int64_t vocab) {
-  auto& c = context::get();
-  if (!c.ready) return false;
-  c.device_read_(table);
-  c.device_read_(d_token);
-  c.device_write_(out);
-  return detail::done_(c, c.f.embed_gather_bf16(table, d_token, out, hidden, vocab));
+  launch L;
+  if (!L.ok) return false;
+  L.reads(table, d_token);
+  L.writes(out);
+  return L.sent(L.lib.embed_gather_bf16(table, d_token, out, hidden, vocab));
 }
 inline bool argmax_async(void* in, int64_t n, void* d_token) {
-  auto& c = context::get();
-  if (!c.ready || !d_token) return false;
-  c.device_read_(in);
-  c.device_write_(d_token);
-  return detail::done_(c, c.f.argmax_async(in, n, d_token));
+  launch L;
+  if (!L.ok || !d_token) return false;
+  L.reads(in);
+  L.writes(d_token);
+  return L.sent(L.lib.argmax_async(in, n, d_token));
 }
 inline bool token_advance(void* d_pos, void* d_token, void* history, int64_t capacity) {
-  auto& c = context::get();
-  if (!c.ready || !d_pos || !d_token) return false;
-  c.device_read_(d_pos);
-  c.device_read_(d_token);
-  c.device_write_(d_pos);
-  if (history) c.device_write_(history);
-  return detail::done_(c, c.f.token_advance(d_pos, d_token, history, capacity));
+  launch L;
+  if (!L.ok || !d_pos || !d_token) return false;
+  L.reads(d_pos, d_token);
+  L.writes(d_pos);
+  if (history) L.writes(history);
+  return L.sent(L.lib.token_advance(d_pos, d_token, history, capacity));
 }
 
 // GEMVs that evaluate the producer of their activation vector while staging it:
@@ -1022,76 +1005,67 @@ inline bool token_advance(void* d_pos, void* d_token, void* history, int64_t cap
 // issues the two separate calls.
 inline bool gemv_q4_swiglu(void* gu, void* qw, void* scales, void* y, int64_t N, int64_t K,
                            int64_t group) {
-  auto& c = context::get();
-  if (!c.ready || group != 32 || (K % 32) != 0) return false;
-  c.device_read_(gu);
-  c.device_read_(qw);
-  c.device_read_(scales);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_q4_swiglu(gu, qw, scales, y, N, K, group));
+  launch L;
+  if (!L.ok || group != 32 || (K % 32) != 0) return false;
+  L.reads(gu, qw, scales);
+  L.writes(y);
+  return L.sent(L.lib.gemv_q4_swiglu(gu, qw, scales, y, N, K, group));
 }
 inline bool gemv_bf16_row_swiglu(void* gu, void* B, void* y, int64_t n, int64_t k) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0) return false;
-  c.device_read_(gu);
-  c.device_read_(B);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_bf16_row_swiglu(gu, B, y, n, k));
+  launch L;
+  if (!L.ok || (k % 8) != 0) return false;
+  L.reads(gu, B);
+  L.writes(y);
+  return L.sent(L.lib.gemv_bf16_row_swiglu(gu, B, y, n, k));
 }
 // s = x (+ delta); xout (optional, distinct from x and delta) receives s;
 // y = W . rmsnorm(s, norm_w, eps)
 inline bool gemv_q4_rmsnorm(void* x, void* delta, void* norm_w, void* xout, void* qw, void* scales,
                             void* y, int64_t N, int64_t K, int64_t group, float eps) {
-  auto& c = context::get();
-  if (!c.ready || group != 32 || (K % 32) != 0 || (xout && (xout == x || xout == delta))) return false;
-  c.device_read_(x);
-  if (delta) c.device_read_(delta);
-  c.device_read_(norm_w);
-  c.device_read_(qw);
-  c.device_read_(scales);
-  if (xout) c.device_write_(xout);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_q4_rmsnorm(x, delta, norm_w, xout, qw, scales, y, N, K, group, eps));
+  launch L;
+  if (!L.ok || group != 32 || (K % 32) != 0 || (xout && (xout == x || xout == delta))) return false;
+  L.reads(x);
+  if (delta) L.reads(delta);
+  L.reads(norm_w, qw, scales);
+  if (xout) L.writes(xout);
+  L.writes(y);
+  return L.sent(L.lib.gemv_q4_rmsnorm(x, delta, norm_w, xout, qw, scales, y, N, K, group, eps));
 }
 inline bool gemv_bf16_row_rmsnorm(void* x, void* delta, void* norm_w, void* xout, void* B, void* y,
                                   int64_t n, int64_t k, float eps) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0 || (xout && (xout == x || xout == delta))) return false;
-  c.device_read_(x);
-  if (delta) c.device_read_(delta);
-  c.device_read_(norm_w);
-  c.device_read_(B);
-  if (xout) c.device_write_(xout);
-  c.device_write_(y);
-  return detail::done_(c, c.f.gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, B, y, n, k, eps));
+  launch L;
+  if (!L.ok || (k % 8) != 0 || (xout && (xout == x || xout == delta))) return false;
+  L.reads(x);
+  if (delta) L.reads(delta);
+  L.reads(norm_w, B);
+  if (xout) L.writes(xout);
+  L.writes(y);
+  return L.sent(L.lib.gemv_bf16_row_rmsnorm(x, delta, norm_w, xout, B, y, n, k, eps));
 }
 // The same with W = [gate rows | up rows] (N2 / 2 each) and the gated activation as the
 // epilogue: act[i] = swiglu(gate_i, up_i), i < N2 / 2.
 inline bool gemv_q4_rmsnorm_gateup(void* x, void* delta, void* norm_w, void* xout, void* qw, void* scales,
                                    void* act, int64_t N2, int64_t K, int64_t group, float eps) {
-  auto& c = context::get();
-  if (!c.ready || group != 32 || (K % 32) != 0 || (N2 % 2) != 0 || (xout && (xout == x || xout == delta)))
+  launch L;
+  if (!L.ok || group != 32 || (K % 32) != 0 || (N2 % 2) != 0 || (xout && (xout == x || xout == delta)))
     return false;
-  c.device_read_(x);
-  if (delta) c.device_read_(delta);
-  c.device_read_(norm_w);
-  c.device_read_(qw);
-  c.device_read_(scales);
-  if (xout) c.device_write_(xout);
-  c.device_write_(act);
-  return detail::done_(c, c.f.gemv_q4_rmsnorm_gateup(x, delta, norm_w, xout, qw, scales, act, N2, K, group, eps));
+  L.reads(x);
+  if (delta) L.reads(delta);
+  L.reads(norm_w, qw, scales);
+  if (xout) L.writes(xout);
+  L.writes(act);
+  return L.sent(L.lib.gemv_q4_rmsnorm_gateup(x, delta, norm_w, xout, qw, scales, act, N2, K, group, eps));
 }
 inline bool gemv_bf16_row_rmsnorm_gateup(void* x, void* delta, void* norm_w, void* xout, void* B, void* act,
                                          int64_t n2, int64_t k, float eps) {
-  auto& c = context::get();
-  if (!c.ready || (k % 8) != 0 || (n2 % 2) != 0 || (xout && (xout == x || xout == delta))) return false;
-  c.device_read_(x);
-  if (delta) c.device_read_(delta);
-  c.device_read_(norm_w);
-  c.device_read_(B);
-  if (xout) c.device_write_(xout);
-  c.device_write_(act);
-  return detail::done_(c, c.f.gemv_bf16_row_rmsnorm_gateup(x, delta, norm_w, xout, B, act, n2, k, eps));
+  launch L;
+  if (!L.ok || (k % 8) != 0 || (n2 % 2) != 0 || (xout && (xout == x || xout == delta))) return false;
+  L.reads(x);
+  if (delta) L.reads(delta);
+  L.reads(norm_w, B);
+  if (xout) L.writes(xout);
+  L.writes(act);
+  return L.sent(L.lib.gemv_bf16_row_rmsnorm_gateup(x, delta, norm_w, xout, B, act, n2, k, eps));
 }
 
 // ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------
@@ -1123,13 +1097,12 @@ inline void* capture_end() {
 inline bool graph_launch(void* g) {
   auto& c = context::get();
   if (!c.ready || !g) return false;
-  if (!detail::done_(c, c.f.graph_launch(g))) return false;
+  if (c.f.graph_launch(g) != 0) return false;
+  c.pending = true;
   auto it = c.graph_writes.find(g);
   if (it != c.graph_writes.end())
-    for (uintptr_t a : it->second) {
-      auto m = c.mirrors.find(a);
-      if (m != c.mirrors.end()) m->second.where = context::DEVICE;
-    }
+    for (uintptr_t base : it->second)
+      if (extent* e = c.buffers.at_base(base)) e->live = extent::side::device;
   return true;
 }
 inline void graph_destroy(void* g) {

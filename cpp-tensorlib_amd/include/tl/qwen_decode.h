@@ -626,14 +626,17 @@ inline void set_cache_pos(model& M, int64_t p) {
 }
 
 // Widen one embedding row into the staged input (host gather, one small H2D).
-inline void stage_embed(model& M, int64_t token) {
+// false for a token id outside [0, vocab): nothing is read or uploaded.
+inline bool stage_embed(model& M, int64_t token) {
   const dims& d = M.d;
+  if (token < 0 || token >= d.vocab) return false;
   const uint16_t* r = M.embed.data() + (size_t)token * d.hidden;
   if (M.embed_f16)
     for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = f16_to_f32(r[j]);
   else
     for (int64_t j = 0; j < d.hidden; j++) M.s.embed_host[j] = bf16_to_f32(r[j]);
   hip::upload(M.s.embedb, M.s.embed_host, d.hidden);
+  return true;
 }
 
 // All layers + final norm + lm_head on the scratch buffers, no allocation, no
@@ -725,8 +728,7 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
 // embed -> layers -> device argmax. Returns the greedy token, or -1 when any
 // launch was declined.
 inline int64_t step_greedy(model& M, int64_t token, int64_t pos) {
-  stage_embed(M, token);
-  if (!run_layers(M, M.s.embedb, pos)) return -1;
+  if (!stage_embed(M, token) || !run_layers(M, M.s.embedb, pos)) return -1;
   int64_t idx = -1;
   if (!hip::argmax(M.s.logitsb, M.d.vocab, &idx)) return -1;
   return idx;
@@ -830,9 +832,12 @@ inline bool prefill_layers(model& M, int64_t T) {
 }
 
 // Gather T embedding rows on the host and upload them as the chunk input.
+// false for a token id outside [0, vocab), before anything is read.
 inline bool stage_chunk(model& M, const int64_t* tokens, int64_t T) {
-  if (!prefill_reserve(M, T)) return false;
   const dims& d = M.d;
+  for (int64_t t = 0; t < T; t++)
+    if (tokens[t] < 0 || tokens[t] >= d.vocab) return false;
+  if (!prefill_reserve(M, T)) return false;
   for (int64_t t = 0; t < T; t++) {
     const uint16_t* r = M.embed.data() + (size_t)tokens[t] * d.hidden;
     float* o = M.ps.emb_host + t * d.hidden;
@@ -917,6 +922,7 @@ struct greedy_loop {
   bool init(model& M, int64_t first_id, int64_t pos) {
     if (M.layers.empty() || !M.fused || !hip::graph_available()) return false;
     const dims& d = M.d;
+    if (first_id < 0 || first_id >= d.vocab) return false;   // later ids are argmax results, in range by construction
     max_ctx = M.layers[0].cache.max_ctx;
     cur_pos = pos;
     if (!upload_embed(M)) return false;
@@ -994,7 +1000,7 @@ struct captured_decoder {
     }
     d_pos = hip::alloc(4, nullptr);
     if (!d_pos) return false;
-    stage_embed(M, first_id);
+    if (!stage_embed(M, first_id)) return false;
     hip::upload_u32(d_pos, (unsigned)pos);
     // warm run: real launches (they also size the library's scratch); it advances d_pos
     // and writes cache row pos, which the first recorded step rewrites identically
@@ -1009,8 +1015,7 @@ struct captured_decoder {
   }
   // Feed token `id` at the current position without reading a token back.
   bool feed(model& M, int64_t id) {
-    if (cur_pos >= max_ctx) return false;
-    stage_embed(M, id);
+    if (cur_pos >= max_ctx || !stage_embed(M, id)) return false;
     bool ok;
     if (graph) ok = hip::graph_launch(graph);
     else ok = run_layers(M, M.s.embedb, cur_pos);

@@ -376,29 +376,10 @@ int tlhip_split_heads(const void* src, const void* bias, void* dst, int64_t T, i
 /* [H,T,D] -> [T,H*D].  cuda.h:866-879 */
 int tlhip_merge_heads(const void* src, void* dst, int64_t T, int64_t H, int64_t D);
 
-/* ---- measurement yardsticks (benchmarks only; no reference counterpart) --------
- * A plain 16-byte-per-lane streaming copy / read of `bytes` bytes, used to find
- * the HBM rate this GPU really sustains and to scale the profiler's traffic
- * counters. blocks <= 0 picks 8 blocks per CU. */
-int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks);
-int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
-
-/* ---- tuning hook (benchmarks only) --------------------------------------------
- * Overrides the int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts
- * sharing one row's K range (a power of two), resident blocks per CU,
- * wavefronts per block (<= 16) and lanes that share a weight row (64 or 16);
- * 0 restores the built-in choice for that field.
- * Results do not depend on it beyond fp32 summation order. */
-int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
-                       int lanes_per_row);
 /* Upper bound on the K splits of the [K,N] GEMVs (tlhip_gemv_f32 / tlhip_gemv_bf16); 1 = no
  * split, 0 = the built-in choice. The reference's diagnostic knob set_no_splitk (cuda.h:193-197,
- * 496-497), which its GEMV benchmark toggles. */
+ * 496-497), which its GEMV benchmark toggles through the backend header. */
 int tlhip_tune_gemv_cols(int max_k_splits);
-/* Which kernel serves tlhip_attn_prefill: 0 = the matrix-pipe one (default), 1 = the VALU kernel
- * that shares its code with decode attention. Same results within fp32 summation order; for A/B
- * timing and tests. No reference counterpart. */
-int tlhip_tune_attn_prefill(int valu_kernel);
 
 #ifdef __cplusplus
 }

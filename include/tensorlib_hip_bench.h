@@ -1,0 +1,41 @@
+/* Benchmark and tuning entry points of libtensorlib_hip.so.
+ *
+ * Not part of the backend boundary: a backend header binds include/tensorlib_hip.h only.
+ * These serve bench.py, the profiles and the tests that force a launch shape. They set
+ * process-wide state: a caller that changes a launch shape restores it with the same call
+ * (zeros) or with tlhip_tune_reset(). None has a counterpart in the reference.
+ */
+#ifndef TENSORLIB_HIP_BENCH_H
+#define TENSORLIB_HIP_BENCH_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- measurement yardsticks ---------------------------------------------------------
+ * A plain 16-byte-per-lane streaming copy / read of `bytes` bytes, used to find
+ * the HBM rate this GPU really sustains and to scale the profiler's traffic
+ * counters. blocks <= 0 picks 8 blocks per CU. */
+int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks);
+int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
+
+/* ---- launch-shape overrides ----------------------------------------------------------
+ * The int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts sharing one row's K
+ * range, resident blocks per CU, wavefronts per block (<= 16; rounded down to a multiple of
+ * the K-sharing wavefronts) and lanes that share a weight row (64 or 16); 0 restores the
+ * built-in choice for that field. Results do not depend on it beyond fp32 summation order. */
+int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
+                       int lanes_per_row);
+/* Which kernel serves tlhip_attn_prefill: 0 = the matrix-pipe one (default), 1 = the VALU kernel
+ * that shares its code with decode attention. Same results within fp32 summation order; for A/B
+ * timing and tests. */
+int tlhip_tune_attn_prefill(int valu_kernel);
+/* Every override back to the built-in choice (tlhip_tune_gemv_cols included). */
+int tlhip_tune_reset(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENSORLIB_HIP_BENCH_H */

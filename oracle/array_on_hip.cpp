@@ -161,6 +161,33 @@ int main() {
       return x1 + m.dot(make(wd, {FF, E}).to_q4());
     }, C_GEMV_Q4, 7);
   }
+  // ---- an op the library refuses in the middle of a graph -----------------------------------------
+  // head_dim 96 is outside what tlhip_attn_decode takes (64 and 128: cuda.h:970-971): the backend
+  // header turns the refusal into `false`, the evaluator runs that one node on its CPU path and
+  // the nodes around it stay on the GPU. Same result as the all-CPU evaluation; the attention
+  // counter must not move, the elementwise and GEMV counters must.
+  {
+    const int64_t H = 4, D = 96, ctx = 50, E = H * D;
+    const auto x = normal(E, 71), wq = normal(E * E, 72, 0.f, 0.02f), k = normal(H * ctx * D, 73), v = normal(H * ctx * D, 74),
+               wo = normal(E * E, 75, 0.f, 0.02f);
+    const auto graph = [&] {
+      array xa = make(x, {1, E});
+      array q = (xa * 2.0f + 0.5f).dot(make(wq, {E, E}).to_q4()).reshape({H, D});
+      array a = array::attn_decode(q, make(k, {H, ctx, D}), make(v, {H, ctx, D}), 0.1f).reshape({1, E});
+      return (a.dot(make(wo, {E, E}).to_q4()) + xa).sigmoid();
+    };
+    tl::use_gpu();
+    const std::vector<uint64_t> before = tl::hip::census();
+    (void)values(graph());
+    const std::vector<uint64_t> after = tl::hip::census();
+    tl::use_cpu();
+    const bool attn_ran = after[C_ATTN] != before[C_ATTN];
+    check("graph with a refused op (attn D=96) in the middle", graph, C_GEMV_Q4, 2);
+    std::printf("%-44s %s  attention launches %lld (must be 0), unary %lld\n", "  refused op stayed on the CPU",
+                attn_ran ? "FAIL" : "PASS", (long long)(after[C_ATTN] - before[C_ATTN]),
+                (long long)(after[C_UNARY] - before[C_UNARY]));
+    if (attn_ran || after[C_UNARY] == before[C_UNARY]) failures++;
+  }
   std::printf(failures ? "%d case(s) FAILED\n" : "ALL OK\n", failures);
   return failures ? 1 : 0;
 }

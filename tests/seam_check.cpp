@@ -5,14 +5,14 @@
 // storage-like buffers obtained from alloc(bytes, &contents). Every case is
 // checked against plain host loops written here. Exit status 0 = all cases ok.
 //
-// Built by build.py into lib/tl_seam_check; needs a gfx950 GPU to run.
+// Built by tests/build_programs.py into tests/bin/tl_seam_check; needs a gfx950 GPU to run.
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <vector>
 
-#include "../include/tl/hip.h"
+#include "tl/hip.h"
 
 namespace hip = tl::hip;
 using tl::hip::kop;

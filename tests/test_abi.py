@@ -10,10 +10,14 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "tensorlib_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(tlhip_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(headers=("tensorlib_hip.h", "tensorlib_hip_bench.h")):
+    """Entry points declared by the boundary header and by the benchmark / tuning header."""
+    names = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(tlhip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_every_declared_symbol_is_exported(pkg):
@@ -22,6 +26,13 @@ def test_every_declared_symbol_is_exported(pkg):
     assert len(names) >= 45
     for n in names:
         assert hasattr(lib, n), "%s declared in tensorlib_hip.h but not exported" % n
+
+
+def test_boundary_header_holds_no_benchmark_or_tuning_hooks():
+    """What a backend binds and what benchmarks use are declared apart."""
+    boundary = declared_symbols(("tensorlib_hip.h",))
+    assert not [n for n in boundary if n.startswith("tlhip_bench_")]
+    assert [n for n in boundary if n.startswith("tlhip_tune_")] == ["tlhip_tune_gemv_cols"]   # the reference's set_no_splitk
 
 
 def test_python_binding_matches_header(pkg):

@@ -247,3 +247,28 @@ def test_greedy_loop_on_the_device(orc, dims, n, q4):
     left = dims["max_ctx"] - (start + n)
     assert g.greedy_run(left + 5) == left
     g.close(); om.close()
+
+
+def test_token_ids_outside_the_vocabulary_are_declined(orc):
+    """An id outside [0, vocab) never indexes the host embedding table: the step, the chunk, the
+    recorded decoder and the on-device loop all decline it, and the model keeps working after."""
+    qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
+    om = orc.qwen_create(SMALL, seed=8, q4=True)
+    g = qwen.QwenGPU.from_blobs(om)
+    V = SMALL["vocab"]
+    for bad in (-1, V, V + 12345, 1 << 40):
+        with pytest.raises(RuntimeError):
+            g.step(bad, 0)
+        with pytest.raises(RuntimeError):
+            g.run_layers(bad, 0)
+        with pytest.raises(RuntimeError):
+            g.prefill([1, 2, bad, 3], want_logits=False)
+        with pytest.raises(RuntimeError):
+            g.stage_chunk([bad])
+        with pytest.raises(RuntimeError):
+            g.greedy_init(bad, 0)
+    want_tok, want_logits = om.step(7, 0)
+    got_tok, got_logits = g.step(7, 0, want_logits=True)
+    assert maxrel(got_logits, want_logits) < 2e-3
+    assert got_tok == want_tok or _near_tie(want_logits)
+    g.close(); om.close()
