@@ -458,8 +458,9 @@ class TlHip:
         self._chk(self.c.tlhip_attn_prefill_tok(q.ptr, K.ptr, V.ptr, out.ptr, Hq, Hkv, T, kv_max, D, scale,
                                                 1 if kv_bf16 else 0, pos0))
 
-    def tune_attn_prefill(self, valu_kernel):
-        self._chk(self.c.tlhip_tune_attn_prefill(1 if valu_kernel else 0))
+    def tune_attn_prefill(self, kernel):
+        """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes."""
+        self._chk(self.c.tlhip_tune_attn_prefill(int(kernel)))
 
     def tune_reset(self):
         self._chk(self.c.tlhip_tune_reset())

@@ -66,42 +66,11 @@ struct QkvFuse {
   int64_t kv_max;
 };
 
-// Rotates elements [d0, d0+4) of a head row that is spread over the 16 lanes of a DPP
-// row (lane c holds D/16 consecutive elements). `own` holds this lane's elements with
-// the bias added; the rotation partner, element d +- D/2, sits in lane c ^ 8 of the
-// same row, which is a rotation of the row by 8 lanes (DPP row_ror:8).
-__device__ __forceinline__ float dpp_ror8(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, true));
-}
-template <int D>
-__device__ __forceinline__ float4 rope4(float4 own, const float2* __restrict__ table, int d0) {
-  constexpr int half = D / 2;
-  const bool lo = d0 < half;
-  const int j0 = lo ? d0 : d0 - half;
-  const float4 oth = make_float4(dpp_ror8(own.x), dpp_ror8(own.y), dpp_ror8(own.z), dpp_ror8(own.w));
-  const float4 a = lo ? own : oth;   // x0: elements j
-  const float4 b = lo ? oth : own;   // x1: elements j + half
-  const float4 t0 = *reinterpret_cast<const float4*>(table + j0);       // (c0, s0, c1, s1)
-  const float4 t1 = *reinterpret_cast<const float4*>(table + j0 + 2);   // (c2, s2, c3, s3)
-  float4 o;
-  if (lo) {
-    o.x = sub_rn(mul_rn(a.x, t0.x), mul_rn(b.x, t0.y));
-    o.y = sub_rn(mul_rn(a.y, t0.z), mul_rn(b.y, t0.w));
-    o.z = sub_rn(mul_rn(a.z, t1.x), mul_rn(b.z, t1.y));
-    o.w = sub_rn(mul_rn(a.w, t1.z), mul_rn(b.w, t1.w));
-  } else {
-    o.x = add_rn(mul_rn(a.x, t0.y), mul_rn(b.x, t0.x));
-    o.y = add_rn(mul_rn(a.y, t0.w), mul_rn(b.y, t0.z));
-    o.z = add_rn(mul_rn(a.z, t1.y), mul_rn(b.z, t1.x));
-    o.w = add_rn(mul_rn(a.w, t1.w), mul_rn(b.w, t1.z));
-  }
-  return o;
-}
-// The same with the four (cos, sin) pairs of elements d0 .. d0+3 already in registers.
-template <int D>
-__device__ __forceinline__ float4 rope4_tab(float4 own, const float4 t0, const float4 t1, int d0) {
-  const bool lo = d0 < D / 2;
-  const float4 oth = make_float4(dpp_ror8(own.x), dpp_ror8(own.y), dpp_ror8(own.z), dpp_ror8(own.w));
+// Rotates four consecutive elements of a head row. `own` holds elements d0 .. d0+3 with the bias
+// added, `oth` their rotation partners (elements d -+ D/2), t0/t1 the four (cos, sin) pairs of
+// j = d mod D/2, lo says whether `own` is the lower half. The arithmetic - two unfused
+// multiplies, then one add or subtract - is that of the stand-alone rotation kernels.
+__device__ __forceinline__ float4 rope4_pair(float4 own, float4 oth, float4 t0, float4 t1, bool lo) {
   const float4 a = lo ? own : oth;   // x0: elements j
   const float4 b = lo ? oth : own;   // x1: elements j + half
   float4 o;
@@ -160,6 +129,10 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     int n_kv_heads, int n_head_groups) {
   constexpr int EPL = D / 16;        // floats of a key row per lane (4 or 8)
   constexpr int NV = EPL / 4;        // float4 loads per lane per key
+  // Lane c of a row holds elements [4c, 4c+4) of each of the NV consecutive 64-element
+  // parts of a key row, so that one load instruction of the 16 lanes covers 256 contiguous
+  // bytes of the row (64 elements) - and, with D = 128, a rotation pair (d, d + 64) in one lane.
+  const auto dim0 = [](int cc, int v) { return v * 64 + cc * 4; };
   constexpr int UNR = 4;             // key steps in flight per lane
   // Decode at short and medium contexts gives a wavefront one or two tiles, and the step
   // is a chain of memory latencies. The first K and V rows of the wavefront's first tile
@@ -235,7 +208,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     for (int g = 0; g < G; g++) {
       const size_t r = (row0 + (size_t)min(g, ng - 1)) * D;
 #pragma unroll
-      for (int v = 0; v < NV; v++) qraw[g][v] = *reinterpret_cast<const float4*>(q + r + c * EPL + v * 4);
+      for (int v = 0; v < NV; v++) qraw[g][v] = *reinterpret_cast<const float4*>(q + r + dim0(c, v));
     }
   } else {
     if (tq < QT) {
@@ -260,8 +233,8 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
       const int key = min(kb0 + u * 4 + slot, kv_rows - 1);
 #pragma unroll
       for (int v = 0; v < NV; v++) {
-        kpre[u][v] = KvLoad<KT>::ld(K + hoff + (size_t)key * D + c * EPL + v * 4);
-        vpre[u][v] = KvLoad<KT>::ld(V + hoff + (size_t)key * D + c * EPL + v * 4);
+        kpre[u][v] = KvLoad<KT>::ld(K + hoff + (size_t)key * D + dim0(c, v));
+        vpre[u][v] = KvLoad<KT>::ld(V + hoff + (size_t)key * D + dim0(c, v));
       }
     }
   }
@@ -308,13 +281,15 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
     for (int g = 0; g < G; g++)
 #pragma unroll
       for (int v = 0; v < NV; v++) {
-        const int d0 = c * EPL + v * 4;
+        const int d0 = dim0(c, v);
         const float4 own = *reinterpret_cast<const float4*>(&qs[g][d0]);
         if constexpr (QKV) {
-          const int j0 = d0 < D / 2 ? d0 : d0 - D / 2;
+          const bool lo = d0 < D / 2;
+          const int j0 = lo ? d0 : d0 - D / 2;
+          const float4 oth = *reinterpret_cast<const float4*>(&qs[g][lo ? d0 + D / 2 : d0 - D / 2]);
           const float4 t0 = *reinterpret_cast<const float4*>(&tabs[2 * j0]);       // (c0, s0, c1, s1)
           const float4 t1 = *reinterpret_cast<const float4*>(&tabs[2 * j0 + 4]);   // (c2, s2, c3, s3)
-          qv[g][v] = rope4_tab<D>(own, t0, t1, d0);
+          qv[g][v] = rope4_pair(own, oth, t0, t1, lo);
         } else {
           qv[g][v] = own;
         }
@@ -367,9 +342,13 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
       float4 kn[NV], vn[NV];
 #pragma unroll
       for (int v = 0; v < NV; v++) {
-        const int d0 = c * EPL + v * 4;
-        const float4 kr =
-            rope4<D>(load_biased4(kraw, fz.bk ? fz.bk + (size_t)kvh * D : nullptr, d0), fz.table, d0);
+        const int d0 = dim0(c, v);
+        const bool lo = d0 < D / 2;
+        const int j0 = lo ? d0 : d0 - D / 2;
+        const float* kb = fz.bk ? fz.bk + (size_t)kvh * D : nullptr;
+        const float4 kr = rope4_pair(load_biased4(kraw, kb, d0), load_biased4(kraw, kb, lo ? d0 + D / 2 : d0 - D / 2),
+                                     *reinterpret_cast<const float4*>(fz.table + j0),
+                                     *reinterpret_cast<const float4*>(fz.table + j0 + 2), lo);
         const float4 vr = load_biased4(vraw, fz.bv ? fz.bv + (size_t)kvh * D : nullptr, d0);
         kn[v] = kv_store4(krow + d0, kr, store);
         vn[v] = kv_store4(vrow + d0, vr, store);
@@ -427,7 +406,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
           const int key = kb + (i0 + u) * 4 + slot;
 #pragma unroll
           for (int v = 0; v < NV; v++)
-            kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + c * EPL + v * 4)
+            kv[u][v] = key < k_end ? KvLoad<KT>::ld(Kh + (size_t)key * D + dim0(c, v))
                                    : make_float4(0.f, 0.f, 0.f, 0.f);
         }
         if (i0 == 0) {
@@ -436,7 +415,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
             const int key = kb + u * 4 + slot;
 #pragma unroll
             for (int v = 0; v < NV; v++)
-              vfirst[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+              vfirst[u][v] = key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + dim0(c, v))
                                          : make_float4(0.f, 0.f, 0.f, 0.f);
           }
         }
@@ -488,7 +467,7 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
 #pragma unroll
         for (int v = 0; v < NV; v++)
           vv[u][v] = i0 == 0 ? vfirst[u][v]
-                     : key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + c * EPL + v * 4)
+                     : key < k_end ? KvLoad<KT>::ld(Vh + (size_t)key * D + dim0(c, v))
                                    : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
@@ -534,10 +513,10 @@ __global__ __launch_bounds__((!PRE && G <= 4) ? 512 : 256) void attn_decode_kern
           const float inv = 1.0f / l[g];
           float4 o = acc[g][v];
           o.x *= inv; o.y *= inv; o.z *= inv; o.w *= inv;
-          *reinterpret_cast<float4*>(out + (row0 + g) * D + c * EPL + v * 4) = o;
+          *reinterpret_cast<float4*>(out + (row0 + g) * D + dim0(c, v)) = o;
         }
       } else {
-        if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][c * EPL + v * 4]) = acc[g][v];
+        if (slot == 0) *reinterpret_cast<float4*>(&st_acc[wave][g][dim0(c, v)]) = acc[g][v];
       }
     }
     if (!PRE && lane == 0) { st_m[wave][g] = m[g]; st_l[wave][g] = l[g]; }
@@ -783,11 +762,27 @@ template <int D, typename KT>
 int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
                         int64_t kv_max, float scale, int pos0, int token_major);
 
+// attn_prefill_x3.hip
+bool prefill_x3_applies(int D, int T, int pos0);
+template <typename KT>
+int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
+                      int64_t kv_max, float scale, int pos0, int token_major);
+
+// Three kernels serve causal prefill attention. Deep in a context (head size 128) the bf16-plane
+// kernels on the matrix cores; otherwise the fp32 matrix-pipe kernel; the VALU kernel that
+// shares its code with decode attention on request. tune_prefill: 0 = that choice, 1 = VALU,
+// 2 = fp32 matrix pipe, 3 = bf16 planes.
 template <int D, typename KT>
 static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
                           int T, int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = tlhip::ctx();
-  if (!c.tune_prefill_valu) {
+  const int mode = c.tune_prefill_valu;
+  if (mode == 3 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: the bf16-plane kernel needs head size 128");
+  if (mode == 3 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
+    if (int rc = launch_prefill_x3<KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
+    TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
+  }
+  if (mode != 1) {
     if (int rc = launch_prefill_mfma<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
     TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
   }

@@ -108,21 +108,37 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
 #pragma unroll
   for (int v = 0; v < 16; v++) { mrow[v] = -INFINITY; lrow[v] = 0.f; }
 
-  for (int kt = wave; kt < nkt; kt += 8) {
-    const int k0 = kt * 32;
-    float4 kreg[kLoads], vreg[kLoads];
+  // K and V rows of a tile travel through registers into the wavefront's LDS region. The
+  // registers are free again as soon as the tile has been written to LDS, so the NEXT tile's
+  // rows are requested at that point - K right after the K tile is stored, V right after the V
+  // tile is stored - and have a whole tile's arithmetic to arrive in. (Rows past the causal
+  // range are clamped to its last row: mapped memory, masked when used.)
+  float4 kreg[kLoads], vreg[kLoads];
+  const auto request = [&](float4* dst, const KT* base, int tile) {
 #pragma unroll
     for (int i = 0; i < kLoads; i++) {
       const int slot = lane + 64 * i, key = slot / (D / 4), c4 = slot % (D / 4);
-      const size_t off = (size_t)min(k0 + key, kend - 1) * D + 4 * c4;
-      kreg[i] = load_kv4(Kh + off);
-      vreg[i] = load_kv4(Vh + off);
+      dst[i] = load_kv4(base + (size_t)min(tile * 32 + key, kend - 1) * D + 4 * c4);
     }
+  };
+  request(kreg, Kh, wave);
+  request(vreg, Vh, wave);
+#ifdef TLHIP_TRACE
+  unsigned long long ph[5] = {0, 0, 0, 0, 0}, tc = __builtin_readcyclecounter();
+  TLHIP_MARK(0);
+#define TLHIP_PHASE(i) do { const unsigned long long n_ = __builtin_readcyclecounter(); ph[i] += n_ - tc; tc = n_; } while (0)
+#else
+#define TLHIP_PHASE(i)
+#endif
+  for (int kt = wave; kt < nkt; kt += 8) {
+    const int k0 = kt * 32;
 #pragma unroll
     for (int i = 0; i < kLoads; i++) {
       const int slot = lane + 64 * i, key = slot / (D / 4), c4 = slot % (D / 4);
       *reinterpret_cast<float4*>(R + key * KS + 4 * c4) = kreg[i];
     }
+    request(kreg, Kh, kt + 8);
+    TLHIP_PHASE(0);
     f32x16 s;
 #pragma unroll
     for (int v = 0; v < 16; v++) s[v] = 0.f;
@@ -135,6 +151,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
       s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.z, kf.z, s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.w, kf.w, s, 0, 0, 0);
     }
+    TLHIP_PHASE(1);
     const int key = k0 + l31;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
@@ -159,18 +176,34 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_mfma_kernel(const float* 
       const int slot = lane + 64 * i, vkey = slot / (D / 4), c4 = slot % (D / 4);
       *reinterpret_cast<float4*>(R + vkey * D + 4 * c4) = vreg[i];
     }
+    request(vreg, Vh, kt + 8);
+    TLHIP_PHASE(2);
+    // (the D/32 output tiles take turns, so consecutive MFMAs never wait for each other's result)
 #pragma unroll
-    for (int dt = 0; dt < D / 32; dt++) {
+    for (int m = 0; m < 4; m++) {
+      const float pj[4] = {pf[m].x, pf[m].y, pf[m].z, pf[m].w};
 #pragma unroll
-      for (int m = 0; m < 4; m++) {
-        const float* vp = R + (8 * m + 4 * hi) * D + dt * 32 + l31;
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].x, vp[0], o[dt], 0, 0, 0);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].y, vp[D], o[dt], 0, 0, 0);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].z, vp[2 * D], o[dt], 0, 0, 0);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[m].w, vp[3 * D], o[dt], 0, 0, 0);
+      for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int dt = 0; dt < D / 32; dt++) {
+          const float* vp = R + (8 * m + 4 * hi + j) * D + dt * 32 + l31;
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pj[j], vp[0], o[dt], 0, 0, 0);
+        }
       }
     }
+    TLHIP_PHASE(3);
   }
+#ifdef TLHIP_TRACE
+  {
+    const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (lane == 0 && b < kTraceBlocks) {
+      unsigned long long* g = &g_trace[(b * kTraceWaves + wave) * kTraceSlots];
+      g[1] = ph[0]; g[2] = ph[1]; g[3] = ph[2]; g[4] = ph[3]; g[5] = (nkt - wave + 7) / 8;
+    }
+  }
+  TLHIP_MARK(6);
+#endif
+#undef TLHIP_PHASE
 
   // merge: each wavefront leaves O [32][D], m [32], l [32] in its region; 16 threads finish a row
   float* Mw = R + 32 * D;

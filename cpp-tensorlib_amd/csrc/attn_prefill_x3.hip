@@ -1,0 +1,537 @@
+// Causal prefill attention on the bf16 matrix cores with fp32-level products
+// (tlhip_attn_prefill deep in a context, cuda.h:1165-1201).
+//
+//   out[h, p, :] = softmax_k( scale * q[h, p, :] . K[kv(h), k, :] ) . V[kv(h), k, :],  k <= pos0 + p
+//
+// The fp32 matrix instructions share the vector ALU's multipliers: a kernel built on them
+// runs its softmax and its products one after the other. v_mfma_f32_16x16x32_bf16 runs on the
+// matrix cores proper, 16 times faster and beside the vector ALU, but multiplies bf16. Every
+// f32 operand x is therefore cut into three bf16 planes x = x1 + x2 + x3 (each the
+// round-to-nearest bf16 of what the planes before it left; |x - x1 - x2 - x3| <= 2^-26 |x|),
+// and a product a.b is formed from the six plane pairs whose weight is at least 2^-16:
+//   a1b1 + (a1b2 + a2b1) + (a1b3 + a2b2 + a3b1)       dropped: a2b3, a3b2, a3b3, < 2^-23 |ab|
+// smallest first, accumulated in fp32 inside the MFMA. A cache that already holds bf16 needs one
+// plane for K and V and three products. Scores and outputs then differ from an fp32 loop by
+// what a different summation order would give.
+//
+// Two kernels per call:
+//  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into planes, written
+//     as the exact register image of the MFMA B operands, one 32-key tile after the other:
+//       K image [plane][k-step 0..3][16-key half 0..1][lane][8]  = K[32t + 16h + l%16][32s + 8(l/16) + j]
+//       V image [plane][16-dim tile 0..7][lane][8]               = V[32t + 8(l/16) + j][16d + l%16]
+//     so that the attention kernel copies a tile to LDS verbatim and every operand is one
+//     conflict-free 16-byte LDS read per lane. Keys at and past pos0 + T are written as zeros.
+//  2. attn_x3_kernel: a block serves ONE kv head and up to 8 (query head, 16-position tile)
+//     pairs, one per wavefront, that all read the same K/V tiles: with grouped-query attention
+//     the query heads of the group, else consecutive position tiles. The 32-key tiles of the
+//     block's causal range are dealt round-robin over `S` blocks (key splits); a tile is staged
+//     into LDS once per block (double buffered, one barrier per tile) and read by every
+//     wavefront. A wavefront keeps its 16 query rows as bf16 planes in registers (the A
+//     operand), the running (max, sum) of its rows and a 16 x 128 output accumulator.
+//     Per tile: 48 MFMAs for the scores, an online-softmax update on 8 scores per lane
+//     (reductions stay inside a 16-lane DPP row), P through a small LDS tile into A-operand
+//     order and into planes, 48 MFMAs for P.V.
+//     S == 1 writes the normalised rows; S > 1 leaves (max, sum, accumulator) per split and
+//  3. attn_x3_merge_kernel combines them in split order.
+#include "common.hpp"
+
+namespace tlhip {
+
+namespace x3 {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a 16-byte unit in registers
+
+constexpr int kD = 128;                      // head size this kernel is built for
+constexpr int kTile = 32;                    // keys per tile
+constexpr int kKUnits = 4 * 2 * 64;          // 16-byte units of one K plane of a tile
+constexpr int kVUnits = 8 * 64;              // ... of one V plane
+constexpr int kPS = 36;                      // floats per row of a wavefront's P tile (16-byte aligned rows)
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// Two floats -> three packed bf16 pairs (element 0 in the low half); hi + mid + lo reproduces x
+// to 2^-26 relative. The conversions are the hardware's packed round-to-nearest-even
+// (v_cvt_pk_bf16_f32); both remainders are exact in f32.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(f32x2 v) {
+  union { bf16x2 b; uint32_t u; } t;
+  t.b = __builtin_convertvector(v, bf16x2);
+  return t.u;
+}
+__device__ __forceinline__ f32x2 widen_bf16x2(uint32_t u) {
+  return f32x2{__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u)};
+}
+__device__ __forceinline__ void split3x2(f32x2 x, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+  hi = pack_bf16x2(x);
+  const f32x2 r1 = x - widen_bf16x2(hi);
+  mid = pack_bf16x2(r1);
+  const f32x2 r2 = r1 - widen_bf16x2(mid);
+  lo = pack_bf16x2(r2);
+}
+
+// 8 floats -> 8 bf16 per plane, packed as the MFMA wants them (element j in bits [16j, 16j+16) of the 128)
+__device__ __forceinline__ void split3x8(const float (&x)[8], uint4& p1, uint4& p2, uint4& p3) {
+  uint32_t a[4], b[4], c[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) split3x2(f32x2{x[2 * j], x[2 * j + 1]}, a[j], b[j], c[j]);
+  p1 = make_uint4(a[0], a[1], a[2], a[3]);
+  p2 = make_uint4(b[0], b[1], b[2], b[3]);
+  p3 = make_uint4(c[0], c[1], c[2], c[3]);
+}
+
+__device__ __forceinline__ bf16x8 as_bf16x8(const uint4& u) {
+  union { uint4 u4; bf16x8 v; } t;
+  t.u4 = u;
+  return t.v;
+}
+__device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 u) {
+  union { u32x4 u4; bf16x8 v; } t;
+  t.u4 = u;
+  return t.v;
+}
+
+__device__ __forceinline__ float cache_elem(const float* p) { return *p; }
+__device__ __forceinline__ float cache_elem(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+
+// ---- 1. planes ---------------------------------------------------------------------------
+// grid = (tiles, Hkv), block = 256. NP = 3 for an f32 cache, 1 for a bf16 cache.
+// planes: per (kv head, tile) a K image of NP * kKUnits uint4, then a V image of NP * kVUnits uint4.
+template <typename KT, int NP>
+__global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K, const KT* __restrict__ V,
+                                                        uint4* __restrict__ planes, int64_t kv_stride,
+                                                        int kend, int ntiles) {
+  const int t = blockIdx.x, kvh = blockIdx.y;
+  const KT* Kh = K + (size_t)kvh * kv_stride;
+  const KT* Vh = V + (size_t)kvh * kv_stride;
+  uint4* img = planes + ((size_t)kvh * ntiles + t) * (size_t)(NP * (kKUnits + kVUnits));
+  for (int u = threadIdx.x; u < kKUnits + kVUnits; u += 256) {
+    float x[8];
+    uint4* dst;
+    int plane_stride;
+    if (u < kKUnits) {
+      const int l = u & 63, half = (u >> 6) & 1, ks = u >> 7;
+      const int key = t * kTile + 16 * half + (l & 15), dim = 32 * ks + 8 * (l >> 4);
+      const bool live = key < kend;
+      const KT* src = Kh + (size_t)min(key, kend - 1) * kD + dim;
+#pragma unroll
+      for (int j = 0; j < 8; j++) x[j] = live ? cache_elem(src + j) : 0.f;
+      dst = img + u;
+      plane_stride = kKUnits;
+    } else {
+      const int v = u - kKUnits, l = v & 63, dt = v >> 6;
+      const int key0 = t * kTile + 8 * (l >> 4), dim = 16 * dt + (l & 15);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int key = key0 + j;
+        x[j] = key < kend ? cache_elem(Vh + (size_t)key * kD + dim) : 0.f;
+      }
+      dst = img + NP * kKUnits + v;
+      plane_stride = kVUnits;
+    }
+    uint4 p1, p2, p3;
+    split3x8(x, p1, p2, p3);
+    dst[0] = p1;
+    if (NP == 3) { dst[plane_stride] = p2; dst[2 * plane_stride] = p3; }
+  }
+}
+
+// max / sum over the 16 lanes of a DPP row, result in every lane of the row
+template <int CTRL>
+__device__ __forceinline__ float dppv(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row_max16(float v) {
+  v = fmaxf(v, dppv<0xB1>(v));
+  v = fmaxf(v, dppv<0x4E>(v));
+  v = fmaxf(v, dppv<0x141>(v));
+  v = fmaxf(v, dppv<0x140>(v));
+  return v;
+}
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dppv<0xB1>(v);
+  v += dppv<0x4E>(v);
+  v += dppv<0x141>(v);
+  v += dppv<0x140>(v);
+  return v;
+}
+
+struct Geometry {
+  int group;        // query heads per kv head
+  int nh, np;       // computing wavefronts of a block: nh heads x np runs of 32 positions (nh * np <= 7)
+  int head_chunks;  // ceil(group / nh)
+  int T, pos0, S, ntiles;
+  int64_t rows;     // Hq * T
+  int64_t o_head, o_row;   // output strides in floats: [Hq,T,D] or [T,Hq*D]
+};
+
+// ---- 2. attention ------------------------------------------------------------------------
+// grid = (Hkv * head_chunks, position blocks, S), block = 512: seven computing wavefronts and
+// one that moves tiles.
+//
+// LDS bandwidth is what bounds this kernel (a 16-byte-per-lane read runs at 64 bytes a clock per
+// CU, and every B operand of every MFMA comes from LDS), so a computing wavefront owns TWO
+// 16-row tiles - 32 consecutive positions of one head - and uses every K/V operand it reads
+// twice. Its registers then hold 96 for the query planes and 64 for the output accumulators,
+// which leaves no room for tiles in transit: wavefront 7 does nothing but copy, K of the next
+// tile and V of this one, global -> registers -> LDS, one 16-byte unit per lane and instruction.
+//
+// A step of the loop is one barrier interval. In interval i a computing wavefront runs one
+// matrix phase - P.V of tile i-1, then Q.K^T of tile i - and one vector phase, the online
+// softmax of one tile. Wavefronts 0-3 run the softmax of tile i AFTER their matrix phase,
+// wavefronts 4-6 run the softmax of tile i-1 BEFORE it. The two wavefronts that share a SIMD
+// (w and w + 4) are therefore never in the same kind of phase: one feeds the matrix core while
+// the other is on the vector ALU. Interval i needs K of tile i and V of tile i-1 in LDS.
+constexpr int kRT = 2;          // 16-row tiles per computing wavefront
+constexpr int kCompute = 7;     // computing wavefronts per block
+
+template <int NP>
+__global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict__ q, const uint4* __restrict__ planes,
+                                                          float* __restrict__ out, float* __restrict__ part_o,
+                                                          float* __restrict__ part_ml, float scale, const Geometry g) {
+  constexpr int kKImg = NP * kKUnits, kVImg = NP * kVUnits;   // 16-byte units of a tile's K and V images
+  constexpr int kImg = kKImg + kVImg;
+  constexpr int kCopyK = kKImg / 64, kCopyV = kVImg / 64;     // units a lane of the copying wavefront moves per tile
+  extern __shared__ u32x4 lds4[];                             // K images [2], V images [2], 7 P tiles of 32 x kPS floats
+  u32x4* kbuf = lds4;
+  u32x4* vbuf = lds4 + 2 * kKImg;
+  float* ptile_base = reinterpret_cast<float*>(lds4 + 2 * kImg);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l15 = lane & 15, lq = lane >> 4;
+  const int kvh = blockIdx.x / g.head_chunks, hc = blockIdx.x - kvh * g.head_chunks;
+  const int nblk = gridDim.y;
+  const int pblock = nblk - 1 - (int)blockIdx.y;          // longest causal ranges first
+  const int split = blockIdx.z;
+  // causal range of the block: tiles up to its last row's limit, dealt round-robin over the splits
+  const int blk_last = min((pblock + 1) * g.np * (16 * kRT), g.T) - 1;
+  const int nkt_blk = (g.pos0 + blk_last) / kTile + 1;
+  const int n = nkt_blk > split ? (nkt_blk - split + g.S - 1) / g.S : 0;   // this block's tiles: split, split + S, ...
+  const auto tile_of = [&](int i) { return split + i * g.S; };
+  const u32x4* img0 = reinterpret_cast<const u32x4*>(planes) + (size_t)kvh * g.ntiles * kImg;
+
+  if (wave == kCompute) {
+    // ---- the copying wavefront (branch-free: tiles past the range are clamped, parked, never read) ----
+    // Interval i needs K of tile i and V of tile i-1. What the interval AFTER it needs - K of
+    // tile i+1, V of tile i - is in registers when interval i begins (requested one interval
+    // earlier) and is parked first thing: those buffers were last read in interval i-1, which
+    // every wavefront has left. The requests for the interval after that go out right behind
+    // and have a whole interval to arrive.
+    u32x4 stk[kCopyK], stv[kCopyV];
+    const auto request = [&](int ik, int iv) {
+      const u32x4* srck = img0 + (size_t)min(tile_of(ik), g.ntiles - 1) * kImg;
+      const u32x4* srcv = img0 + (size_t)min(tile_of(iv), g.ntiles - 1) * kImg + kKImg;
+#pragma unroll
+      for (int c = 0; c < kCopyK; c++) stk[c] = srck[lane + 64 * c];
+#pragma unroll
+      for (int c = 0; c < kCopyV; c++) stv[c] = srcv[lane + 64 * c];
+    };
+    request(0, 0);
+#pragma unroll
+    for (int c = 0; c < kCopyK; c++) kbuf[lane + 64 * c] = stk[c];
+    request(1, 0);
+    __syncthreads();
+    for (int i = 0; i <= n; i++) {
+#pragma unroll
+      for (int c = 0; c < kCopyK; c++) kbuf[((i + 1) & 1) * kKImg + lane + 64 * c] = stk[c];
+#pragma unroll
+      for (int c = 0; c < kCopyV; c++) vbuf[(i & 1) * kVImg + lane + 64 * c] = stv[c];
+      request(i + 2, i + 1);
+      __syncthreads();
+    }
+    return;
+  }
+
+  const int hh = wave % g.nh, pt = wave / g.nh;
+  const int hloc = hc * g.nh + hh;                        // head inside the group
+  const int p_first = (pblock * g.np + pt) * (16 * kRT);  // this wavefront's first query position
+  const bool active = pt < g.np && hloc < g.group && p_first < g.T;
+  const bool late = wave >= 4;                            // softmax before the matrix phase
+  const int h = kvh * g.group + min(hloc, g.group - 1);
+  const int my_last_key = g.pos0 + min(p_first + 16 * kRT - 1, g.T - 1);
+  const int kend = g.pos0 + g.T;
+
+  // ---- the wavefront's query rows as A-operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
+  uint4 qa[kRT][3][4];
+#pragma unroll
+  for (int rt = 0; rt < kRT; rt++) {
+    const float* qrow = q + ((size_t)h * g.T + min(p_first + 16 * rt + l15, g.T - 1)) * kD;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq);
+      const float4 b = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq + 4);
+      const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      split3x8(x, qa[rt][0][ks], qa[rt][1][ks], qa[rt][2][ks]);
+    }
+  }
+
+  f32x4 o[kRT][8];
+  float mrow[kRT][4], lrow[kRT][4];   // rows 16 rt + 4(l/16) + r; lrow is this lane's share of the row sum
+  f32x4 s[kRT][2];                    // scores of the tile whose softmax is pending
+  uint4 pa3[kRT][3];                  // P planes of the tile whose P.V is pending
+#pragma unroll
+  for (int rt = 0; rt < kRT; rt++) {
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; r++) { mrow[rt][r] = -INFINITY; lrow[rt][r] = 0.f; }
+    s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    pa3[rt][0] = pa3[rt][1] = pa3[rt][2] = make_uint4(0, 0, 0, 0);
+  }
+  float* ptile = ptile_base + wave * (16 * kRT) * kPS;
+
+  // the vector phase of tile number i: masks, running maxima and sums, rescale of the output
+  // accumulators, P into operand order and planes
+  const auto softmax_tile = [&](int i) {
+    const int kt = tile_of(i);
+#pragma unroll
+    for (int rt = 0; rt < kRT; rt++) {
+      float pr[2][4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int limit = min(g.pos0 + p_first + 16 * rt + 4 * lq + r, kend - 1);   // last key the row sees
+        float sv[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+          const int key = kt * kTile + 16 * hf + l15;
+          sv[hf] = key <= limit ? s[rt][hf][r] * scale : -INFINITY;
+        }
+        const float mnew = fmaxf(mrow[rt][r], row_max16(fmaxf(sv[0], sv[1])));
+        const float mref = mnew == -INFINITY ? 0.f : mnew;
+        const float corr = __expf(mrow[rt][r] - mref);
+        pr[0][r] = __expf(sv[0] - mref);
+        pr[1][r] = __expf(sv[1] - mref);
+        lrow[rt][r] = lrow[rt][r] * corr + (pr[0][r] + pr[1][r]);
+        mrow[rt][r] = mnew;
+#pragma unroll
+        for (int dt = 0; dt < 8; dt++) o[rt][dt][r] *= corr;
+      }
+      // P: result order (row 4(l/16)+r, key l%16) -> operand order (row l%16, keys 8(l/16)+j)
+      float* pt_ = ptile + rt * 16 * kPS;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        pt_[(4 * lq + r) * kPS + l15] = pr[0][r];
+        pt_[(4 * lq + r) * kPS + 16 + l15] = pr[1][r];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int rt = 0; rt < kRT; rt++) {
+      const float* pt_ = ptile + rt * 16 * kPS;
+      const float4 a = *reinterpret_cast<const float4*>(pt_ + l15 * kPS + 8 * lq);
+      const float4 b = *reinterpret_cast<const float4*>(pt_ + l15 * kPS + 8 * lq + 4);
+      const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      split3x8(x, pa3[rt][0], pa3[rt][1], pa3[rt][2]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // the tile is rewritten by the next softmax
+  };
+  const auto mine = [&](int i) { return active && i >= 0 && i < n && tile_of(i) * kTile <= my_last_key; };
+
+#ifdef TLHIP_TRACE
+  unsigned long long ph[4] = {0, 0, 0, 0}, tc;
+  TLHIP_MARK(0);
+#define TLHIP_X3_T0() tc = __builtin_readcyclecounter()
+#define TLHIP_X3_T(k) do { const unsigned long long n_ = __builtin_readcyclecounter(); ph[k] += n_ - tc; tc = n_; } while (0)
+#else
+#define TLHIP_X3_T0()
+#define TLHIP_X3_T(k)
+#endif
+  __syncthreads();   // K of tile 0 is in LDS
+  TLHIP_X3_T0();
+  for (int i = 0; i <= n; i++) {   // interval n drains: P.V of the last tile (and, for the late half, its softmax)
+    if (late && mine(i - 1)) softmax_tile(i - 1);
+    TLHIP_X3_T(0);
+    // ---- matrix phase; plane pairs (a, b) with a + b <= 2, smallest products first ----
+    if (mine(i - 1)) {   // O[32 x 128] += P[32 x 32] . V[32 x 128] of tile i-1, eight 16-column tiles
+      const u32x4* vimg = vbuf + ((i - 1) & 1) * kVImg;
+      // two column tiles at a time: four independent accumulators take turns, so that an MFMA
+      // never waits for the result of the one issued just before it
+#pragma unroll
+      for (int dt = 0; dt < 8; dt += 2) {
+        bf16x8 vb[2][NP];
+#pragma unroll
+        for (int d2 = 0; d2 < 2; d2++)
+#pragma unroll
+          for (int p = 0; p < NP; p++) vb[d2][p] = as_bf16x8(vimg[p * kVUnits + (dt + d2) * 64 + lane]);
+#pragma unroll
+        for (int w = 2; w >= 0; w--)
+#pragma unroll
+          for (int pb = NP - 1; pb >= 0; pb--) {
+            const int pa = w - pb;
+            if (pa >= 0 && pa <= 2) {
+#pragma unroll
+              for (int d2 = 0; d2 < 2; d2++)
+#pragma unroll
+                for (int rt = 0; rt < kRT; rt++)
+                  o[rt][dt + d2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(pa3[rt][pa]), vb[d2][pb], o[rt][dt + d2], 0, 0, 0);
+            }
+          }
+      }
+    }
+    if (mine(i)) {       // S[32 rows x 32 keys] of tile i as 16 x 16 tiles
+      const u32x4* kimg = kbuf + (i & 1) * kKImg;
+#pragma unroll
+      for (int rt = 0; rt < kRT; rt++) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        bf16x8 kb[2][NP];
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+          for (int p = 0; p < NP; p++) kb[hf][p] = as_bf16x8(kimg[p * kKUnits + (ks * 2 + hf) * 64 + lane]);
+#pragma unroll
+        for (int w = 2; w >= 0; w--)
+#pragma unroll
+          for (int pb = NP - 1; pb >= 0; pb--) {
+            const int pa = w - pb;
+            if (pa >= 0 && pa <= 2) {
+#pragma unroll
+              for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+                for (int rt = 0; rt < kRT; rt++)
+                  s[rt][hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(qa[rt][pa][ks]), kb[hf][pb], s[rt][hf], 0, 0, 0);
+            }
+          }
+      }
+    }
+    TLHIP_X3_T(1);
+    if (!late && mine(i)) softmax_tile(i);
+    TLHIP_X3_T(0);
+    __syncthreads();
+    TLHIP_X3_T(2);
+  }
+#ifdef TLHIP_TRACE
+  {
+    const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (lane == 0 && b < kTraceBlocks) {
+      unsigned long long* gt = &g_trace[(b * kTraceWaves + wave) * kTraceSlots];
+      gt[1] = ph[0]; gt[2] = ph[1]; gt[3] = ph[2]; gt[4] = n + 1;
+    }
+  }
+  TLHIP_MARK(6);
+#endif
+#undef TLHIP_X3_T0
+#undef TLHIP_X3_T
+
+  // ---- rows complete for this split: sum l over the row's 16 lanes, store ----
+  if (!active) return;
+#pragma unroll
+  for (int rt = 0; rt < kRT; rt++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int p = p_first + 16 * rt + 4 * lq + r;
+      const float lsum = row_sum16(lrow[rt][r]);
+      if (p >= g.T) continue;
+      if (g.S == 1) {
+        const float inv = 1.0f / lsum;
+        float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row;
+#pragma unroll
+        for (int dt = 0; dt < 8; dt++) op[16 * dt + l15] = o[rt][dt][r] * inv;
+      } else {
+        const size_t row = (size_t)h * g.T + p, rows = (size_t)g.rows;   // row number in [Hq * T)
+        float* po = part_o + ((size_t)split * rows + row) * kD;
+#pragma unroll
+        for (int dt = 0; dt < 8; dt++) po[16 * dt + l15] = o[rt][dt][r];
+        if (l15 == 0) {
+          part_ml[((size_t)split * rows + row) * 2] = mrow[rt][r];
+          part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
+        }
+      }
+    }
+}
+
+// ---- 3. merge of the key splits ---------------------------------------------------------------
+// One thread per (row, 4 columns); splits are combined in split order.
+__global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml,
+                                                            float* __restrict__ out, int rows, int T, int S,
+                                                            int64_t o_head, int64_t o_row) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = i / (kD / 4);
+  const int c4 = (int)(i - row * (kD / 4)) * 4;
+  if (row >= rows) return;
+  float M = -INFINITY;
+  for (int s = 0; s < S; s++) M = fmaxf(M, part_ml[((size_t)s * rows + row) * 2]);
+  float L = 0.f;
+  float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s = 0; s < S; s++) {
+    const float m = part_ml[((size_t)s * rows + row) * 2];
+    const float f = m == -INFINITY ? 0.f : __expf(m - M);
+    L = fmaf(part_ml[((size_t)s * rows + row) * 2 + 1], f, L);
+    const float4 v = *reinterpret_cast<const float4*>(part_o + ((size_t)s * rows + row) * kD + c4);
+    a.x = fmaf(v.x, f, a.x); a.y = fmaf(v.y, f, a.y); a.z = fmaf(v.z, f, a.z); a.w = fmaf(v.w, f, a.w);
+  }
+  const float inv = 1.0f / L;
+  const int64_t h = row / T, p = row - h * T;
+  *reinterpret_cast<float4*>(out + h * o_head + p * o_row + c4) = make_float4(a.x * inv, a.y * inv, a.z * inv, a.w * inv);
+}
+
+}  // namespace x3
+
+// Whether the bf16-plane kernels serve this call (head size 128, enough keys for the extra
+// pass to pay), and the launch. Returns 0 when launched, a negative status on failure.
+bool prefill_x3_applies(int D, int T, int pos0) { return D == x3::kD && pos0 + T >= 1024 && T >= 16; }
+
+template <typename KT>
+int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
+                      int64_t kv_max, float scale, int pos0, int token_major) {
+  using namespace x3;
+  constexpr int NP = sizeof(KT) == 4 ? 3 : 1;
+  Context& c = ctx();
+  Geometry g{};
+  g.group = Hq / Hkv;
+  g.nh = g.group < kCompute ? g.group : kCompute;
+  g.np = kCompute / g.nh;
+  if (g.np * 16 * kRT > T) g.np = (T + 16 * kRT - 1) / (16 * kRT);
+  g.head_chunks = (g.group + g.nh - 1) / g.nh;
+  g.T = T;
+  g.pos0 = pos0;
+  const int kend = pos0 + T;
+  g.ntiles = (kend + kTile - 1) / kTile;
+  g.o_head = token_major ? kD : (int64_t)T * kD;
+  g.o_row = token_major ? (int64_t)Hq * kD : kD;
+  g.rows = (int64_t)Hq * T;
+  const int pblocks = (T + g.np * 16 * kRT - 1) / (g.np * 16 * kRT);
+  const int base = Hkv * g.head_chunks * pblocks;
+  // key splits: fill the chip once, keep at least 8 tiles per block
+  int S = (c.cus + base - 1) / base;
+  if (S > g.ntiles / 8) S = g.ntiles / 8;
+  if (S < 1) S = 1;
+  if (S > 64) S = 64;
+  g.S = S;
+  constexpr size_t kImgBytes = (size_t)NP * (kKUnits + kVUnits) * 16;
+  const size_t plane_bytes = (size_t)Hkv * g.ntiles * kImgBytes;
+  const size_t rows = (size_t)Hq * T;
+  const size_t part_o_bytes = S > 1 ? (size_t)S * rows * kD * 4 : 0;
+  const size_t part_ml_bytes = S > 1 ? (size_t)S * rows * 2 * 4 : 0;
+  char* buf = static_cast<char*>(scratch(plane_bytes + part_o_bytes + part_ml_bytes + 256));
+  if (!buf) return fail(TLHIP_ENOMEM, "tlhip_attn_prefill: no scratch for %zu bytes of key/value planes", plane_bytes);
+  uint4* planes = reinterpret_cast<uint4*>(buf);
+  float* part_o = reinterpret_cast<float*>(buf + plane_bytes);
+  float* part_ml = reinterpret_cast<float*>(buf + plane_bytes + part_o_bytes);
+  const size_t lds = 2 * kImgBytes + (size_t)kCompute * 16 * kRT * kPS * 4;
+  if (lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
+  auto fn = attn_x3_kernel<NP>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
+  hipLaunchKernelGGL((kv_planes_kernel<KT, NP>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes,
+                     kv_max * (int64_t)kD, kend, g.ntiles);
+  hipLaunchKernelGGL(fn, dim3(Hkv * g.head_chunks, pblocks, S), dim3(512), lds, c.stream, q, planes, out, part_o,
+                     part_ml, scale, g);
+  if (S > 1) {
+    const int64_t threads = (int64_t)rows * (kD / 4);
+    hipLaunchKernelGGL(attn_x3_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c.stream, part_o,
+                       part_ml, out, (int)rows, T, S, g.o_head, g.o_row);
+  }
+  return 0;
+}
+
+template int launch_prefill_x3<float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+
+}  // namespace tlhip

@@ -497,14 +497,18 @@ static RowCfg pick_rows_cfg(int64_t N, int upr, int E, int cus, int lds_per_cu, 
   if (lpr == 64) {
     if (rows_per_cu >= 512) { nw = 16; R = 4; KW = 2; want_bpc = 1; }        // LM head
     else if (rows_per_cu >= 128) { nw = 8; R = 4; KW = 1; want_bpc = 1; }    // 7B gate|up
-    else if (rows_per_cu >= 32) { nw = 8; R = 2; KW = 1; want_bpc = 2; }     // 7B up-projection alone
-    else if (rows_per_cu >= 17) { nw = 8; R = 2; KW = 2; want_bpc = 2; }     // 7B q|k|v
-    else if (rows_per_cu >= 8) {
+    else if (rows_per_cu >= 32) { nw = 8; R = 2; KW = 1; want_bpc = 1; }     // 7B up-projection alone
+    else if (rows_per_cu >= 17) {                                            // 7B q|k|v
+      // one tile per CU: as many 4-row groups as a CU's share of the rows needs, K over two wavefronts
+      const int groups = (int)(((N + cus - 1) / cus + 3) / 4);
+      R = 4; KW = 2; nw = 2 * (groups < 8 ? groups : 8); want_bpc = 2;
+    } else if (rows_per_cu >= 8) {
       if (chunks <= 3) { nw = 8; R = 4; KW = 2; want_bpc = 2; }              // 7B o-projection
-      else { nw = 16; R = 1; KW = 2; want_bpc = 1; }                         // 7B down-projection (K = 18944)
+      else { nw = 16; R = 2; KW = 2; want_bpc = 1; }                         // 7B down-projection (K = 18944)
     } else {                                                                 // a few rows per CU
       KW = chunks < 3 ? chunks : 3;
-      nw = 2 * KW; R = 2; want_bpc = 2;
+      nw = 2 * KW; want_bpc = 2;
+      R = N / 4 >= cus ? 2 : 1;                                              // two row groups a block: keep every CU busy
     }
   } else {
     if (rows_per_cu >= 256) { nw = 8; R = 1; KW = 1; want_bpc = 2; }         // 0.5B LM head

@@ -347,30 +347,37 @@ def test_gemm_bf16_nt_declines(lib):
         b.free()
 
 
-def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, valu=False):
-    """valu: the VALU kernel instead of the matrix-pipe one (tlhip_tune_attn_prefill)."""
+KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "planes": 3}
+
+
+def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, kernel="auto"):
+    """kernel (tlhip_tune_attn_prefill): the library's own choice, the VALU kernel, the fp32
+    matrix-pipe kernel, or the bf16-plane kernels on the matrix cores (head size 128 only)."""
     Hq, T, D = q.shape
     Hkv, kv_max, _ = K.shape
+    if kernel == "planes" and D != 128:
+        pytest.skip("the bf16-plane kernels are built for head size 128")
     dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, T, D))
-    lib.tune_attn_prefill(valu)
+    lib.tune_attn_prefill(KERNELS[kernel])
     try:
         lib.attn_prefill(dq, dk, dv, do, Hq, Hkv, T, kv_max, D, scale, kv_bf16, pos0)
     finally:
-        lib.tune_attn_prefill(False)
+        lib.tune_attn_prefill(0)
     out = do.numpy()
     for b in (dq, dk, dv, do):
         b.free()
     return out
 
 
-@pytest.mark.parametrize("valu", [False, True])
+@pytest.mark.parametrize("kernel", list(KERNELS))
 @pytest.mark.parametrize("D,Hq,Hkv,T,pos0", [
     (128, 28, 4, 64, 0), (64, 14, 2, 100, 0), (128, 4, 2, 7, 0), (128, 8, 8, 33, 300),
     (64, 6, 2, 257, 19), (128, 2, 1, 1, 0), (128, 2, 1, 1, 77), (64, 4, 4, 130, 513),
     (128, 7, 1, 512, 0), (64, 2, 2, 512, 0), (128, 2, 1, 200, 1000), (128, 1, 1, 31, 32), (64, 3, 1, 32, 31),
     (128, 7, 1, 512, 3584), (128, 4, 4, 256, 7680),      # deep in a context: > 120 key tiles per wavefront
+    (128, 12, 1, 50, 1500), (128, 3, 1, 100, 990), (128, 16, 2, 17, 2047),   # head groups of 12, 3 and 8; ragged chunk lengths
 ])
-def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, valu):
+def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, kernel):
     """Causal prefill over a cache: query p at absolute position pos0+p sees keys
     0..pos0+p (cuda.h:1165-1200). Rows past pos0+T hold poison that must not leak; so
     must, per query, the chunk's own later keys."""
@@ -382,14 +389,14 @@ def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, valu):
     K[:, pos0 + T:, :] = 1e30
     V[:, pos0 + T:, :] = np.nan
     scale = 1.0 / np.sqrt(float(D))
-    got = _prefill(lib, q, K, V, scale, pos0, valu=valu)
+    got = _prefill(lib, q, K, V, scale, pos0, kernel=kernel)
     want = orc.attn_prefill(q, K, V, scale, pos0)
     assert np.all(np.isfinite(got))
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
-@pytest.mark.parametrize("valu", [False, True])
-def test_attn_prefill_rows_equal_decode(lib, orc, valu):
+@pytest.mark.parametrize("kernel", list(KERNELS))
+def test_attn_prefill_rows_equal_decode(lib, orc, kernel):
     """Row p of a prefill equals a decode step with ctx = pos0 + p + 1 (the equivalence the
     reference's prefill bench relies on, bench_qwen_prefill.cpp:283-310), and the first query
     of a fresh cache returns V[0] exactly."""
@@ -399,7 +406,7 @@ def test_attn_prefill_rows_equal_decode(lib, orc, valu):
     K = orc.normal(Hkv * kv_max * D, 42).reshape(Hkv, kv_max, D)
     V = orc.normal(Hkv * kv_max * D, 43).reshape(Hkv, kv_max, D)
     scale = 1.0 / np.sqrt(float(D))
-    got = _prefill(lib, q, K, V, scale, pos0, valu=valu)
+    got = _prefill(lib, q, K, V, scale, pos0, kernel=kernel)
     dk, dv, do = lib.to_device(K), lib.to_device(V), lib.empty((Hq, D))
     for p in (0, 1, 17, T - 1):
         dq = lib.to_device(np.ascontiguousarray(q[:, p, :]))
@@ -408,20 +415,20 @@ def test_attn_prefill_rows_equal_decode(lib, orc, valu):
         dq.free()
     for b in (dk, dv, do):
         b.free()
-    fresh = _prefill(lib, q, K, V, scale, 0, valu=valu)
+    fresh = _prefill(lib, q, K, V, scale, 0, kernel=kernel)
     assert np.array_equal(fresh[:, 0, :], np.repeat(V[:, 0, :], Hq // Hkv, axis=0))
 
 
-@pytest.mark.parametrize("valu", [False, True])
+@pytest.mark.parametrize("kernel", list(KERNELS))
 @pytest.mark.parametrize("D", [128, 64])
-def test_attn_prefill_bf16_cache(lib, orc, D, valu):
+def test_attn_prefill_bf16_cache(lib, orc, D, kernel):
     Hq, Hkv, T, pos0 = 4, 2, 70, 10
     kv_max = pos0 + T
     q = orc.normal(Hq * T * D, 51).reshape(Hq, T, D)
     Kb = orc.to_bf16(orc.normal(Hkv * kv_max * D, 52)).reshape(Hkv, kv_max, D)
     Vb = orc.to_bf16(orc.normal(Hkv * kv_max * D, 53)).reshape(Hkv, kv_max, D)
     scale = 1.0 / np.sqrt(float(D))
-    got = _prefill(lib, q, Kb, Vb, scale, pos0, kv_bf16=True, valu=valu)
+    got = _prefill(lib, q, Kb, Vb, scale, pos0, kv_bf16=True, kernel=kernel)
     want = orc.attn_prefill(q, orc.bf16_widen(Kb).reshape(Kb.shape),
                             orc.bf16_widen(Vb).reshape(Vb.shape), scale, pos0)
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
