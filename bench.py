@@ -31,7 +31,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 SHAPES = [(3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584)]  # (N, K)
 HBM_PEAK_GBS = 8000.0
 RING_BYTES = 1.2e9      # distinct weight bytes per shape, > 4x the Infinity Cache
-LMHEAD_HBM_BYTES_PER_LAUNCH = 356_645_000   # (173845.2 KiB * 2.000 + 595.6 KiB) * 1024
+LMHEAD_HBM_BYTES_PER_LAUNCH = 341_917_491   # (166654.9 KiB * 2.000 + 594.0 KiB) * 1024
 
 
 def q4_nbytes(N, K):
@@ -467,11 +467,35 @@ def prefill_7b(lib, rounds=3):
         for b in (A, W, C):
             b.free()
     gemm_tf = flops / d.n_layers / gemm_ms / 1e9
+    # one layer's causal attention for the chunk at three depths of the context (f32 cache)
+    attn = {}
+    Hq, Hkv, D = d.n_q_heads, d.n_kv_heads, d.head_dim
+    scale = float(1.0 / np.sqrt(D))
+    for pos0 in (0, 3584, 7680):
+        kv_max = pos0 + T
+        K = lib.to_device(rng.standard_normal(Hkv * kv_max * D, dtype=np.float32))
+        V = lib.to_device(rng.standard_normal(Hkv * kv_max * D, dtype=np.float32))
+        q = lib.to_device(rng.standard_normal(Hq * T * D, dtype=np.float32))
+        out = lib.empty(Hq * T * D)
+        for _ in range(2):
+            lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
+        lib.record(e0)
+        for _ in range(10):
+            lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
+        lib.record(e1)
+        ms = lib.elapsed_ms(e0, e1) / 10
+        fl = 4.0 * Hq * D * (T * pos0 + T * (T + 1) / 2)
+        attn["pos0_%d" % pos0] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(fl / ms / 1e9, 1)}
+        for b in (K, V, q, out):
+            b.free()
     return {
         "workload": "Qwen2.5-7B-shape 512-token prompt chunk at pos0 0, bf16 weights, f32 KV",
         "ms_per_chunk": round(best, 3), "tok_s": round(T / best * 1e3, 1),
         "tflops_chunk": round(flops / best / 1e9, 1),
         "int4_weights": {"ms_per_chunk": round(best_q4, 3), "tok_s": round(T / best_q4 * 1e3, 1)},
+        "attention_per_layer": dict(attn, note="causal attention of the 512-token chunk, 28/4 heads of 128, f32 cache; "
+                                               "from 1024 keys on: bf16 planes on the matrix cores, six plane products per "
+                                               "fp32 product (157.3 TFLOP/s is the fp32 matrix-pipe peak)"),
         "gemm": {"per_shape": per_gemm, "TFLOP/s": round(gemm_tf, 1),
                  "roofline": {"bound": "mfma", "achieved": round(3 * gemm_tf, 1), "peak": 2500.0,
                               "unit": "TFLOP/s", "frac": round(3 * gemm_tf / 2500.0, 4),
@@ -598,7 +622,7 @@ def main():
                    "per_shape": per_shape},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_rows_kernel<FmtQ4,4,0,64> on 152064x3584 (LM head)",
+                     "kernel": "gemv_rows_kernel<FmtQ4,4,0,64,0> on 152064x3584 (LM head)",
                      "bytes_per_launch": dom["nb"], "avg_launch_us": round(dom_ms * 1e3, 2),
                      "avg_us_between_events_inside_step": round(in_step_ms * 1e3, 2)},
     }

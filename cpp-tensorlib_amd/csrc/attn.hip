@@ -112,7 +112,8 @@ __device__ __forceinline__ float4 kv_store4(uint16_t* p, float4 v, bool store) {
 
 // grid = (Hkv, S, ceil(group/G)); block = nw*64 threads (nw in 1,2,4).
 // A wavefront works on tiles of TK keys (16, 32 or 64): 4 keys per load step
-// (one per DPP row), each lane holding EPL = D/16 consecutive floats of its key.
+// (one per DPP row), each lane holding EPL = D/16 floats of its key: four consecutive
+// ones of each 64-element part of the row.
 // part_m/part_l: [Hq*S], part_acc: [Hq*S*D]; used when S > 1, else `out` is final.
 //
 // PRE = true is causal prefill over q/out [Hq, T, D]: grid = (Hq, 1, ceil(T/(4G))).

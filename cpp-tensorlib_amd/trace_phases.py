@@ -1,0 +1,130 @@
+"""Where the time goes inside a kernel: accumulated phase clocks per wavefront.
+
+The kernels carry TLHIP_MARK points that compile to nothing in the product library. The trace
+build (python cpp-tensorlib_amd/build.py --trace -> lib/libtensorlib_hip_trace.so) makes lane 0 of
+every wavefront record the shader clock (s_memtime) there; this script runs one launch and prints
+the distribution over wavefronts. Times are clocks of the 100 MHz-referenced shader counter
+divided by the frequency given with --ghz (default 2.1).
+
+  python cpp-tensorlib_amd/trace_phases.py attn_decode [pos]      7B decode attention (fused q/k/v, device position)
+  python cpp-tensorlib_amd/trace_phases.py attn_prefill [pos0]    7B causal prefill attention of a 512-token chunk (bf16 planes)
+"""
+import ctypes as C
+import importlib
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+SLOTS, WAVES, BLOCKS = 8, 16, 1024
+
+
+def load():
+    capi = importlib.import_module("cpp-tensorlib_amd.capi")
+    path = os.path.join(HERE, "lib", "libtensorlib_hip_trace.so")
+    if not os.path.exists(path):
+        sys.exit("build the trace library first: python cpp-tensorlib_amd/build.py --trace")
+    lib = capi.TlHip(path=path)
+    lib.c.tlhip_trace_read.restype = C.c_int
+    lib.c.tlhip_trace_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int]
+    return lib
+
+
+def read_trace(lib, clear=True):
+    tr = np.zeros(BLOCKS * WAVES * SLOTS, np.uint64)
+    if lib.c.tlhip_trace_read(tr.ctypes.data, tr.nbytes, 1 if clear else 0) != 0:
+        sys.exit("tlhip_trace_read failed")
+    return tr.reshape(BLOCKS, WAVES, SLOTS).astype(np.float64)
+
+
+def pct(name, d):
+    print("   %-58s p10 %7.2f  med %7.2f  p90 %7.2f  max %7.2f us" % (name, np.percentile(d, 10), np.median(d), np.percentile(d, 90), d.max()))
+
+
+def attn_decode(lib, pos, ghz):
+    Hq, Hkv, D, kv_max = 28, 4, 128, 4352
+    rng = np.random.default_rng(1)
+    qkv = lib.to_device(rng.standard_normal((Hq + 2 * Hkv) * D, dtype=np.float32))
+    layers = 8
+    Ks = [lib.to_device(rng.standard_normal((Hkv, kv_max, D), dtype=np.float32)) for _ in range(layers)]
+    Vs = [lib.to_device(rng.standard_normal((Hkv, kv_max, D), dtype=np.float32)) for _ in range(layers)]
+    bq, bk, bv = (lib.to_device(np.zeros(m, np.float32)) for m in (Hq * D, Hkv * D, Hkv * D))
+    tab, out = lib.empty(D), lib.empty((Hq, D))
+    dpos = lib.to_device(np.array([pos], np.uint32))
+    part = lib.empty_bytes(lib.attn_partials_bytes(Hq, Hkv, kv_max, D))
+    lib.rope_table(tab, D, pos, 1e6)
+    scale = float(1 / np.sqrt(D))
+    run = lambda i: lib.attn_decode_qkv(qkv, bq, bk, bv, Ks[i % layers], Vs[i % layers], out, Hq, Hkv, pos, kv_max, D,
+                                        scale, tab, d_pos=dpos, partials=part)
+    for i in range(layers):
+        run(i)
+    lib.sync()
+    e0, e1 = lib.event(), lib.event()
+    lib.record(e0)
+    for i in range(4 * layers):
+        run(i)
+    lib.record(e1)
+    lib.sync()
+    print("tlhip_attn_decode_qkv (attention + combine), position %d, caches rotating: %.2f us per call"
+          % (pos, lib.elapsed_ms(e0, e1) * 1e3 / (4 * layers)))
+    read_trace(lib)
+    run(0)
+    lib.sync()
+    t = read_trace(lib)
+    live = t[:, :, 0] > 0
+    print("%d wavefronts; time since the wavefront's first instruction:" % int(live.sum()))
+    names = {7: "all requests issued (query rows, rotary table, first K/V tile)",
+             1: "query rows staged in LDS, rotated; position read",
+             2: "new key/value row formed (wavefront 0 of split 0)",
+             3: "tile loop done (scores, softmax, P.V)",
+             4: "wave totals (sums over lanes and key slots) in LDS",
+             5: "block barrier passed",
+             6: "block merge done, partials stored"}
+    for sl in (7, 1, 2, 3, 4, 5, 6):
+        ok = live & (t[:, :, sl] > 0)
+        pct(names[sl], ((t[:, :, sl] - t[:, :, 0])[ok]) / (ghz * 1e3))
+
+
+def attn_prefill(lib, pos0, ghz):
+    Hq, Hkv, D, T = 28, 4, 128, 512
+    rng = np.random.default_rng(3)
+    kv_max = pos0 + T
+    scale = float(1 / np.sqrt(D))
+    K = lib.to_device(rng.standard_normal(Hkv * kv_max * D, dtype=np.float32))
+    V = lib.to_device(rng.standard_normal(Hkv * kv_max * D, dtype=np.float32))
+    q = lib.to_device(rng.standard_normal(Hq * T * D, dtype=np.float32))
+    out = lib.empty(Hq * T * D)
+    lib.tune_attn_prefill(3)
+    for _ in range(2):
+        lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
+    lib.sync()
+    read_trace(lib)
+    e0, e1 = lib.event(), lib.event()
+    lib.record(e0)
+    lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
+    lib.record(e1)
+    lib.sync()
+    print("tlhip_attn_prefill, bf16-plane kernels (planes + attention + merge), pos0 %d: %.1f us" % (pos0, lib.elapsed_ms(e0, e1) * 1e3))
+    t = read_trace(lib)
+    for grp, ws in (("wavefronts 0-3 (matrix phase, then softmax)", range(0, 4)), ("wavefronts 4-6 (softmax, then matrix phase)", range(4, 7))):
+        tt = t[:, list(ws), :]
+        live = tt[:, :, 4] > 0
+        iv = tt[:, :, 4][live]
+        print("%s: %d wavefronts, %d barrier intervals each (median); per interval:" % (grp, int(live.sum()), int(np.median(iv))))
+        for k, nm in ((1, "softmax phase"), (2, "matrix phase (P.V of the tile before, Q.K^T of this one)"), (3, "barrier wait")):
+            pct(nm, tt[:, :, k][live] / iv / (ghz * 1e3))
+        pct("whole interval", (tt[:, :, 6] - tt[:, :, 0])[live] / iv / (ghz * 1e3))
+
+
+if __name__ == "__main__":
+    args = [a for a in sys.argv[1:] if not a.startswith("--ghz")]
+    ghz = next((float(a.split("=")[1]) for a in sys.argv[1:] if a.startswith("--ghz=")), 2.1)
+    if not args or args[0] not in ("attn_decode", "attn_prefill"):
+        sys.exit(__doc__)
+    lib = load()
+    if args[0] == "attn_decode":
+        attn_decode(lib, int(args[1]) if len(args) > 1 else 4095, ghz)
+    else:
+        attn_prefill(lib, int(args[1]) if len(args) > 1 else 7680, ghz)
