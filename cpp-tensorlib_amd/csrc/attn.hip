@@ -765,11 +765,11 @@ int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, in
 
 // attn_prefill_x3.hip
 bool prefill_x3_applies(int D, int T, int pos0);
-template <typename KT>
+template <int D, typename KT>
 int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
                       int64_t kv_max, float scale, int pos0, int token_major);
 
-// Three kernels serve causal prefill attention. Deep in a context (head size 128) the bf16-plane
+// Three kernels serve causal prefill attention. Deep in a context the bf16-plane
 // kernels on the matrix cores; otherwise the fp32 matrix-pipe kernel; the VALU kernel that
 // shares its code with decode attention on request. tune_prefill: 0 = that choice, 1 = VALU,
 // 2 = fp32 matrix pipe, 3 = bf16 planes.
@@ -778,9 +778,8 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
                           int T, int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = tlhip::ctx();
   const int mode = c.tune_prefill_valu;
-  if (mode == 3 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: the bf16-plane kernel needs head size 128");
   if (mode == 3 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
-    if (int rc = launch_prefill_x3<KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
+    if (int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
     TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
   }
   if (mode != 1) {

@@ -43,10 +43,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a 16-byte unit in registers
 
-constexpr int kD = 128;                      // head size this kernel is built for
 constexpr int kTile = 32;                    // keys per tile
-constexpr int kKUnits = 4 * 2 * 64;          // 16-byte units of one K plane of a tile
-constexpr int kVUnits = 8 * 64;              // ... of one V plane
+// 16-byte units of one K plane of a tile (D/32 k-steps x 2 key halves x 64 lanes) and of one V
+// plane (D/16 column tiles x 64 lanes): 4 D either way. Head sizes 64 and 128 are built.
+template <int D> struct Img { static constexpr int kKUnits = (D / 32) * 2 * 64, kVUnits = (D / 16) * 64; };
 constexpr int kPS = 36;                      // floats per row of a wavefront's P tile (16-byte aligned rows)
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
@@ -99,10 +99,11 @@ __device__ __forceinline__ float cache_elem(const uint16_t* p) { return bf16_bit
 // ---- 1. planes ---------------------------------------------------------------------------
 // grid = (tiles, Hkv), block = 256. NP = 3 for an f32 cache, 1 for a bf16 cache.
 // planes: per (kv head, tile) a K image of NP * kKUnits uint4, then a V image of NP * kVUnits uint4.
-template <typename KT, int NP>
+template <typename KT, int NP, int D>
 __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K, const KT* __restrict__ V,
                                                         uint4* __restrict__ planes, int64_t kv_stride,
                                                         int kend, int ntiles) {
+  constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
   const int t = blockIdx.x, kvh = blockIdx.y;
   const KT* Kh = K + (size_t)kvh * kv_stride;
   const KT* Vh = V + (size_t)kvh * kv_stride;
@@ -187,10 +188,12 @@ struct Geometry {
 constexpr int kRT = 2;          // 16-row tiles per computing wavefront
 constexpr int kCompute = 7;     // computing wavefronts per block
 
-template <int NP>
+template <int NP, int D>
 __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict__ q, const uint4* __restrict__ planes,
                                                           float* __restrict__ out, float* __restrict__ part_o,
                                                           float* __restrict__ part_ml, float scale, const Geometry g) {
+  constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
+  constexpr int kKS = D / 32, kDT = D / 16;                   // k-steps of Q.K^T, column tiles of P.V
   constexpr int kKImg = NP * kKUnits, kVImg = NP * kVUnits;   // 16-byte units of a tile's K and V images
   constexpr int kImg = kKImg + kVImg;
   constexpr int kCopyK = kKImg / 64, kCopyV = kVImg / 64;     // units a lane of the copying wavefront moves per tile
@@ -254,12 +257,12 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
   const int kend = g.pos0 + g.T;
 
   // ---- the wavefront's query rows as A-operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
-  uint4 qa[kRT][3][4];
+  uint4 qa[kRT][3][kKS];
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
     const float* qrow = q + ((size_t)h * g.T + min(p_first + 16 * rt + l15, g.T - 1)) * kD;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
+    for (int ks = 0; ks < kKS; ks++) {
       const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq);
       const float4 b = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq + 4);
       const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -267,14 +270,14 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
     }
   }
 
-  f32x4 o[kRT][8];
+  f32x4 o[kRT][kDT];
   float mrow[kRT][4], lrow[kRT][4];   // rows 16 rt + 4(l/16) + r; lrow is this lane's share of the row sum
   f32x4 s[kRT][2];                    // scores of the tile whose softmax is pending
   uint4 pa3[kRT][3];                  // P planes of the tile whose P.V is pending
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
 #pragma unroll
-    for (int dt = 0; dt < 8; dt++) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt < kDT; dt++) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < 4; r++) { mrow[rt][r] = -INFINITY; lrow[rt][r] = 0.f; }
     s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -306,7 +309,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
         lrow[rt][r] = lrow[rt][r] * corr + (pr[0][r] + pr[1][r]);
         mrow[rt][r] = mnew;
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) o[rt][dt][r] *= corr;
+        for (int dt = 0; dt < kDT; dt++) o[rt][dt][r] *= corr;
       }
       // P: result order (row 4(l/16)+r, key l%16) -> operand order (row l%16, keys 8(l/16)+j)
       float* pt_ = ptile + rt * 16 * kPS;
@@ -352,7 +355,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
       // two column tiles at a time: four independent accumulators take turns, so that an MFMA
       // never waits for the result of the one issued just before it
 #pragma unroll
-      for (int dt = 0; dt < 8; dt += 2) {
+      for (int dt = 0; dt < kDT; dt += 2) {
         bf16x8 vb[2][NP];
 #pragma unroll
         for (int d2 = 0; d2 < 2; d2++)
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
 #pragma unroll
       for (int rt = 0; rt < kRT; rt++) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
+      for (int ks = 0; ks < kKS; ks++) {
         bf16x8 kb[2][NP];
 #pragma unroll
         for (int hf = 0; hf < 2; hf++)
@@ -431,12 +434,12 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
         const float inv = 1.0f / lsum;
         float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row;
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) op[16 * dt + l15] = o[rt][dt][r] * inv;
+        for (int dt = 0; dt < kDT; dt++) op[16 * dt + l15] = o[rt][dt][r] * inv;
       } else {
         const size_t row = (size_t)h * g.T + p, rows = (size_t)g.rows;   // row number in [Hq * T)
         float* po = part_o + ((size_t)split * rows + row) * kD;
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) po[16 * dt + l15] = o[rt][dt][r];
+        for (int dt = 0; dt < kDT; dt++) po[16 * dt + l15] = o[rt][dt][r];
         if (l15 == 0) {
           part_ml[((size_t)split * rows + row) * 2] = mrow[rt][r];
           part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
@@ -447,10 +450,12 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
 
 // ---- 3. merge of the key splits ---------------------------------------------------------------
 // One thread per (row, 4 columns); splits are combined in split order.
+template <int D>
 __global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restrict__ part_o,
                                                             const float* __restrict__ part_ml,
                                                             float* __restrict__ out, int rows, int T, int S,
                                                             int64_t o_head, int64_t o_row) {
+  constexpr int kD = D;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t row = i / (kD / 4);
   const int c4 = (int)(i - row * (kD / 4)) * 4;
@@ -473,15 +478,22 @@ __global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restr
 
 }  // namespace x3
 
-// Whether the bf16-plane kernels serve this call (head size 128, enough keys for the extra
-// pass to pay), and the launch. Returns 0 when launched, a negative status on failure.
-bool prefill_x3_applies(int D, int T, int pos0) { return D == x3::kD && pos0 + T >= 1024 && T >= 16; }
+// Whether the bf16-plane kernels serve this call: head size 64 or 128 and enough keys for the
+// extra passes to pay (measured crossover against the fp32 matrix-pipe kernel at the 7B and
+// 0.5B head shapes: about 1024 keys at head size 128, about 2048 at 64).
+bool prefill_x3_applies(int D, int T, int pos0) {
+  if (T < 16) return false;
+  if (D == 128) return pos0 + T >= 1024;
+  if (D == 64) return pos0 + T >= 2048;
+  return false;
+}
 
-template <typename KT>
+template <int D, typename KT>
 int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
                       int64_t kv_max, float scale, int pos0, int token_major) {
   using namespace x3;
   constexpr int NP = sizeof(KT) == 4 ? 3 : 1;
+  constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
   Context& c = ctx();
   Geometry g{};
   g.group = Hq / Hkv;
@@ -516,22 +528,24 @@ int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int 
   float* part_ml = reinterpret_cast<float*>(buf + plane_bytes + part_o_bytes);
   const size_t lds = 2 * kImgBytes + (size_t)kCompute * 16 * kRT * kPS * 4;
   if (lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
-  auto fn = attn_x3_kernel<NP>;
+  auto fn = attn_x3_kernel<NP, D>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  hipLaunchKernelGGL((kv_planes_kernel<KT, NP>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes,
+  hipLaunchKernelGGL((kv_planes_kernel<KT, NP, D>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes,
                      kv_max * (int64_t)kD, kend, g.ntiles);
   hipLaunchKernelGGL(fn, dim3(Hkv * g.head_chunks, pblocks, S), dim3(512), lds, c.stream, q, planes, out, part_o,
                      part_ml, scale, g);
   if (S > 1) {
     const int64_t threads = (int64_t)rows * (kD / 4);
-    hipLaunchKernelGGL(attn_x3_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c.stream, part_o,
+    hipLaunchKernelGGL(attn_x3_merge_kernel<D>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c.stream, part_o,
                        part_ml, out, (int)rows, T, S, g.o_head, g.o_row);
   }
   return 0;
 }
 
-template int launch_prefill_x3<float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
-template int launch_prefill_x3<uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
 
 }  // namespace tlhip

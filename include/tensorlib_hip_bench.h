@@ -29,9 +29,9 @@ int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
 int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int waves_per_block,
                        int lanes_per_row);
 /* Which kernel serves tlhip_attn_prefill: 0 = the built-in choice (bf16 planes on the matrix
- * cores deep in a context at head size 128, else the fp32 matrix pipe), 1 = the VALU kernel that
- * shares its code with decode attention, 2 = the fp32 matrix-pipe kernel, 3 = the bf16-plane
- * kernels (head size 128 only). Same results within fp32 summation order; for A/B timing and tests. */
+ * cores from 1024 keys on, else the fp32 matrix pipe), 1 = the VALU kernel that shares its code
+ * with decode attention, 2 = the fp32 matrix-pipe kernel, 3 = the bf16-plane kernels.
+ * Same results within fp32 summation order; for A/B timing and tests. */
 int tlhip_tune_attn_prefill(int kernel);
 /* Every override back to the built-in choice (tlhip_tune_gemv_cols included). */
 int tlhip_tune_reset(void);

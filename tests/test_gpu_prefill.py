@@ -352,11 +352,9 @@ KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "planes": 3}
 
 def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, kernel="auto"):
     """kernel (tlhip_tune_attn_prefill): the library's own choice, the VALU kernel, the fp32
-    matrix-pipe kernel, or the bf16-plane kernels on the matrix cores (head size 128 only)."""
+    matrix-pipe kernel, or the bf16-plane kernels on the matrix cores."""
     Hq, T, D = q.shape
     Hkv, kv_max, _ = K.shape
-    if kernel == "planes" and D != 128:
-        pytest.skip("the bf16-plane kernels are built for head size 128")
     dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, T, D))
     lib.tune_attn_prefill(KERNELS[kernel])
     try:
@@ -376,6 +374,7 @@ def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, kernel="auto"):
     (128, 7, 1, 512, 0), (64, 2, 2, 512, 0), (128, 2, 1, 200, 1000), (128, 1, 1, 31, 32), (64, 3, 1, 32, 31),
     (128, 7, 1, 512, 3584), (128, 4, 4, 256, 7680),      # deep in a context: > 120 key tiles per wavefront
     (128, 12, 1, 50, 1500), (128, 3, 1, 100, 990), (128, 16, 2, 17, 2047),   # head groups of 12, 3 and 8; ragged chunk lengths
+    (64, 14, 2, 512, 1536), (64, 5, 1, 33, 3000),                            # head size 64 deep in a context (0.5B shape)
 ])
 def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, kernel):
     """Causal prefill over a cache: query p at absolute position pos0+p sees keys
