@@ -14,23 +14,24 @@
 // plane for K and V and three products. Scores and outputs then differ from an fp32 loop by
 // what a different summation order would give.
 //
-// Two kernels per call:
+// Three kernels per call:
 //  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into planes, written
-//     as the exact register image of the MFMA B operands, one 32-key tile after the other:
-//       K image [plane][k-step 0..3][16-key half 0..1][lane][8]  = K[32t + 16h + l%16][32s + 8(l/16) + j]
-//       V image [plane][16-dim tile 0..7][lane][8]               = V[32t + 8(l/16) + j][16d + l%16]
+//     as the exact register image of the MFMA operands, one 32-key tile after the other:
+//       K image [plane][k-step][16-key half 0..1][lane][8]  = K[32t + 16h + l%16][32s + 8(l/16) + j]
+//       V image [plane][16-column tile][lane][8]            = V[32t + tile_key(l/16, j)][16d + l%16]
 //     so that the attention kernel copies a tile to LDS verbatim and every operand is one
 //     conflict-free 16-byte LDS read per lane. Keys at and past pos0 + T are written as zeros.
-//  2. attn_x3_kernel: a block serves ONE kv head and up to 8 (query head, 16-position tile)
-//     pairs, one per wavefront, that all read the same K/V tiles: with grouped-query attention
-//     the query heads of the group, else consecutive position tiles. The 32-key tiles of the
+//  2. attn_x3_kernel: a block serves ONE kv head and up to 7 wavefronts of 32 query rows each
+//     that all read the same K/V tiles: with grouped-query attention the query heads of the
+//     group (32 positions each), else consecutive runs of positions. The 32-key tiles of the
 //     block's causal range are dealt round-robin over `S` blocks (key splits); a tile is staged
-//     into LDS once per block (double buffered, one barrier per tile) and read by every
-//     wavefront. A wavefront keeps its 16 query rows as bf16 planes in registers (the A
-//     operand), the running (max, sum) of its rows and a 16 x 128 output accumulator.
-//     Per tile: 48 MFMAs for the scores, an online-softmax update on 8 scores per lane
-//     (reductions stay inside a 16-lane DPP row), P through a small LDS tile into A-operand
-//     order and into planes, 48 MFMAs for P.V.
+//     into LDS once per block (double buffered, one barrier per tile) by an eighth wavefront
+//     and read by every computing wavefront. Both products are formed transposed
+//     (S^T = K . Q^T, O^T = V^T . P^T): a lane's scores, probabilities and output columns all
+//     belong to one query row, so the softmax needs no exchange through LDS and P goes from
+//     the score registers - cut into planes - straight back into the matrix core.
+//     Per tile and wavefront: 96 MFMAs for the scores, an online-softmax update on 16 scores
+//     per lane, 96 MFMAs for P.V.
 //     S == 1 writes the normalised rows; S > 1 leaves (max, sum, accumulator) per split and
 //  3. attn_x3_merge_kernel combines them in split order.
 #include "common.hpp"
@@ -46,8 +47,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a 16-byte unit 
 constexpr int kTile = 32;                    // keys per tile
 // 16-byte units of one K plane of a tile (D/32 k-steps x 2 key halves x 64 lanes) and of one V
 // plane (D/16 column tiles x 64 lanes): 4 D either way. Head sizes 64 and 128 are built.
+// The scores of a 32-key tile leave the two 16x16 MFMAs with lane (g = l/16, c = l%16) holding,
+// for query row c, the keys 16h + 4g + r (h = 0, 1; r = 0..3). Those 8 values, in the order
+// j = 4h + r, are the lane's 8 elements of the P.V reduction index, so the V image lists the keys
+// in the same order: element j of lane group g is key 16 (j / 4) + 4 g + j % 4 of the tile.
+__host__ __device__ constexpr int tile_key(int g, int j) { return 16 * (j >> 2) + 4 * g + (j & 3); }
+
 template <int D> struct Img { static constexpr int kKUnits = (D / 32) * 2 * 64, kVUnits = (D / 16) * 64; };
-constexpr int kPS = 36;                      // floats per row of a wavefront's P tile (16-byte aligned rows)
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
@@ -123,10 +129,10 @@ __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K
       plane_stride = kKUnits;
     } else {
       const int v = u - kKUnits, l = v & 63, dt = v >> 6;
-      const int key0 = t * kTile + 8 * (l >> 4), dim = 16 * dt + (l & 15);
+      const int dim = 16 * dt + (l & 15);
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        const int key = key0 + j;
+        const int key = t * kTile + tile_key(l >> 4, j);
         x[j] = key < kend ? cache_elem(Vh + (size_t)key * kD + dim) : 0.f;
       }
       dst = img + NP * kKUnits + v;
@@ -172,12 +178,12 @@ struct Geometry {
 // grid = (Hkv * head_chunks, position blocks, S), block = 512: seven computing wavefronts and
 // one that moves tiles.
 //
-// LDS bandwidth is what bounds this kernel (a 16-byte-per-lane read runs at 64 bytes a clock per
-// CU, and every B operand of every MFMA comes from LDS), so a computing wavefront owns TWO
-// 16-row tiles - 32 consecutive positions of one head - and uses every K/V operand it reads
-// twice. Its registers then hold 96 for the query planes and 64 for the output accumulators,
-// which leaves no room for tiles in transit: wavefront 7 does nothing but copy, K of the next
-// tile and V of this one, global -> registers -> LDS, one 16-byte unit per lane and instruction.
+// A computing wavefront owns TWO 16-row tiles - 32 consecutive positions of one head - and uses
+// every K/V operand it reads from LDS twice (with one tile per wavefront the operand reads took
+// as long as the MFMAs they feed). Its registers then hold 96 for the query planes and 64 for
+// the output accumulators, which leaves no room for tiles in transit: wavefront 7 does nothing
+// but copy, K of the next tile and V of this one, global -> registers -> LDS, one 16-byte unit
+// per lane and instruction.
 //
 // A step of the loop is one barrier interval. In interval i a computing wavefront runs one
 // matrix phase - P.V of tile i-1, then Q.K^T of tile i - and one vector phase, the online
@@ -197,10 +203,9 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
   constexpr int kKImg = NP * kKUnits, kVImg = NP * kVUnits;   // 16-byte units of a tile's K and V images
   constexpr int kImg = kKImg + kVImg;
   constexpr int kCopyK = kKImg / 64, kCopyV = kVImg / 64;     // units a lane of the copying wavefront moves per tile
-  extern __shared__ u32x4 lds4[];                             // K images [2], V images [2], 7 P tiles of 32 x kPS floats
+  extern __shared__ u32x4 lds4[];                             // K images [2], V images [2]
   u32x4* kbuf = lds4;
   u32x4* vbuf = lds4 + 2 * kKImg;
-  float* ptile_base = reinterpret_cast<float*>(lds4 + 2 * kImg);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l15 = lane & 15, lq = lane >> 4;
@@ -256,7 +261,15 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
   const int my_last_key = g.pos0 + min(p_first + 16 * kRT - 1, g.T - 1);
   const int kend = g.pos0 + g.T;
 
-  // ---- the wavefront's query rows as A-operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
+  // Both products are formed transposed, S^T = K . Q^T and O^T = V^T . P^T, so that a lane's
+  // results all belong to ONE query row (row l%16 of each of the wavefront's two 16-row tiles):
+  // its 8 scores of a tile are 8 keys of that row, they stay in the lane through the softmax,
+  // become - cut into planes - the lane's B operand of P.V as they are, and the output
+  // accumulators they feed hold 4 columns of the same row. No exchange through LDS, one
+  // running maximum and one running sum per lane and tile; a row's keys are spread over the 4
+  // lanes c, c+16, c+32, c+48, which meet in two register swaps.
+
+  // ---- the wavefront's query rows as operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
   uint4 qa[kRT][3][kKS];
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
@@ -270,68 +283,55 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
     }
   }
 
-  f32x4 o[kRT][kDT];
-  float mrow[kRT][4], lrow[kRT][4];   // rows 16 rt + 4(l/16) + r; lrow is this lane's share of the row sum
-  f32x4 s[kRT][2];                    // scores of the tile whose softmax is pending
+  f32x4 o[kRT][kDT];                  // O^T: columns 16 dt + 4(l/16) + r of row l%16
+  float mrow[kRT], lrow[kRT];         // row l%16: running maximum; this lane's share of the running sum
+  f32x4 s[kRT][2];                    // S^T of the tile whose softmax is pending: keys 16 h + 4(l/16) + r
   uint4 pa3[kRT][3];                  // P planes of the tile whose P.V is pending
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
 #pragma unroll
     for (int dt = 0; dt < kDT; dt++) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < 4; r++) { mrow[rt][r] = -INFINITY; lrow[rt][r] = 0.f; }
+    mrow[rt] = -INFINITY;
+    lrow[rt] = 0.f;
     s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
     pa3[rt][0] = pa3[rt][1] = pa3[rt][2] = make_uint4(0, 0, 0, 0);
   }
-  float* ptile = ptile_base + wave * (16 * kRT) * kPS;
 
-  // the vector phase of tile number i: masks, running maxima and sums, rescale of the output
-  // accumulators, P into operand order and planes
+  // the vector phase of tile number i: masks, running maximum and sum, rescale of the output
+  // accumulators, P cut into planes
   const auto softmax_tile = [&](int i) {
     const int kt = tile_of(i);
+    // only a tile that reaches past the first row's causal limit (or the chunk's last key) needs masks
+    const bool masked = (kt + 1) * kTile - 1 > min(g.pos0 + p_first, kend - 1);   // (uniform for the wavefront)
 #pragma unroll
     for (int rt = 0; rt < kRT; rt++) {
-      float pr[2][4];
+      float v[8];
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int limit = min(g.pos0 + p_first + 16 * rt + 4 * lq + r, kend - 1);   // last key the row sees
-        float sv[2];
+      for (int j = 0; j < 8; j++) v[j] = s[rt][j >> 2][j & 3] * scale;
+      if (masked) {
+        const int limit = min(g.pos0 + p_first + 16 * rt + l15, kend - 1);   // last key the row sees
 #pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-          const int key = kt * kTile + 16 * hf + l15;
-          sv[hf] = key <= limit ? s[rt][hf][r] * scale : -INFINITY;
-        }
-        const float mnew = fmaxf(mrow[rt][r], row_max16(fmaxf(sv[0], sv[1])));
-        const float mref = mnew == -INFINITY ? 0.f : mnew;
-        const float corr = __expf(mrow[rt][r] - mref);
-        pr[0][r] = __expf(sv[0] - mref);
-        pr[1][r] = __expf(sv[1] - mref);
-        lrow[rt][r] = lrow[rt][r] * corr + (pr[0][r] + pr[1][r]);
-        mrow[rt][r] = mnew;
-#pragma unroll
-        for (int dt = 0; dt < kDT; dt++) o[rt][dt][r] *= corr;
+        for (int j = 0; j < 8; j++) v[j] = kt * kTile + tile_key(lq, j) <= limit ? v[j] : -INFINITY;
       }
-      // P: result order (row 4(l/16)+r, key l%16) -> operand order (row l%16, keys 8(l/16)+j)
-      float* pt_ = ptile + rt * 16 * kPS;
+      float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+      LanePair e = swap16(mx, mx);
+      mx = fmaxf(e.first, e.second);
+      e = swap32(mx, mx);
+      mx = fmaxf(e.first, e.second);               // over the row's 32 keys
+      const float mnew = fmaxf(mrow[rt], mx);
+      const float mref = mnew == -INFINITY ? 0.f : mnew;
+      const float corr = __expf(mrow[rt] - mref);
+      float p[8];
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        pt_[(4 * lq + r) * kPS + l15] = pr[0][r];
-        pt_[(4 * lq + r) * kPS + 16 + l15] = pr[1][r];
+      for (int j = 0; j < 8; j++) p[j] = __expf(v[j] - mref);
+      lrow[rt] = lrow[rt] * corr + (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7])));
+      mrow[rt] = mnew;
+#pragma unroll
+      for (int dt = 0; dt < kDT; dt++) {
+        o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
       }
+      split3x8(p, pa3[rt][0], pa3[rt][1], pa3[rt][2]);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int rt = 0; rt < kRT; rt++) {
-      const float* pt_ = ptile + rt * 16 * kPS;
-      const float4 a = *reinterpret_cast<const float4*>(pt_ + l15 * kPS + 8 * lq);
-      const float4 b = *reinterpret_cast<const float4*>(pt_ + l15 * kPS + 8 * lq + 4);
-      const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-      split3x8(x, pa3[rt][0], pa3[rt][1], pa3[rt][2]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();   // the tile is rewritten by the next softmax
   };
   const auto mine = [&](int i) { return active && i >= 0 && i < n && tile_of(i) * kTile <= my_last_key; };
 
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
     if (late && mine(i - 1)) softmax_tile(i - 1);
     TLHIP_X3_T(0);
     // ---- matrix phase; plane pairs (a, b) with a + b <= 2, smallest products first ----
-    if (mine(i - 1)) {   // O[32 x 128] += P[32 x 32] . V[32 x 128] of tile i-1, eight 16-column tiles
+    if (mine(i - 1)) {   // O^T[D x 32 rows] += V^T[D x 32 keys] . P^T[32 keys x 32 rows] of tile i-1, 16-column tiles
       const u32x4* vimg = vbuf + ((i - 1) & 1) * kVImg;
       // two column tiles at a time: four independent accumulators take turns, so that an MFMA
       // never waits for the result of the one issued just before it
@@ -371,12 +371,12 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
               for (int d2 = 0; d2 < 2; d2++)
 #pragma unroll
                 for (int rt = 0; rt < kRT; rt++)
-                  o[rt][dt + d2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(pa3[rt][pa]), vb[d2][pb], o[rt][dt + d2], 0, 0, 0);
+                  o[rt][dt + d2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb[d2][pb], as_bf16x8(pa3[rt][pa]), o[rt][dt + d2], 0, 0, 0);
             }
           }
       }
     }
-    if (mine(i)) {       // S[32 rows x 32 keys] of tile i as 16 x 16 tiles
+    if (mine(i)) {       // S^T[32 keys x 32 rows] of tile i as 16 x 16 tiles
       const u32x4* kimg = kbuf + (i & 1) * kKImg;
 #pragma unroll
       for (int rt = 0; rt < kRT; rt++) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
               for (int hf = 0; hf < 2; hf++)
 #pragma unroll
                 for (int rt = 0; rt < kRT; rt++)
-                  s[rt][hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(qa[rt][pa][ks]), kb[hf][pb], s[rt][hf], 0, 0, 0);
+                  s[rt][hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[hf][pb], as_bf16x8(qa[rt][pa][ks]), s[rt][hf], 0, 0, 0);
             }
           }
       }
@@ -421,31 +421,35 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
 #undef TLHIP_X3_T0
 #undef TLHIP_X3_T
 
-  // ---- rows complete for this split: sum l over the row's 16 lanes, store ----
+  // ---- rows complete for this split: the row's sum over its 4 lanes, store 4 columns per lane and tile ----
   if (!active) return;
 #pragma unroll
-  for (int rt = 0; rt < kRT; rt++)
+  for (int rt = 0; rt < kRT; rt++) {
+    const int p = p_first + 16 * rt + l15;
+    LanePair e = swap16(lrow[rt], lrow[rt]);
+    float lsum = e.first + e.second;
+    e = swap32(lsum, lsum);
+    lsum = e.first + e.second;
+    if (p >= g.T) continue;
+    if (g.S == 1) {
+      const float inv = 1.0f / lsum;
+      float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row + 4 * lq;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const int p = p_first + 16 * rt + 4 * lq + r;
-      const float lsum = row_sum16(lrow[rt][r]);
-      if (p >= g.T) continue;
-      if (g.S == 1) {
-        const float inv = 1.0f / lsum;
-        float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row;
+      for (int dt = 0; dt < kDT; dt++)
+        *reinterpret_cast<float4*>(op + 16 * dt) =
+            make_float4(o[rt][dt][0] * inv, o[rt][dt][1] * inv, o[rt][dt][2] * inv, o[rt][dt][3] * inv);
+    } else {
+      const size_t row = (size_t)h * g.T + p, rows = (size_t)g.rows;   // row number in [Hq * T)
+      float* po = part_o + ((size_t)split * rows + row) * kD + 4 * lq;
 #pragma unroll
-        for (int dt = 0; dt < kDT; dt++) op[16 * dt + l15] = o[rt][dt][r] * inv;
-      } else {
-        const size_t row = (size_t)h * g.T + p, rows = (size_t)g.rows;   // row number in [Hq * T)
-        float* po = part_o + ((size_t)split * rows + row) * kD;
-#pragma unroll
-        for (int dt = 0; dt < kDT; dt++) po[16 * dt + l15] = o[rt][dt][r];
-        if (l15 == 0) {
-          part_ml[((size_t)split * rows + row) * 2] = mrow[rt][r];
-          part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
-        }
+      for (int dt = 0; dt < kDT; dt++)
+        *reinterpret_cast<float4*>(po + 16 * dt) = make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+      if (lq == 0) {
+        part_ml[((size_t)split * rows + row) * 2] = mrow[rt];
+        part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
       }
     }
+  }
 }
 
 // ---- 3. merge of the key splits ---------------------------------------------------------------
@@ -526,7 +530,7 @@ int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int 
   uint4* planes = reinterpret_cast<uint4*>(buf);
   float* part_o = reinterpret_cast<float*>(buf + plane_bytes);
   float* part_ml = reinterpret_cast<float*>(buf + plane_bytes + part_o_bytes);
-  const size_t lds = 2 * kImgBytes + (size_t)kCompute * 16 * kRT * kPS * 4;
+  const size_t lds = 2 * kImgBytes;
   if (lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
   auto fn = attn_x3_kernel<NP, D>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
