@@ -779,8 +779,11 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
   Context& c = tlhip::ctx();
   const int mode = c.tune_prefill_valu;
   if (mode == 3 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
-    if (int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
-    TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
+    const int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major);
+    if (rc < 0) return rc;
+    if (rc == 0) TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
+    if (mode == 3) return fail(TLHIP_ENOMEM, "tlhip_attn_prefill: no scratch for the key/value planes");
+    // no scratch for the planes: the fp32 matrix-pipe kernel needs none
   }
   if (mode != 1) {
     if (int rc = launch_prefill_mfma<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)) return rc;
