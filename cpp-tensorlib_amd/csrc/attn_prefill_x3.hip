@@ -145,26 +145,6 @@ __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K
   }
 }
 
-// max / sum over the 16 lanes of a DPP row, result in every lane of the row
-template <int CTRL>
-__device__ __forceinline__ float dppv(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float row_max16(float v) {
-  v = fmaxf(v, dppv<0xB1>(v));
-  v = fmaxf(v, dppv<0x4E>(v));
-  v = fmaxf(v, dppv<0x141>(v));
-  v = fmaxf(v, dppv<0x140>(v));
-  return v;
-}
-__device__ __forceinline__ float row_sum16(float v) {
-  v += dppv<0xB1>(v);
-  v += dppv<0x4E>(v);
-  v += dppv<0x141>(v);
-  v += dppv<0x140>(v);
-  return v;
-}
-
 struct Geometry {
   int group;        // query heads per kv head
   int nh, np;       // computing wavefronts of a block: nh heads x np runs of 32 positions (nh * np <= 7)
