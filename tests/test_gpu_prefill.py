@@ -394,6 +394,85 @@ def test_attn_prefill_matches_oracle(lib, orc, D, Hq, Hkv, T, pos0, kernel):
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
+def _attn_f64(q, K, V, scale, pos0):
+    """Causal attention in float64: what the arithmetic fixes, independent of any summation order."""
+    Hq, T, D = q.shape
+    Hkv = K.shape[0]
+    out = np.empty((Hq, T, D))
+    for h in range(Hq):
+        kh, vh = K[h // (Hq // Hkv)].astype(np.float64), V[h // (Hq // Hkv)].astype(np.float64)
+        for t in range(T):
+            s = (kh[:pos0 + t + 1] @ q[h, t].astype(np.float64)) * scale
+            p = np.exp(s - s.max())
+            out[h, t] = (p / p.sum()) @ vh[:pos0 + t + 1]
+    return out
+
+
+@pytest.mark.parametrize("kernel", ["fp32pipe", "planes"])
+@pytest.mark.parametrize("case", ["one_dominant_key", "equal_scores", "large_values", "tiny_values", "cancelling_values"])
+def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
+    """Rows chosen against the bf16-plane products (three planes per operand, six plane pairs per
+    product: what is dropped is below 2^-23 of |a b|) and against the online softmax:
+      one_dominant_key    one key's score exceeds the others by ~40: the softmax is one-hot to
+                          fp32 and the output must be that key's value row;
+      equal_scores        every key of a row scores the same to 1e-6: the output is a plain mean,
+                          where an error in the scores is not damped by a peaked softmax;
+      large_values        |q|, |k|, |v| around 2^10 (scores around 1e5 before the maximum is
+                          taken): plane residuals of large numbers;
+      tiny_values         values around 2^-40: the third plane is near the bottom of bf16's range;
+      cancelling_values   V alternates +-(1000 + small) so that the output is a small difference
+                          of large terms (tests the value planes and the fp32 accumulation).
+    Both matrix kernels against the CPU oracle at allclose(1e-4, 1e-5) and against float64 with the
+    bound an fp32 evaluation obeys: 2^-22 (4 + max_k sum_i |q_i k_i| scale) sum_k p_k |v_k| (the
+    CPU oracle itself uses up to 0.7 of it on these rows; the plane kernel measured at or below the
+    oracle's error on every case)."""
+    print("case attn_prefill adversarial", case, kernel, flush=True)
+    D, Hq, Hkv, T, pos0 = 128, 7, 1, 48, 1200
+    kv_max = pos0 + T
+    rng = np.random.default_rng(17)
+    q = rng.standard_normal((Hq, T, D)).astype(np.float32)
+    K = rng.standard_normal((Hkv, kv_max, D)).astype(np.float32)
+    V = rng.standard_normal((Hkv, kv_max, D)).astype(np.float32)
+    scale = np.float32(1.0 / np.sqrt(float(D)))
+    if case == "one_dominant_key":
+        # key 777 is 4 q-directions long for every row: its score leads by ~ 4 |q|^2 scale ~ 45
+        K[0, 777] = 0.0
+        q[:] = np.abs(q)
+        K[0, 777] = 4.0 * np.sign(q.mean(axis=(0, 1)))
+    elif case == "equal_scores":
+        K[0, :] = K[0, 0] + (1e-6 * rng.standard_normal((kv_max, D))).astype(np.float32)
+    elif case == "large_values":
+        q *= np.float32(1024.0); K *= np.float32(1024.0); V *= np.float32(1024.0)
+        scale = np.float32(scale / 1024.0 / 1024.0 * 8.0)
+    elif case == "tiny_values":
+        q *= np.float32(2.0 ** -40); K *= np.float32(2.0 ** -40); V *= np.float32(2.0 ** -40)
+        scale = np.float32(scale * 2.0 ** 80)
+    elif case == "cancelling_values":
+        sign = np.where(np.arange(kv_max) % 2 == 0, 1.0, -1.0).astype(np.float32)
+        V[0] = sign[:, None] * (1000.0 + V[0])
+        K[0, :] = K[0, 0] + (1e-3 * rng.standard_normal((kv_max, D))).astype(np.float32)   # near-uniform softmax
+    got = _prefill(lib, q, K, V, float(scale), pos0, kernel=kernel)
+    want = orc.attn_prefill(q, K, V, float(scale), pos0)
+    assert np.all(np.isfinite(got))
+    exact = _attn_f64(q, K, V, float(scale), pos0)
+    # sum_k p_k |v_k| per output element, the scale an fp32 evaluation's error goes with
+    mag = _attn_f64(q, K, np.abs(V), float(scale), pos0)
+    err, err_ref = np.abs(got - exact), np.abs(want - exact)
+    # An fp32 score carries up to 2^-24 sum_i |q_i k_i| scale of rounding per product, and an error
+    # d in a score is a relative error d in its probability: the bound grows with the largest
+    # sum_i |q_i k_i| scale of a row (its own dot products are what the planes must reproduce).
+    absdot = np.einsum("htd,kd->htk", np.abs(q).astype(np.float64), np.abs(K[0]).astype(np.float64)).max(axis=2) * float(scale)
+    bound = 2.0 ** -22 * (4.0 + absdot)[:, :, None] * mag + 1e-37
+    print("   max err / bound: kernel %.3f, CPU oracle %.3f" % ((err / bound).max(), (err_ref / bound).max()), flush=True)
+    assert np.all(err <= bound), float((err / bound).max())
+    # (with sharp softmaxes over large scores, or outputs that are small differences of large
+    # terms, two correct fp32 evaluations differ by more than allclose(1e-4, 1e-5) allows)
+    if case in ("one_dominant_key", "equal_scores"):
+        assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+    if case == "one_dominant_key":
+        assert allclose(got, np.broadcast_to(V[0, 777], got.shape), 1e-6, 1e-6)
+
+
 @pytest.mark.parametrize("kernel", list(KERNELS))
 def test_attn_prefill_rows_equal_decode(lib, orc, kernel):
     """Row p of a prefill equals a decode step with ctx = pos0 + p + 1 (the equivalence the
