@@ -80,6 +80,11 @@ SIGNATURES = {
     "tlhip_gemm_q4_nt_swiglu": (cint, [P, P, P, P, i64, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_swiglu": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_parts": (cint, [P, P, P, i64, i64, i64, i64, P]),
+    "tlhip_gemm_f16w_bytes": (i64, [i64, i64, cint]),
+    "tlhip_gemm_f16w_prepare": (cint, [P, i64, i64, cint, P, P]),
+    "tlhip_gemm_f16w_nt": (cint, [P, P, P, P, i64, i64, i64]),
+    "tlhip_gemm_f16w_nt_parts": (cint, [P, P, P, P, i64, i64, i64, i64, P]),
+    "tlhip_gemm_f16w_nt_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
     "tlhip_rmsnorm_res_parts": (cint, [P, P, i64, P, P, P, i64, f32, i64]),
     "tlhip_split_heads": (cint, [P, P, P, i64, i64, i64, i64, i64]),
     "tlhip_merge_heads": (cint, [P, P, i64, i64, i64]),
@@ -112,6 +117,7 @@ SIGNATURES = {
     "tlhip_tune_gemv_q4": (cint, [cint, cint, cint, cint, cint]),
     "tlhip_tune_gemv_cols": (cint, [cint]),
     "tlhip_tune_attn_prefill": (cint, [cint]),
+    "tlhip_tune_gemm_planes": (cint, [cint]),
     "tlhip_tune_reset": (cint, []),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
@@ -332,6 +338,29 @@ class TlHip:
         self._chk(self.c.tlhip_gemm_bf16_nt_parts(A.ptr, W.ptr, parts.ptr, parts.nbytes, M, N, K, C.byref(n)))
         return n.value
 
+    def gemm_f16w_prepare(self, W, N, K, gated=False):
+        """The prepared form of the bf16 weight W ([N, K], or [2 * N, K] = gate rows | up rows when
+        gated): returns (image, exps) device buffers for the gemm_f16w_* products."""
+        nbytes = self.c.tlhip_gemm_f16w_bytes(N, K, int(gated))
+        if nbytes <= 0:
+            raise ValueError("gemm_f16w_prepare: need positive N, K and K % 32 == 0")
+        image = self.empty_bytes(nbytes)
+        exps = self.empty_bytes((2 * N if gated else N))
+        self._chk(self.c.tlhip_gemm_f16w_prepare(W.ptr, N, K, int(gated), image.ptr, exps.ptr))
+        return image, exps
+
+    def gemm_f16w_nt(self, A, image, exps, out, M, N, K):
+        self._chk(self.c.tlhip_gemm_f16w_nt(A.ptr, image.ptr, exps.ptr, out.ptr, M, N, K))
+
+    def gemm_f16w_nt_swiglu(self, A, image, exps, act, M, ff, K):
+        self._chk(self.c.tlhip_gemm_f16w_nt_swiglu(A.ptr, image.ptr, exps.ptr, act.ptr, M, ff, K))
+
+    def gemm_f16w_nt_parts(self, A, image, exps, parts, M, N, K):
+        n = C.c_int(0)
+        self._chk(self.c.tlhip_gemm_f16w_nt_parts(A.ptr, image.ptr, exps.ptr, parts.ptr, parts.nbytes, M, N, K,
+                                                  C.byref(n)))
+        return n.value
+
     def rmsnorm_res_parts(self, x, parts, n_parts, w, xout, hout, n, eps, rows=1):
         self._chk(self.c.tlhip_rmsnorm_res_parts(x.ptr, parts.ptr, n_parts, w.ptr, xout.ptr, hout.ptr,
                                                  n, eps, rows))
@@ -461,6 +490,10 @@ class TlHip:
     def tune_attn_prefill(self, kernel):
         """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes."""
         self._chk(self.c.tlhip_tune_attn_prefill(int(kernel)))
+
+    def tune_gemm_planes(self, planes):
+        """3: the int4 prompt GEMMs cut activations into three bf16 terms; 0: built-in choice (two f16)."""
+        self._chk(self.c.tlhip_tune_gemm_planes(int(planes)))
 
     def tune_reset(self):
         self._chk(self.c.tlhip_tune_reset())

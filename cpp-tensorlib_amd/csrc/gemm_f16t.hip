@@ -1,0 +1,474 @@
+// Prompt-chunk GEMM over a PREPARED bf16 weight: C[M,N] = A[M,K] f32 . W[N,K]^T, on f16 operands
+// copied global -> LDS without passing through registers.
+//
+// Why a second GEMM. Measured per K slab, gemm_bf16_nt_kernel (prefill.hip) is not bound by the
+// matrix pipe: its 128 x 256 tile pulls 32 KB per slab through the CU's vector memory path, which
+// moves about 45 bytes a clock for rows that are 64 or 128 bytes long and kilobytes apart, and it
+// spends 100-140 vector ALU instructions per lane and slab on cutting activations into planes -
+// together more clocks than the slab's MFMAs. Both costs are removed here by doing the work once,
+// outside the loop:
+//   * the weight is prepared when it is loaded (tlhip_gemm_f16w_prepare): every row times
+//     2^ew[n], converted to f16 (a bf16 weight has 8 significant bits, an f16 holds 11; ew[n]
+//     brings the row's largest magnitude into [2^14, 2^15), so every weight within 2^-29 of it
+//     converts exactly and smaller ones carry an absolute error below 2^-40 of it), stored as the
+//     LDS image of each (256 rows, 32 k) slab: 16 KB, rows already in the bank-conflict-free order
+//     the fragment reads expect;
+//   * the activations are cut once per call (a_image_kernel): row m times 2^ea[m], then TWO f16
+//     terms, both rounded to nearest - a * 2^ea = hi + lo + r with |r| <= 2^-24 |a * 2^ea| where lo
+//     is a normal f16 (<= 2^-39 of the row's largest where it is not): the accuracy of one fp32
+//     rounding, from two MFMAs per product instead of the three of the bf16 split - again stored
+//     as slab images, 32 KB per (256 rows, 32 k).
+// The GEMM then has no vector ALU work and no address arithmetic in its loop: a slab is 48
+// contiguous kilobytes, copied by 48 global_load_lds_dwordx4 (1 KB each, whole cache lines, no
+// registers), six per wavefront. A block is eight wavefronts (4 x 2) on a 256 x 256 tile, 64 x 128
+// per wavefront (128 x 256 and 32 x 128 where N is small), one block per CU, a ring of three slabs
+// in LDS (144 KB), one barrier per slab; a copy has two slab times to land. Products of f16 are exact in fp32, the MFMA sums in fp32, and
+// the result leaves as acc * 2^-(ea[m] + ew[n]), an exact scaling: the error is fp32 summation
+// error plus one fp32-rounding-sized term per product, as in the reference's fp32 FMA loop
+// (tensorlib_cuda.cu:509-519).
+#include "gemm_shared.hpp"
+
+namespace tlhip {
+namespace f16t {
+
+template <int N> struct Idx { static constexpr int value = N; };
+
+constexpr int kBK = 32;                 // K slab
+constexpr int kTile = 256;              // block tile, both ways
+constexpr int kRing = 3;
+constexpr int kRowBytes = kBK * 2;      // one row of one plane of a slab: 64 bytes, four 16-byte chunks
+constexpr int kPlaneBytes = kTile * kRowBytes;          // 16 KB
+constexpr int kAImage = 2 * kPlaneBytes;                // hi plane, lo plane
+constexpr int kWImage = kPlaneBytes;
+
+// Byte offset of 16-byte chunk `chunk` (8 k) of row `row` inside a plane image: the chunk index is
+// XORed with bits of the row so that both the fragment reads (32 consecutive rows, same chunk) and
+// linear copies spread over all LDS banks.
+__host__ __device__ __forceinline__ int image_off(int row, int chunk) {
+  return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4);
+}
+
+// W row behind tile column `col` (0..255) of column tile `tn`; -1 past the edge. Gated: the tile's
+// two 128-column strips are 64 gate features followed by the same features' up rows (ff rows
+// further down), so that a lane of the GEMM holds both accumulators of a feature.
+__host__ __device__ __forceinline__ int weight_row(bool gated, int tn, int col, int n, int ff) {
+  if (gated) {
+    const int j = col & 127, f = tn * 128 + (col >> 7) * 64 + (j & 63);
+    return f < n ? f + (j >= 64 ? ff : 0) : -1;
+  }
+  const int r = tn * kTile + col;
+  return r < n ? r : -1;
+}
+
+// One block per (column tile, slab): 256 rows x 32 k of the bf16 weight -> its f16 slab image.
+// n = rows of W (plain) or features (gated: W has 2 * ff rows).
+__global__ __launch_bounds__(256) void w_image_kernel(const uint16_t* __restrict__ W,
+                                                      const int8_t* __restrict__ ew, char* __restrict__ img,
+                                                      int n, int K, int ff, int gated) {
+  const int tn = blockIdx.x, slab = blockIdx.y, nslab = gridDim.y, t = threadIdx.x;
+  char* dst = img + ((size_t)tn * nslab + slab) * kWImage;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int col = (t >> 2) + 64 * i, c8 = t & 3;
+    const int r = weight_row(gated != 0, tn, col, n, ff);
+    frag16 v = {0u, 0u, 0u, 0u};
+    if (r >= 0)
+      v = bf16x8_to_f16(*reinterpret_cast<const frag16*>(W + (size_t)r * K + slab * kBK + c8 * 8), pow2f(ew[r]));
+    *reinterpret_cast<frag16*>(dst + image_off(col, c8)) = v;
+  }
+}
+
+// One block per (row tile, slab): 256 rows x 32 k of the activations -> hi and lo f16 slab images.
+__global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ A, const int* __restrict__ ea,
+                                                      char* __restrict__ img, int M, int K) {
+  const int tm = blockIdx.x, slab = blockIdx.y, nslab = gridDim.y, t = threadIdx.x;
+  char* dst = img + ((size_t)tm * nslab + slab) * kAImage;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int row = (t >> 3) + 32 * i, c4 = t & 7, gm = tm * kTile + row;
+    uint32_t h01 = 0, l01 = 0, h23 = 0, l23 = 0;
+    if (gm < M) {
+      const float4 a = *reinterpret_cast<const float4*>(A + (size_t)gm * K + slab * kBK + c4 * 4);
+      const float s = pow2f(ea[gm]);
+      split2_f16(a.x * s, a.y * s, h01, l01);
+      split2_f16(a.z * s, a.w * s, h23, l23);
+    }
+    const int o = image_off(row, c4 >> 1) + (c4 & 1) * 8;
+    *reinterpret_cast<uint2*>(dst + o) = make_uint2(h01, h23);
+    *reinterpret_cast<uint2*>(dst + kPlaneBytes + o) = make_uint2(l01, l23);
+  }
+}
+
+// Grid: x = tiles (row tiles fastest, one contiguous run of tiles per XCD), y = K-split parts of
+// `part_slabs` slabs each; part y goes to C + y * M * ldc. N = columns of this launch (gated:
+// features), tn0 = first column tile (the launch may cover a column range of the weight).
+// TM = 2: a 256 x 256 tile, 64 x 128 per wavefront. TM = 1: 128 x 256 (32 x 128 per wavefront, one
+// half of an activation image): twice the tiles for the products whose N is a few thousand, which
+// then need half the K splits and write half the parts.
+// GU: the result is the gated activation act[m][f] = swiglu(A . gate_f, A . up_f)
+// (array.h:2435-2439) when K is not split; under a split the raw parts are stored in tile column
+// order and splitk_sum_swiglu_kernel gates after the sum.
+template <int TM, bool GU>
+__global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restrict__ Aimg,
+                                                           const char* __restrict__ Wimg,
+                                                           float* __restrict__ C, int M, int N, int nslab,
+                                                           int part_slabs, int ldc, int tn0, int ff,
+                                                           const int* __restrict__ ea,
+                                                           const int8_t* __restrict__ ew) {
+  constexpr int BM = 128 * TM;
+  constexpr int kAPlane = BM * kRowBytes;            // one plane of this block's rows in a stage
+  constexpr int kStage = 2 * kAPlane + kWImage;
+  constexpr int kCopies = 2 * TM + 2;                // 1 KB copies per wavefront and slab
+  extern __shared__ __attribute__((aligned(1024))) char ring[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;           // 4 x 2 wavefronts, (32 * TM) x 128 each
+  const int mt = (M + BM - 1) / BM;
+  const int nb = gridDim.x, xcd = blockIdx.x & 7, within = blockIdx.x >> 3;
+  const int q8 = nb >> 3, r8 = nb & 7;
+  const int lid = xcd * q8 + min(xcd, r8) + within;
+  const int tm = lid % mt, tn = tn0 + lid / mt;
+  const int sbeg = blockIdx.y * part_slabs, ns = min(nslab, sbeg + part_slabs) - sbeg;
+  C += (size_t)blockIdx.y * M * ldc;
+
+  // this wavefront's share of a slab copy: TM KB of each plane of A (TM = 1: of the half image
+  // that holds this block's rows), two of the 16 KB of W
+  const int img = TM == 2 ? tm : tm >> 1, half = TM == 2 ? 0 : (tm & 1) * kAPlane;
+  const char* asrc = Aimg + ((size_t)img * nslab + sbeg) * kAImage + half + (wave * TM) * 1024 + lane * 16;
+  const char* wsrc = Wimg + ((size_t)tn * nslab + sbeg) * kWImage + (wave * 2) * 1024 + lane * 16;
+  auto issue = [&](int slab, int stage) {   // past the end: the last slab again, into a stage nobody reads
+    const int s = min(slab, ns - 1);
+    char* base = ring + stage * kStage;
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+      for (int j = 0; j < TM; j++)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(asrc + (size_t)s * kAImage + p * kPlaneBytes + j * 1024),
+            (__attribute__((address_space(3))) void*)(base + p * kAPlane + (wave * TM + j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (size_t)s * kWImage + j * 1024),
+                                       (__attribute__((address_space(3))) void*)(base + 2 * kAPlane + (wave * 2 + j) * 1024), 16, 0, 0);
+  };
+
+  f32x16 acc[TM][4];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  // this lane's first fragment of A (hi plane, tile row 0) and of W (tile column 0) within a
+  // stage, per 16-k step; the other fragments are constant offsets from these
+  int aoff[2], boff[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) {
+    const int kc = ks * 2 + (lane >> 5);
+    aoff[ks] = image_off(wm * 32 * TM + (lane & 31), kc);
+    boff[ks] = 2 * kAPlane + image_off(wn * 128 + (lane & 31), kc);
+  }
+  // fragment sets: F[0] for the first 16 k of a slab, F[1] for the second
+  frag16 af[2][TM][2], bf[2][4];
+  auto fetch = [&](const char* stage, auto KS) {
+    constexpr int ks = decltype(KS)::value;
+#pragma unroll
+    for (int j = 0; j < 4; j++) bf[ks][j] = *reinterpret_cast<const frag16*>(stage + boff[ks] + j * 32 * kRowBytes);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int p = 0; p < 2; p++)
+        af[ks][i][p] = *reinterpret_cast<const frag16*>(stage + aoff[ks] + p * kAPlane + i * 32 * kRowBytes);
+  };
+  // one half of the products of fragment set KS: TM of its 2 * TM (tile row, plane) pairs, 4 MFMAs each
+  auto mul = [&](auto KS, auto HALF) {
+    constexpr int ks = decltype(KS)::value, h = decltype(HALF)::value;
+#pragma unroll
+    for (int q = h * TM; q < (h + 1) * TM; q++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        acc[q >> 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[ks][q >> 1][q & 1]),
+                                                                __builtin_bit_cast(f16x8, bf[ks][j]), acc[q >> 1][j], 0, 0, 0);
+  };
+  // The block's barrier without the fence __syncthreads() puts before it: that fence would wait for
+  // EVERY copy in flight (they write LDS). What has to be complete is waited for by count instead.
+  auto barrier = [] {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  // Three slabs in flight. Invariant at the top of iteration k: slab k has landed in stage k % 3
+  // for every wavefront and its first fragment set is on its way to registers; slabs k + 1 and
+  // k + 2 are being copied.
+  issue(0, 0);
+  issue(1, 1);
+  issue(2, 2);
+#ifdef TLHIP_TRACE
+  unsigned long long ph[2] = {0, 0}, tc = __builtin_readcyclecounter();
+  TLHIP_MARK(0);
+#define TLHIP_PHASE(i) do { const unsigned long long n_ = __builtin_readcyclecounter(); ph[i] += n_ - tc; tc = n_; } while (0)
+#else
+#define TLHIP_PHASE(i)
+#endif
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kCopies) : "memory");   // my copies of slab 0
+  barrier();
+  fetch(ring, Idx<0>{});
+  TLHIP_MARK(1);
+  // A fragment set is requested half a set of MFMAs before the set that uses it starts, and
+  // nothing younger is outstanding when it is waited for.
+  int st = 0;
+  for (int k = 0; k < ns; k++) {
+    const char* stage = ring + st * kStage;
+    const int nx = st == 2 ? 0 : st + 1;
+    mul(Idx<0>{}, Idx<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(stage, Idx<1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mul(Idx<0>{}, Idx<1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    TLHIP_PHASE(0);
+    // my reads of slab k are complete and my copies of slab k + 1 have landed (those of slab
+    // k + 2 may still be in flight); past the barrier that holds for every wavefront
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
+    barrier();
+    TLHIP_PHASE(1);
+    issue(k + 3, st);                                  // into the stage slab k has just left
+    __builtin_amdgcn_sched_barrier(0);
+    mul(Idx<1>{}, Idx<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (k + 1 < ns) fetch(ring + nx * kStage, Idx<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mul(Idx<1>{}, Idx<1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    st = nx;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the copies past the end
+#ifdef TLHIP_TRACE
+  {
+    const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (lane == 0 && b < kTraceBlocks) {
+      unsigned long long* g = &g_trace[(b * kTraceWaves + wave) * kTraceSlots];
+      g[2] = ph[0]; g[3] = ph[1]; g[7] = ns;
+    }
+  }
+  TLHIP_MARK(5);
+#endif
+#undef TLHIP_PHASE
+
+  // acc[v] of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32x32 tile. The exponents
+  // come back out, -(ea[row] + ew[W row of the column]); ldexpf is exact.
+  int ec[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int r = weight_row(GU, tn, wn * 128 + j * 32 + (lane & 31), N + (GU ? tn0 * 128 : tn0 * kTile), ff);
+    ec[j] = r >= 0 ? (int)ew[r] : 0;
+  }
+  const int ltn = tn - tn0;                          // column tile within this launch
+  if (GU && gridDim.y == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int gm = tm * BM + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (gm >= M) continue;
+        const int em = ea[gm];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const int f = ltn * 128 + wn * 64 + j * 32 + (lane & 31);
+          if (f >= N) continue;
+          const float g = ldexpf(acc[i][j][v], -(em + ec[j])), sg = 1.0f / (1.0f + expf(-g));
+          C[(size_t)gm * ldc + f] = (g * sg) * ldexpf(acc[i][j + 2][v], -(em + ec[j + 2]));
+        }
+      }
+    TLHIP_MARK(6);
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int gm = tm * BM + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+      if (gm >= M) continue;
+      const int em = ea[gm];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int gn = ltn * kTile + wn * 128 + j * 32 + (lane & 31);
+        if (!GU && gn >= N) continue;   // gated parts are whole tiles wide
+        C[(size_t)gm * ldc + gn] = ldexpf(acc[i][j][v], -(em + ec[j]));
+      }
+    }
+  TLHIP_MARK(6);
+}
+
+}  // namespace f16t
+}  // namespace tlhip
+
+using namespace tlhip;
+
+namespace {
+
+int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// plain: C[M][N]; parts (S_out != nullptr): C is the caller's [S][M][N]; gated: N = features, C[M][N] the activation
+int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N, int64_t K,
+                   size_t parts_bytes, int* S_out, bool gu) {
+  TLHIP_REQUIRE_READY();
+  const bool want_parts = S_out != nullptr;
+  if (!A || !image || !exps || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt: null pointer");
+  if (M <= 0 || N <= 0 || K <= 0 || (K % f16t::kBK) != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: need positive M, N, K and K %% 32 == 0");
+  if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: dimension too large");
+  if (!aligned16(A) || !aligned16(image) || !aligned16(C))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt: operands must be 16-byte aligned");
+  Context& c = ctx();
+  const int per = gu ? 2 : 1;                       // tile columns per unit of N
+  const int64_t w = f16t::kTile / per;              // units of N per column tile
+  const int64_t nslab = K / f16t::kBK, tn = cdiv64(N, w);
+  const int64_t slots = c.cus;                      // one block per CU
+  // 256-row tiles unless they leave more than half of the CUs to K splits; then 128-row tiles
+  const int tmh = (cdiv64(M, 256) * tn * 2 <= slots) ? 1 : 2;
+  const int64_t bm = 128 * tmh, tm = cdiv64(M, bm), tiles = tm * tn;
+  const bool can_split = (N % 4) == 0;              // the part sums work on float4s
+  // Work is shaped to whole rounds of the block slots, as in tlhip_gemm_bf16_nt: fewer tiles than
+  // slots -> K split so that tiles * S comes close to the slots; more -> the columns that make
+  // whole rounds with full K, the remaining columns split over K in a second launch.
+  struct Piece { int64_t tn0, tcols; int S; };
+  Piece pieces[2];
+  int npieces = 0;
+  auto pick_S = [&](int64_t t) {
+    if (!can_split || t >= slots) return 1;
+    int64_t S = slots / t;
+    if (S > 16) S = 16;
+    while (S > 1 && nslab / S < 8) S--;             // at least 256 k per part
+    if (want_parts)
+      while (S > 1 && (size_t)S * M * N * sizeof(float) > parts_bytes) S--;
+    return (int)S;
+  };
+  const int64_t cols_per_round = slots / tm;
+  if (tiles <= slots || cols_per_round == 0 || !can_split || want_parts) {
+    pieces[npieces++] = Piece{0, tn, pick_S(tiles)};
+  } else {
+    const int64_t main_tn = tn / cols_per_round * cols_per_round;
+    pieces[npieces++] = Piece{0, main_tn, 1};
+    if (main_tn < tn) pieces[npieces++] = Piece{main_tn, tn - main_tn, pick_S(tm * (tn - main_tn))};
+  }
+  // scratch: exponents of A's rows, the slab images of A, room for the largest piece's parts
+  const size_t ea_bytes = ((size_t)M * sizeof(int) + 1023) & ~(size_t)1023;
+  const int64_t timg = cdiv64(M, f16t::kTile);      // activation images are 256 rows tall
+  const size_t aimg_bytes = (size_t)timg * nslab * f16t::kAImage;
+  size_t parts_need = 0;
+  if (!want_parts)
+    for (int pi = 0; pi < npieces; pi++)
+      if (pieces[pi].S > 1) {
+        const int64_t part_w = gu ? pieces[pi].tcols * f16t::kTile : std::min<int64_t>(pieces[pi].tcols * w, N - pieces[pi].tn0 * w);
+        parts_need = std::max(parts_need, (size_t)pieces[pi].S * M * part_w * sizeof(float));
+      }
+  char* sbase = static_cast<char*>(scratch(ea_bytes + aimg_bytes + parts_need));
+  if (!sbase) return fail(TLHIP_ENOMEM, "tlhip_gemm_f16w_nt: no scratch for the activation planes and K-split parts");
+  int* ea = reinterpret_cast<int*>(sbase);
+  char* aimg = sbase + ea_bytes;
+  const float* pa = static_cast<const float*>(A);
+  row_exponent_f32_kernel<<<dim3((unsigned)M), dim3(256), 0, c.stream>>>(pa, (int)K, ea);
+  f16t::a_image_kernel<<<dim3((unsigned)timg, (unsigned)nslab), dim3(256), 0, c.stream>>>(pa, ea, aimg, (int)M, (int)K);
+  const size_t lds = (size_t)f16t::kRing * (2 * bm * f16t::kRowBytes + f16t::kWImage);
+  float* pc = static_cast<float*>(C);
+  for (int pi = 0; pi < npieces; pi++) {
+    const Piece& P = pieces[pi];
+    const int64_t n0 = P.tn0 * w, pn = std::min<int64_t>(P.tcols * w, N - n0);   // units of N in this piece
+    const int64_t part_w = gu ? P.tcols * f16t::kTile : pn;
+    int S = P.S, part_slabs = (int)nslab;
+    float* dst = pc + n0;
+    int ldc = (int)N;
+    if (S > 1) {
+      part_slabs = (int)cdiv64(nslab, S);
+      S = (int)cdiv64(nslab, part_slabs);
+    }
+    if (want_parts) {
+      *S_out = S;
+      dst = pc;
+    } else if (S > 1) {
+      dst = reinterpret_cast<float*>(sbase + ea_bytes + aimg_bytes);
+      ldc = (int)part_w;
+    }
+    const int64_t nblk = tm * P.tcols;
+    if (nblk > 0x7fffffff || part_w > 0x7fffffff)
+      return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: too many tiles for one grid");
+    const dim3 grid((unsigned)nblk, (unsigned)S);
+    auto launch = [&](auto fn) -> hipError_t {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      fn<<<grid, dim3(512), lds, c.stream>>>(aimg, static_cast<const char*>(image), dst, (int)M, (int)pn, (int)nslab,
+                                             part_slabs, ldc, (int)P.tn0, (int)N, ea, static_cast<const int8_t*>(exps));
+      return hipSuccess;
+    };
+    const hipError_t e = tmh == 2 ? (gu ? launch(f16t::gemm_f16t_kernel<2, true>) : launch(f16t::gemm_f16t_kernel<2, false>))
+                                  : (gu ? launch(f16t::gemm_f16t_kernel<1, true>) : launch(f16t::gemm_f16t_kernel<1, false>));
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
+    if (S > 1 && !want_parts) {
+      const size_t total4 = (size_t)M * pn / 4;
+      const dim3 sgrid((unsigned)((total4 + 255) / 256));
+      if (gu)
+        splitk_sum_swiglu_kernel<<<sgrid, dim3(256), 0, c.stream>>>(
+            reinterpret_cast<const float4*>(dst), reinterpret_cast<float4*>(pc + n0), (int)M, (int)(pn / 4),
+            (int)(part_w / 4), (int)(N / 4), S, 64 / 4);
+      else
+        splitk_sum_kernel<<<sgrid, dim3(256), 0, c.stream>>>(reinterpret_cast<const float4*>(dst),
+                                                              reinterpret_cast<float4*>(pc + n0), (int)M,
+                                                              (int)(pn / 4), (int)(N / 4), S);
+    }
+  }
+  TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t tlhip_gemm_f16w_bytes(int64_t N, int64_t K, int gated) {
+  if (N <= 0 || K <= 0 || (K % f16t::kBK) != 0) return 0;
+  const int64_t tn = cdiv64(N, gated ? 128 : f16t::kTile);
+  return tn * (K / f16t::kBK) * f16t::kWImage;
+}
+
+int tlhip_gemm_f16w_prepare(const void* W, int64_t N, int64_t K, int gated, void* image, void* exps) {
+  TLHIP_REQUIRE_READY();
+  if (!W || !image || !exps) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_prepare: null pointer");
+  const int64_t rows = gated ? 2 * N : N;
+  if (N <= 0 || K <= 0 || (K % f16t::kBK) != 0 || rows > 0x7fffffff || K > 0x3fffffff)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_prepare: need positive N, K and K %% 32 == 0");
+  if (!aligned16(W) || !aligned16(image))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_prepare: weight and image must be 16-byte aligned");
+  Context& c = ctx();
+  const uint16_t* pw = static_cast<const uint16_t*>(W);
+  int8_t* pe = static_cast<int8_t*>(exps);
+  row_exponent_bf16_kernel<<<dim3((unsigned)rows), dim3(256), 0, c.stream>>>(pw, (int)K, pe);
+  const int64_t tn = cdiv64(N, gated ? 128 : f16t::kTile), nslab = K / f16t::kBK;
+  if (tn > 0x7fffffff || nslab > 65535)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_prepare: weight too large for one grid");
+  f16t::w_image_kernel<<<dim3((unsigned)tn, (unsigned)nslab), dim3(256), 0, c.stream>>>(
+      pw, pe, static_cast<char*>(image), (int)N, (int)K, (int)N, gated ? 1 : 0);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
+}
+
+int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N,
+                       int64_t K) {
+  return gemm_f16w_impl(A, image, exps, C, M, N, K, 0, nullptr, false);
+}
+
+int tlhip_gemm_f16w_nt_swiglu(const void* A, const void* image, const void* exps, void* act, int64_t M,
+                              int64_t ff, int64_t K) {
+  return gemm_f16w_impl(A, image, exps, act, M, ff, K, 0, nullptr, true);
+}
+
+int tlhip_gemm_f16w_nt_parts(const void* A, const void* image, const void* exps, void* parts,
+                             int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int* n_parts) {
+  if (!n_parts) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_parts: null n_parts");
+  if (M > 0 && N > 0 && parts_bytes < (int64_t)(M * N * sizeof(float)))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_parts: the buffer must hold at least one [M, N] part");
+  *n_parts = 0;
+  return gemm_f16w_impl(A, image, exps, parts, M, N, K, (size_t)parts_bytes, n_parts, false);
+}
+
+}  // extern "C"

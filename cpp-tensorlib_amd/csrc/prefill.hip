@@ -19,12 +19,11 @@
 // W is [N,K]), which is exactly the MFMA operand layout: one ds_read_b128 per
 // fragment. Global loads of the next slab are in flight while the current one is
 // multiplied.
-#include "common.hpp"
+#include "gemm_shared.hpp"
 
 namespace tlhip {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kBK = 32;        // K slab: an LDS row is 32 bf16 = four 16-byte chunks
 
@@ -57,12 +56,22 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {   // in bf16 elemen
 // arithmetic on the matrix pipe. The second set holds one row block of MFMA tiles at a time; with
 // it, 64-column wavefront tiles (TN = 2) fit the registers, 128-column ones spill (and then run
 // at half the speed).
-template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false, bool Q4 = false>
+//
+// H = true (int4 weights): the operands go to the matrix cores as f16 instead. Row m of A is first
+// multiplied by 2^ea[m], which brings its largest magnitude into [2^14, 2^15), and then cut into
+// TWO f16 terms, both rounded to nearest: a * 2^ea = hi + lo + r with |r| <= 2^-24 |a * 2^ea|
+// wherever lo is a normal f16 (and <= 2^-25 absolute, 2^-39 of the row's largest, where it is not)
+// - the accuracy of one fp32 rounding, from two MFMAs per product instead of three. The nibbles
+// are small integers, exact in f16; the result leaves as acc * 2^-ea[m], an exact scaling.
+template <int TM, int TN, int WM = 2, int WN = 2, bool GU = false, bool Q4 = false, bool H = false>
 __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const float* __restrict__ A,
                                                            const uint16_t* __restrict__ W,
                                                            float* __restrict__ C, int M, int N,
                                                            int K, int kchunk, int ldc, int ff,
-                                                           const float* __restrict__ scales) {
+                                                           const float* __restrict__ scales,
+                                                           const int* __restrict__ ea) {
+  static_assert(!H || Q4, "f16 planes here are for int4 weights; prepared bf16 weights have their own kernel");
+  constexpr int PL = H ? 2 : 3;                 // planes of A
   static_assert(!GU || TN % 2 == 0, "gate and up accumulators of a feature must share a lane");
   static_assert(!Q4 || ((32 * TN * WN == 128 || 32 * TN * WN == 256) && 64 * WM * WN == 256),
                 "int4 slab copy: one or two threads per tile column");
@@ -73,7 +82,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
   constexpr int A_LOADS = BM * kBK / 4 / NT;    // float4 per thread per slab
   constexpr int B_LOADS = BN * kBK / 8 / NT;    // uint4 (8 bf16) per thread per slab
   static_assert(A_LOADS >= 1 && B_LOADS >= 1 && BM * kBK / 4 % NT == 0 && BN * kBK / 8 % NT == 0, "tile vs threads");
-  __shared__ __attribute__((aligned(16))) uint16_t As[3][BM * kBK];
+  __shared__ __attribute__((aligned(16))) uint16_t As[PL][BM * kBK];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * kBK];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -110,6 +119,15 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     }
     return n0 + col < N ? n0 + col : -1;
   };
+  // H: 2^exponent of the rows of A this thread copies (the same rows in every slab)
+  float sa[H ? A_LOADS : 1];
+  if (H) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) {
+      const int gm = m0 + ((tid + i * NT) >> 3);
+      sa[i] = gm < M ? pow2f(ea[gm]) : 1.0f;
+    }
+  }
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
@@ -152,6 +170,17 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     }
     return o;
   };
+  auto nib8h = [](uint32_t w) {   // the same as f16
+    const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;
+    uint4 o;
+    uint32_t* po = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      const f32x2 x = {(float)((lo >> (8 * b)) & 0xffu) - 8.0f, (float)((hi >> (8 * b)) & 0xffu) - 8.0f};
+      po[b] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+    }
+    return o;
+  };
   auto split3 = [](float a, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
     const uint32_t h = __float_as_uint(a) & 0xffff0000u;
     const float r1 = a - __uint_as_float(h);            // exact
@@ -165,6 +194,16 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
+      if (H) {
+        uint32_t h01, l01, h23, l23;
+        const float s = sa[H ? i : 0];
+        split2_f16(ra[i].x * s, ra[i].y * s, h01, l01);
+        split2_f16(ra[i].z * s, ra[i].w * s, h23, l23);
+        const int o = lds_off(row, c4 >> 1) + (c4 & 1) * 4;
+        *reinterpret_cast<uint2*>(&As[0][o]) = make_uint2(h01, h23);
+        *reinterpret_cast<uint2*>(&As[1][o]) = make_uint2(l01, l23);
+        continue;
+      }
       uint32_t h[4], m[4], l[4];
       split3(ra[i].x, h[0], m[0], l[0]);
       split3(ra[i].y, h[1], m[1], l[1]);
@@ -173,12 +212,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       const int o = lds_off(row, c4 >> 1) + (c4 & 1) * 4;
       *reinterpret_cast<uint2*>(&As[0][o]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
       *reinterpret_cast<uint2*>(&As[1][o]) = make_uint2(m[0] | (m[1] << 16), m[2] | (m[3] << 16));
-      *reinterpret_cast<uint2*>(&As[2][o]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
+      *reinterpret_cast<uint2*>(&As[PL - 1][o]) = make_uint2(l[0] | (l[1] << 16), l[2] | (l[3] << 16));
     }
     if (Q4) {
       const int row = tid / TPC, c8 = (tid % TPC) * (4 / TPC);
 #pragma unroll
-      for (int u = 0; u < 4 / TPC; u++) *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + u)]) = nib8(rq[u]);
+      for (int u = 0; u < 4 / TPC; u++) *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + u)]) = H ? nib8h(rq[u]) : nib8(rq[u]);
 #pragma unroll
       for (int j = 0; j < TN; j++) sc[j] = sc_next[j];
     } else {
@@ -190,11 +229,32 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     }
   };
 
+  // one 32x32x16 product step on two 16-byte fragments
+  auto mma = [](frag16 a, frag16 b, f32x16 c) {
+    if (H)
+      return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  };
   gload(kbeg);
+#ifdef TLHIP_TRACE
+  unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, tc = __builtin_readcyclecounter();
+  TLHIP_MARK(0);
+#define TLHIP_PHASE(i) do { const unsigned long long n_ = __builtin_readcyclecounter(); ph[i] += n_ - tc; tc = n_; } while (0)
+#else
+#define TLHIP_PHASE(i)
+#endif
   for (int k0 = kbeg; k0 < kend; k0 += kBK) {
+    TLHIP_PHASE(4);           // products of the slab before
     __syncthreads();          // the previous slab has been consumed
+    TLHIP_PHASE(0);
+#ifdef TLHIP_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    TLHIP_PHASE(1);
+#endif
     lstore();
+    TLHIP_PHASE(2);
     __syncthreads();
+    TLHIP_PHASE(3);
     if (k0 + kBK < kend) gload(k0 + kBK);
     if (Q4) {
       // one row block of MFMA tiles at a time: its sums over this slab (= this scale group) in a
@@ -210,16 +270,16 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ks++) {
           const int kc = ks * 2 + (lane >> 5);
-          bf16x8 bfrag[TN];
+          frag16 bfrag[TN];
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            bfrag[j] = *reinterpret_cast<const bf16x8*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
+            bfrag[j] = *reinterpret_cast<const frag16*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
 #pragma unroll
-          for (int p = 0; p < 3; p++) {
-            const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
+          for (int p = 0; p < PL; p++) {
+            const frag16 afrag = *reinterpret_cast<const frag16*>(&As[p][lds_off(row, kc)]);
 #pragma unroll
             for (int j = 0; j < TN; j++)
-              grp[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], grp[j], 0, 0, 0);
+              grp[j] = mma(afrag, bfrag[j], grp[j]);
           }
         }
 #pragma unroll
@@ -232,38 +292,54 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ks++) {
       const int kc = ks * 2 + (lane >> 5);   // 16-byte chunk of the slab this lane multiplies
-      bf16x8 bfrag[TN];
+      frag16 bfrag[TN];
 #pragma unroll
       for (int j = 0; j < TN; j++)
-        bfrag[j] = *reinterpret_cast<const bf16x8*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
+        bfrag[j] = *reinterpret_cast<const frag16*>(&Bs[lds_off(wn * 32 * TN + j * 32 + (lane & 31), kc)]);
 #pragma unroll
       for (int i = 0; i < TM; i++) {
         const int row = wm * 32 * TM + i * 32 + (lane & 31);
 #pragma unroll
-        for (int p = 0; p < 3; p++) {
-          const bf16x8 afrag = *reinterpret_cast<const bf16x8*>(&As[p][lds_off(row, kc)]);
+        for (int p = 0; p < PL; p++) {
+          const frag16 afrag = *reinterpret_cast<const frag16*>(&As[p][lds_off(row, kc)]);
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag, bfrag[j], acc[i][j], 0, 0, 0);
+            acc[i][j] = mma(afrag, bfrag[j], acc[i][j]);
         }
       }
     }
   }
 
-  // acc[v] of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32x32 tile
+#ifdef TLHIP_TRACE
+  {
+    TLHIP_PHASE(4);
+    const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (lane == 0 && b < kTraceBlocks) {
+      unsigned long long* g = &g_trace[(b * kTraceWaves + wave) * kTraceSlots];
+      g[1] = ph[0]; g[2] = ph[1]; g[3] = ph[2]; g[4] = ph[3]; g[5] = ph[4]; g[7] = (kend - kbeg + kBK - 1) / kBK;
+    }
+  }
+  TLHIP_MARK(6);
+#endif
+#undef TLHIP_PHASE
+  // acc[v] of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32x32 tile.
+  // H: the exponent of the row comes back out; ldexpf is exact.
+  auto out = [&](float x, int e) { return H ? ldexpf(x, -e) : x; };
   if (GU && gridDim.y == 1) {
     // act = (g * sigmoid(g)) * u, the arithmetic of swiglu_kernel (array.h:2435-2439)
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < TN / 2; j++) {
-        const int f = (n0 >> 1) + wn * HW + j * 32 + (lane & 31);
-        if (f >= N) continue;
+      for (int v = 0; v < 16; v++) {
+        const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (gm >= M) continue;
+        const int em = H ? ea[gm] : 0;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-          const float g = acc[i][j][v], sg = 1.0f / (1.0f + expf(-g));
-          if (gm < M) C[(size_t)gm * ldc + f] = (g * sg) * acc[i][j + TN / 2][v];
+        for (int j = 0; j < TN / 2; j++) {
+          const int f = (n0 >> 1) + wn * HW + j * 32 + (lane & 31);
+          if (f >= N) continue;
+          const float g = out(acc[i][j][v], em), sg = 1.0f / (1.0f + expf(-g));
+          C[(size_t)gm * ldc + f] = (g * sg) * out(acc[i][j + TN / 2][v], em);
         }
       }
     return;
@@ -271,15 +347,68 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const int gn = n0 + wn * 32 * TN + j * 32 + (lane & 31);
-      if (!GU && gn >= N) continue;   // GU parts are whole tiles wide
+    for (int v = 0; v < 16; v++) {
+      const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+      if (gm >= M) continue;
+      const int em = H ? ea[gm] : 0;
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int gm = m0 + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (gm < M) C[(size_t)gm * ldc + gn] = acc[i][j][v];
+      for (int j = 0; j < TN; j++) {
+        const int gn = n0 + wn * 32 * TN + j * 32 + (lane & 31);
+        if (!GU && gn >= N) continue;   // GU parts are whole tiles wide
+        C[(size_t)gm * ldc + gn] = out(acc[i][j][v], em);
       }
     }
+}
+
+// Exponent that brings the largest magnitude of a row into [2^14, 2^15): 14 - floor(log2(max)),
+// kept within [-126, 126] so that 2^e is a normal float; 0 for a row of zeros. `field` is the
+// biased exponent field of the row's largest magnitude (255 for inf / NaN: they stay what they are).
+__device__ __forceinline__ int row_exponent(int field, bool all_zero) {
+  return all_zero ? 0 : max(-126, min(126, 14 - (field - 127)));
+}
+
+// ea[m] for the rows of an f32 matrix [M][K] (K % 4 == 0, rows 16-byte aligned). One block per row.
+__global__ __launch_bounds__(256) void row_exponent_f32_kernel(const float* __restrict__ A, int K,
+                                                               int* __restrict__ ea) {
+  __shared__ uint32_t part[4];
+  const uint4* row = reinterpret_cast<const uint4*>(A + (size_t)blockIdx.x * K);
+  uint32_t mx = 0;
+  for (int i = threadIdx.x; i < K / 4; i += 256) {
+    const uint4 v = row[i];
+    mx = max(max(mx, v.x & 0x7fffffffu), max(max(v.y & 0x7fffffffu, v.z & 0x7fffffffu), v.w & 0x7fffffffu));
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, d));
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mx = max(max(part[0], part[1]), max(part[2], part[3]));
+    ea[blockIdx.x] = row_exponent((int)(mx >> 23), mx == 0);
+  }
+}
+
+// ew[n] for the rows of a bf16 matrix [N][K] (K % 8 == 0, rows 16-byte aligned). One block per row.
+__global__ __launch_bounds__(256) void row_exponent_bf16_kernel(const uint16_t* __restrict__ W, int K,
+                                                                int8_t* __restrict__ ew) {
+  __shared__ uint32_t part[4];
+  const uint4* row = reinterpret_cast<const uint4*>(W + (size_t)blockIdx.x * K);
+  uint32_t mx = 0;   // two 15-bit magnitudes, compared half by half
+  auto both = [](uint32_t a, uint32_t b) {
+    return max(a & 0x7fff0000u, b & 0x7fff0000u) | max(a & 0x7fffu, b & 0x7fffu);
+  };
+  for (int i = threadIdx.x; i < K / 8; i += 256) {
+    const uint4 v = row[i];
+    mx = both(both(mx, v.x), both(both(v.y, v.z), v.w));
+  }
+  mx = max(mx >> 16, mx & 0x7fffu);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, d));
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mx = max(max(part[0], part[1]), max(part[2], part[3]));
+    ew[blockIdx.x] = (int8_t)row_exponent((int)(mx >> 7), mx == 0);
+  }
 }
 
 // C[m][n] = sum_s part[s][m][n], s in ascending order. Parts are dense [M][n4 * 4]; C rows
@@ -337,6 +466,8 @@ extern "C" {
 //   gu: W = [gate rows | up rows], N = features (rows of each), C[M][N] = the gated activation.
 //   scales != nullptr: W is an int4 weight (packed nibbles [rows][K/2], scales [rows][K/32]); any of
 //     the three forms above.
+//     Prompt chunks (M > 64) of an int4 weight run on two f16 planes of A instead of three bf16
+//     ones (the nibbles are exact in either format); the exponents of A's rows are taken here.
 static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, int64_t N, int64_t K,
                              size_t parts_bytes, int* S_out, bool gu, const void* scales = nullptr) {
   TLHIP_REQUIRE_READY();
@@ -369,6 +500,8 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
   const int64_t slots = (int64_t)c.cus * 2;
   const int per = gu ? 2 : 1;                             // tile columns per unit of N
   const bool can_split = (N % 4) == 0 && aligned16(C);   // the part sum works on float4s
+  const bool half = q4 && M > 64 && c.tune_gemm_planes != 3;
+  const size_t ea_bytes = half ? (((size_t)M * sizeof(int) + 255) & ~(size_t)255) : 0;
   struct Piece { int64_t n0, n; int S; int variant; };    // columns (features) [n0, n0 + n)
   Piece pieces[2];
   int npieces = 0;
@@ -402,9 +535,26 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
     if (gu || q4 || t128 >= slots || pick_S(t128) > 1) pieces[npieces++] = Piece{0, N, pick_S(t128), 1};
     else pieces[npieces++] = Piece{0, N, pick_S(t64), 2};
   }
+  static const int kBm[4] = {128, 64, 64, 128}, kBn[4] = {256, 128, 64, 128};
+  // One scratch request for the whole call (a second, larger one could move the buffer): the
+  // exponents of A's rows first, then room for the largest piece's K-split parts.
+  size_t parts_need = 0;
+  if (!want_parts)
+    for (int pi = 0; pi < npieces; pi++) {
+      const Piece& P = pieces[pi];
+      const int bn = kBn[P.variant];
+      const int64_t part_w = gu ? cdiv(P.n, bn / per) * bn : P.n;
+      if (P.S > 1) parts_need = std::max(parts_need, (size_t)P.S * M * part_w * sizeof(float));
+    }
+  char* sbase = nullptr;
+  if (ea_bytes + parts_need > 0) {
+    sbase = static_cast<char*>(scratch(ea_bytes + parts_need));
+    if (!sbase) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for row exponents and K-split parts");
+  }
+  int* ea = reinterpret_cast<int*>(sbase);
+  if (half) row_exponent_f32_kernel<<<dim3((unsigned)M), dim3(256), 0, c.stream>>>(pa, (int)K, ea);
   for (int pi = 0; pi < npieces; pi++) {
     const Piece& P = pieces[pi];
-    static const int kBm[4] = {128, 64, 64, 128}, kBn[4] = {256, 128, 64, 128};
     const int bm = kBm[P.variant], bn = kBn[P.variant];
     const int64_t tcols = cdiv(P.n, bn / per);            // tile columns of this piece
     const int64_t part_w = gu ? tcols * bn : P.n;         // row width of a K-split part
@@ -419,8 +569,7 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
       *S_out = S;             // one piece: dst is the caller's parts, [S][M][N]
       if (S == 1) kchunk = (int)K;
     } else if (S > 1) {
-      dst = static_cast<float*>(scratch((size_t)S * M * part_w * sizeof(float)));
-      if (!dst) return fail(TLHIP_ENOMEM, "tlhip_gemm_bf16_nt: no scratch for %d K-splits", S);
+      dst = reinterpret_cast<float*>(sbase + ea_bytes);
       ldc = (int)part_w;
     } else {
       kchunk = (int)K;
@@ -433,19 +582,21 @@ static int gemm_bf16_nt_impl(const void* A, const void* W, void* C, int64_t M, i
     const uint16_t* wp = q4 ? reinterpret_cast<const uint16_t*>(static_cast<const uint8_t*>(W) + (size_t)P.n0 * K / 2)
                             : pw + (size_t)P.n0 * K;
     const float* sp = q4 ? static_cast<const float*>(scales) + (size_t)P.n0 * (K / 32) : nullptr;
-#define TLHIP_GEMM(TM_, TN_, GU_, Q4_)                                                         \
-  gemm_bf16_nt_kernel<TM_, TN_, 2, 2, GU_, Q4_><<<grid, dim3(256), 0, c.stream>>>(             \
-      pa, wp, dst, (int)M, (int)P.n, (int)K, kchunk, ldc, (int)N, sp)
-    switch (P.variant + (gu ? 4 : 0) + (q4 ? 8 : 0)) {
-      case 0: TLHIP_GEMM(2, 4, false, false); break;
-      case 1: TLHIP_GEMM(1, 2, false, false); break;
-      case 2: TLHIP_GEMM(1, 1, false, false); break;
-      case 4: TLHIP_GEMM(2, 4, true, false); break;
-      case 5: TLHIP_GEMM(1, 2, true, false); break;
-      case 9: TLHIP_GEMM(1, 2, false, true); break;
-      case 11: TLHIP_GEMM(2, 2, false, true); break;
-      case 13: TLHIP_GEMM(1, 2, true, true); break;
-      case 15: TLHIP_GEMM(2, 2, true, true); break;
+#define TLHIP_GEMM(TM_, TN_, GU_, Q4_, H_)                                                     \
+  gemm_bf16_nt_kernel<TM_, TN_, 2, 2, GU_, Q4_, H_><<<grid, dim3(256), 0, c.stream>>>(         \
+      pa, wp, dst, (int)M, (int)P.n, (int)K, kchunk, ldc, (int)N, sp, ea)
+    switch (P.variant + (gu ? 4 : 0) + (q4 ? 8 : 0) + (half ? 16 : 0)) {
+      case 0: TLHIP_GEMM(2, 4, false, false, false); break;
+      case 1: TLHIP_GEMM(1, 2, false, false, false); break;
+      case 2: TLHIP_GEMM(1, 1, false, false, false); break;
+      case 4: TLHIP_GEMM(2, 4, true, false, false); break;
+      case 5: TLHIP_GEMM(1, 2, true, false, false); break;
+      case 9: TLHIP_GEMM(1, 2, false, true, false); break;
+      case 11: TLHIP_GEMM(2, 2, false, true, false); break;
+      case 13: TLHIP_GEMM(1, 2, true, true, false); break;
+      case 15: TLHIP_GEMM(2, 2, true, true, false); break;
+      case 27: TLHIP_GEMM(2, 2, false, true, true); break;
+      case 31: TLHIP_GEMM(2, 2, true, true, true); break;
       default: return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_bf16_nt: no kernel for this plan");
     }
 #undef TLHIP_GEMM

@@ -355,6 +355,7 @@ int tlhip_tune_reset(void) {
   c.tune_q4_rows = c.tune_q4_kw = c.tune_q4_bpc = c.tune_q4_nw = c.tune_q4_lpr = 0;
   c.tune_cols_max_splits = 0;
   c.tune_prefill_valu = 0;
+  c.tune_gemm_planes = 0;
   return TLHIP_OK;
 }
 
@@ -367,6 +368,13 @@ int tlhip_tune_attn_prefill(int valu_kernel) {
   TLHIP_REQUIRE_READY();
   if (valu_kernel < 0 || valu_kernel > 3) return fail(TLHIP_EINVAL, "tlhip_tune_attn_prefill: 0 (built-in choice) .. 3");
   ctx().tune_prefill_valu = valu_kernel;
+  return 0;
+}
+
+int tlhip_tune_gemm_planes(int planes) {
+  TLHIP_REQUIRE_READY();
+  if (planes != 0 && planes != 3) return fail(TLHIP_EINVAL, "tlhip_tune_gemm_planes: 0 (built-in choice) or 3");
+  ctx().tune_gemm_planes = planes;
   return 0;
 }
 

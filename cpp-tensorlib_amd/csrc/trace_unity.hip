@@ -12,6 +12,7 @@
 #include "attn_prefill_mfma.hip"
 #include "attn_prefill_x3.hip"
 #include "prefill.hip"
+#include "gemm_f16t.hip"
 #include "convert.hip"
 #include "sgemm.hip"
 

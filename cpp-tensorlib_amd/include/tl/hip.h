@@ -112,6 +112,12 @@ struct api {
   int (*gemm_q4_nt_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
                            int64_t) = nullptr;
   int (*gemm_bf16_nt_swiglu)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int64_t (*gemm_f16w_bytes)(int64_t, int64_t, int) = nullptr;
+  int (*gemm_f16w_prepare)(const void*, int64_t, int64_t, int, void*, void*) = nullptr;
+  int (*gemm_f16w_nt)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
+  int (*gemm_f16w_nt_parts)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
+                            int*) = nullptr;
+  int (*gemm_f16w_nt_swiglu)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*gemm_bf16_nt_parts)(const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
                             int*) = nullptr;
   int (*rmsnorm_res_parts)(const void*, const void*, int64_t, const void*, void*, void*, int64_t, float,
@@ -278,6 +284,9 @@ struct context {
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.gemm_bf16_nt_parts, "tlhip_gemm_bf16_nt_parts") &&
               bind(f.gemm_bf16_nt_swiglu, "tlhip_gemm_bf16_nt_swiglu") &&
+              bind(f.gemm_f16w_bytes, "tlhip_gemm_f16w_bytes") && bind(f.gemm_f16w_prepare, "tlhip_gemm_f16w_prepare") &&
+              bind(f.gemm_f16w_nt, "tlhip_gemm_f16w_nt") && bind(f.gemm_f16w_nt_parts, "tlhip_gemm_f16w_nt_parts") &&
+              bind(f.gemm_f16w_nt_swiglu, "tlhip_gemm_f16w_nt_swiglu") &&
               bind(f.gemm_q4_nt, "tlhip_gemm_q4_nt") && bind(f.gemm_q4_nt_parts, "tlhip_gemm_q4_nt_parts") &&
               bind(f.gemm_q4_nt_swiglu, "tlhip_gemm_q4_nt_swiglu") &&
               bind(f.rmsnorm_res_parts, "tlhip_rmsnorm_res_parts") &&
@@ -649,6 +658,43 @@ inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_byte
   L.reads(a, B);
   L.writes(parts);
   return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
+}
+
+// The prepared form of a bf16 weight for prompt chunks (the library's f16 slab images and row
+// exponents): its size, its construction from the bf16 rows, and the three products over it.
+// No counterpart in the reference's seam; for a harness that owns its weights.
+inline int64_t gemm_f16w_bytes(int64_t n, int64_t k, bool gated) {
+  launch L;
+  return L.ok ? L.lib.gemm_f16w_bytes(n, k, gated ? 1 : 0) : 0;
+}
+inline bool gemm_f16w_prepare(void* B, int64_t n, int64_t k, bool gated, void* image, void* exps) {
+  launch L;
+  if (!L.ok || n <= 0 || k <= 0 || (k % 32) != 0) return false;
+  L.reads(B);
+  L.writes(image, exps);
+  return L.sent(L.lib.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, image, exps));
+}
+inline bool gemm_f16w_nt(void* a, void* image, void* exps, void* out, int64_t m, int64_t n, int64_t k) {
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0) return false;
+  L.reads(a, image, exps);
+  L.writes(out);
+  return L.sent(L.lib.gemm_f16w_nt(a, image, exps, out, m, n, k));
+}
+inline bool gemm_f16w_nt_swiglu(void* a, void* image, void* exps, void* act, int64_t m, int64_t ff, int64_t k) {
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || ff <= 0) return false;
+  L.reads(a, image, exps);
+  L.writes(act);
+  return L.sent(L.lib.gemm_f16w_nt_swiglu(a, image, exps, act, m, ff, k));
+}
+inline bool gemm_f16w_nt_parts(void* a, void* image, void* exps, void* parts, int64_t parts_bytes, int64_t m,
+                               int64_t n, int64_t k, int* n_parts) {
+  launch L;
+  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
+  L.reads(a, image, exps);
+  L.writes(parts);
+  return L.sent(L.lib.gemm_f16w_nt_parts(a, image, exps, parts, parts_bytes, m, n, k, n_parts));
 }
 
 inline bool attn_decode(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,

@@ -62,6 +62,7 @@ def _load():
             "tlq_set_fused_attn": (None, [P, cint]),
             "tlq_set_gateup_epilogue": (None, [P, cint]),
             "tlq_set_fused_prefill": (None, [P, cint]),
+            "tlq_set_prompt_f16": (None, [P, cint]),
             "tlq_greedy_init": (cint, [P, i64, i64]),
             "tlq_greedy_run": (i64, [P, i64]),
             "tlq_greedy_tokens": (cint, [P, i64, i64, P]),
@@ -340,6 +341,10 @@ class QwenGPU:
     def set_fused_prefill(self, on):
         """Prompt chunks: one launch for split_heads + rope + kv_fill and token-major attention output (default), or the reference's op sequence."""
         self.L.tlq_set_fused_prefill(self.h, 1 if on else 0)
+
+    def set_prompt_f16(self, on):
+        """Prompt chunks of bf16 weights: on their prepared f16 images (default; a second copy of the weights, made on the first chunk) or on the bf16 rows."""
+        self.L.tlq_set_prompt_f16(self.h, 1 if on else 0)
 
     def set_gateup_epilogue(self, on):
         """Within the fused path: swiglu as the epilogue of the gate|up GEMV (default) or as the producer of the down GEMV."""

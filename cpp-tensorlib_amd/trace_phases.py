@@ -8,6 +8,7 @@ divided by the frequency given with --ghz (default 2.1).
 
   python cpp-tensorlib_amd/trace_phases.py attn_decode [pos]      7B decode attention (fused q/k/v, device position)
   python cpp-tensorlib_amd/trace_phases.py attn_prefill [pos0]    7B causal prefill attention of a 512-token chunk (bf16 planes)
+  python cpp-tensorlib_amd/trace_phases.py gemm [f16w|bf16]       a 512 x 32768 x 3584 prompt GEMM: prepared weight, or plain bf16
 """
 import ctypes as C
 import importlib
@@ -118,13 +119,61 @@ def attn_prefill(lib, pos0, ghz):
         pct("whole interval", (tt[:, :, 6] - tt[:, :, 0])[live] / iv / (ghz * 1e3))
 
 
+def gemm(lib, kind, ghz):
+    M, N, K = 512, 32768, 3584
+    rng = np.random.default_rng(5)
+    A = lib.to_device(rng.standard_normal((M, K), dtype=np.float32))
+    w = (rng.standard_normal((N, K), dtype=np.float32) * 0.02).view(np.uint32) >> 16
+    W = lib.to_device(w.astype(np.uint16))
+    Cm = lib.empty((M, N))
+    us = lambda x: x / (ghz * 1e3)
+    if kind == "f16w":
+        img, ex = lib.gemm_f16w_prepare(W, N, K)
+        run = lambda: lib.gemm_f16w_nt(A, img, ex, Cm, M, N, K)
+    else:
+        run = lambda: lib.gemm_bf16_nt(A, W, Cm, M, N, K)
+    for _ in range(2):
+        run()
+    lib.sync()
+    read_trace(lib)
+    e0, e1 = lib.event(), lib.event()
+    lib.record(e0)
+    run()
+    lib.record(e1)
+    lib.sync()
+    print("prompt GEMM %d x %d x %d, %s: %.1f us" % (M, N, K, kind, lib.elapsed_ms(e0, e1) * 1e3))
+    t = read_trace(lib)
+    if kind != "f16w":
+        t = t[:, :4, :]
+        live = t[:, :, 7] > 0
+        slabs = t[:, :, 7][live]
+        print("%d wavefronts, %d K slabs each; per slab:" % (int(live.sum()), int(np.median(slabs))))
+        for k, nm in ((1, "barrier: the slab before consumed by every wavefront"), (2, "wait for the slab's global loads"),
+                      (3, "convert and store to LDS"), (4, "barrier: slab complete in LDS"),
+                      (5, "next slab requested, fragments read, matrix products")):
+            pct(nm, us(t[:, :, k][live] / slabs))
+        pct("whole slab", us((t[:, :, 6] - t[:, :, 0])[live] / slabs))
+        return
+    t = t[:, :8, :]
+    live = t[:, :, 7] > 0
+    slabs = t[:, :, 7][live]
+    print("%d wavefronts, %d K slabs each" % (int(live.sum()), int(np.median(slabs))))
+    pct("first three slab copies issued -> slab 0 landed everywhere", us((t[:, :, 1] - t[:, :, 0])[live]))
+    pct("per slab: fragment reads, matrix products, copy requests", us(t[:, :, 2][live] / slabs))
+    pct("per slab: wait for own reads and copies, barrier", us(t[:, :, 3][live] / slabs))
+    pct("loop", us((t[:, :, 5] - t[:, :, 1])[live]))
+    pct("result scaled and stored", us((t[:, :, 6] - t[:, :, 5])[live]))
+
+
 if __name__ == "__main__":
     args = [a for a in sys.argv[1:] if not a.startswith("--ghz")]
     ghz = next((float(a.split("=")[1]) for a in sys.argv[1:] if a.startswith("--ghz=")), 2.1)
-    if not args or args[0] not in ("attn_decode", "attn_prefill"):
+    if not args or args[0] not in ("attn_decode", "attn_prefill", "gemm"):
         sys.exit(__doc__)
     lib = load()
-    if args[0] == "attn_decode":
+    if args[0] == "gemm":
+        gemm(lib, args[1] if len(args) > 1 else "f16w", ghz)
+    elif args[0] == "attn_decode":
         attn_decode(lib, int(args[1]) if len(args) > 1 else 4095, ghz)
     else:
         attn_prefill(lib, int(args[1]) if len(args) > 1 else 7680, ghz)

@@ -356,6 +356,31 @@ int tlhip_gemm_bf16_nt_parts(const void* A, const void* W, void* parts, int64_t 
  * tlhip_gemm_bf16_nt on the same W; where K is split, it is split for other columns than there,
  * so the two agree to fp32 summation order, not bit for bit. */
 int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M, int64_t ff, int64_t K);
+/* The same three products over a PREPARED weight, for a harness that owns its weights (no reference
+ * counterpart: gemm_bf16_nt of cuda.h:787-841 takes the weight alone). tlhip_gemm_f16w_prepare, once
+ * when the weight is loaded, writes
+ *   exps[r] (int8, one per row of W) = 14 - floor(log2(max_k |W[r][k]|)), what brings the row's
+ *     largest magnitude into [2^14, 2^15) (0 for a row of zeros), and
+ *   image (tlhip_gemm_f16w_bytes(N, K, gated) bytes) = every weight times 2^exps[r] as f16, laid out
+ *     slab by slab (256 rows x 32 k, 16 KB) in the order the kernel's LDS reads expect. A bf16
+ *     weight has 8 significant bits and an f16 holds 11, so each weight is exact unless it lies more
+ *     than 2^29 below its row's largest (then its absolute error is below 2^-40 of that).
+ * gated != 0: W = [gate rows | up rows], [2*N, K], N = features (the operand of
+ * tlhip_gemm_bf16_nt_swiglu); the image then serves tlhip_gemm_f16w_nt_swiglu only, a plain image
+ * the other two. K % 32 == 0.
+ * The products cut every activation row, scaled the same way, into two f16 terms, both rounded to
+ * nearest (2^-24 relative), and run two matrix-core products per weight instead of three, fp32
+ * sums, the result scaled back exactly: the error is that of one fp32 rounding per product, as in
+ * tlhip_gemm_bf16_nt, which these agree with to fp32 summation order. The image replaces W for
+ * prompt chunks; the decode GEMV still reads the bf16 weight. */
+int64_t tlhip_gemm_f16w_bytes(int64_t N, int64_t K, int gated);
+int tlhip_gemm_f16w_prepare(const void* W, int64_t N, int64_t K, int gated, void* image, void* exps);
+int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N,
+                       int64_t K);
+int tlhip_gemm_f16w_nt_parts(const void* A, const void* image, const void* exps, void* parts,
+                             int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int* n_parts);
+int tlhip_gemm_f16w_nt_swiglu(const void* A, const void* image, const void* exps, void* act, int64_t M,
+                              int64_t ff, int64_t K);
 /* The three prompt-chunk products over an int4 weight (qw = packed nibbles [N][K/2], scales
  * [N][K/32], group 32 - the operand of tlhip_gemv_q4): C = A . dequant(W)^T formed as
  * sum over groups of scale * (A . q) with exact products on the matrix pipe, fp32 sums - the decode

@@ -33,6 +33,10 @@ int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int wa
  * with decode attention, 2 = the fp32 matrix-pipe kernel, 3 = the bf16-plane kernels.
  * Same results within fp32 summation order; for A/B timing and tests. */
 int tlhip_tune_attn_prefill(int kernel);
+/* How the prompt GEMMs over an int4 weight (M > 64) cut the f32 activations: 0 = the built-in
+ * choice (two f16 terms), 3 = three bf16 terms. Same results within fp32 summation order; for A/B
+ * timing and tests. */
+int tlhip_tune_gemm_planes(int planes);
 /* Every override back to the built-in choice (tlhip_tune_gemv_cols included). */
 int tlhip_tune_reset(void);
 
