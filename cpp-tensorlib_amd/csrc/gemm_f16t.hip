@@ -78,24 +78,51 @@ __global__ __launch_bounds__(256) void w_image_kernel(const uint16_t* __restrict
   }
 }
 
-// One block per (row tile, slab): 256 rows x 32 k of the activations -> hi and lo f16 slab images.
-__global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ A, const int* __restrict__ ea,
+// One block per row of the activation images (rows past M are zero rows): the row's largest
+// magnitude and from it ea[m], then its two f16 terms into the slab images - one read of A.
+// The row stays in registers between the two steps: up to kRowRegs float4s per thread.
+constexpr int kRowRegs = 32;            // K <= 256 * 4 * 32 = 32768
+__global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ A, int* __restrict__ ea,
                                                       char* __restrict__ img, int M, int K) {
-  const int tm = blockIdx.x, slab = blockIdx.y, nslab = gridDim.y, t = threadIdx.x;
-  char* dst = img + ((size_t)tm * nslab + slab) * kAImage;
+  __shared__ uint32_t part[4];
+  const int gm = blockIdx.x, t = threadIdx.x, nslab = K / kBK, k4 = K / 4;
+  const int tm = gm / kTile, row = gm % kTile;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  f32x4 v[kRowRegs];
+  uint32_t mx = 0;
+  if (gm < M) {
+    const f32x4* src = reinterpret_cast<const f32x4*>(A + (size_t)gm * K);
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const int row = (t >> 3) + 32 * i, c4 = t & 7, gm = tm * kTile + row;
-    uint32_t h01 = 0, l01 = 0, h23 = 0, l23 = 0;
-    if (gm < M) {
-      const float4 a = *reinterpret_cast<const float4*>(A + (size_t)gm * K + slab * kBK + c4 * 4);
-      const float s = pow2f(ea[gm]);
-      split2_f16(a.x * s, a.y * s, h01, l01);
-      split2_f16(a.z * s, a.w * s, h23, l23);
+    for (int i = 0; i < kRowRegs; i++) {
+      const int q = t + 256 * i;
+      v[i] = q < k4 ? src[q] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; e++) mx = max(mx, __float_as_uint(v[i][e]) & 0x7fffffffu);
     }
-    const int o = image_off(row, c4 >> 1) + (c4 & 1) * 8;
-    *reinterpret_cast<uint2*>(dst + o) = make_uint2(h01, h23);
-    *reinterpret_cast<uint2*>(dst + kPlaneBytes + o) = make_uint2(l01, l23);
+  } else {
+#pragma unroll
+    for (int i = 0; i < kRowRegs; i++) v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, d));
+  if ((t & 63) == 0) part[t >> 6] = mx;
+  __syncthreads();
+  mx = max(max(part[0], part[1]), max(part[2], part[3]));
+  const int e = row_exponent((int)(mx >> 23), mx == 0);
+  if (t == 0 && gm < M) ea[gm] = e;
+  const float s = pow2f(e);
+  char* dst = img + (size_t)tm * nslab * kAImage;
+#pragma unroll
+  for (int i = 0; i < kRowRegs; i++) {
+    const int q = t + 256 * i;               // float4 q of the row: slab q / 8, 8-byte piece q % 8 of its 64 bytes
+    if (q >= k4) break;
+    uint32_t h01, l01, h23, l23;
+    split2_f16(v[i][0] * s, v[i][1] * s, h01, l01);
+    split2_f16(v[i][2] * s, v[i][3] * s, h23, l23);
+    const int c4 = q & 7;
+    char* o = dst + (size_t)(q >> 3) * kAImage + image_off(row, c4 >> 1) + (c4 & 1) * 8;
+    *reinterpret_cast<uint2*>(o) = make_uint2(h01, h23);
+    *reinterpret_cast<uint2*>(o + kPlaneBytes) = make_uint2(l01, l23);
   }
 }
 
@@ -233,10 +260,9 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
     barrier();
     TLHIP_PHASE(1);
-    issue(k + 3, st);                                  // into the stage slab k has just left
-    __builtin_amdgcn_sched_barrier(0);
     mul(Idx<1>{}, Idx<0>{});
     __builtin_amdgcn_sched_barrier(0);
+    issue(k + 3, st);                                  // into the stage slab k has just left
     if (k + 1 < ns) fetch(ring + nx * kStage, Idx<0>{});
     __builtin_amdgcn_sched_barrier(0);
     mul(Idx<1>{}, Idx<1>{});
@@ -316,8 +342,8 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
   TLHIP_REQUIRE_READY();
   const bool want_parts = S_out != nullptr;
   if (!A || !image || !exps || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt: null pointer");
-  if (M <= 0 || N <= 0 || K <= 0 || (K % f16t::kBK) != 0)
-    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: need positive M, N, K and K %% 32 == 0");
+  if (M <= 0 || N <= 0 || K <= 0 || (K % f16t::kBK) != 0 || K > 256 * 4 * f16t::kRowRegs)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: need positive M, N, K, K %% 32 == 0 and K <= 32768");
   if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: dimension too large");
   if (!aligned16(A) || !aligned16(image) || !aligned16(C))
@@ -370,8 +396,7 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
   int* ea = reinterpret_cast<int*>(sbase);
   char* aimg = sbase + ea_bytes;
   const float* pa = static_cast<const float*>(A);
-  row_exponent_f32_kernel<<<dim3((unsigned)M), dim3(256), 0, c.stream>>>(pa, (int)K, ea);
-  f16t::a_image_kernel<<<dim3((unsigned)timg, (unsigned)nslab), dim3(256), 0, c.stream>>>(pa, ea, aimg, (int)M, (int)K);
+  f16t::a_image_kernel<<<dim3((unsigned)(timg * f16t::kTile)), dim3(256), 0, c.stream>>>(pa, ea, aimg, (int)M, (int)K);
   const size_t lds = (size_t)f16t::kRing * (2 * bm * f16t::kRowBytes + f16t::kWImage);
   float* pc = static_cast<float*>(C);
   for (int pi = 0; pi < npieces; pi++) {
@@ -449,7 +474,8 @@ int tlhip_gemm_f16w_prepare(const void* W, int64_t N, int64_t K, int gated, void
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_prepare: weight too large for one grid");
   f16t::w_image_kernel<<<dim3((unsigned)tn, (unsigned)nslab), dim3(256), 0, c.stream>>>(
       pw, pe, static_cast<char*>(image), (int)N, (int)K, (int)N, gated ? 1 : 0);
-  TLHIP_CHECK_LAUNCH(TLHIP_C_GEMM_BF16_NT);
+  const hipError_t e = hipGetLastError();   // a preparation is not a product: not in the census
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "kernel launch");
 }
 
 int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N,

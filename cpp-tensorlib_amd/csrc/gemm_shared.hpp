@@ -19,6 +19,12 @@ __global__ void row_exponent_f32_kernel(const float* __restrict__ A, int K, int*
 __global__ void row_exponent_bf16_kernel(const uint16_t* __restrict__ W, int K, int8_t* __restrict__ ew);
 
 #if defined(__HIPCC__)
+// Exponent that brings the largest magnitude of a row into [2^14, 2^15): 14 - floor(log2(max)),
+// kept within [-126, 126] so that 2^e is a normal float; 0 for a row of zeros. `field` is the
+// biased exponent field of the row's largest magnitude (255 for inf / NaN: they stay what they are).
+__device__ __forceinline__ int row_exponent(int field, bool all_zero) {
+  return all_zero ? 0 : max(-126, min(126, 14 - (field - 127)));
+}
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // e in [-126, 127]
 
 // two scaled floats -> their f16 terms, both round-to-nearest; x - hi is exact in fp32

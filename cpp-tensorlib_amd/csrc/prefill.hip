@@ -360,13 +360,6 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     }
 }
 
-// Exponent that brings the largest magnitude of a row into [2^14, 2^15): 14 - floor(log2(max)),
-// kept within [-126, 126] so that 2^e is a normal float; 0 for a row of zeros. `field` is the
-// biased exponent field of the row's largest magnitude (255 for inf / NaN: they stay what they are).
-__device__ __forceinline__ int row_exponent(int field, bool all_zero) {
-  return all_zero ? 0 : max(-126, min(126, 14 - (field - 127)));
-}
-
 // ea[m] for the rows of an f32 matrix [M][K] (K % 4 == 0, rows 16-byte aligned). One block per row.
 __global__ __launch_bounds__(256) void row_exponent_f32_kernel(const float* __restrict__ A, int K,
                                                                int* __restrict__ ea) {

@@ -151,16 +151,19 @@ def test_prefill_chunk_at_7b_dims(orc, q4):
         Vc[:] = 0.0
         _seed_caches(orc, om, g, pos0, 800 + pos0)
         want = _oracle_chunk_rows(orc, om, tokens, pos0, rows)
-        for fused in (True, False):
-            print("case 7B chunk", "q4" if q4 else "bf16", "pos0", pos0, "fused" if fused else "plain", flush=True)
+        # fused twice for bf16 weights: on their prepared f16 images (the default) and on the bf16 rows
+        for fused, f16 in ((True, True), (True, False), (False, True)) if not q4 else ((True, True), (False, True)):
+            print("case 7B chunk", "q4" if q4 else "bf16", "pos0", pos0, "fused" if fused else "plain",
+                  "f16 images" if f16 else "bf16 rows", flush=True)
             g.set_fused_prefill(fused)
+            g.set_prompt_f16(f16)
             g.set_cache_pos(pos0)
             g.prefill(tokens, chunk=T, want_logits=False)
             got = g.prefill_hidden(T)[rows]
             mr = maxrel(got, want)
             print("   final-norm rows maxrel %.2e" % mr, flush=True)
             assert np.all(np.isfinite(got))
-            assert mr < 2e-4, (pos0, fused, mr)
+            assert mr < 2e-4, (pos0, fused, f16, mr)
         # decode continues on the caches the chunk filled
         tok = int(tokens[-1])
         want_tok, want_logits = om.step(tok, pos0 + T)

@@ -135,7 +135,7 @@ def test_bf16_decode_loop_matches_oracle(orc):
 
 @pytest.mark.parametrize("q4", [False, True])
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("dims,n_prompt,chunk", [(SMALL, 50, 32), (SMALL128, 130, 64), (SMALL, 40, 512)])
+@pytest.mark.parametrize("dims,n_prompt,chunk", [(SMALL, 50, 32), (SMALL128, 130, 64), (SMALL, 40, 512), (SMALL128, 280, 100)])
 def test_prefill_chunks_match_token_by_token_oracle(orc, dims, n_prompt, chunk, fused, q4):
     """A prompt consumed in chunks through the MFMA GEMM + causal prefill attention
     (bench/cuda/qwen_model.h:357-401) gives the logits of feeding the same tokens one at a
