@@ -159,23 +159,39 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
 
   // this wavefront's share of a slab copy: TM KB of each plane of A (TM = 1: of the half image
   // that holds this block's rows), two of the 16 KB of W
+  // Everything but the lane's 16-byte slot is uniform over the wavefront and kept in scalars.
   const int img = TM == 2 ? tm : tm >> 1, half = TM == 2 ? 0 : (tm & 1) * kAPlane;
-  const char* asrc = Aimg + ((size_t)img * nslab + sbeg) * kAImage + half + (wave * TM) * 1024 + lane * 16;
-  const char* wsrc = Wimg + ((size_t)tn * nslab + sbeg) * kWImage + (wave * 2) * 1024 + lane * 16;
-  auto issue = [&](int slab, int stage) {   // past the end: the last slab again, into a stage nobody reads
+  const int uw = __builtin_amdgcn_readfirstlane(wave);
+  const char* asrc = Aimg + ((size_t)img * nslab + sbeg) * kAImage + half + (uw * TM) * 1024;
+  const char* wsrc = Wimg + ((size_t)tn * nslab + sbeg) * kWImage + (uw * 2) * 1024;
+  const uint32_t slot = lane * 16;
+  // copy C of this wavefront's kCopies for slab `slab` into ring stage `stage`
+  // (past the end: the last slab again, into a stage nobody reads)
+  auto copy = [&](int slab, int stage, auto CI) {
+    constexpr int ci = decltype(CI)::value;
     const int s = min(slab, ns - 1);
     char* base = ring + stage * kStage;
-#pragma unroll
-    for (int p = 0; p < 2; p++)
-#pragma unroll
-      for (int j = 0; j < TM; j++)
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(asrc + (size_t)s * kAImage + p * kPlaneBytes + j * 1024),
-            (__attribute__((address_space(3))) void*)(base + p * kAPlane + (wave * TM + j) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (size_t)s * kWImage + j * 1024),
-                                       (__attribute__((address_space(3))) void*)(base + 2 * kAPlane + (wave * 2 + j) * 1024), 16, 0, 0);
+    if (ci < 2 * TM) {
+      constexpr int p = ci / TM, j = ci % TM;
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(asrc + (size_t)s * kAImage + p * kPlaneBytes + j * 1024 + slot),
+          (__attribute__((address_space(3))) void*)(base + p * kAPlane + (uw * TM + j) * 1024), 16, 0, 0);
+    } else {
+      constexpr int j = ci - 2 * TM;
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(wsrc + (size_t)s * kWImage + j * 1024 + slot),
+          (__attribute__((address_space(3))) void*)(base + 2 * kAPlane + (uw * 2 + j) * 1024), 16, 0, 0);
+    }
+  };
+  auto issue = [&](int slab, int stage) {
+    copy(slab, stage, Idx<0>{});
+    copy(slab, stage, Idx<1>{});
+    copy(slab, stage, Idx<2>{});
+    copy(slab, stage, Idx<3>{});
+    if (TM == 2) {
+      copy(slab, stage, Idx<4>{});
+      copy(slab, stage, Idx<5>{});
+    }
   };
 
   f32x16 acc[TM][4];
@@ -207,15 +223,14 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
       for (int p = 0; p < 2; p++)
         af[ks][i][p] = *reinterpret_cast<const frag16*>(stage + aoff[ks] + p * kAPlane + i * 32 * kRowBytes);
   };
-  // one half of the products of fragment set KS: TM of its 2 * TM (tile row, plane) pairs, 4 MFMAs each
-  auto mul = [&](auto KS, auto HALF) {
-    constexpr int ks = decltype(KS)::value, h = decltype(HALF)::value;
+  // four products: fragment set KS, (tile row, plane) pair Q against the four tile columns
+  auto mul4 = [&](auto KS, auto Q) {
+    constexpr int ks = decltype(KS)::value, q = decltype(Q)::value;
 #pragma unroll
-    for (int q = h * TM; q < (h + 1) * TM; q++)
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        acc[q >> 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[ks][q >> 1][q & 1]),
-                                                                __builtin_bit_cast(f16x8, bf[ks][j]), acc[q >> 1][j], 0, 0, 0);
+    for (int j = 0; j < 4; j++)
+      acc[q >> 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[ks][q >> 1][q & 1]),
+                                                              __builtin_bit_cast(f16x8, bf[ks][j]), acc[q >> 1][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
   };
   // The block's barrier without the fence __syncthreads() puts before it: that fence would wait for
   // EVERY copy in flight (they write LDS). What has to be complete is waited for by count instead.
@@ -242,30 +257,49 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
   barrier();
   fetch(ring, Idx<0>{});
   TLHIP_MARK(1);
-  // A fragment set is requested half a set of MFMAs before the set that uses it starts, and
-  // nothing younger is outstanding when it is waited for.
+  // A fragment set is requested a few MFMAs before the set that uses it starts, and nothing
+  // younger is outstanding when it is waited for. The copies of slab k + 3 go out one or two at a
+  // time between groups of MFMAs: issued together, the 48 of a block queue up in front of the
+  // CU's one vector memory path and hold back the MFMAs that follow them in each wavefront.
   int st = 0;
   for (int k = 0; k < ns; k++) {
     const char* stage = ring + st * kStage;
     const int nx = st == 2 ? 0 : st + 1;
-    mul(Idx<0>{}, Idx<0>{});
-    __builtin_amdgcn_sched_barrier(0);
+    mul4(Idx<0>{}, Idx<0>{});
     fetch(stage, Idx<1>{});
     __builtin_amdgcn_sched_barrier(0);
-    mul(Idx<0>{}, Idx<1>{});
-    __builtin_amdgcn_sched_barrier(0);
+    mul4(Idx<0>{}, Idx<1>{});
+    if (TM == 2) {
+      mul4(Idx<0>{}, Idx<2>{});
+      mul4(Idx<0>{}, Idx<3>{});
+    }
     TLHIP_PHASE(0);
     // my reads of slab k are complete and my copies of slab k + 1 have landed (those of slab
     // k + 2 may still be in flight); past the barrier that holds for every wavefront
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
     barrier();
     TLHIP_PHASE(1);
-    mul(Idx<1>{}, Idx<0>{});
-    __builtin_amdgcn_sched_barrier(0);
-    issue(k + 3, st);                                  // into the stage slab k has just left
+    // slab k + 3 into the stage slab k has just left
+    mul4(Idx<1>{}, Idx<0>{});
+    copy(k + 3, st, Idx<0>{});
+    if (TM == 1) copy(k + 3, st, Idx<1>{});
     if (k + 1 < ns) fetch(ring + nx * kStage, Idx<0>{});
     __builtin_amdgcn_sched_barrier(0);
-    mul(Idx<1>{}, Idx<1>{});
+    mul4(Idx<1>{}, Idx<1>{});
+    if (TM == 1) {
+      copy(k + 3, st, Idx<2>{});
+      copy(k + 3, st, Idx<3>{});
+    } else {
+      copy(k + 3, st, Idx<1>{});
+      copy(k + 3, st, Idx<2>{});
+      __builtin_amdgcn_sched_barrier(0);
+      mul4(Idx<1>{}, Idx<2>{});
+      copy(k + 3, st, Idx<3>{});
+      copy(k + 3, st, Idx<4>{});
+      __builtin_amdgcn_sched_barrier(0);
+      mul4(Idx<1>{}, Idx<3>{});
+      copy(k + 3, st, Idx<5>{});
+    }
     __builtin_amdgcn_sched_barrier(0);
     st = nx;
   }
@@ -353,14 +387,14 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
   const int64_t w = f16t::kTile / per;              // units of N per column tile
   const int64_t nslab = K / f16t::kBK, tn = cdiv64(N, w);
   const int64_t slots = c.cus;                      // one block per CU
-  // 256-row tiles unless they leave more than half of the CUs to K splits; then 128-row tiles
-  const int tmh = (cdiv64(M, 256) * tn * 2 <= slots) ? 1 : 2;
-  const int64_t bm = 128 * tmh, tm = cdiv64(M, bm), tiles = tm * tn;
+  const int64_t tm256 = cdiv64(M, 256), tm128 = cdiv64(M, 128);
   const bool can_split = (N % 4) == 0;              // the part sums work on float4s
   // Work is shaped to whole rounds of the block slots, as in tlhip_gemm_bf16_nt: fewer tiles than
   // slots -> K split so that tiles * S comes close to the slots; more -> the columns that make
-  // whole rounds with full K, the remaining columns split over K in a second launch.
-  struct Piece { int64_t tn0, tcols; int S; };
+  // whole rounds with full K, the remaining columns split over K in a second launch. A piece runs
+  // on 256-row tiles unless those would leave more than half of the CUs to K splits; then on
+  // 128-row tiles: twice the tiles, half the splits, half the parts to write and add up.
+  struct Piece { int64_t tn0, tcols; int S; int tmh; };
   Piece pieces[2];
   int npieces = 0;
   auto pick_S = [&](int64_t t) {
@@ -372,13 +406,17 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
       while (S > 1 && (size_t)S * M * N * sizeof(float) > parts_bytes) S--;
     return (int)S;
   };
-  const int64_t cols_per_round = slots / tm;
-  if (tiles <= slots || cols_per_round == 0 || !can_split || want_parts) {
-    pieces[npieces++] = Piece{0, tn, pick_S(tiles)};
+  auto piece = [&](int64_t tn0, int64_t tcols, bool split) {
+    const int tmh = tm256 * tcols * 2 <= slots ? 1 : 2;
+    return Piece{tn0, tcols, split ? pick_S((tmh == 1 ? tm128 : tm256) * tcols) : 1, tmh};
+  };
+  const int64_t cols_per_round = slots / tm256;
+  if (tm256 * tn <= slots || cols_per_round == 0 || !can_split || want_parts) {
+    pieces[npieces++] = piece(0, tn, true);
   } else {
     const int64_t main_tn = tn / cols_per_round * cols_per_round;
-    pieces[npieces++] = Piece{0, main_tn, 1};
-    if (main_tn < tn) pieces[npieces++] = Piece{main_tn, tn - main_tn, pick_S(tm * (tn - main_tn))};
+    pieces[npieces++] = Piece{0, main_tn, 1, 2};
+    if (main_tn < tn) pieces[npieces++] = piece(main_tn, tn - main_tn, true);
   }
   // scratch: exponents of A's rows, the slab images of A, room for the largest piece's parts
   const size_t ea_bytes = ((size_t)M * sizeof(int) + 1023) & ~(size_t)1023;
@@ -397,7 +435,6 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
   char* aimg = sbase + ea_bytes;
   const float* pa = static_cast<const float*>(A);
   f16t::a_image_kernel<<<dim3((unsigned)(timg * f16t::kTile)), dim3(256), 0, c.stream>>>(pa, ea, aimg, (int)M, (int)K);
-  const size_t lds = (size_t)f16t::kRing * (2 * bm * f16t::kRowBytes + f16t::kWImage);
   float* pc = static_cast<float*>(C);
   for (int pi = 0; pi < npieces; pi++) {
     const Piece& P = pieces[pi];
@@ -417,7 +454,8 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
       dst = reinterpret_cast<float*>(sbase + ea_bytes + aimg_bytes);
       ldc = (int)part_w;
     }
-    const int64_t nblk = tm * P.tcols;
+    const int64_t nblk = (P.tmh == 1 ? tm128 : tm256) * P.tcols;
+    const size_t lds = (size_t)f16t::kRing * (2 * 128 * P.tmh * f16t::kRowBytes + f16t::kWImage);
     if (nblk > 0x7fffffff || part_w > 0x7fffffff)
       return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: too many tiles for one grid");
     const dim3 grid((unsigned)nblk, (unsigned)S);
@@ -428,7 +466,7 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
                                              part_slabs, ldc, (int)P.tn0, (int)N, ea, static_cast<const int8_t*>(exps));
       return hipSuccess;
     };
-    const hipError_t e = tmh == 2 ? (gu ? launch(f16t::gemm_f16t_kernel<2, true>) : launch(f16t::gemm_f16t_kernel<2, false>))
+    const hipError_t e = P.tmh == 2 ? (gu ? launch(f16t::gemm_f16t_kernel<2, true>) : launch(f16t::gemm_f16t_kernel<2, false>))
                                   : (gu ? launch(f16t::gemm_f16t_kernel<1, true>) : launch(f16t::gemm_f16t_kernel<1, false>));
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
     if (S > 1 && !want_parts) {
