@@ -178,6 +178,17 @@ struct extent {
   float* staging = nullptr;
   size_t size = 0;
   side live = side::staging;
+  // What the library derived from a bf16 weight inside this extent for prompt-chunk products
+  // (its f16 slab images and row exponents): made on the first such product, dropped as soon as
+  // the extent's device bytes can change (an upload, a launch that writes it, its release).
+  struct prepared {
+    size_t off = 0;            // of the weight inside the extent
+    int64_t n = 0, k = 0;      // rows (gated: features) and depth
+    bool gated = false;
+    void* image = nullptr;
+    void* exps = nullptr;
+  };
+  std::vector<prepared> derived;
 };
 
 // The extents in use, ordered by base address so that an address INSIDE one (q4 scales at
@@ -230,6 +241,9 @@ struct context {
   std::vector<uintptr_t> capture_writes;
   std::unordered_map<void*, std::vector<uintptr_t>> graph_writes;
   std::string why;  // why the backend is unavailable (diagnostics only)
+  // Prompt-chunk products over bf16 weights run on the library's prepared f16 form of the weight
+  // (a second copy of it, made on first use). TENSORLIB_HIP_PROMPT_F16=0 keeps them on the bf16 rows.
+  bool prompt_f16 = true;
 
   ledger buffers;   // every extent handed out, and the idle ones waiting for reuse
 
@@ -249,6 +263,7 @@ struct context {
     // TENSORLIB_HIP_LIB names the library explicitly; otherwise the usual
     // dynamic-loader search applies.
     std::vector<std::string> paths;
+    if (const char* e = std::getenv("TENSORLIB_HIP_PROMPT_F16")) prompt_f16 = std::strcmp(e, "0") != 0;
     if (const char* e = std::getenv("TENSORLIB_HIP_LIB")) paths.emplace_back(e);
     paths.emplace_back("libtensorlib_hip.so");
     for (const auto& p : paths) {
@@ -339,13 +354,49 @@ struct context {
     extent* e = buffers.containing(p);
     if (!e) return;
     if (e->live == extent::side::staging && static_cast<char*>(p) != e->base) push(*e, e->size);
+    forget_derived(*e);
     e->live = extent::side::device;
     if (capturing) capture_writes.push_back(reinterpret_cast<uintptr_t>(e->base));
   }
   // staging -> device, blocking and ordered after the queued launches
   void push(extent& e, size_t n) {
     f.memcpy_h2d(e.base, e.staging, n < e.size ? n : e.size);
+    forget_derived(e);
     e.live = extent::side::either;
+  }
+  // The extent's device bytes are changing: what was derived from them goes. (free_ drains the
+  // device first, so a queued product that still reads an image finishes with it.)
+  void forget_derived(extent& e) {
+    for (auto& d : e.derived) {
+      f.free_(d.image);
+      f.free_(d.exps);
+    }
+    e.derived.clear();
+  }
+  // The prepared form of the bf16 weight B [n, k] (gated: [2n, k], gate rows | up rows), made now
+  // if this is its first prompt-chunk product. nullptr: not a managed buffer, not a shape the
+  // prepared products take, no memory, or a capture is open - the caller uses the bf16 rows.
+  const extent::prepared* prepared_weight(void* B, int64_t n, int64_t k, bool gated) {
+    if (!prompt_f16 || capturing) return nullptr;
+    extent* e = buffers.containing(B);
+    if (!e) return nullptr;
+    const size_t off = static_cast<size_t>(static_cast<char*>(B) - e->base);
+    for (const auto& d : e->derived)
+      if (d.off == off && d.n == n && d.k == k && d.gated == gated) return &d;
+    const int64_t rows = gated ? 2 * n : n, bytes = f.gemm_f16w_bytes(n, k, gated ? 1 : 0);
+    if (bytes <= 0 || off + static_cast<size_t>(rows * k * 2) > e->size) return nullptr;
+    extent::prepared d;
+    d.off = off; d.n = n; d.k = k; d.gated = gated;
+    if (f.malloc_(&d.image, static_cast<size_t>(bytes)) != 0) return nullptr;
+    if (f.malloc_(&d.exps, static_cast<size_t>((rows + 15) & ~int64_t(15))) != 0 ||
+        f.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, d.image, d.exps) != 0) {
+      f.free_(d.image);
+      if (d.exps) f.free_(d.exps);
+      return nullptr;
+    }
+    pending = true;
+    e->derived.push_back(d);
+    return &e->derived.back();
   }
   // device -> staging
   void pull(extent& e) {
@@ -368,6 +419,8 @@ class launch {
   void reads(P... p) { (c_.refresh_device(p), ...); }
   template <class... P>
   void writes(P... p) { (c_.claim_device(p), ...); }
+  // see context::prepared_weight; call after reads() has brought the weight up to date
+  const extent::prepared* prepared(void* B, int64_t n, int64_t k, bool gated) { return c_.prepared_weight(B, n, k, gated); }
   bool sent(int rc) {
     if (rc != 0) return false;   // declined or failed: the caller falls back
     c_.pending = true;
@@ -463,6 +516,7 @@ inline void release(void* buf, int64_t, float*) {
   if (c.pending && !c.capturing) flush();
   extent e;
   c.buffers.leave(buf, e);
+  c.forget_derived(e);
   if (e.staging) c.buffers.park(e);
   else c.f.free_(e.base);   // device-only extents are not kept for reuse
 }
@@ -610,16 +664,19 @@ inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int6
   if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0) return false;
   L.reads(a, B);
   L.writes(out);
+  if (m > 64)   // a prompt chunk: on the weight's prepared f16 form where there is one
+    if (const auto* p = L.prepared(B, n, k, false)) return L.sent(L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k));
   return L.sent(L.lib.gemm_bf16_nt(a, B, out, m, n, k));
 }
 
-// act[m, ff] = swiglu(a . gate^T, a . up^T) for B = [gate rows | up rows] ([2*ff, k] bf16):
 // gemm_bf16_nt + swiglu in one launch.
 inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t ff, int64_t k) {
   launch L;
   if (!L.ok || (k % 8) != 0 || m <= 0 || ff <= 0) return false;
   L.reads(a, B);
   L.writes(act);
+  if (m > 64)
+    if (const auto* p = L.prepared(B, ff, k, true)) return L.sent(L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k));
   return L.sent(L.lib.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
 }
 
@@ -657,45 +714,16 @@ inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_byte
   if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
   L.reads(a, B);
   L.writes(parts);
+  if (m > 64)
+    if (const auto* p = L.prepared(B, n, k, false))
+      return L.sent(L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts));
   return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
 }
 
-// The prepared form of a bf16 weight for prompt chunks (the library's f16 slab images and row
-// exponents): its size, its construction from the bf16 rows, and the three products over it.
-// No counterpart in the reference's seam; for a harness that owns its weights.
-inline int64_t gemm_f16w_bytes(int64_t n, int64_t k, bool gated) {
-  launch L;
-  return L.ok ? L.lib.gemm_f16w_bytes(n, k, gated ? 1 : 0) : 0;
-}
-inline bool gemm_f16w_prepare(void* B, int64_t n, int64_t k, bool gated, void* image, void* exps) {
-  launch L;
-  if (!L.ok || n <= 0 || k <= 0 || (k % 32) != 0) return false;
-  L.reads(B);
-  L.writes(image, exps);
-  return L.sent(L.lib.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, image, exps));
-}
-inline bool gemm_f16w_nt(void* a, void* image, void* exps, void* out, int64_t m, int64_t n, int64_t k) {
-  launch L;
-  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0) return false;
-  L.reads(a, image, exps);
-  L.writes(out);
-  return L.sent(L.lib.gemm_f16w_nt(a, image, exps, out, m, n, k));
-}
-inline bool gemm_f16w_nt_swiglu(void* a, void* image, void* exps, void* act, int64_t m, int64_t ff, int64_t k) {
-  launch L;
-  if (!L.ok || (k % 32) != 0 || m <= 0 || ff <= 0) return false;
-  L.reads(a, image, exps);
-  L.writes(act);
-  return L.sent(L.lib.gemm_f16w_nt_swiglu(a, image, exps, act, m, ff, k));
-}
-inline bool gemm_f16w_nt_parts(void* a, void* image, void* exps, void* parts, int64_t parts_bytes, int64_t m,
-                               int64_t n, int64_t k, int* n_parts) {
-  launch L;
-  if (!L.ok || (k % 32) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
-  L.reads(a, image, exps);
-  L.writes(parts);
-  return L.sent(L.lib.gemm_f16w_nt_parts(a, image, exps, parts, parts_bytes, m, n, k, n_parts));
-}
+// Prompt-chunk products over bf16 weights (the three above, m > 64) run on the library's prepared
+// f16 form of the weight, made and cached per weight on first use: `false` keeps them on the bf16
+// rows (and stops new images; existing ones stay until their buffer changes).
+inline void set_prompt_f16(bool on) { context::get().prompt_f16 = on; }
 
 inline bool attn_decode(void* q, void* K, void* V, void* out, int64_t n_q_heads, int64_t n_kv_heads,
                         int64_t ctx, int64_t kv_max, int64_t D, float scale, bool kv_bf16 = false) {

@@ -61,30 +61,8 @@ struct linear {
   void* w = nullptr;
   int64_t N = 0, K = 0;
   wfmt fmt = wfmt::q4;
-  // bf16 rows only, made on the first prompt chunk (prepare_prompt): the weight as f16 slab
-  // images with one exponent per row, the operand of the prompt-chunk products below
-  void* image = nullptr;
-  void* exps = nullptr;
   int64_t bytes() const { return fmt == wfmt::q4 ? q4_bytes(N, K) : N * K * 2; }
 };
-
-// The prepared form of a bf16 weight (gated: the fused [gate | up] rows). false leaves L as it
-// was and the prompt products on the bf16 rows.
-inline bool prepare_prompt(linear& L, bool gated) {
-  if (L.fmt != wfmt::bf16_row || L.image || (L.K % 32) != 0) return L.image != nullptr;
-  const int64_t n = gated ? L.N / 2 : L.N, bytes = hip::gemm_f16w_bytes(n, L.K, gated);
-  if (bytes <= 0) return false;
-  void* image = hip::alloc_device(bytes);
-  void* exps = hip::alloc_device((L.N + 15) & ~int64_t(15));
-  if (!image || !exps || !hip::gemm_f16w_prepare(L.w, n, L.K, gated, image, exps)) {
-    if (image) hip::release(image, 0, nullptr);
-    if (exps) hip::release(exps, 0, nullptr);
-    return false;
-  }
-  L.image = image;
-  L.exps = exps;
-  return true;
-}
 
 // y[N] = a[K] . W
 inline bool gemv(const linear& L, void* a, void* y) {
@@ -107,14 +85,12 @@ inline bool gemm_parts(const linear& L, void* a, void* parts, int64_t parts_byte
   if (L.fmt == wfmt::q4)
     return hip::gemm_q4_nt_parts(a, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, parts, parts_bytes, T, L.N,
                                  L.K, n_parts, kQ4Group);
-  if (L.image && T > 64) return hip::gemm_f16w_nt_parts(a, L.image, L.exps, parts, parts_bytes, T, L.N, L.K, n_parts);
   return hip::gemm_bf16_nt_parts(a, L.w, parts, parts_bytes, T, L.N, L.K, n_parts);
 }
 inline bool gemm_swiglu(const linear& L, void* a, void* act, int64_t T) {
   if (L.fmt == wfmt::q4)
     return hip::gemm_q4_nt_swiglu(a, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, act, T, L.N / 2, L.K,
                                   kQ4Group);
-  if (L.image && T > 64) return hip::gemm_f16w_nt_swiglu(a, L.image, L.exps, act, T, L.N / 2, L.K);
   return hip::gemm_bf16_nt_swiglu(a, L.w, act, T, L.N / 2, L.K);
 }
 
@@ -194,7 +170,7 @@ struct model {
   bool fused = true;
   bool fused_attn = true;   // within the fused path: q/k/v epilogue + append inside the attention launch
   bool fused_prefill = true;     // prompt chunks: one launch for split_heads + rope + kv_fill, attention writes token-major
-  bool prompt_f16 = true;        // prompt chunks of bf16 weights on their prepared f16 images (a second copy of the weights)
+  bool prompt_f16 = true;        // prompt chunks of bf16 weights on the backend's prepared f16 form of them (a second copy, made on first use)
   bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
 };
 
@@ -810,13 +786,7 @@ inline bool prefill_layers(model& M, int64_t T) {
   void* x = P.emb;
   ok &= hip::rmsnorm(x, M.layers[0].an, P.h, E, d.eps, T);
   const bool fused = M.fused_prefill;
-  if (fused && M.prompt_f16 && T > 64)   // first chunk: the f16 images of the bf16 weights (a refusal keeps the bf16 rows)
-    for (layer& L : M.layers) {
-      prepare_prompt(L.wqkv, false);
-      prepare_prompt(L.wo, false);
-      prepare_prompt(L.wgu, true);
-      prepare_prompt(L.wd, false);
-    }
+  hip::set_prompt_f16(M.prompt_f16);
   if (fused) ok &= hip::rope_table_range(P.rope, HD, pos0, T, d.rope_base);   // once for all layers
   for (int64_t l = 0; l < d.n_layers; l++) {
     layer& L = M.layers[(size_t)l];
