@@ -185,7 +185,7 @@ struct extent {
     size_t off = 0;            // of the weight inside the extent
     int64_t n = 0, k = 0;      // rows (gated: features) and depth
     bool gated = false;
-    void* image = nullptr;
+    void* image = nullptr;     // one allocation: the images, then the exponents
     void* exps = nullptr;
   };
   std::vector<prepared> derived;
@@ -367,10 +367,7 @@ struct context {
   // The extent's device bytes are changing: what was derived from them goes. (free_ drains the
   // device first, so a queued product that still reads an image finishes with it.)
   void forget_derived(extent& e) {
-    for (auto& d : e.derived) {
-      f.free_(d.image);
-      f.free_(d.exps);
-    }
+    for (auto& d : e.derived) f.free_(d.image);
     e.derived.clear();
   }
   // The prepared form of the bf16 weight B [n, k] (gated: [2n, k], gate rows | up rows), made now
@@ -387,11 +384,10 @@ struct context {
     if (bytes <= 0 || off + static_cast<size_t>(rows * k * 2) > e->size) return nullptr;
     extent::prepared d;
     d.off = off; d.n = n; d.k = k; d.gated = gated;
-    if (f.malloc_(&d.image, static_cast<size_t>(bytes)) != 0) return nullptr;
-    if (f.malloc_(&d.exps, static_cast<size_t>((rows + 15) & ~int64_t(15))) != 0 ||
-        f.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, d.image, d.exps) != 0) {
+    if (f.malloc_(&d.image, static_cast<size_t>(bytes + ((rows + 15) & ~int64_t(15)))) != 0) return nullptr;
+    d.exps = static_cast<char*>(d.image) + bytes;
+    if (f.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, d.image, d.exps) != 0) {
       f.free_(d.image);
-      if (d.exps) f.free_(d.exps);
       return nullptr;
     }
     pending = true;
@@ -659,12 +655,19 @@ inline bool gemv_q4(void* a, void* qw, void* scales, void* y, int64_t N, int64_t
   return L.sent(L.lib.gemv_q4(a, qw, scales, y, N, K, group));
 }
 
+// The prepared-weight products pay one more launch (the activation planes) and win it back on the
+// matrix cores only when the product is large: measured, from about 4 * 10^9 multiply-adds on
+// (512 x 4608 x 3584 gains 13 %, 512 x 896 x 4864 loses 10 %).
+inline bool prompt_product_is_large(int64_t m, int64_t n, int64_t k) {
+  return m > 64 && (double)m * (double)n * (double)k >= 4e9;
+}
+
 inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int64_t k) {
   launch L;
   if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0) return false;
   L.reads(a, B);
   L.writes(out);
-  if (m > 64)   // a prompt chunk: on the weight's prepared f16 form where there is one
+  if (prompt_product_is_large(m, n, k))   // on the weight's prepared f16 form where there is one
     if (const auto* p = L.prepared(B, n, k, false)) return L.sent(L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k));
   return L.sent(L.lib.gemm_bf16_nt(a, B, out, m, n, k));
 }
@@ -675,7 +678,7 @@ inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t 
   if (!L.ok || (k % 8) != 0 || m <= 0 || ff <= 0) return false;
   L.reads(a, B);
   L.writes(act);
-  if (m > 64)
+  if (prompt_product_is_large(m, 2 * ff, k))
     if (const auto* p = L.prepared(B, ff, k, true)) return L.sent(L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k));
   return L.sent(L.lib.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
 }
@@ -714,7 +717,7 @@ inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_byte
   if (!L.ok || (k % 8) != 0 || m <= 0 || n <= 0 || !n_parts) return false;
   L.reads(a, B);
   L.writes(parts);
-  if (m > 64)
+  if (prompt_product_is_large(m, n, k))
     if (const auto* p = L.prepared(B, n, k, false))
       return L.sent(L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts));
   return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
