@@ -460,8 +460,14 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
       return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: too many tiles for one grid");
     const dim3 grid((unsigned)nblk, (unsigned)S);
     auto launch = [&](auto fn) -> hipError_t {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return e;
+      // more than 64 KB of LDS per block has to be asked for once per kernel (and device)
+      static int asked_on[2] = {-1, -1};             // per instantiation of this lambda: [tile height - 1]
+      if (asked_on[P.tmh - 1] != c.device) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)((size_t)f16t::kRing * (2 * 128 * P.tmh * f16t::kRowBytes + f16t::kWImage)));
+        if (e != hipSuccess) return e;
+        asked_on[P.tmh - 1] = c.device;
+      }
       fn<<<grid, dim3(512), lds, c.stream>>>(aimg, static_cast<const char*>(image), dst, (int)M, (int)pn, (int)nslab,
                                              part_slabs, ldc, (int)P.tn0, (int)N, ea, static_cast<const int8_t*>(exps));
       return hipSuccess;
