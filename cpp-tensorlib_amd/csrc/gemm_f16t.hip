@@ -223,13 +223,15 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
       for (int p = 0; p < 2; p++)
         af[ks][i][p] = *reinterpret_cast<const frag16*>(stage + aoff[ks] + p * kAPlane + i * 32 * kRowBytes);
   };
-  // four products: fragment set KS, (tile row, plane) pair Q against the four tile columns
+  // four products: fragment set KS, (tile row, plane) pair Q against the four tile columns. The
+  // weight fragment is the MFMA's first operand: the tile comes out transposed, D[n][m], so that a
+  // lane ends up with four consecutive COLUMNS of one row of C - a 16-byte store, not four 4-byte ones.
   auto mul4 = [&](auto KS, auto Q) {
     constexpr int ks = decltype(KS)::value, q = decltype(Q)::value;
 #pragma unroll
     for (int j = 0; j < 4; j++)
-      acc[q >> 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[ks][q >> 1][q & 1]),
-                                                              __builtin_bit_cast(f16x8, bf[ks][j]), acc[q >> 1][j], 0, 0, 0);
+      acc[q >> 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, bf[ks][j]),
+                                                              __builtin_bit_cast(f16x8, af[ks][q >> 1][q & 1]), acc[q >> 1][j], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
   // The block's barrier without the fence __syncthreads() puts before it: that fence would wait for
@@ -316,48 +318,83 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
 #endif
 #undef TLHIP_PHASE
 
-  // acc[v] of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32x32 tile. The exponents
-  // come back out, -(ea[row] + ew[W row of the column]); ldexpf is exact.
-  int ec[4];
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int r = weight_row(GU, tn, wn * 128 + j * 32 + (lane & 31), N + (GU ? tn0 * 128 : tn0 * kTile), ff);
-    ec[j] = r >= 0 ? (int)ew[r] : 0;
-  }
+  // acc[v] of lane l (transposed tile): column of C 8*(v/4) + 4*(l/32) + v%4 of the tile, row of C
+  // l%32. Four consecutive v are four consecutive columns: one 16-byte store where the row stride
+  // allows it. The exponents come back out, -(ea[row] + ew[W row of the column]); ldexpf is exact.
   const int ltn = tn - tn0;                          // column tile within this launch
+  const int nlim = N + (GU ? tn0 * 128 : tn0 * kTile);   // first unit of N past this launch, absolute
+  const bool wide = (ldc & 3) == 0;
+  // exponents of the W rows behind tile columns c .. c + 3 of this block
+  auto wexp4 = [&](int c, int e4[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int r = weight_row(GU, tn, c + e, nlim, ff);
+      e4[e] = r >= 0 ? (int)ew[r] : 0;
+    }
+  };
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
   if (GU && gridDim.y == 1) {
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < TM; i++) {
+      const int gm = tm * BM + wm * 32 * TM + i * 32 + (lane & 31);
+      if (gm >= M) continue;
+      const int em = ea[gm];
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int gm = tm * BM + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (gm >= M) continue;
-        const int em = ea[gm];
+      for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-          const int f = ltn * 128 + wn * 64 + j * 32 + (lane & 31);
+        for (int g = 0; g < 4; g++) {
+          const int c = wn * 128 + j * 32 + 8 * g + 4 * (lane >> 5);      // gate column of the tile; its up value is 64 further
+          const int f = ltn * 128 + wn * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
           if (f >= N) continue;
-          const float g = ldexpf(acc[i][j][v], -(em + ec[j])), sg = 1.0f / (1.0f + expf(-g));
-          C[(size_t)gm * ldc + f] = (g * sg) * ldexpf(acc[i][j + 2][v], -(em + ec[j + 2]));
+          int eg[4], eu[4];
+          wexp4(c, eg);
+          wexp4(c + 64, eu);
+          f32x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float gt = ldexpf(acc[i][j][4 * g + e], -(em + eg[e])), sg = 1.0f / (1.0f + expf(-gt));
+            o[e] = (gt * sg) * ldexpf(acc[i][j + 2][4 * g + e], -(em + eu[e]));
+          }
+          float* dst = C + (size_t)gm * ldc + f;
+          if (wide && f + 3 < N) {
+            *reinterpret_cast<f32x4*>(dst) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (f + e < N) dst[e] = o[e];
+          }
         }
-      }
+    }
     TLHIP_MARK(6);
     return;
   }
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+  for (int i = 0; i < TM; i++) {
+    const int gm = tm * BM + wm * 32 * TM + i * 32 + (lane & 31);
+    if (gm >= M) continue;
+    const int em = ea[gm];
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const int gm = tm * BM + wm * 32 * TM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-      if (gm >= M) continue;
-      const int em = ea[gm];
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int gn = ltn * kTile + wn * 128 + j * 32 + (lane & 31);
+      for (int g = 0; g < 4; g++) {
+        const int c = wn * 128 + j * 32 + 8 * g + 4 * (lane >> 5);
+        const int gn = ltn * kTile + c;
         if (!GU && gn >= N) continue;   // gated parts are whole tiles wide
-        C[(size_t)gm * ldc + gn] = ldexpf(acc[i][j][v], -(em + ec[j]));
+        int e4[4];
+        wexp4(c, e4);
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = ldexpf(acc[i][j][4 * g + e], -(em + e4[e]));
+        float* dst = C + (size_t)gm * ldc + gn;
+        if (wide && (GU || gn + 3 < N)) {
+          *reinterpret_cast<f32x4*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (GU || gn + e < N) dst[e] = o[e];
+        }
       }
-    }
+  }
   TLHIP_MARK(6);
 }
 
