@@ -278,7 +278,7 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
     TLHIP_PHASE(0);
     // my reads of slab k are complete and my copies of slab k + 1 have landed (those of slab
     // k + 2 may still be in flight); past the barrier that holds for every wavefront
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
     barrier();
     TLHIP_PHASE(1);
     // slab k + 3 into the stage slab k has just left
