@@ -228,6 +228,52 @@ int main() {
     check("rope", ok);
   }
 
+  {  // a large prompt product runs on a form of the bf16 weight the header prepares once and keeps
+     // with the buffer: a host edit of the weight and a device-side overwrite must both reach the
+     // next product, and switching the prepared form off must give the same rows
+    const int64_t m = 512, n = 1024, k = 8192;      // m * n * k = 4.3e9: large enough to be prepared
+    buf a(m * k), w(n * k / 2), w2(n * k / 2), o(m * n);
+    fill(a);
+    auto fill_bf16 = [&](buf& b, float scale) {     // two bf16 per float slot
+      uint16_t* p = reinterpret_cast<uint16_t*>(b.write());
+      for (int64_t i = 0; i < n * k; i++) {
+        const float v = scale * rnd();
+        uint32_t u;
+        std::memcpy(&u, &v, 4);
+        p[i] = (uint16_t)(u >> 16);
+      }
+    };
+    auto widen = [](uint16_t h) { const uint32_t u = (uint32_t)h << 16; float f; std::memcpy(&f, &u, 4); return f; };
+    auto rows_match = [&](buf& wb, const char* what) {
+      std::vector<uint16_t> hw(reinterpret_cast<const uint16_t*>(wb.host), reinterpret_cast<const uint16_t*>(wb.host) + n * k);
+      std::vector<float> ha(a.host, a.host + a.n);
+      const float* got = o.read();
+      for (int64_t r : {int64_t(0), m / 2, m - 1})
+        for (int64_t c : {int64_t(0), int64_t(17), n - 1}) {
+          double want = 0;
+          for (int64_t i = 0; i < k; i++) want += (double)ha[r * k + i] * (double)widen(hw[c * k + i]);
+          if (!close(got[r * n + c], want)) {
+            std::printf("  %s at (%lld, %lld): got %.9g want %.9g\n", what, (long long)r, (long long)c, got[r * n + c], want);
+            return false;
+          }
+        }
+      return true;
+    };
+    fill_bf16(w, 0.05f);
+    fill_bf16(w2, 0.3f);
+    bool ok = hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "first product");
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "second product (cached form)");
+    reinterpret_cast<uint16_t*>(w.write())[17 * k + 5] = 0x4080;          // host edit: one weight becomes 4.0
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "after a host edit");
+    w2.read();                                                              // keep w2's host half current for the comparison
+    ok = ok && hip::copy_d2d(w.native, w2.native, n * k * 2);             // device-side overwrite
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w2, "after a device copy into the weight");
+    hip::set_prompt_f16(false);
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w2, "on the bf16 rows");
+    hip::set_prompt_f16(true);
+    check("prepared weight follows host edits and device writes of its buffer", ok);
+  }
+
   {  // pool: a released buffer comes back for the same size, contents pointer included
     float* h1 = nullptr;
     void* n1 = hip::alloc(4096, &h1);
