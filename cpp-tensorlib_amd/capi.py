@@ -488,7 +488,7 @@ class TlHip:
                                                 1 if kv_bf16 else 0, pos0))
 
     def tune_attn_prefill(self, kernel):
-        """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes."""
+        """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes, 4: f16 terms."""
         self._chk(self.c.tlhip_tune_attn_prefill(int(kernel)))
 
     def tune_gemm_planes(self, planes):

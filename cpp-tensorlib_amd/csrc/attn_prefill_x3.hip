@@ -14,8 +14,19 @@
 // plane for K and V and three products. Scores and outputs then differ from an fp32 loop by
 // what a different summation order would give.
 //
+// The f16 form (what the library picks; the bf16 planes remain selectable) does the same with TWO
+// f16 terms per operand, each rounded to nearest, and the three term pairs a1b1 + (a1b2 + a2b1);
+// a2b2 <= 2^-24 |ab| is dropped - three MFMAs per product instead of six, two instead of three
+// over a bf16 cache. f16 has 11 significant bits but a narrow exponent, so the
+// operand is first multiplied by a power of two that brings its block's largest magnitude into
+// [2^14, 2^15): one exponent per query row, one each for K and V per 32-key tile (kept beside the
+// planes). Two terms then carry 23 bits of a value whose magnitude is within 2^14 of its block's
+// largest and an absolute 2^-39 of that largest below. The Q and K exponents leave through the
+// score scale; P enters as p * 2^14 and the output accumulators move from one tile's V exponent to
+// the next in the multiplication that applies the softmax correction.
+//
 // Three kernels per call:
-//  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into planes, written
+//  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into planes (or terms), written
 //     as the exact register image of the MFMA operands, one 32-key tile after the other:
 //       K image [plane][k-step][16-key half 0..1][lane][8]  = K[32t + 16h + l%16][32s + 8(l/16) + j]
 //       V image [plane][16-column tile][lane][8]            = V[32t + tile_key(l/16, j)][16d + l%16]
@@ -30,8 +41,8 @@
 //     (S^T = K . Q^T, O^T = V^T . P^T): a lane's scores, probabilities and output columns all
 //     belong to one query row, so the softmax needs no exchange through LDS and P goes from
 //     the score registers - cut into planes - straight back into the matrix core.
-//     Per tile and wavefront: 96 MFMAs for the scores, an online-softmax update on 16 scores
-//     per lane, 96 MFMAs for P.V.
+//     Per tile and wavefront (head size 128, f32 cache): 96 MFMAs for the scores, an online-softmax
+//     update on 16 scores per lane, 96 MFMAs for P.V; 48 and 48 in the f16 form.
 //     S == 1 writes the normalised rows; S > 1 leaves (max, sum, accumulator) per split and
 //  3. attn_x3_merge_kernel combines them in split order.
 #include "common.hpp"
@@ -99,49 +110,133 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 u) {
   return t.v;
 }
 
+// The f16 form (template flag H): an operand, first multiplied by a power of two that brings it
+// into the f16 range, is cut into TWO f16 terms, both rounded to nearest (2^-24 relative while
+// the second term is a normal f16), and a product is formed from the three term pairs that hold
+// a first term - three MFMAs where the bf16 planes need six.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void split2x8_f16(const float (&x)[8], float s, uint4& p1, uint4& p2) {
+  uint32_t a[4], b[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const f32x2 v = {x[2 * j] * s, x[2 * j + 1] * s};
+    const f16x2 h = __builtin_convertvector(v, f16x2);
+    const f16x2 l = __builtin_convertvector(v - __builtin_convertvector(h, f32x2), f16x2);
+    a[j] = __builtin_bit_cast(uint32_t, h);
+    b[j] = __builtin_bit_cast(uint32_t, l);
+  }
+  p1 = make_uint4(a[0], a[1], a[2], a[3]);
+  p2 = make_uint4(b[0], b[1], b[2], b[3]);
+}
+__device__ __forceinline__ void split2x8_f16(const float (&x)[8], uint4& p1, uint4& p2) {   // (already in range)
+  uint32_t a[4], b[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const f32x2 v = {x[2 * j], x[2 * j + 1]};
+    const f16x2 h = __builtin_convertvector(v, f16x2);
+    const f16x2 l = __builtin_convertvector(v - __builtin_convertvector(h, f32x2), f16x2);
+    a[j] = __builtin_bit_cast(uint32_t, h);
+    b[j] = __builtin_bit_cast(uint32_t, l);
+  }
+  p1 = make_uint4(a[0], a[1], a[2], a[3]);
+  p2 = make_uint4(b[0], b[1], b[2], b[3]);
+}
+// exponent that brings a largest magnitude (as f32 bits, sign cleared) into [2^14, 2^15); 0 for 0
+__device__ __forceinline__ int f16_exponent(uint32_t maxbits) {
+  return maxbits == 0 ? 0 : max(-100, min(100, 14 - ((int)(maxbits >> 23) - 127)));
+}
+__device__ __forceinline__ float pow2i(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // e in [-126, 127]
+template <bool H>
+__device__ __forceinline__ f32x4 mma16(const u32x4 a, const u32x4 b, f32x4 c) {
+  if (H) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ u32x4 as_u32x4(const uint4& u) { return u32x4{u.x, u.y, u.z, u.w}; }
+
 __device__ __forceinline__ float cache_elem(const float* p) { return *p; }
 __device__ __forceinline__ float cache_elem(const uint16_t* p) { return bf16_bits_to_f32(*p); }
 
 // ---- 1. planes ---------------------------------------------------------------------------
-// grid = (tiles, Hkv), block = 256. NP = 3 for an f32 cache, 1 for a bf16 cache.
+// grid = (tiles, Hkv), block = 256. NP planes: bf16 form 3 for an f32 cache, 1 for a bf16 cache;
+// f16 form (H) 2 and 1.
 // planes: per (kv head, tile) a K image of NP * kKUnits uint4, then a V image of NP * kVUnits uint4.
-template <typename KT, int NP, int D>
+// H: K and V of a tile are scaled by 2^ek and 2^ev, one exponent each per tile (from the tile's
+// largest magnitude), left in texp[(kv head * tiles + tile) * 2 + {0, 1}]; the attention kernel
+// folds them into its score scale and its running output scale.
+template <typename KT, int NP, int D, bool H>
 __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K, const KT* __restrict__ V,
-                                                        uint4* __restrict__ planes, int64_t kv_stride,
-                                                        int kend, int ntiles) {
+                                                        uint4* __restrict__ planes, int* __restrict__ texp,
+                                                        int64_t kv_stride, int kend, int ntiles) {
   constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
+  constexpr int kPer = (kKUnits + kVUnits) / 256;       // units per thread: the first half of them K, the rest V
+  static_assert(kKUnits % 256 == 0 && kVUnits % 256 == 0, "a thread's units are all K or all V per step");
+  __shared__ uint32_t red[2][4];
   const int t = blockIdx.x, kvh = blockIdx.y;
   const KT* Kh = K + (size_t)kvh * kv_stride;
   const KT* Vh = V + (size_t)kvh * kv_stride;
   uint4* img = planes + ((size_t)kvh * ntiles + t) * (size_t)(NP * (kKUnits + kVUnits));
-  for (int u = threadIdx.x; u < kKUnits + kVUnits; u += 256) {
-    float x[8];
-    uint4* dst;
-    int plane_stride;
+  float x[kPer][8];
+  uint32_t mxk = 0, mxv = 0;
+#pragma unroll
+  for (int i = 0; i < kPer; i++) {
+    const int u = threadIdx.x + 256 * i;
     if (u < kKUnits) {
       const int l = u & 63, half = (u >> 6) & 1, ks = u >> 7;
       const int key = t * kTile + 16 * half + (l & 15), dim = 32 * ks + 8 * (l >> 4);
       const bool live = key < kend;
       const KT* src = Kh + (size_t)min(key, kend - 1) * kD + dim;
 #pragma unroll
-      for (int j = 0; j < 8; j++) x[j] = live ? cache_elem(src + j) : 0.f;
-      dst = img + u;
-      plane_stride = kKUnits;
+      for (int j = 0; j < 8; j++) x[i][j] = live ? cache_elem(src + j) : 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) mxk = max(mxk, __float_as_uint(x[i][j]) & 0x7fffffffu);
     } else {
       const int v = u - kKUnits, l = v & 63, dt = v >> 6;
       const int dim = 16 * dt + (l & 15);
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const int key = t * kTile + tile_key(l >> 4, j);
-        x[j] = key < kend ? cache_elem(Vh + (size_t)key * kD + dim) : 0.f;
+        x[i][j] = key < kend ? cache_elem(Vh + (size_t)key * kD + dim) : 0.f;
       }
-      dst = img + NP * kKUnits + v;
-      plane_stride = kVUnits;
+#pragma unroll
+      for (int j = 0; j < 8; j++) mxv = max(mxv, __float_as_uint(x[i][j]) & 0x7fffffffu);
     }
+  }
+  float sk = 1.0f, sv = 1.0f;
+  if (H) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      mxk = max(mxk, (uint32_t)__shfl_xor((int)mxk, d));
+      mxv = max(mxv, (uint32_t)__shfl_xor((int)mxv, d));
+    }
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = mxk; red[1][threadIdx.x >> 6] = mxv; }
+    __syncthreads();
+    mxk = max(max(red[0][0], red[0][1]), max(red[0][2], red[0][3]));
+    mxv = max(max(red[1][0], red[1][1]), max(red[1][2], red[1][3]));
+    const int ek = f16_exponent(mxk), ev = f16_exponent(mxv);
+    if (threadIdx.x == 0) {
+      texp[((size_t)kvh * ntiles + t) * 2] = ek;
+      texp[((size_t)kvh * ntiles + t) * 2 + 1] = ev;
+    }
+    sk = pow2i(ek);
+    sv = pow2i(ev);
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; i++) {
+    const int u = threadIdx.x + 256 * i;
+    const bool isk = u < kKUnits;
+    uint4* dst = isk ? img + u : img + NP * kKUnits + (u - kKUnits);
+    const int plane_stride = isk ? kKUnits : kVUnits;
     uint4 p1, p2, p3;
-    split3x8(x, p1, p2, p3);
-    dst[0] = p1;
-    if (NP == 3) { dst[plane_stride] = p2; dst[2 * plane_stride] = p3; }
+    if (H) {
+      split2x8_f16(x[i], isk ? sk : sv, p1, p2);
+      dst[0] = p1;
+      if (NP == 2) dst[plane_stride] = p2;
+    } else {
+      split3x8(x[i], p1, p2, p3);
+      dst[0] = p1;
+      if (NP == 3) { dst[plane_stride] = p2; dst[2 * plane_stride] = p3; }
+    }
   }
 }
 
@@ -172,12 +267,16 @@ struct Geometry {
 // (w and w + 4) are therefore never in the same kind of phase: one feeds the matrix core while
 // the other is on the vector ALU. Interval i needs K of tile i and V of tile i-1 in LDS.
 constexpr int kRT = 2;          // 16-row tiles per computing wavefront
+constexpr int kF16Weight = 1;   // f16 form: term pairs (a, b) with a + b <= this; 1 leaves out lo x lo, <= 2^-24 |a b|
 constexpr int kCompute = 7;     // computing wavefronts per block
 
-template <int NP, int D>
+template <int NP, int D, bool H>
 __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict__ q, const uint4* __restrict__ planes,
+                                                          const int* __restrict__ texp,
                                                           float* __restrict__ out, float* __restrict__ part_o,
                                                           float* __restrict__ part_ml, float scale, const Geometry g) {
+  constexpr int QP = H ? 2 : 3;                               // planes of Q and of P
+  constexpr int kW = H ? kF16Weight : 2;                      // products keep the plane pairs (a, b) with a + b <= this
   constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
   constexpr int kKS = D / 32, kDT = D / 16;                   // k-steps of Q.K^T, column tiles of P.V
   constexpr int kKImg = NP * kKUnits, kVImg = NP * kVUnits;   // 16-byte units of a tile's K and V images
@@ -199,6 +298,7 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
   const int n = nkt_blk > split ? (nkt_blk - split + g.S - 1) / g.S : 0;   // this block's tiles: split, split + S, ...
   const auto tile_of = [&](int i) { return split + i * g.S; };
   const u32x4* img0 = reinterpret_cast<const u32x4*>(planes) + (size_t)kvh * g.ntiles * kImg;
+  const int* texp0 = texp + (size_t)kvh * g.ntiles * 2;     // H: (ek, ev) of each tile of this kv head
 
   if (wave == kCompute) {
     // ---- the copying wavefront (branch-free: tiles past the range are clamped, parked, never read) ----
@@ -250,23 +350,57 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
   // lanes c, c+16, c+32, c+48, which meet in two register swaps.
 
   // ---- the wavefront's query rows as operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
-  uint4 qa[kRT][3][kKS];
+  uint4 qa[kRT][QP][kKS];
+  int eq[kRT];                        // H: exponent the row was scaled by
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
     const float* qrow = q + ((size_t)h * g.T + min(p_first + 16 * rt + l15, g.T - 1)) * kD;
+    float x[kKS][8];
+    uint32_t mx = 0;
 #pragma unroll
     for (int ks = 0; ks < kKS; ks++) {
       const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq);
       const float4 b = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq + 4);
-      const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-      split3x8(x, qa[rt][0][ks], qa[rt][1][ks], qa[rt][2][ks]);
+      x[ks][0] = a.x; x[ks][1] = a.y; x[ks][2] = a.z; x[ks][3] = a.w;
+      x[ks][4] = b.x; x[ks][5] = b.y; x[ks][6] = b.z; x[ks][7] = b.w;
+      if (scale < 0.f) {   // the sign of the scale goes into Q: the softmax below multiplies by |scale|
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[ks][j] = -x[ks][j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) mx = max(mx, __float_as_uint(x[ks][j]) & 0x7fffffffu);
+    }
+    eq[rt] = 0;
+    if (H) {   // the row's largest magnitude: its dims are spread over the 4 lanes c, c+16, c+32, c+48
+      LanePair e = swap16(__uint_as_float(mx), __uint_as_float(mx));
+      mx = max(__float_as_uint(e.first), __float_as_uint(e.second));
+      e = swap32(__uint_as_float(mx), __uint_as_float(mx));
+      mx = max(__float_as_uint(e.first), __float_as_uint(e.second));
+      eq[rt] = f16_exponent(mx);
+    }
+#pragma unroll
+    for (int ks = 0; ks < kKS; ks++) {
+      if (H) split2x8_f16(x[ks], pow2i(eq[rt]), qa[rt][0][ks], qa[rt][1][ks]);
+      else split3x8(x[ks], qa[rt][0][ks], qa[rt][1][ks], qa[rt][QP - 1][ks]);
     }
   }
 
   f32x4 o[kRT][kDT];                  // O^T: columns 16 dt + 4(l/16) + r of row l%16
   float mrow[kRT], lrow[kRT];         // row l%16: running maximum; this lane's share of the running sum
   f32x4 s[kRT][2];                    // S^T of the tile whose softmax is pending: keys 16 h + 4(l/16) + r
-  uint4 pa3[kRT][3];                  // P planes of the tile whose P.V is pending
+  uint4 pa3[kRT][QP];                 // P planes of the tile whose P.V is pending
+  // H: P of a tile enters its MFMAs as p * 2^14 against V * 2^ev(tile), so the tile's products come
+  // in units of 2^-(14 + ev(tile)). The output accumulators are kept in the unit of the tile last
+  // added, 2^-(14 + unit): moving on to the next tile multiplies them by 2^(unit' - unit) in the
+  // same multiplication as the softmax correction. unit = ev(tile), except that it stays within
+  // kUnitSpan of the smallest ev seen (the largest V): a tile whose values are more than 2^64 below
+  // an earlier tile's gets its P scaled down instead, which keeps the accumulators far from overflow.
+  constexpr int kUnitSpan = 64;
+  int evmin = 1 << 20, unit = 0;
+  // (ek, ev) of the tile whose softmax comes next: asked for one tile ahead, so that the load's
+  // latency passes behind a matrix phase
+  int2 next_exp = make_int2(0, 0);
+  if (H) next_exp = *reinterpret_cast<const int2*>(texp0 + 2 * min(tile_of(0), g.ntiles - 1));
 #pragma unroll
   for (int rt = 0; rt < kRT; rt++) {
 #pragma unroll
@@ -274,43 +408,73 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
     mrow[rt] = -INFINITY;
     lrow[rt] = 0.f;
     s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    pa3[rt][0] = pa3[rt][1] = pa3[rt][2] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int pl = 0; pl < QP; pl++) pa3[rt][pl] = make_uint4(0, 0, 0, 0);
   }
 
   // the vector phase of tile number i: masks, running maximum and sum, rescale of the output
-  // accumulators, P cut into planes
+  // accumulators, P cut into planes. Scores are taken to base-2 units (score * |scale| * log2 e) in
+  // the same fused multiply-add that subtracts the running maximum; mrow is kept in those units.
+  const float ascale = fabsf(scale) * 1.44269504088896341f;
   const auto softmax_tile = [&](int i) {
     const int kt = tile_of(i);
     // only a tile that reaches past the first row's causal limit (or the chunk's last key) needs masks
     const bool masked = (kt + 1) * kTile - 1 > min(g.pos0 + p_first, kend - 1);   // (uniform for the wavefront)
+    int ek = 0, down = 0, pexp = 0;   // H: P enters the MFMAs as p * 2^pexp
+    if (H) {
+      ek = next_exp.x;
+      const int ev = next_exp.y;
+      next_exp = *reinterpret_cast<const int2*>(texp0 + 2 * min(tile_of(i + 1), g.ntiles - 1));
+      evmin = min(evmin, ev);
+      const int nunit = min(ev, evmin + kUnitSpan);
+      down = max(nunit - unit, -200);              // (the first tile finds the accumulators at zero)
+      pexp = max(14 + nunit - ev, -120);
+      unit = nunit;
+    }
 #pragma unroll
     for (int rt = 0; rt < kRT; rt++) {
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = s[rt][j >> 2][j & 3] * scale;
+      const float c2 = H ? ldexpf(ascale, -(eq[rt] + ek)) : ascale;
+      float v[8], mx;
       if (masked) {
         const int limit = min(g.pos0 + p_first + 16 * rt + l15, kend - 1);   // last key the row sees
 #pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = kt * kTile + tile_key(lq, j) <= limit ? v[j] : -INFINITY;
+        for (int j = 0; j < 8; j++) v[j] = kt * kTile + tile_key(lq, j) <= limit ? s[rt][j >> 2][j & 3] * c2 : -INFINITY;
+        mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = s[rt][j >> 2][j & 3];
+        mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7]))) * c2;   // c2 >= 0
       }
-      float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
       LanePair e = swap16(mx, mx);
       mx = fmaxf(e.first, e.second);
       e = swap32(mx, mx);
       mx = fmaxf(e.first, e.second);               // over the row's 32 keys
       const float mnew = fmaxf(mrow[rt], mx);
       const float mref = mnew == -INFINITY ? 0.f : mnew;
-      const float corr = __expf(mrow[rt] - mref);
+      const float lcorr = __builtin_amdgcn_exp2f(mrow[rt] - mref);
+      const float off = (float)pexp - mref;
       float p[8];
+      if (masked) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) p[j] = __expf(v[j] - mref);
-      lrow[rt] = lrow[rt] * corr + (((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7])));
-      mrow[rt] = mnew;
+        for (int j = 0; j < 8; j++) p[j] = __builtin_amdgcn_exp2f(v[j] + off);
+      } else {
 #pragma unroll
-      for (int dt = 0; dt < kDT; dt++) {
-        o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
+        for (int j = 0; j < 8; j++) p[j] = __builtin_amdgcn_exp2f(fmaf(v[j], c2, off));
       }
-      split3x8(p, pa3[rt][0], pa3[rt][1], pa3[rt][2]);
+      const float psum = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      lrow[rt] = fmaf(lrow[rt], lcorr, H ? ldexpf(psum, -pexp) : psum);
+      mrow[rt] = mnew;
+      const float corr = H ? ldexpf(lcorr, down) : lcorr;
+      // deep in a context the running maximum of a row seldom moves: skip the 64 multiplications
+      // when no row of the tile needs them
+      if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < kDT; dt++) {
+          o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
+        }
+      }
+      if (H) split2x8_f16(p, pa3[rt][0], pa3[rt][1]);
+      else split3x8(p, pa3[rt][0], pa3[rt][1], pa3[rt][QP - 1]);
     }
   };
   const auto mine = [&](int i) { return active && i >= 0 && i < n && tile_of(i) * kTile <= my_last_key; };
@@ -336,22 +500,22 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
       // never waits for the result of the one issued just before it
 #pragma unroll
       for (int dt = 0; dt < kDT; dt += 2) {
-        bf16x8 vb[2][NP];
+        u32x4 vb[2][NP];
 #pragma unroll
         for (int d2 = 0; d2 < 2; d2++)
 #pragma unroll
-          for (int p = 0; p < NP; p++) vb[d2][p] = as_bf16x8(vimg[p * kVUnits + (dt + d2) * 64 + lane]);
+          for (int p = 0; p < NP; p++) vb[d2][p] = vimg[p * kVUnits + (dt + d2) * 64 + lane];
 #pragma unroll
-        for (int w = 2; w >= 0; w--)
+        for (int w = kW; w >= 0; w--)
 #pragma unroll
           for (int pb = NP - 1; pb >= 0; pb--) {
             const int pa = w - pb;
-            if (pa >= 0 && pa <= 2) {
+            if (pa >= 0 && pa < QP) {
 #pragma unroll
               for (int d2 = 0; d2 < 2; d2++)
 #pragma unroll
                 for (int rt = 0; rt < kRT; rt++)
-                  o[rt][dt + d2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb[d2][pb], as_bf16x8(pa3[rt][pa]), o[rt][dt + d2], 0, 0, 0);
+                  o[rt][dt + d2] = mma16<H>(vb[d2][pb], as_u32x4(pa3[rt][pa]), o[rt][dt + d2]);
             }
           }
       }
@@ -362,22 +526,22 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
       for (int rt = 0; rt < kRT; rt++) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < kKS; ks++) {
-        bf16x8 kb[2][NP];
+        u32x4 kb[2][NP];
 #pragma unroll
         for (int hf = 0; hf < 2; hf++)
 #pragma unroll
-          for (int p = 0; p < NP; p++) kb[hf][p] = as_bf16x8(kimg[p * kKUnits + (ks * 2 + hf) * 64 + lane]);
+          for (int p = 0; p < NP; p++) kb[hf][p] = kimg[p * kKUnits + (ks * 2 + hf) * 64 + lane];
 #pragma unroll
-        for (int w = 2; w >= 0; w--)
+        for (int w = kW; w >= 0; w--)
 #pragma unroll
           for (int pb = NP - 1; pb >= 0; pb--) {
             const int pa = w - pb;
-            if (pa >= 0 && pa <= 2) {
+            if (pa >= 0 && pa < QP) {
 #pragma unroll
               for (int hf = 0; hf < 2; hf++)
 #pragma unroll
                 for (int rt = 0; rt < kRT; rt++)
-                  s[rt][hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[hf][pb], as_bf16x8(qa[rt][pa][ks]), s[rt][hf], 0, 0, 0);
+                  s[rt][hf] = mma16<H>(kb[hf][pb], as_u32x4(qa[rt][pa][ks]), s[rt][hf]);
             }
           }
       }
@@ -411,8 +575,9 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
     e = swap32(lsum, lsum);
     lsum = e.first + e.second;
     if (p >= g.T) continue;
+    const int back = H ? -(14 + unit) : 0;   // H: the accumulators are in units of 2^-(14 + unit)
     if (g.S == 1) {
-      const float inv = 1.0f / lsum;
+      const float inv = H ? ldexpf(1.0f / lsum, back) : 1.0f / lsum;
       float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row + 4 * lq;
 #pragma unroll
       for (int dt = 0; dt < kDT; dt++)
@@ -423,7 +588,9 @@ __global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict
       float* po = part_o + ((size_t)split * rows + row) * kD + 4 * lq;
 #pragma unroll
       for (int dt = 0; dt < kDT; dt++)
-        *reinterpret_cast<float4*>(po + 16 * dt) = make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+        *reinterpret_cast<float4*>(po + 16 * dt) =
+            H ? make_float4(ldexpf(o[rt][dt][0], back), ldexpf(o[rt][dt][1], back), ldexpf(o[rt][dt][2], back), ldexpf(o[rt][dt][3], back))
+              : make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
       if (lq == 0) {
         part_ml[((size_t)split * rows + row) * 2] = mrow[rt];
         part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
@@ -450,7 +617,7 @@ __global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restr
   float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
   for (int s = 0; s < S; s++) {
     const float m = part_ml[((size_t)s * rows + row) * 2];
-    const float f = m == -INFINITY ? 0.f : __expf(m - M);
+    const float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);   // maxima are in base-2 units
     L = fmaf(part_ml[((size_t)s * rows + row) * 2 + 1], f, L);
     const float4 v = *reinterpret_cast<const float4*>(part_o + ((size_t)s * rows + row) * kD + c4);
     a.x = fmaf(v.x, f, a.x); a.y = fmaf(v.y, f, a.y); a.z = fmaf(v.z, f, a.z); a.w = fmaf(v.w, f, a.w);
@@ -462,23 +629,25 @@ __global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restr
 
 }  // namespace x3
 
-// Whether the bf16-plane kernels serve this call: head size 64 or 128 and enough keys for the
-// extra passes to pay (measured crossover against the fp32 matrix-pipe kernel at the 7B and
-// 0.5B head shapes: about 1024 keys at head size 128, about 2048 at 64).
+// Whether the matrix-core kernels serve this call: head size 64 or 128 and enough keys for the
+// extra passes to pay. Measured crossover of the f16 form against the fp32 matrix-pipe kernel at the
+// 7B and 0.5B head shapes, in query-key pairs of one head (T pos0 + T^2 / 2): about 200 thousand at
+// head size 128, 300 thousand at 64; short chunks deep in a context stay with the older rule by keys.
 bool prefill_x3_applies(int D, int T, int pos0) {
   if (T < 16) return false;
-  if (D == 128) return pos0 + T >= 1024;
-  if (D == 64) return pos0 + T >= 2048;
+  const int64_t keys = (int64_t)pos0 + T, pairs = (int64_t)T * pos0 + (int64_t)T * T / 2;
+  if (D == 128) return keys >= 1024 || (keys >= 768 && pairs >= 200000);
+  if (D == 64) return keys >= 2048 || pairs >= 300000;
   return false;
 }
 
 // Launches the three kernels. Returns 0 when launched, a negative status on failure, 1 when the
 // scratch for the planes could not be had (the caller then uses the fp32 matrix-pipe kernel).
-template <int D, typename KT>
-int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
-                      int64_t kv_max, float scale, int pos0, int token_major) {
+template <int D, typename KT, bool H>
+static int launch_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
+                     int64_t kv_max, float scale, int pos0, int token_major) {
   using namespace x3;
-  constexpr int NP = sizeof(KT) == 4 ? 3 : 1;
+  constexpr int NP = sizeof(KT) == 4 ? (H ? 2 : 3) : 1;
   constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
   Context& c = ctx();
   Geometry g{};
@@ -507,20 +676,22 @@ int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int 
   const size_t rows = (size_t)Hq * T;
   const size_t part_o_bytes = S > 1 ? (size_t)S * rows * kD * 4 : 0;
   const size_t part_ml_bytes = S > 1 ? (size_t)S * rows * 2 * 4 : 0;
-  char* buf = static_cast<char*>(scratch(plane_bytes + part_o_bytes + part_ml_bytes + 256));
+  const size_t texp_bytes = ((size_t)Hkv * g.ntiles * 2 * sizeof(int) + 255) & ~(size_t)255;
+  char* buf = static_cast<char*>(scratch(plane_bytes + part_o_bytes + part_ml_bytes + texp_bytes + 256));
   if (!buf) return 1;   // no room for the planes: the caller takes the kernel that needs none
   uint4* planes = reinterpret_cast<uint4*>(buf);
   float* part_o = reinterpret_cast<float*>(buf + plane_bytes);
   float* part_ml = reinterpret_cast<float*>(buf + plane_bytes + part_o_bytes);
+  int* texp = reinterpret_cast<int*>(buf + plane_bytes + part_o_bytes + part_ml_bytes);
   const size_t lds = 2 * kImgBytes;
   if (lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
-  auto fn = attn_x3_kernel<NP, D>;
+  auto fn = attn_x3_kernel<NP, D, H>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  hipLaunchKernelGGL((kv_planes_kernel<KT, NP, D>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes,
+  hipLaunchKernelGGL((kv_planes_kernel<KT, NP, D, H>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes, texp,
                      kv_max * (int64_t)kD, kend, g.ntiles);
-  hipLaunchKernelGGL(fn, dim3(Hkv * g.head_chunks, pblocks, S), dim3(512), lds, c.stream, q, planes, out, part_o,
-                     part_ml, scale, g);
+  hipLaunchKernelGGL(fn, dim3(Hkv * g.head_chunks, pblocks, S), dim3(512), lds, c.stream, q, planes, texp, out,
+                     part_o, part_ml, scale, g);
   if (S > 1) {
     const int64_t threads = (int64_t)rows * (kD / 4);
     hipLaunchKernelGGL(attn_x3_merge_kernel<D>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c.stream, part_o,
@@ -529,9 +700,17 @@ int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int 
   return 0;
 }
 
-template int launch_prefill_x3<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
-template int launch_prefill_x3<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
-template int launch_prefill_x3<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
-template int launch_prefill_x3<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+// f16_terms: the f16 form (two terms per operand) instead of the three bf16 planes
+template <int D, typename KT>
+int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
+                      int64_t kv_max, float scale, int pos0, int token_major, bool f16_terms) {
+  return f16_terms ? launch_x3<D, KT, true>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)
+                   : launch_x3<D, KT, false>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major);
+}
+
+template int launch_prefill_x3<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int, bool);
+template int launch_prefill_x3<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int, bool);
+template int launch_prefill_x3<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int, bool);
+template int launch_prefill_x3<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int, bool);
 
 }  // namespace tlhip

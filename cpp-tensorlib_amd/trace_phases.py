@@ -7,7 +7,7 @@ the distribution over wavefronts. Times are clocks of the 100 MHz-referenced sha
 divided by the frequency given with --ghz (default 2.1).
 
   python cpp-tensorlib_amd/trace_phases.py attn_decode [pos]      7B decode attention (fused q/k/v, device position)
-  python cpp-tensorlib_amd/trace_phases.py attn_prefill [pos0]    7B causal prefill attention of a 512-token chunk (bf16 planes)
+  python cpp-tensorlib_amd/trace_phases.py attn_prefill [pos0 [bf16]]  7B causal prefill attention of a 512-token chunk: f16 terms, or bf16 planes
   python cpp-tensorlib_amd/trace_phases.py gemm [f16w|bf16]       a 512 x 32768 x 3584 prompt GEMM: prepared weight, or plain bf16
 """
 import ctypes as C
@@ -88,7 +88,7 @@ def attn_decode(lib, pos, ghz):
         pct(names[sl], ((t[:, :, sl] - t[:, :, 0])[ok]) / (ghz * 1e3))
 
 
-def attn_prefill(lib, pos0, ghz):
+def attn_prefill(lib, pos0, ghz, mode=4):
     Hq, Hkv, D, T = 28, 4, 128, 512
     rng = np.random.default_rng(3)
     kv_max = pos0 + T
@@ -97,7 +97,7 @@ def attn_prefill(lib, pos0, ghz):
     V = lib.to_device(rng.standard_normal(Hkv * kv_max * D, dtype=np.float32))
     q = lib.to_device(rng.standard_normal(Hq * T * D, dtype=np.float32))
     out = lib.empty(Hq * T * D)
-    lib.tune_attn_prefill(3)
+    lib.tune_attn_prefill(mode)
     for _ in range(2):
         lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
     lib.sync()
@@ -107,7 +107,8 @@ def attn_prefill(lib, pos0, ghz):
     lib.attn_prefill(q, K, V, out, Hq, Hkv, T, kv_max, D, scale, pos0=pos0)
     lib.record(e1)
     lib.sync()
-    print("tlhip_attn_prefill, bf16-plane kernels (planes + attention + merge), pos0 %d: %.1f us" % (pos0, lib.elapsed_ms(e0, e1) * 1e3))
+    print("tlhip_attn_prefill, %s (planes + attention + merge), pos0 %d: %.1f us"
+          % ("f16-term kernels" if mode == 4 else "bf16-plane kernels", pos0, lib.elapsed_ms(e0, e1) * 1e3))
     t = read_trace(lib)
     for grp, ws in (("wavefronts 0-3 (matrix phase, then softmax)", range(0, 4)), ("wavefronts 4-6 (softmax, then matrix phase)", range(4, 7))):
         tt = t[:, list(ws), :]
@@ -176,4 +177,4 @@ if __name__ == "__main__":
     elif args[0] == "attn_decode":
         attn_decode(lib, int(args[1]) if len(args) > 1 else 4095, ghz)
     else:
-        attn_prefill(lib, int(args[1]) if len(args) > 1 else 7680, ghz)
+        attn_prefill(lib, int(args[1]) if len(args) > 1 else 7680, ghz, 3 if "bf16" in args[2:] else 4)

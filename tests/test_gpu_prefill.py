@@ -347,12 +347,13 @@ def test_gemm_bf16_nt_declines(lib):
         b.free()
 
 
-KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "planes": 3}
+KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "planes": 3, "f16terms": 4}
 
 
 def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, kernel="auto"):
     """kernel (tlhip_tune_attn_prefill): the library's own choice, the VALU kernel, the fp32
-    matrix-pipe kernel, or the bf16-plane kernels on the matrix cores."""
+    matrix-pipe kernel, the bf16-plane kernels on the matrix cores, or their f16 form (two f16 terms
+    per operand; what the library's own choice takes deep in a context)."""
     Hq, T, D = q.shape
     Hkv, kv_max, _ = K.shape
     dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, T, D))
@@ -408,8 +409,9 @@ def _attn_f64(q, K, V, scale, pos0):
     return out
 
 
-@pytest.mark.parametrize("kernel", ["fp32pipe", "planes"])
-@pytest.mark.parametrize("case", ["one_dominant_key", "equal_scores", "large_values", "tiny_values", "cancelling_values"])
+@pytest.mark.parametrize("kernel", ["fp32pipe", "planes", "f16terms"])
+@pytest.mark.parametrize("case", ["one_dominant_key", "equal_scores", "large_values", "tiny_values", "cancelling_values",
+                                  "value_scale_by_tile"])
 def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
     """Rows chosen against the bf16-plane products (three planes per operand, six plane pairs per
     product: what is dropped is below 2^-23 of |a b|) and against the online softmax:
@@ -421,7 +423,11 @@ def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
                           taken): plane residuals of large numbers;
       tiny_values         values around 2^-40: the third plane is near the bottom of bf16's range;
       cancelling_values   V alternates +-(1000 + small) so that the output is a small difference
-                          of large terms (tests the value planes and the fp32 accumulation).
+                          of large terms (tests the value planes and the fp32 accumulation);
+      value_scale_by_tile every run of 32 keys has its V rows scaled by its own power of two between
+                          2^-24 and 2^24 and its K rows by one between 2^-2 and 2^2 (the f16 form
+                          scales K and V per 32-key tile and carries the output accumulators from
+                          one tile's unit to the next).
     Both matrix kernels against the CPU oracle at allclose(1e-4, 1e-5) and against float64 with the
     bound an fp32 evaluation obeys: 2^-22 (4 + max_k sum_i |q_i k_i| scale) sum_k p_k |v_k| (the
     CPU oracle itself uses up to 0.7 of it on these rows; the plane kernel measured at or below the
@@ -451,6 +457,12 @@ def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
         sign = np.where(np.arange(kv_max) % 2 == 0, 1.0, -1.0).astype(np.float32)
         V[0] = sign[:, None] * (1000.0 + V[0])
         K[0, :] = K[0, 0] + (1e-3 * rng.standard_normal((kv_max, D))).astype(np.float32)   # near-uniform softmax
+    elif case == "value_scale_by_tile":
+        tiles = (kv_max + 31) // 32
+        ev = np.repeat(rng.integers(-24, 25, tiles), 32)[:kv_max]
+        ek = np.repeat(rng.integers(-2, 3, tiles), 32)[:kv_max]
+        V[0] *= np.exp2(ev).astype(np.float32)[:, None]
+        K[0] *= np.exp2(ek).astype(np.float32)[:, None]
     got = _prefill(lib, q, K, V, float(scale), pos0, kernel=kernel)
     want = orc.attn_prefill(q, K, V, float(scale), pos0)
     assert np.all(np.isfinite(got))
@@ -477,7 +489,7 @@ def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
 def test_attn_prefill_rows_equal_decode(lib, orc, kernel):
     """Row p of a prefill equals a decode step with ctx = pos0 + p + 1 (the equivalence the
     reference's prefill bench relies on, bench_qwen_prefill.cpp:283-310), and the first query
-    of a fresh cache returns V[0] exactly."""
+    of a fresh cache returns V[0] (exactly; to one rounding from the f16 form)."""
     D, Hq, Hkv, T, pos0 = 128, 8, 2, 40, 24
     kv_max = pos0 + T
     q = orc.normal(Hq * T * D, 41).reshape(Hq, T, D)
@@ -494,7 +506,11 @@ def test_attn_prefill_rows_equal_decode(lib, orc, kernel):
     for b in (dk, dv, do):
         b.free()
     fresh = _prefill(lib, q, K, V, scale, 0, kernel=kernel)
-    assert np.array_equal(fresh[:, 0, :], np.repeat(V[:, 0, :], Hq // Hkv, axis=0))
+    v0 = np.repeat(V[:, 0, :], Hq // Hkv, axis=0)
+    if kernel == "f16terms":   # two f16 terms carry 23 bits of a value, not 24: one rounding, like any fp32 operation
+        assert np.all(np.abs(fresh[:, 0, :] - v0) <= 2.0 ** -23 * np.abs(v0))
+    else:
+        assert np.array_equal(fresh[:, 0, :], v0)
 
 
 @pytest.mark.parametrize("kernel", list(KERNELS))
