@@ -778,7 +778,7 @@ static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, 
                           int T, int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = tlhip::ctx();
   const int mode = c.tune_prefill_valu;
-  if (mode == 3 || mode == 4 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
+  if (mode >= 3 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
     const int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major, mode != 3);
     if (rc < 0) return rc;
     if (rc == 0) TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
