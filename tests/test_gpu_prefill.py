@@ -414,7 +414,8 @@ def _attn_f64(q, K, V, scale, pos0):
                                   "value_scale_by_tile"])
 def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
     """Rows chosen against the bf16-plane products (three planes per operand, six plane pairs per
-    product: what is dropped is below 2^-23 of |a b|) and against the online softmax:
+    product: what is dropped is below 2^-23 of |a b|), the f16-term products (two terms per operand
+    scaled per query row and per 32-key tile, three term pairs) and the online softmax:
       one_dominant_key    one key's score exceeds the others by ~40: the softmax is one-hot to
                           fp32 and the output must be that key's value row;
       equal_scores        every key of a row scores the same to 1e-6: the output is a plain mean,
