@@ -502,7 +502,7 @@ def prefill_7b(lib, rounds=3):
         "tflops_chunk": round(flops / best / 1e9, 1),
         "int4_weights": {"ms_per_chunk": round(best_q4, 3), "tok_s": round(T / best_q4 * 1e3, 1)},
         "attention_per_layer": dict(attn, note="causal attention of the 512-token chunk, 28/4 heads of 128, f32 cache; "
-                                               "deep in a context: two f16 terms per operand on the matrix cores, four term products per "
+                                               "deep in a context: two f16 terms per operand on the matrix cores, three term products per "
                                                "fp32 product (157.3 TFLOP/s is the fp32 matrix-pipe peak)"),
         "gemm": {"per_shape": per_gemm, "TFLOP/s": round(gemm_tf, 1), "bf16_rows_TFLOP/s": round(rows_tf, 1),
                  "roofline": {"bound": "mfma", "achieved": round(2 * gemm_tf, 1), "peak": 2500.0,

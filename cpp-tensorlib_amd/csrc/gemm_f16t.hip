@@ -271,14 +271,14 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
     fetch(stage, Idx<1>{});
     __builtin_amdgcn_sched_barrier(0);
     mul4(Idx<0>{}, Idx<1>{});
-    if (TM == 2) {
+    if constexpr (TM == 2) {
       mul4(Idx<0>{}, Idx<2>{});
       mul4(Idx<0>{}, Idx<3>{});
     }
     TLHIP_PHASE(0);
     // my reads of slab k are complete and my copies of slab k + 1 have landed (those of slab
     // k + 2 may still be in flight); past the barrier that holds for every wavefront
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kCopies) : "memory");
     barrier();
     TLHIP_PHASE(1);
     // slab k + 3 into the stage slab k has just left
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
     if (k + 1 < ns) fetch(ring + nx * kStage, Idx<0>{});
     __builtin_amdgcn_sched_barrier(0);
     mul4(Idx<1>{}, Idx<1>{});
-    if (TM == 1) {
+    if constexpr (TM == 1) {
       copy(k + 3, st, Idx<2>{});
       copy(k + 3, st, Idx<3>{});
     } else {
