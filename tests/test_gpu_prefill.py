@@ -515,9 +515,11 @@ def test_attn_prefill_rows_equal_decode(lib, orc, kernel):
 
 
 @pytest.mark.parametrize("kernel", list(KERNELS))
+@pytest.mark.parametrize("pos0", [10, 2100])
 @pytest.mark.parametrize("D", [128, 64])
-def test_attn_prefill_bf16_cache(lib, orc, D, kernel):
-    Hq, Hkv, T, pos0 = 4, 2, 70, 10
+def test_attn_prefill_bf16_cache(lib, orc, D, pos0, kernel):
+    """A bf16 cache, fresh and deep in a context (one plane / one term of K and V in the matrix-core kernels)."""
+    Hq, Hkv, T = 4, 2, 70
     kv_max = pos0 + T
     q = orc.normal(Hq * T * D, 51).reshape(Hq, T, D)
     Kb = orc.to_bf16(orc.normal(Hkv * kv_max * D, 52)).reshape(Hkv, kv_max, D)
@@ -526,6 +528,20 @@ def test_attn_prefill_bf16_cache(lib, orc, D, kernel):
     got = _prefill(lib, q, Kb, Vb, scale, pos0, kv_bf16=True, kernel=kernel)
     want = orc.attn_prefill(q, orc.bf16_widen(Kb).reshape(Kb.shape),
                             orc.bf16_widen(Vb).reshape(Vb.shape), scale, pos0)
+    assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS))
+def test_attn_prefill_negative_scale(lib, orc, kernel):
+    """The scale is an argument like any other: a negative one turns the softmax towards the
+    smallest dot products (the matrix-core kernels fold its sign into Q)."""
+    D, Hq, Hkv, T, pos0 = 128, 4, 2, 40, 1100
+    kv_max = pos0 + T
+    q = orc.normal(Hq * T * D, 71).reshape(Hq, T, D)
+    K = orc.normal(Hkv * kv_max * D, 72).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 73).reshape(Hkv, kv_max, D)
+    got = _prefill(lib, q, K, V, -0.07, pos0, kernel=kernel)
+    want = orc.attn_prefill(q, K, V, -0.07, pos0)
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
