@@ -894,14 +894,14 @@ __global__ __launch_bounds__(256) void attn_x3_merge_kernel(const float* __restr
 }  // namespace x3
 
 // Whether the matrix-core kernels serve this call: head size 64 or 128 and enough keys for the
-// extra passes to pay. Measured crossover of the f16 form against the fp32 matrix-pipe kernel at the
-// 7B and 0.5B head shapes, in query-key pairs of one head (T pos0 + T^2 / 2): about 200 thousand at
-// head size 128, 300 thousand at 64; short chunks deep in a context stay with the older rule by keys.
+// extra passes (planes, merge) to pay. Measured crossover of the f16 form against the fp32
+// matrix-pipe kernel at the 7B and 0.5B head shapes, chunks of 32 to 512 tokens: from 640 keys on
+// at head size 128 (512 for a chunk of 512), from 1024 at head size 64 (768 for chunks of 256 up).
 bool prefill_x3_applies(int D, int T, int pos0) {
   if (T < 16) return false;
-  const int64_t keys = (int64_t)pos0 + T, pairs = (int64_t)T * pos0 + (int64_t)T * T / 2;
-  if (D == 128) return keys >= 1024 || (keys >= 768 && pairs >= 200000);
-  if (D == 64) return keys >= 2048 || pairs >= 300000;
+  const int64_t keys = (int64_t)pos0 + T;
+  if (D == 128) return keys >= 640 || (keys >= 512 && T >= 512);
+  if (D == 64) return keys >= 1024 || (keys >= 768 && T >= 256);
   return false;
 }
 
@@ -929,9 +929,9 @@ static int launch_x3(const float* q, const KT* K, const KT* V, float* out, int H
   g.rows = (int64_t)Hq * T;
   const int pblocks = (T + g.np * 16 * kRT - 1) / (g.np * 16 * kRT);
   const int base = Hkv * g.head_chunks * pblocks;
-  // key splits: fill the chip once, keep at least 8 tiles per block
+  // key splits: fill the chip once, keep at least 4 tiles per block
   int S = (c.cus + base - 1) / base;
-  if (S > g.ntiles / 8) S = g.ntiles / 8;
+  if (S > g.ntiles / 4) S = g.ntiles / 4;
   if (S < 1) S = 1;
   if (S > 64) S = 64;
   g.S = S;
