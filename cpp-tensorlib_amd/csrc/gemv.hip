@@ -90,7 +90,8 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   constexpr int XS = LPR + (J == 8 ? 2 : 8);
   float4* xs = smem4;
   float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * XS);  // [chunks*LPR], int4 only
-  float* red = xsum + (Fmt::kScaled ? chunks * LPR : 0);
+  float* red = xsum + (Fmt::kScaled ? chunks * LPR : 0);   // [nw * QN * 8] K-split partials
+  float* nsum = red + nw * QN * 8;                          // [16] per-wavefront sums of squares (norm producer)
 
   const int kw = wave % KW;          // which K split this wavefront takes
   const int wn = wave / KW;          // which row group of the block tile
@@ -163,8 +164,11 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
       if (PRO == kSwiglu) { v.x = gated(v.x, aux.x); v.y = gated(v.y, aux.y); v.z = gated(v.z, aux.z); v.w = gated(v.w, aux.w); }
       return v;
     };
-    float inv = 0.f;
-    if (PRO == kRmsnorm) {   // mean square of the row, summed in a fixed order
+    if (PRO == kRmsnorm) {
+      // Mean square of the row, summed in a fixed order. The row goes into LDS as x * w without
+      // the 1 / rms factor, which is one number for the whole row: every row total is multiplied
+      // by it at the end instead (W . (x w / rms) = (W . (x w)) / rms), so the staging pass does
+      // not wait for this sum and the block needs no barrier of its own for it.
       float ss = 0.f;
       int k = 0;
       for (int i = tid; i < n4; i += blockDim.x, k++) {
@@ -173,12 +177,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
       }
       ss = wave_sum(ss);
-      if (lane == 0) red[wave] = ss;
-      __syncthreads();
-      float tot = red[0];
-      for (int w = 1; w < nw; w++) tot += red[w];
-      inv = 1.0f / sqrtf(tot * (1.0f / (float)(n4 * 4)) + pro.eps);
-      // red is reused only after the barrier that ends the staging pass
+      if (lane == 0) nsum[wave] = ss;
     }
     int k2 = 0;
     for (int i = tid; i < n4_padded; i += blockDim.x, k2++) {
@@ -189,8 +188,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         v = raw(k2, i, nv);
         if (PRO == kRmsnorm) {
           if (pro.xout && blockIdx.x == 0) reinterpret_cast<float4*>(pro.xout)[i] = v;
-          v.x = (v.x * inv) * nv.x; v.y = (v.y * inv) * nv.y;
-          v.z = (v.z * inv) * nv.z; v.w = (v.w * inv) * nv.w;
+          v.x *= nv.x; v.y *= nv.y; v.z *= nv.z; v.w *= nv.w;
         }
       }
       const int u = i / J, j = i - u * J;
@@ -211,6 +209,12 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   }
   __syncthreads();
   TLHIP_MARK(2);
+  float inv = 1.0f;
+  if (PRO == kRmsnorm) {
+    float tot = nsum[0];
+    for (int w = 1; w < nw; w++) tot += nsum[w];
+    inv = 1.0f / sqrtf(tot * (1.0f / (float)(upr * Fmt::E)) + pro.eps);
+  }
 
   float acc[R];
 #pragma unroll
@@ -256,6 +260,7 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
         r = li;
         writer = li < R;
       }
+      if (PRO == kRmsnorm) v *= inv;
       if (KW == 1) {
         if constexpr (kPair) {
           // the up row's total sits half a wavefront (64-lane form) or R/2 lanes (16-lane form) away
