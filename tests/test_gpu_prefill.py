@@ -531,6 +531,28 @@ def test_attn_prefill_bf16_cache(lib, orc, D, pos0, kernel):
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
 
 
+@pytest.mark.parametrize("D,T,pos0,expect", [
+    (128, 64, 100, "fp32pipe"), (128, 64, 576, "f16terms"), (128, 512, 0, "f16terms"), (128, 256, 256, "fp32pipe"),
+    (64, 64, 700, "fp32pipe"), (64, 64, 960, "f16terms"), (64, 256, 512, "f16terms"), (128, 8, 4000, "fp32pipe"),
+])
+def test_attn_prefill_builtin_choice(lib, orc, D, T, pos0, expect):
+    """Which kernel the library picks by itself: the f16-term kernels from 640 keys on at head size
+    128 (512 for a chunk of 512) and from 1024 at head size 64 (768 for chunks of 256 up), chunks
+    of at least 16 tokens; the fp32 matrix-pipe kernel otherwise. Checked bit for bit against the
+    forced kernel."""
+    Hq, Hkv = 4, 2
+    kv_max = pos0 + T
+    q = orc.normal(Hq * T * D, 81).reshape(Hq, T, D)
+    K = orc.normal(Hkv * kv_max * D, 82).reshape(Hkv, kv_max, D)
+    V = orc.normal(Hkv * kv_max * D, 83).reshape(Hkv, kv_max, D)
+    scale = 1.0 / np.sqrt(float(D))
+    auto = _prefill(lib, q, K, V, scale, pos0, kernel="auto")
+    forced = _prefill(lib, q, K, V, scale, pos0, kernel=expect)
+    assert np.array_equal(auto, forced)
+    other = _prefill(lib, q, K, V, scale, pos0, kernel="fp32pipe" if expect == "f16terms" else "f16terms")
+    assert not np.array_equal(auto, other)      # (the two kernels differ in the last bits, so the check above tells them apart)
+
+
 @pytest.mark.parametrize("kernel", list(KERNELS))
 def test_attn_prefill_negative_scale(lib, orc, kernel):
     """The scale is an argument like any other: a negative one turns the softmax towards the
