@@ -107,17 +107,6 @@ __device__ __forceinline__ void split3x8(const float (&x)[8], uint4& p1, uint4& 
   p3 = make_uint4(c[0], c[1], c[2], c[3]);
 }
 
-__device__ __forceinline__ bf16x8 as_bf16x8(const uint4& u) {
-  union { uint4 u4; bf16x8 v; } t;
-  t.u4 = u;
-  return t.v;
-}
-__device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 u) {
-  union { u32x4 u4; bf16x8 v; } t;
-  t.u4 = u;
-  return t.v;
-}
-
 // The f16 form: an operand, first multiplied by a power of two that brings it
 // into the f16 range, is cut into TWO f16 terms, both rounded to nearest (2^-24 relative while
 // the second term is a normal f16), and a product is formed from the three term pairs that hold
