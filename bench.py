@@ -531,7 +531,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; every GPU box of this run has one. "
-              "Run with --gpus 1 (DESIGN.md says how the path would shard).", file=sys.stderr)
+              "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     pkg = importlib.import_module("cpp-tensorlib_amd")

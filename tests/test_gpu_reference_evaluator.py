@@ -1,6 +1,6 @@
 """The reference's REAL evaluator on this backend. oracle/_ref/array_on_hip is the reference's
 unmodified array.h / storage.h / types.h compiled (in the build container, by oracle/Makefile)
-on top of cpp-tensorlib_amd/include/tl/hip.h through the gpu.h arm INTEGRATION.md describes.
+on top of cpp-tensorlib_amd/include/tl/hip.h through a gpu.h with one more backend arm (oracle/seam_gpu.h).
 It evaluates every case twice with the reference's own code - use_cpu() and use_gpu() - and
 compares with allclose(rtol 1e-4, atol 1e-5); the dispatch census shows that the GPU run
 launched kernels. This is the drop-in claim itself: dot (int4 / bf16 / f32, with and without
