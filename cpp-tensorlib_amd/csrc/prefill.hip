@@ -128,7 +128,43 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       sa[i] = gm < M ? pow2f(ea[gm]) : 1.0f;
     }
   }
+  // Q4: where this thread's loads of a slab start at k = 0 (the same rows in every slab). Every
+  // address is clamped into the operands and what lies past an edge is replaced when the slab is
+  // stored to LDS, so that no load sits under a condition and nothing waits for a load where it
+  // is issued: the requests of a slab go out back to back, in front of the products.
+  const float* a_src[Q4 ? A_LOADS : 1];
+  const uint8_t* q_src = nullptr;
+  const float* s_src[Q4 ? TN : 1];
+  bool a_in[Q4 ? A_LOADS : 1], s_in[Q4 ? TN : 1], q_in = false;
+  if constexpr (Q4) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) {
+      const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
+      a_in[i] = m0 + row < M;
+      a_src[i] = A + (size_t)min(m0 + row, M - 1) * K + c4 * 4;
+    }
+    const int gn = wrow(tid / TPC);
+    q_in = gn >= 0;
+    q_src = reinterpret_cast<const uint8_t*>(W) + ((size_t)max(gn, 0) * K + (tid % TPC) * (32 / TPC)) / 2;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int gn2 = wrow(wn * WT + j * 32 + (lane & 31));
+      s_in[j] = gn2 >= 0;
+      s_src[j] = scales + (size_t)max(gn2, 0) * (K >> 5);
+    }
+  }
   auto gload = [&](int k0) {
+    if constexpr (Q4) {   // (k0 < kend: the loop asks for slabs that exist)
+#pragma unroll
+      for (int i = 0; i < A_LOADS; i++) ra[i] = *reinterpret_cast<const float4*>(a_src[i] + k0);
+      // thread t: tile column t / TPC, nibbles of k0 + (32 / TPC) * (t % TPC) .. (16 / TPC bytes)
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(q_src + (k0 >> 1));
+#pragma unroll
+      for (int u = 0; u < 4 / TPC; u++) rq[u] = src[u];
+#pragma unroll
+      for (int j = 0; j < TN; j++) sc_next[j] = s_src[j][k0 >> 5];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
@@ -136,26 +172,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       ra[i] = (gm < M && gk < kend) ? *reinterpret_cast<const float4*>(A + (size_t)gm * K + gk)
                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    if (Q4) {
-      // thread t: tile column t / TPC, nibbles of k0 + (32 / TPC) * (t % TPC) .. (16 / TPC bytes)
-      const int gn = wrow(tid / TPC), gk = k0 + (tid % TPC) * (32 / TPC);
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(W) + ((size_t)max(gn, 0) * K + gk) / 2);
-      const bool in = gn >= 0 && gk < kend;
-#pragma unroll
-      for (int u = 0; u < 4 / TPC; u++) rq[u] = in ? src[u] : 0x88888888u;   // nibble 8 = weight 0
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-        const int gn2 = wrow(wn * WT + j * 32 + (lane & 31));
-        sc_next[j] = (gn2 >= 0 && k0 < kend) ? scales[(size_t)gn2 * (K >> 5) + (k0 >> 5)] : 0.f;
-      }
-    } else {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 2, c8 = idx & 3;
       const int gk = k0 + c8 * 8, gn = wrow(row);
       rb[i] = (gn >= 0 && gk < kend) ? *reinterpret_cast<const uint4*>(W + (size_t)gn * K + gk)
                                      : make_uint4(0u, 0u, 0u, 0u);
-    }
     }
   };
   // 4 bytes = 8 nibbles -> 8 bf16 (k ascending): float(nibble) - 8 is an integer in [-8, 7], exact in bf16
@@ -194,6 +216,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
 #pragma unroll
     for (int i = 0; i < A_LOADS; i++) {
       const int idx = tid + i * NT, row = idx >> 3, c4 = idx & 7;
+      if (Q4 && !a_in[Q4 ? i : 0]) ra[i] = make_float4(0.f, 0.f, 0.f, 0.f);
       if (H) {
         uint32_t h01, l01, h23, l23;
         const float s = sa[H ? i : 0];
@@ -217,9 +240,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     if (Q4) {
       const int row = tid / TPC, c8 = (tid % TPC) * (4 / TPC);
 #pragma unroll
-      for (int u = 0; u < 4 / TPC; u++) *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + u)]) = H ? nib8h(rq[u]) : nib8(rq[u]);
+      for (int u = 0; u < 4 / TPC; u++) {
+        const uint32_t w = q_in ? rq[u] : 0x88888888u;   // nibble 8 = weight 0
+        *reinterpret_cast<uint4*>(&Bs[lds_off(row, c8 + u)]) = H ? nib8h(w) : nib8(w);
+      }
 #pragma unroll
-      for (int j = 0; j < TN; j++) sc[j] = sc_next[j];
+      for (int j = 0; j < TN; j++) sc[j] = s_in[Q4 ? j : 0] ? sc_next[j] : 0.f;
     } else {
 #pragma unroll
     for (int i = 0; i < B_LOADS; i++) {

@@ -8,7 +8,7 @@ divided by the frequency given with --ghz (default 2.1).
 
   python cpp-tensorlib_amd/trace_phases.py attn_decode [pos]      7B decode attention (fused q/k/v, device position)
   python cpp-tensorlib_amd/trace_phases.py attn_prefill [pos0 [bf16]]  7B causal prefill attention of a 512-token chunk: f16 terms, or bf16 planes
-  python cpp-tensorlib_amd/trace_phases.py gemm [f16w|bf16]       a 512 x 32768 x 3584 prompt GEMM: prepared weight, or plain bf16
+  python cpp-tensorlib_amd/trace_phases.py gemm [f16w|bf16|q4]    a 512 x 32768 x 3584 prompt GEMM: prepared weight, plain bf16, or int4
 """
 import ctypes as C
 import importlib
@@ -131,6 +131,12 @@ def gemm(lib, kind, ghz):
     if kind == "f16w":
         img, ex = lib.gemm_f16w_prepare(W, N, K)
         run = lambda: lib.gemm_f16w_nt(A, img, ex, Cm, M, N, K)
+    elif kind == "q4":
+        host = np.empty(N * K // 2 + N * (K // 32) * 4, np.uint8)       # packed nibbles, then f32 scales
+        host[:N * K // 2] = rng.integers(0, 256, N * K // 2, dtype=np.uint8)
+        host[N * K // 2:] = rng.uniform(0.005, 0.02, N * (K // 32)).astype(np.float32).view(np.uint8)
+        q4 = lib.to_device(host)
+        run = lambda: lib.gemm_q4_nt(A, q4, Cm, M, N, K)
     else:
         run = lambda: lib.gemm_bf16_nt(A, W, Cm, M, N, K)
     for _ in range(2):
