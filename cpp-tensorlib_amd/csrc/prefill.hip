@@ -192,14 +192,18 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
     }
     return o;
   };
-  auto nib8h = [](uint32_t w) {   // the same as f16
-    const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;
+  // the same as f16: 0x6400 | n is the f16 number 1024 + n (one unit in the last place there), so
+  // a nibble becomes its weight n - 8 by a byte permute, an OR and one packed f16 subtraction
+  auto nib8h = [](uint32_t w) {
+    const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;   // even k, odd k
     uint4 o;
     uint32_t* po = reinterpret_cast<uint32_t*>(&o);
+    const f16x2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
 #pragma unroll
     for (int b = 0; b < 4; b++) {
-      const f32x2 x = {(float)((lo >> (8 * b)) & 0xffu) - 8.0f, (float)((hi >> (8 * b)) & 0xffu) - 8.0f};
-      po[b] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+      // bytes of the pair: [lo.byte b, 0, hi.byte b, 0]
+      const uint32_t pair = __builtin_amdgcn_perm(hi, lo, (uint32_t)b | 0x0c00u | ((uint32_t)(4 + b) << 16) | 0x0c000000u);
+      po[b] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, pair | 0x64006400u) - bias);
     }
     return o;
   };
