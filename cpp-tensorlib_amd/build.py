@@ -90,24 +90,5 @@ def build_host(force=False, verbose=True):
     return QWEN_LIB
 
 
-TRACE_LIB = os.path.join(LIBDIR, "libtensorlib_hip_trace.so")
-
-
-def build_trace(verbose=True):
-    """libtensorlib_hip_trace.so: every kernel in one translation unit with the in-kernel phase
-    timestamps on (csrc/trace_unity.hip). A tuning aid for trace_phases.py, built on request only."""
-    os.makedirs(LIBDIR, exist_ok=True)
-    cmd = [hipcc()] + FLAGS + ["-w", "-shared", os.path.join(CSRC, "trace_unity.hip"), "-o", TRACE_LIB]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for the trace build:\n%s" % r.stderr)
-    return TRACE_LIB
-
-
 if __name__ == "__main__":
-    if "--trace" in sys.argv:
-        print(build_trace())
-    else:
-        print(build(force="--force" in sys.argv))
+    print(build(force="--force" in sys.argv))

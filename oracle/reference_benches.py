@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """The reference's own benchmark programs on this backend (test infrastructure, not the bench line).
 
-  python tests/reference_benches.py
+  python oracle/reference_benches.py
 """
 import json
 import os
