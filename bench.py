@@ -102,7 +102,7 @@ def cpu_baseline(guards, budget_s=25.0):
 
     total_bytes, total_s, timed, per_shape_s = 0, 0.0, [], {}
     t_start = time.time()
-    for (N, K) in sorted(SHAPES, key=lambda s: s[0] * s[1]):
+    for (N, K) in [(4864, 896)] + sorted(SHAPES, key=lambda s: s[0] * s[1]):
         big = N * K > 10 ** 8
         est = 0.62 * N * K / 0.1e9 * (3.3 if big else 4.2)     # ~0.1 GB/s, calls incl. warm-up
         if time.time() - t_start + est > budget_s and timed:
@@ -119,6 +119,9 @@ def cpu_baseline(guards, budget_s=25.0):
         sec = med3(run, warm=not big)
         if refl is not None:
             refl.lib.tlref_gemv_free(h)
+        if (N, K) not in SHAPES:        # BASELINE configs[0]: reported beside the sweep, not in it
+            config0_ms = sec * 1e3
+            continue
         total_bytes += q4_nbytes(N, K)
         total_s += sec
         per_shape_s["%dx%d" % (N, K)] = sec
@@ -131,6 +134,7 @@ def cpu_baseline(guards, budget_s=25.0):
                   "call except for the LM head); the reference's dot at M=1 runs on one thread whatever the core "
                   "count" % (", ".join(timed), len(timed)),
         "ms": round(total_s * 1e3, 2), "host_cores_online": os.cpu_count(),
+        "config0_4864x896_ms": round(config0_ms, 3),
     }
     # ---- the other ops of a 7B-shape decode step at ctx 4096, one thread like the dots
     if len(timed) == len(SHAPES):
@@ -196,7 +200,7 @@ def decode_guard(lib):
             "logits_maxrel": float("%.3g" % worst), "bar": 2e-3, "graph_captured": bool(ok)}
 
 
-def decode_7b(lib, steps, eager=False):
+def decode_7b(lib, steps, eager=False, warm=None):
     """Qwen2.5-7B-shape int4 decode step at ctx 4096 (BASELINE configs[4], decode half):
     random-init weights, cache rows [0,4095) pre-filled, one step captured as a hipGraph
     at position 4095 and replayed. eager=True launches the same kernels one by one, without
@@ -207,6 +211,8 @@ def decode_7b(lib, steps, eager=False):
     ctx = 4096
     g.fill_cache_random(ctx - 1, 2)
     pos = ctx - 1
+    if warm:        # (mode, blocks): weight warm-up reads on a second stream beside each layer
+        g.set_warm(warm[1], False, warm[0])
     for _ in range(2):
         g.step(11, pos)
     if eager:
@@ -218,6 +224,9 @@ def decode_7b(lib, steps, eager=False):
         g.close()
         return {"workload": "Qwen2.5-7B-shape int4 decode step, ctx 4096, eager launches",
                 "ms_per_token": round(ms, 4), "tok_s": round(1e3 / ms, 1)}
+    # where the step's GPU time goes: events between the launches of five eager steps (the role
+    # of the reference's StepProf, bench_qwen_decode.cpp:212-237); the events cost a little themselves
+    layer_us = {k: round(v, 2) for k, v in g.profile_steps(11, pos, 5).items()}
     g.capture(11, pos)
     for _ in range(3):
         g.replay()
@@ -283,6 +292,8 @@ def decode_7b(lib, steps, eager=False):
                  "tok_s_greedy_token_loop_on_device": round(1e3 / greedy_dev, 1)},
         "algorithmic_bytes": int(wbytes + kvbytes),
         "hbm_frac": round((wbytes + kvbytes) / (best * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "layer_us": dict(layer_us, what="eager step with an event between its regions: microseconds per layer "
+                                        "(lm_head, step: per token); attention = q/k/v epilogue + attention + split combine"),
     }
 
 
@@ -523,6 +534,11 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the 7B-shape decode leg")
     ap.add_argument("--eager-decode", action="store_true",
                     help="decode leg without the hipGraph (for kernel traces)")
+    ap.add_argument("--decode-warm", default="", metavar="MODE:BLOCKS",
+                    help="decode leg with weight warm-up reads on a second stream beside each layer "
+                         "(an experiment that does not pay; off by default). MODE 0: o-proj, gate|up, down "
+                         "and the next q|k|v from the layer's start; 3: o-proj and gate|up beside attention. "
+                         "BLOCKS < 0: short-lived 32 KB blocks")
     ap.add_argument("--no-side", action="store_true",
                     help="skip the bf16 GEMV and decode attention legs")
     ap.add_argument("--no-prefill", action="store_true", help="skip the 7B-shape prompt-chunk leg")
@@ -538,20 +554,21 @@ def main():
     lib = pkg.load()                      # raises when the HIP library or the GPU is missing
 
     # ---- device-resident inputs: a ring of weight copies per shape -----------------
-    rings = []
-    for si, (N, K) in enumerate(SHAPES):
+    def make_ring(N, K, wseed, xseed):
         nb = q4_nbytes(N, K)
         stride = (nb + 255) // 256 * 256
         copies = max(2, int(RING_BYTES // nb) + 1)
-        host = make_q4_host(lib, N, K, 100 + si)
+        host = make_q4_host(lib, N, K, wseed)
         first = lib.empty_bytes(stride * copies)
         first.upload(host)
         for c in range(1, copies):
             lib._chk(lib.c.tlhip_memcpy_d2d_async(first.ptr + c * stride, first.ptr, nb))
-        x = lib.to_device(normal(K, 200 + si))
+        x = lib.to_device(normal(K, xseed))
         y = lib.empty(N)
-        rings.append(dict(N=N, K=K, nb=nb, stride=stride, copies=copies, buf=first, x=x, y=y, it=0,
-                          host=None if a.no_cpu else host))
+        return dict(N=N, K=K, nb=nb, stride=stride, copies=copies, buf=first, x=x, y=y, it=0,
+                    host=None if a.no_cpu else host)
+
+    rings = [make_ring(N, K, 100 + si, 200 + si) for si, (N, K) in enumerate(SHAPES)]
     lib.sync()
 
     # every shape's GPU result (through the last copy of its ring), kept for the CPU leg's check
@@ -589,22 +606,49 @@ def main():
     dom = rings[-1]
     in_step_ms = float(np.mean([lib.elapsed_ms(e0, e1) for (e0, e1) in evs]))
 
-    # per-shape rates (events around R back-to-back launches, rotating copies)
+    # per-shape rates (events around R back-to-back launches, rotating copies), and beside each:
+    # a kernel that only READS the same bytes of the same rotating copies (the floor any GEMV
+    # launch over them has, launch included) and the GEMV over ONE copy read again and again
+    # (what it would take if its weights already waited in the last-level cache)
     per_shape = {}
     e0, e1 = lib.event(), lib.event()
-    for r in rings:
-        n = max(10, min(r["copies"], 60))
+    sink = lib.empty(4)
+
+    def median_us(call, n):
         rounds = []
         for _ in range(5):      # median of 5 rounds, the reference's discipline (bench_q4_gemv.cpp:106-119)
             lib.record(e0)
             for i in range(n):
-                lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"], wq_off=((r["it"] + i) % r["copies"]) * r["stride"])
+                call(i)
             lib.record(e1)
-            rounds.append(lib.elapsed_ms(e0, e1) / n)
-            r["it"] += n
-        ms = float(np.median(rounds))
-        per_shape["%dx%d" % (r["N"], r["K"])] = {"us": round(ms * 1e3, 2),
-                                                 "GB/s": round(r["nb"] / ms / 1e6, 1)}
+            rounds.append(lib.elapsed_ms(e0, e1) / n * 1e3)
+        return float(np.median(rounds))
+
+    def shape_line(r):
+        n = max(10, min(r["copies"], 60))
+        off = lambda i: ((r["it"] + i) % r["copies"]) * r["stride"]
+        us = median_us(lambda i: lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"], wq_off=off(i)), n)
+        r["it"] += n
+        nb16 = r["nb"] & ~15
+        floor = min(median_us(lambda i: lib.bench_read(r["buf"], nb16, sink, blocks, off=off(i)), n)
+                    for blocks in (256, 512, 1024))
+        line = {"us": round(us, 2), "GB/s": round(r["nb"] / us / 1e3, 1),
+                "read_floor_us": round(floor, 2), "frac_of_read": round(floor / us, 3)}
+        if r["nb"] <= 100e6:
+            line["resident_us"] = round(median_us(lambda i: lib.gemv_q4(r["x"], r["buf"], r["y"], r["N"], r["K"]), n), 2)
+        return line
+
+    for r in rings:
+        per_shape["%dx%d" % (r["N"], r["K"])] = shape_line(r)
+    # BASELINE configs[0], the reference's own CPU-runnable case (bench_q4_gemv.cpp's first shape):
+    # a 2.7 MB weight, i.e. a launch and little else; outside `value`, which is configs[1]'s sweep
+    r0 = make_ring(4864, 896, 99, 299)
+    config0 = shape_line(r0)
+    if not a.no_cpu:
+        lib.gemv_q4(r0["x"], r0["buf"], r0["y"], r0["N"], r0["K"], wq_off=(r0["copies"] - 1) * r0["stride"])
+        guards.append((r0["x"].numpy(), r0["host"], r0["N"], r0["K"], r0["y"].numpy()))
+    r0["buf"].free()
+    sink.free()
     # dominant kernel: average launch duration over back-to-back launches of the LM-head
     # GEMV (events on the library's stream), the figure rocprofv3 --kernel-trace reports too
     dom_ms = per_shape["152064x3584"]["us"] * 1e-3
@@ -629,7 +673,8 @@ def main():
                                "3584x3584, 512x3584, 18944x3584, 3584x18944, 152064x3584, batch 1, "
                                "group-32 scales, weights rotated through >1.2 GB of copies per shape",
                    "bytes_per_step": step_bytes, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-                   "per_shape": per_shape},
+                   "per_shape": per_shape,
+                   "config0_4864x896": config0},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": "gemv_rows_kernel<FmtQ4,4,0,64,0> on 152064x3584 (LM head)",
@@ -645,7 +690,10 @@ def main():
         out["cpu_baseline"] = cpu_baseline(guards)
     if not a.no_decode:
         guard7b = None if a.no_cpu else decode_guard(lib)
-        out["decode"] = decode_7b(lib, max(10, a.steps), eager=a.eager_decode)
+        warm = tuple(int(v) for v in a.decode_warm.split(":")) if a.decode_warm else None
+        out["decode"] = decode_7b(lib, max(10, a.steps), eager=a.eager_decode, warm=warm)
+        if warm:
+            out["decode"]["warm"] = {"mode": warm[0], "blocks": warm[1]}
         if guard7b is not None:
             out["decode"]["checked_against_oracle"] = guard7b
         cpu_dec = out.get("cpu_baseline", {}).get("decode_7b_ctx4096")

@@ -121,6 +121,8 @@ SIGNATURES = {
     "tlhip_tune_reset": (cint, []),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
+    "tlhip_warm_fork": (cint, [P, P, cint, cint, cint]),
+    "tlhip_warm_join": (cint, []),
 }
 
 

@@ -22,6 +22,11 @@ struct Context {
   int lds_per_cu = 0;
   int64_t hbm_bytes = 0;
   hipStream_t stream = nullptr;   // every launch and async copy goes here
+  // A second stream of the same priority that only ever runs weight warm-up reads
+  // (tlhip_warm_fork / tlhip_warm_join); created on first use.
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  bool side_open = false;         // reads queued on `side` that the main stream has not joined yet
   bool capturing = false;
   // grow-only device scratch (split-K / split-KV partials, argmax partials)
   void* scratch = nullptr;

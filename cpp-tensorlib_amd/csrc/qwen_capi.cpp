@@ -229,6 +229,21 @@ int tlq_run_layers(void* hv, int64_t token, int64_t pos) {
   return qwen::run_layers(h->M, h->M.s.embedb, pos) ? 0 : -1;
 }
 
+// n eager steps at one position with events between the regions of the step; out[0..6] = qkv,
+// attention, o-proj, gate|up, down (each per layer), LM head and the whole step, microseconds.
+int tlq_profile_steps(void* hv, int64_t token, int64_t pos, int64_t n, double* out) {
+  auto* h = static_cast<handle*>(hv);
+  qwen::step_prof p;
+  for (int64_t i = 0; i < n; i++)
+    if (!qwen::profile_step(h->M, token, pos, p)) return -1;
+  if (p.n == 0) return -1;
+  const double per_layer = 1e3 / ((double)p.n * (double)h->M.d.n_layers), per_step = 1e3 / (double)p.n;
+  out[0] = p.qkv * per_layer; out[1] = p.attn * per_layer; out[2] = p.oproj * per_layer;
+  out[3] = p.gateup * per_layer; out[4] = p.down * per_layer; out[5] = p.head * per_step;
+  out[6] = p.total * per_step;
+  return 0;
+}
+
 int64_t tlq_argmax(void* hv) {
   auto* h = static_cast<handle*>(hv);
   int64_t idx = -1;
@@ -290,6 +305,10 @@ void tlq_set_fused_prefill(void* hv, int on) { static_cast<handle*>(hv)->M.fused
 // prompt chunks of bf16 weights on their prepared f16 images (default) or on the bf16 rows
 void tlq_set_prompt_f16(void* hv, int on) { static_cast<handle*>(hv)->M.prompt_f16 = on != 0; }
 void tlq_set_gateup_epilogue(void* hv, int on) { static_cast<handle*>(hv)->M.gateup_epilogue = on != 0; }
+void tlq_set_warm(void* hv, int blocks, int nt, int mode) {
+  auto& M = static_cast<handle*>(hv)->M;
+  M.warm_blocks = blocks; M.warm_nt = nt != 0; M.warm_mode = mode;
+}
 int tlq_replay(void* hv) { return static_cast<handle*>(hv)->cap.replay() ? 0 : -1; }
 void tlq_flush() { hip::flush(); }
 

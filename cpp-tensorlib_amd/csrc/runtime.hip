@@ -81,6 +81,64 @@ __global__ __launch_bounds__(256) void read16_kernel(const u32x4* __restrict__ s
   if (acc == 0x9e3779b9u) sink[0] = acc;  // practically never: keeps the loads alive
 }
 
+// Reads up to four byte ranges, one after the other, and keeps nothing: what it leaves behind is
+// the ranges' lines in the last-level cache (and in the L2 of the XCD that read them).
+struct WarmRanges { const u32x4* p[4]; uint32_t n16[4]; };
+template <bool NT>
+__global__ __launch_bounds__(256) void warm_kernel(WarmRanges r, uint32_t* __restrict__ sink) {
+  uint32_t acc = 0;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+#pragma unroll 1
+  for (int j = 0; j < 4; j++) {
+    const u32x4* __restrict__ src = r.p[j];
+    const size_t n16 = r.n16[j];
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+      u32x4 a, b, c, d;
+      if (NT) {
+        a = __builtin_nontemporal_load(&src[i]);
+        b = __builtin_nontemporal_load(&src[i + stride]);
+        c = __builtin_nontemporal_load(&src[i + 2 * stride]);
+        d = __builtin_nontemporal_load(&src[i + 3 * stride]);
+      } else {
+        a = src[i]; b = src[i + stride]; c = src[i + 2 * stride]; d = src[i + 3 * stride];
+      }
+      acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < n16; i += stride) {
+      const u32x4 a = NT ? __builtin_nontemporal_load(&src[i]) : src[i];
+      acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+  }
+  if (acc == 0x9e3779b9u && r.n16[0] == 0xffffffffu) sink[0] = acc;  // never: keeps the loads alive
+}
+
+// The same reads by short-lived blocks: block b reads 32 KB (eight 16-byte loads per thread, all in
+// flight at once) of the ranges laid end to end and exits, so the blocks fit into whatever room
+// the launches of the main stream leave.
+__global__ __launch_bounds__(256) void warm_short_kernel(WarmRanges r, uint32_t* __restrict__ sink) {
+  size_t u = (size_t)blockIdx.x * 2048 + threadIdx.x;     // first 16-byte unit of this thread
+  const u32x4* src = nullptr;
+  size_t n16 = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const size_t nj = (r.n16[j] + 2047) & ~size_t(2047);  // each range starts a new block
+    if (!src && u < nj) { src = r.p[j]; n16 = r.n16[j]; }
+    if (!src) u -= nj;
+  }
+  if (!src) return;
+  u32x4 v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const size_t k = u + (size_t)i * 256;
+    v[i] = src[k < n16 ? k : n16 - 1];
+  }
+  uint32_t acc = 0;
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+  if (acc == 0x9e3779b9u && r.n16[0] == 0xffffffffu) sink[0] = acc;  // never: keeps the loads alive
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;
@@ -240,6 +298,7 @@ int tlhip_graph_end(void** graph_exec) {
   if (!c.capturing) return fail(TLHIP_EINVAL, "no capture open");
   if (!graph_exec) return fail(TLHIP_EINVAL, "tlhip_graph_end: null out pointer");
   *graph_exec = nullptr;
+  if (c.side_open) (void)tlhip_warm_join();   // a capture cannot end with a branch left open
   hipGraph_t g = nullptr;
   hipError_t e = hipStreamEndCapture(c.stream, &g);
   c.capturing = false;
@@ -296,6 +355,50 @@ int tlhip_event_destroy(void* ev) {
   if (!ev) return TLHIP_OK;
   hipError_t e = hipEventDestroy(static_cast<hipEvent_t>(ev));
   return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipEventDestroy");
+}
+
+int tlhip_warm_fork(const void* const* ptrs, const int64_t* bytes, int n, int blocks, int nontemporal) {
+  TLHIP_REQUIRE_READY();
+  Context& c = ctx();
+  if (n < 0 || n > 4 || (n > 0 && (!ptrs || !bytes))) return fail(TLHIP_EINVAL, "tlhip_warm_fork: 0..4 ranges");
+  WarmRanges r = {};
+  for (int i = 0; i < n; i++) {
+    if (!ptrs[i] || bytes[i] < 0 || !aligned16(ptrs[i]) || (bytes[i] >> 4) > 0xfffffff0ll)
+      return fail(TLHIP_EINVAL, "tlhip_warm_fork: ranges are 16-byte aligned and below 64 GiB");
+    r.p[i] = static_cast<const u32x4*>(ptrs[i]);
+    r.n16[i] = (uint32_t)(bytes[i] >> 4);
+  }
+  if (n == 0) return TLHIP_OK;
+  hipError_t e = hipSuccess;
+  if (!c.side) {
+    if (c.capturing) return fail(TLHIP_EUNSUPPORTED, "tlhip_warm_fork: first call inside a capture");
+    if ((e = hipStreamCreate(&c.side)) != hipSuccess) return hip_fail(e, "hipStreamCreate");
+    if ((e = hipEventCreateWithFlags(&c.ev_fork, hipEventDisableTiming)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&c.ev_join, hipEventDisableTiming)) != hipSuccess)
+      return hip_fail(e, "hipEventCreate");
+  }
+  if (blocks == 0) blocks = 32;
+  if (blocks > 4096) blocks = 4096;
+  size_t short_blocks = 0;
+  for (int i = 0; i < n; i++) short_blocks += ((size_t)r.n16[i] + 2047) / 2048;
+  if ((e = hipEventRecord(c.ev_fork, c.stream)) != hipSuccess) return hip_fail(e, "hipEventRecord");
+  if ((e = hipStreamWaitEvent(c.side, c.ev_fork, 0)) != hipSuccess) return hip_fail(e, "hipStreamWaitEvent");
+  c.side_open = true;
+  if (blocks < 0) warm_short_kernel<<<dim3((unsigned)short_blocks), dim3(256), 0, c.side>>>(r, (uint32_t*)c.argmax_dev + 8);
+  else if (nontemporal) warm_kernel<true><<<dim3(blocks), dim3(256), 0, c.side>>>(r, (uint32_t*)c.argmax_dev + 8);
+  else warm_kernel<false><<<dim3(blocks), dim3(256), 0, c.side>>>(r, (uint32_t*)c.argmax_dev + 8);
+  e = hipGetLastError();
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "warm kernel");
+}
+
+int tlhip_warm_join(void) {
+  TLHIP_REQUIRE_READY();
+  Context& c = ctx();
+  if (!c.side_open) return TLHIP_OK;
+  c.side_open = false;
+  hipError_t e = hipEventRecord(c.ev_join, c.side);
+  if (e == hipSuccess) e = hipStreamWaitEvent(c.stream, c.ev_join, 0);
+  return e == hipSuccess ? TLHIP_OK : hip_fail(e, "tlhip_warm_join");
 }
 
 int tlhip_census(uint64_t* counts, int n) {

@@ -166,6 +166,12 @@ struct api {
                                 void*, int64_t, int64_t, int64_t, float) = nullptr;
   int (*gemv_bf16_row_rmsnorm_gateup)(const void*, const void*, const void*, void*, const void*, void*,
                                       int64_t, int64_t, float) = nullptr;
+  int (*warm_fork)(const void* const*, const int64_t*, int, int, int) = nullptr;
+  int (*warm_join)() = nullptr;
+  int (*event_create)(void**) = nullptr;
+  int (*event_record)(void*) = nullptr;
+  int (*event_elapsed_ms)(void*, void*, float*) = nullptr;
+  int (*event_destroy)(void*) = nullptr;
 };
 
 // ---- buffer ledger ----------------------------------------------------------------
@@ -329,6 +335,11 @@ struct context {
               bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm") &&
               bind(f.gemv_q4_rmsnorm_gateup, "tlhip_gemv_q4_rmsnorm_gateup") &&
               bind(f.gemv_bf16_row_rmsnorm_gateup, "tlhip_gemv_bf16_row_rmsnorm_gateup");
+    if (!ok) return;
+    bind(f.warm_fork, "tlhip_warm_fork") && bind(f.warm_join, "tlhip_warm_join");   // optional
+    why.clear();
+    ok = bind(f.event_create, "tlhip_event_create") && bind(f.event_record, "tlhip_event_record") &&
+         bind(f.event_elapsed_ms, "tlhip_event_elapsed_ms") && bind(f.event_destroy, "tlhip_event_destroy");
     if (!ok) return;
     if (f.abi_version() != 1) {
       why = "libtensorlib_hip.so has a different ABI version";
@@ -883,6 +894,19 @@ inline bool incr_u32(void* d_pos) {
   L.writes(d_pos);
   return L.sent(L.lib.incr_u32(d_pos));
 }
+// Weights that launches further down the stream will stream: read them now on a second stream
+// (up to four device ranges, in the order given) so that they wait in the last-level cache.
+// No counterpart in the reference. warm_join makes the stream wait for the reads.
+inline bool warm_fork(const void* const* ptrs, const int64_t* bytes, int n, int blocks, bool nontemporal) {
+  launch L;
+  if (!L.ok || !L.lib.warm_fork) return false;
+  for (int i = 0; i < n; i++) L.reads(ptrs[i]);
+  return L.sent(L.lib.warm_fork(ptrs, bytes, n, blocks, nontemporal ? 1 : 0));
+}
+inline bool warm_join() {
+  launch L;
+  return L.ok && L.lib.warm_join && L.sent(L.lib.warm_join());
+}
 inline bool kv_append_dpos(void* Kc, void* Vc, void* k_new, void* v_new, void* d_pos, int64_t kv_max,
                            int64_t n_kv_heads, int64_t D, bool kv_bf16 = false) {
   launch L;
@@ -1143,6 +1167,28 @@ inline bool gemv_bf16_row_rmsnorm_gateup(void* x, void* delta, void* norm_w, voi
   if (xout) L.writes(xout);
   L.writes(act);
   return L.sent(L.lib.gemv_bf16_row_rmsnorm_gateup(x, delta, norm_w, xout, B, act, n2, k, eps));
+}
+
+// ---- events on the library's stream: GPU time between two points of the launch sequence ------
+inline void* event_create() {
+  auto& c = context::get();
+  void* ev = nullptr;
+  return c.ready && c.f.event_create(&ev) == 0 ? ev : nullptr;
+}
+inline bool event_record(void* ev) {
+  auto& c = context::get();
+  return c.ready && ev && c.f.event_record(ev) == 0;
+}
+// Waits for `stop`; negative when either event is unusable.
+inline float event_elapsed_ms(void* start, void* stop) {
+  auto& c = context::get();
+  float ms = -1.0f;
+  if (!c.ready || !start || !stop || c.f.event_elapsed_ms(start, stop, &ms) != 0) return -1.0f;
+  return ms;
+}
+inline void event_destroy(void* ev) {
+  auto& c = context::get();
+  if (c.ready && ev) c.f.event_destroy(ev);
 }
 
 // ---- graph capture (cuda.h:508-551), hipGraph underneath --------------------------

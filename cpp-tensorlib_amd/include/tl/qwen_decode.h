@@ -151,6 +151,16 @@ struct prefill_scratch {
   float* emb_host = nullptr;
 };
 
+// GPU time per region of a decode step, from events on the library's stream around the launches
+// of each region (the role of the reference harness's StepProf, qm:543-552, whose regions are
+// host-side because its step is host-bound; this step is a chain of launches, so the regions are
+// the launches). Sums over layers and steps, in milliseconds; `n` counts steps. The events cost
+// a little GPU time themselves: read the shares, not the total, against an unprofiled step.
+struct step_prof {
+  double qkv = 0, attn = 0, oproj = 0, gateup = 0, down = 0, head = 0, total = 0;
+  int64_t n = 0;
+};
+
 struct model {
   dims d{};
   prefill_scratch ps;
@@ -172,6 +182,12 @@ struct model {
   bool fused_prefill = true;     // prompt chunks: one launch for split_heads + rope + kv_fill, attention writes token-major
   bool prompt_f16 = true;        // prompt chunks of bf16 weights on the backend's prepared f16 form of them (a second copy, made on first use)
   bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
+  // within the fused path: blocks of the weight warm-up that runs beside each layer on a second
+  // stream (0 = none); warm_nt: with streaming loads; warm_mode picks what is read when
+  int warm_blocks = 0;
+  bool warm_nt = false;
+  int warm_mode = 0;
+  std::vector<void*> prof_events;   // profile_step's events: 5 per layer + 2, recorded by run_layers when set
 };
 
 namespace detail {
@@ -665,9 +681,23 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     void* din = nullptr;     // MLP output of the previous layer, not yet added
     if (!M.rope_tab) M.rope_tab = hip::alloc_device(d.head_dim * 4);
     ok &= M.rope_tab && hip::rope_table(M.rope_tab, d.head_dim, pos, d_pos, d.rope_base);
+    size_t marks = 0;
+    auto mark = [&] { if (marks < M.prof_events.size()) ok &= hip::event_record(M.prof_events[marks++]); };
     for (int64_t l = 0; l < d.n_layers; l++) {
       layer& L = M.layers[(size_t)l];
+      mark();
+      auto warm = [&](int mode) {
+        if (M.warm_blocks == 0 || M.warm_mode != mode) return;
+        const linear& nx = (l + 1 < d.n_layers) ? M.layers[(size_t)l + 1].wqkv : M.lm_head;
+        const void* p[4] = {L.wo.w, L.wgu.w, L.wd.w, nx.w};
+        int64_t b[4] = {L.wo.bytes(), L.wgu.bytes(), L.wd.bytes(), std::min<int64_t>(nx.bytes(), int64_t(16) << 20)};
+        for (auto& x : b) x &= ~int64_t(15);
+        ok &= hip::warm_fork(p, b, mode == 1 || mode == 3 ? 2 : mode == 4 ? 3 : 4, M.warm_blocks, M.warm_nt);
+      };
+      warm(0); warm(1);            // beside the whole layer: everything / o-proj and gate|up only
       ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
+      warm(2); warm(3); warm(4);   // beside attention: everything / o-proj and gate|up / + down
+      mark();
       if (M.fused_attn) {
         if (!d_pos) L.cache.pos = pos;
         ok &= L.cache.attn_qkv(S.qkvb, L.bq, L.bk, L.bv, S.ab, d.n_q_heads, scale, M.rope_tab, d_pos,
@@ -681,18 +711,25 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
         ok &= L.cache.rope_append_tab(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, M.rope_tab);
         ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
       }
+      mark();
       ok &= gemv(L.wo, S.ab, S.hb);
+      mark();
       if (M.gateup_epilogue) {
         ok &= gemv_rmsnorm_gateup(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.mb, d.eps);
+        mark();
         ok &= gemv(L.wd, S.mb, S.mdb);
       } else {
         ok &= gemv_rmsnorm(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.gub, d.eps);
+        mark();
         ok &= gemv_swiglu(L.wd, S.gub, S.mdb);
       }
       rin = S.res[1];
       din = S.mdb;
     }
+    mark();
     ok &= gemv_rmsnorm(M.lm_head, rin, din, M.onorm, nullptr, logits_out ? logits_out : S.logitsb, d.eps);
+    mark();
+    if (M.warm_blocks != 0) ok &= hip::warm_join();
     if (d_pos && advance) ok &= hip::incr_u32(d_pos);
     return ok;
   }
@@ -723,6 +760,37 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     x = ro;
   }
   ok &= gemv(M.lm_head, S.hb, logits_out ? logits_out : S.logitsb);
+  return ok;
+}
+
+// One eager step of the fused launch sequence with an event between its regions; the regions'
+// GPU times are added to `p`. false when a launch or an event was declined.
+inline bool profile_step(model& M, int64_t token, int64_t pos, step_prof& p) {
+  if (!M.fused || !stage_embed(M, token)) return false;
+  const size_t L = (size_t)M.d.n_layers, want = 5 * L + 2;
+  while (M.prof_events.size() < want) {
+    void* ev = hip::event_create();
+    if (!ev) break;
+    M.prof_events.push_back(ev);
+  }
+  bool ok = M.prof_events.size() == want && run_layers(M, M.s.embedb, pos);
+  hip::flush();
+  std::vector<void*> ev;
+  ev.swap(M.prof_events);          // later steps run without marks
+  if (ok) {
+    auto ms = [&](size_t a, size_t b) { return (double)hip::event_elapsed_ms(ev[a], ev[b]); };
+    for (size_t l = 0; l < L; l++) {
+      p.qkv += ms(5 * l, 5 * l + 1);
+      p.attn += ms(5 * l + 1, 5 * l + 2);
+      p.oproj += ms(5 * l + 2, 5 * l + 3);
+      p.gateup += ms(5 * l + 3, 5 * l + 4);
+      p.down += ms(5 * l + 4, 5 * l + 5);
+    }
+    p.head += ms(5 * L, 5 * L + 1);
+    p.total += ms(0, 5 * L + 1);
+    p.n++;
+  }
+  for (void* e : ev) hip::event_destroy(e);
   return ok;
 }
 

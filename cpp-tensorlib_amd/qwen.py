@@ -59,6 +59,8 @@ def _load():
             "tlq_capture": (cint, [P, i64, i64]),
             "tlq_replay": (cint, [P]),
             "tlq_set_fused": (None, [P, cint]),
+            "tlq_set_warm": (None, [P, cint, cint, cint]),
+            "tlq_profile_steps": (cint, [P, i64, i64, i64, C.POINTER(C.c_double)]),
             "tlq_set_fused_attn": (None, [P, cint]),
             "tlq_set_gateup_epilogue": (None, [P, cint]),
             "tlq_set_fused_prefill": (None, [P, cint]),
@@ -333,6 +335,19 @@ class QwenGPU:
 
     def set_fused(self, on):
         self.L.tlq_set_fused(self.h, 1 if on else 0)
+
+    def profile_steps(self, token, pos, n=5):
+        """GPU microseconds per region of the fused decode step (events between the launches of
+        n eager steps): per layer qkv / attention / o-proj / gate|up / down, then the LM head and the step."""
+        out = (C.c_double * 7)()
+        if self.L.tlq_profile_steps(self.h, token, pos, n, out) != 0:
+            raise RuntimeError("profile_steps: a launch or an event was declined")
+        names = ("qkv_gemv", "attention", "o_proj_gemv", "gateup_gemv", "down_gemv", "lm_head", "step")
+        return {k: float(v) for k, v in zip(names, out)}
+
+    def set_warm(self, blocks, nt=False, mode=0):
+        """Within the fused path: weight warm-up reads on a second stream beside each layer (0 blocks = off)."""
+        self.L.tlq_set_warm(self.h, int(blocks), 1 if nt else 0, int(mode))
 
     def set_fused_attn(self, on):
         """Within the fused path: run the q/k/v epilogue inside the attention launch (default) or alone."""

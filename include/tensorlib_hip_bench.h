@@ -9,6 +9,7 @@
 #define TENSORLIB_HIP_BENCH_H
 
 #include <stddef.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -20,6 +21,17 @@ extern "C" {
  * counters. blocks <= 0 picks 8 blocks per CU. */
 int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks);
 int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
+
+/* ---- weight warm-up on a second stream ---------------------------------------------------
+ * tlhip_warm_fork: up to four byte ranges (16-byte aligned) are read once, in the order given, by
+ * `blocks` blocks of 256 threads (<= 0: 32) on a second stream of the same priority that starts
+ * where the main stream stands now; nothing is written. What the reads leave behind is the
+ * ranges' lines in the last-level cache, so that a later launch on the main stream finds them
+ * there. nontemporal != 0 reads with streaming loads. tlhip_warm_join makes the main stream wait
+ * for every fork since the last join (a capture must join before it ends; tlhip_graph_end does it
+ * if the caller did not). Both record into an open capture as a parallel branch. */
+int tlhip_warm_fork(const void* const* ptrs, const int64_t* bytes, int n, int blocks, int nontemporal);
+int tlhip_warm_join(void);
 
 /* ---- launch-shape overrides ----------------------------------------------------------
  * The int4 GEMV launch shape: rows per wavefront (1,2,4,8), wavefronts sharing one row's K
