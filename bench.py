@@ -174,8 +174,10 @@ def decode_guard(lib):
     one-layer model with the 7B dimensions (hidden 3584, 28/4 heads of 128, MLP 18944; a small
     vocabulary - the LM-head shape is checked by the sweep's guard) built from the oracle's
     seeded weights, caches of 4352 rows seeded up to row 4095 on both sides, one fused step at
-    position 4095 eagerly and one from a recorded graph with the position on the device. Bar: the
-    reference's own for a decode loop, logits maxrel < 2e-3 (check_llm_decode.cpp:268-276)."""
+    position 4095 eagerly and one from a recorded graph with the position on the device. Bar:
+    logits max |d| / (1 + |ref|) < 1e-4 (a few times what the step measures; the reference's own
+    bar for a decode loop is 2e-3, check_llm_decode.cpp:268-276); the share of logits inside
+    allclose(rtol 1e-4, atol 1e-5) is reported beside it."""
     from oraclelib import QWEN_7B, maxrel, oracle
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
     orc = oracle()
@@ -192,12 +194,14 @@ def decode_guard(lib):
     ok = g.decoder_init(1234, pos)
     _, replay = g.decoder_step(1234, want_logits=True)
     worst = max(maxrel(eager, want), maxrel(replay, want))
+    inside = min(float(np.mean(np.abs(r.astype(np.float64) - want) <= 1e-5 + 1e-4 * np.abs(want))) for r in (eager, replay))
     g.close(); om.close()
-    if not (worst < 2e-3):
+    if not (worst < 1e-4):
         print("bench.py: 7B-shape decode step differs from the CPU oracle (maxrel %.2e)" % worst, file=sys.stderr)
         sys.exit(3)
     return {"what": "one-layer 7B-dims model, step at position 4095, eager and recorded graph, vs the CPU oracle",
-            "logits_maxrel": float("%.3g" % worst), "bar": 2e-3, "graph_captured": bool(ok)}
+            "logits_maxrel": float("%.3g" % worst), "bar": 1e-4, "logits_inside_allclose_1e-4_1e-5": round(inside, 5),
+            "graph_captured": bool(ok)}
 
 
 def decode_7b(lib, steps, eager=False, warm=None):

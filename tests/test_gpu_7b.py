@@ -4,17 +4,30 @@ model with the full 152064-row LM head, and one layer's 512-token prompt chunk a
 and deep in a context, against the CPU oracle on the same weight bytes and the same seeded
 cache rows.
 
-Bars are the reference's own: logits maxrel < 2e-3 and identical greedy ids for a decode loop
+The reference checks these with logits maxrel < 2e-3 and identical greedy ids for a decode loop
 (check_llm_decode.cpp:268-276; ids may differ only where the top-2 logits are within
-rtol 1e-4 / atol 1e-5), maxrel < 2e-4 for one decoder block (check_llm_block.cpp:94-98, 242)."""
+rtol 1e-4 / atol 1e-5), maxrel < 2e-4 for one decoder block (check_llm_block.cpp:94-98, 242);
+the bars asserted here are tighter (below) and the share of elements inside allclose(rtol 1e-4,
+atol 1e-5) is asserted beside them."""
 import importlib
 
 import numpy as np
 import pytest
 
-from oraclelib import QWEN_7B, maxrel
+from oraclelib import QWEN_7B, check_logits
 
 pytestmark = pytest.mark.gpu
+
+# Bars: max |d| / (1 + |ref|) at under five times what these tests measure on the MI355X (3.8e-5
+# for the step two tokens past position 4095; the reference's own bars for the same checks are
+# 2e-3 and 2e-4), and the least fraction of elements that must sit inside allclose(rtol 1e-4,
+# atol 1e-5) of the oracle. Random-init logits are a few hundredths in size, so it is the atol that
+# binds: the fp32 chains of the two sides differ by up to 4e-5 on them (98.9 % inside, the worst
+# element 3.1 tolerances out). The chunk's final-norm rows divide a residual of size ~0.03 by its
+# rms, which magnifies the two sides' 1e-6 differences thirty times: 4.6e-5 measured, 5.2e-5 on the
+# logits of the step that follows the chunk (97.5 % inside).
+STEP_BAR, STEP_FRAC = 1.5e-4, 0.97
+CHUNK_BAR, CHUNK_FRAC = 2e-4, 0.95
 
 
 def _near_tie(logits, rtol=1e-4, atol=1e-5):
@@ -56,9 +69,7 @@ def test_decode_step_at_7b_dims_deep_in_a_context(orc):
         print("case 7B step", name, flush=True)
         g.set_fused(fused); g.set_fused_attn(fattn); g.set_gateup_epilogue(gu)
         got_tok, got_logits = g.step(tok, pos, want_logits=True)      # rewrites cache row 4095 identically
-        mr = maxrel(got_logits, want_logits)
-        print("   logits maxrel %.2e" % mr, flush=True)
-        assert mr < 2e-3, (name, mr)
+        check_logits(got_logits, want_logits, STEP_BAR, "logits " + name, STEP_FRAC)
         assert got_tok == want_tok or _near_tie(want_logits), (name, got_tok, want_tok)
     g.set_fused(True); g.set_fused_attn(True); g.set_gateup_epilogue(True)
     # one recorded graph, position on the device: positions 4095 (again), 4096, 4097
@@ -69,9 +80,7 @@ def test_decode_step_at_7b_dims_deep_in_a_context(orc):
         if p > pos:
             want_tok, want_logits = om.step(feed, p)
         got_tok, got_logits = g.decoder_step(feed, want_logits=True)
-        mr = maxrel(got_logits, want_logits)
-        print("   pos %d logits maxrel %.2e" % (p, mr), flush=True)
-        assert mr < 2e-3, (p, mr)
+        check_logits(got_logits, want_logits, STEP_BAR, "logits pos %d" % p, STEP_FRAC)
         assert got_tok == want_tok or _near_tie(want_logits), (p, got_tok, want_tok)
         feed = want_tok
     g.decoder_sync_host_pos()
@@ -160,14 +169,11 @@ def test_prefill_chunk_at_7b_dims(orc, q4):
             g.set_cache_pos(pos0)
             g.prefill(tokens, chunk=T, want_logits=False)
             got = g.prefill_hidden(T)[rows]
-            mr = maxrel(got, want)
-            print("   final-norm rows maxrel %.2e" % mr, flush=True)
-            assert np.all(np.isfinite(got))
-            assert mr < 2e-4, (pos0, fused, f16, mr)
+            check_logits(got, want, CHUNK_BAR, "final-norm rows", CHUNK_FRAC)
         # decode continues on the caches the chunk filled
         tok = int(tokens[-1])
         want_tok, want_logits = om.step(tok, pos0 + T)
         got_tok, got_logits = g.step(tok, pos0 + T, want_logits=True)
-        assert maxrel(got_logits, want_logits) < 2e-3
+        check_logits(got_logits, want_logits, CHUNK_BAR, "logits of the step after the chunk", CHUNK_FRAC)
         assert got_tok == want_tok or _near_tie(want_logits)
     g.close(); om.close()

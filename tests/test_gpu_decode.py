@@ -10,9 +10,16 @@ import importlib
 import numpy as np
 import pytest
 
-from oraclelib import maxrel
+from oraclelib import check_logits
 
 pytestmark = pytest.mark.gpu
+
+# max |d| / (1 + |ref|) of the logits, at under five times what these loops measure on the MI355X
+# (2.3e-6 at the small dims, 6.9e-6 at config 4's; the reference's own bar for a decode loop is
+# 2e-3), and the fraction of a logits vector that must sit inside allclose(rtol 1e-4, atol 1e-5)
+# of the oracle's: all of it (the worst element measured uses 0.21 / 0.62 of its tolerance).
+BAR, FRAC = 1e-5, 1.0
+CFG4_BAR = 3e-5
 
 SMALL = dict(n_layers=3, hidden=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ff=1024, vocab=1000,
              max_ctx=96, eps=1e-6, rope_base=1e6)
@@ -38,17 +45,17 @@ def test_decode_loop_matches_oracle(orc, dims, steps, mode):
     g.set_gateup_epilogue(mode != "fused_swiglu_in_down")
     rng = np.random.default_rng(5)
     tok = int(rng.integers(0, dims["vocab"]))
-    worst = 0.0
+    worst, least = 0.0, 1.0
     for pos in range(steps):
         want_tok, want_logits = om.step(tok, pos)
         got_tok, got_logits = g.step(tok, pos, want_logits=True)
-        worst = max(worst, maxrel(got_logits, want_logits))
-        assert maxrel(got_logits, want_logits) < 2e-3, (pos, worst)
+        mr, frac = check_logits(got_logits, want_logits, BAR, "pos %d" % pos, FRAC)
+        worst, least = max(worst, mr), min(least, frac)
         if got_tok != want_tok:
             assert _near_tie(want_logits), (pos, got_tok, want_tok)
         # feed the oracle's token so one near-tie cannot fork the two runs
         tok = want_tok if pos >= 8 else int(rng.integers(0, dims["vocab"]))
-    print("decode loop worst logits maxrel: %.2e" % worst)
+    print("decode loop worst logits maxrel: %.2e, least allclose fraction %.5f" % (worst, least))
     c = g.census()
     assert c["gemv_q4"] >= steps * (4 * dims["n_layers"] + 1) and c["attn_decode"] >= steps * dims["n_layers"]
     g.close(); om.close()
@@ -74,19 +81,15 @@ def test_graph_replay_equals_eager(orc):
     g.close(); om.close()
 
 
-def test_config4_qwen05b_greedy_tokens_match_reference_golden(orc):
-    """BASELINE config 4: Qwen2.5-0.5B architecture (24 layers, hidden 896, 14/2 heads,
-    head_dim 64, MLP 4864, vocab 151936), int4 weights with bf16 embeddings, 128 prompt
-    ids + 256 greedy tokens. The golden argmax sequence and top-2 margins come from the
-    REAL reference's CPU path (tests/golden/make_golden.py qwen05b). The GPU run is fed
-    the golden tokens (so one near-tie cannot fork the runs) and must pick the same
-    token at every position unless the reference's own top-2 logits are within
-    rtol=1e-4 / atol=1e-5 of each other."""
+@pytest.fixture(scope="module")
+def config4(orc):
+    """BASELINE config 4 once per module: the Qwen2.5-0.5B-architecture model (24 layers, hidden 896,
+    14/2 heads of 64, MLP 4864, vocab 151936; int4 weights, bf16 embeddings) on both sides, and the
+    golden greedy run of the REAL reference's CPU path over it (tests/golden/make_golden.py qwen05b):
+    128 prompt ids + 256 generated tokens, with the top-1 logit and the top-2 margin per position."""
     import json
     import os
     g_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-    if not os.path.exists(os.path.join(g_dir, "qwen05b_decode.npz")):
-        pytest.skip("tests/golden/qwen05b_decode.npz not generated")
     z = np.load(os.path.join(g_dir, "qwen05b_decode.npz"))
     meta = json.load(open(os.path.join(g_dir, "qwen05b_decode.json")))
     qwen = importlib.import_module("cpp-tensorlib_amd.qwen")
@@ -94,26 +97,97 @@ def test_config4_qwen05b_greedy_tokens_match_reference_golden(orc):
     om = orc.qwen_create(meta["dims"], seed=meta["seed"], q4=True)
     assert orc.crc32(om.weight(-1, "outw")) == meta["crc_outw"], "weights not regenerated identically"
     g = qwen.QwenGPU.from_blobs(om)
-    prompt, gold, margin, top1 = meta["prompt"], z["argmax"], z["margin"], z["top1"]
+    gold, margin, top1 = z["argmax"], z["margin"], z["top1"]
+    near = margin <= 1e-5 + 1e-4 * np.abs(top1)       # positions where the reference's own top two tie
+    yield dict(om=om, g=g, prompt=meta["prompt"], gold=gold, near=near, margin=margin)
+    g.close(); om.close()
+
+
+def test_config4_qwen05b_greedy_tokens_match_reference_golden(config4):
+    """Config 4 one eager step at a time. The GPU run is fed the golden tokens (so one near-tie cannot
+    fork the runs) and must pick the golden token at every position unless the reference's own
+    top-2 logits are within rtol=1e-4 / atol=1e-5 of each other there; the logits of the first
+    prompt positions are compared with the oracle model's in full."""
+    c = config4
+    g, om, prompt, gold, near = c["g"], c["om"], c["prompt"], c["gold"], c["near"]
+    g.set_cache_pos(0)
     tok, mismatches, ties = prompt[0], 0, 0
     for pos in range(len(gold)):
         got = g.step(tok, pos)
         if got != int(gold[pos]):
-            near = margin[pos] <= 1e-5 + 1e-4 * abs(top1[pos])
-            assert near, (pos, got, int(gold[pos]), float(margin[pos]))
-            ties += 1
+            if near[pos]:
+                ties += 1
+            else:
+                mismatches += 1
+                print("   pos %d: got %d, golden %d, golden margin %.3g" % (pos, got, int(gold[pos]), float(c["margin"][pos])))
         tok = prompt[pos + 1] if pos + 1 < 128 else int(gold[pos])
-    print("0.5B decode: %d positions, %d near-tie differences" % (len(gold), ties))
-    # spot-check full logits against the oracle model at the last position
-    want_tok, want_logits = None, None
-    for pos in range(0, 3):                     # oracle cache must be warm from position 0
-        want_tok, want_logits = om.step(prompt[pos], pos)
-    g2_tok, g2_logits = None, None
-    for pos in range(0, 3):
-        g2_tok, g2_logits = g.step(prompt[pos], pos, want_logits=True)
-    assert maxrel(g2_logits, want_logits) < 2e-3
+    print("0.5B decode: %d positions, %d near-tie differences of %d near-tie positions, %d mismatches"
+          % (len(gold), ties, int(near.sum()), mismatches))
     assert mismatches == 0
-    g.close(); om.close()
+    assert ties <= int(near.sum())
+    # full logits against the oracle model at the first positions (its cache must be warm from 0)
+    for pos in range(0, 3):
+        want_tok, want_logits = om.step(prompt[pos], pos)
+        got_tok, got_logits = g.step(prompt[pos], pos, want_logits=True)
+        check_logits(got_logits, want_logits, CFG4_BAR, "config 4 pos %d" % pos, FRAC)
+
+
+@pytest.mark.parametrize("chunk", [128, 48])
+def test_config4_through_the_fast_paths(config4, chunk):
+    """Config 4 the way a user runs it: the 128 golden prompt ids through prefill() (the int4 prompt
+    GEMM, causal prefill attention, the q/k/v epilogue that fills the caches; one chunk, or ragged
+    chunks of 48), then the 256 generated tokens twice - by the recorded graph with the position on
+    the device (fed the golden tokens) and by the greedy loop whose token never leaves the device.
+    Every token must be the golden one unless the reference's own top two logits tie there; after
+    such a permitted difference the on-device loop is started again from the golden token, since its
+    own sequence has left the golden one."""
+    c = config4
+    g, prompt, gold, near = c["g"], c["prompt"], c["gold"], c["near"]
+    n_prompt, n_gen = 128, len(gold) - 127
+    g.set_cache_pos(0)
+    logits = g.prefill(prompt[:n_prompt], chunk=chunk)
+    first = int(np.argmax(logits))
+    assert first == int(gold[n_prompt - 1]) or near[n_prompt - 1], (first, int(gold[n_prompt - 1]))
+    # (b0) the same logits from 128 eager steps, the path the golden test above holds to the golden
+    # tokens (the CPU oracle needs seconds per position at this size)
+    g.set_cache_pos(0)
+    for pos in range(n_prompt - 1):
+        g.step(prompt[pos], pos)
+    _, eager_logits = g.step(prompt[n_prompt - 1], n_prompt - 1, want_logits=True)
+    check_logits(logits, eager_logits, CFG4_BAR, "config 4 prompt logits, chunk %d, against eager steps" % chunk, FRAC)
+    g.set_cache_pos(0)
+    g.prefill(prompt[:n_prompt], chunk=chunk, want_logits=False)     # the caches the loops below continue on
+    # (a) recorded graph, position on the device
+    tok = int(gold[n_prompt - 1])
+    assert g.decoder_init(tok, n_prompt), "graph capture unavailable"
+    ties = mismatches = 0
+    for i in range(1, n_gen):
+        pos = n_prompt - 1 + i              # this step consumes position pos and predicts gold[pos]
+        got = g.decoder_step(tok)
+        if got != int(gold[pos]):
+            ties += bool(near[pos]); mismatches += not near[pos]
+        tok = int(gold[pos])
+    print("config 4 recorded decoder: %d tokens, %d near-tie differences, %d mismatches" % (n_gen - 1, ties, mismatches))
+    assert mismatches == 0 and ties <= int(near.sum())
+    g.decoder_sync_host_pos()
+    # (b) token loop on the device, over the caches the prompt left (rows from 128 on are rewritten)
+    pos, tok, restarts = n_prompt, int(gold[n_prompt - 1]), 0
+    while pos < len(gold):
+        g.set_cache_pos(pos)
+        g.greedy_init(tok, pos)
+        n = len(gold) - pos
+        assert g.greedy_run(n) == n
+        got = g.greedy_tokens(pos, n)
+        bad = [i for i in range(n) if int(got[i]) != int(gold[pos + i])]
+        if not bad:
+            break
+        i = bad[0]
+        assert near[pos + i], ("greedy loop left the golden sequence", pos + i, int(got[i]), int(gold[pos + i]))
+        restarts += 1
+        tok, pos = int(gold[pos + i]), pos + i + 1
+    print("config 4 greedy loop on the device: %d restarts after near-ties" % restarts)
+    assert restarts <= int(near.sum())
+    g.greedy_sync_host_pos()
 
 
 def test_bf16_decode_loop_matches_oracle(orc):
@@ -127,7 +201,7 @@ def test_bf16_decode_loop_matches_oracle(orc):
         tok = int(rng.integers(0, SMALL["vocab"]))
         want_tok, want_logits = om.step(tok, pos)
         got_tok, got_logits = g.step(tok, pos, want_logits=True)
-        assert maxrel(got_logits, want_logits) < 2e-3, pos
+        check_logits(got_logits, want_logits, BAR, "bf16 pos %d" % pos, FRAC)
         assert got_tok == want_tok or _near_tie(want_logits), pos
     assert g.census()["gemv_bf16_row"] >= 24 * (4 * SMALL["n_layers"] + 1)
     g.close(); om.close()
@@ -158,13 +232,13 @@ def test_prefill_chunks_match_token_by_token_oracle(orc, dims, n_prompt, chunk, 
     n_chunks = -(-n_prompt // chunk)
     assert after["gemm_bf16_nt"] - before["gemm_bf16_nt"] == 4 * dims["n_layers"] * n_chunks
     assert after["attn_prefill"] - before["attn_prefill"] == dims["n_layers"] * n_chunks
-    assert maxrel(got_logits, want_logits) < 2e-3, maxrel(got_logits, want_logits)
+    check_logits(got_logits, want_logits, BAR, "prompt logits", FRAC)
     assert int(np.argmax(got_logits)) == want_tok or _near_tie(want_logits)
     tok = want_tok
     for pos in range(n_prompt, n_prompt + 12):        # decode on top of the prefilled caches
         want_tok, want_logits = om.step(tok, pos)
         got_tok, got_logits = g.step(tok, pos, want_logits=True)
-        assert maxrel(got_logits, want_logits) < 2e-3, pos
+        check_logits(got_logits, want_logits, BAR, "pos %d" % pos, FRAC)
         assert got_tok == want_tok or _near_tie(want_logits), pos
         tok = want_tok
     g.close(); om.close()
@@ -194,7 +268,7 @@ def test_captured_decoder_advances_position_on_the_device(orc, dims, steps, q4):
         want_tok, want_logits = om.step(tok, pos)
         got_tok, got_logits = g.decoder_step(tok, want_logits=True)
         assert g.decoder_pos() == pos + 1
-        assert maxrel(got_logits, want_logits) < 2e-3, (pos, maxrel(got_logits, want_logits))
+        check_logits(got_logits, want_logits, BAR, "replay pos %d" % pos, FRAC)
         assert got_tok == want_tok or _near_tie(want_logits), pos
         tok = want_tok
     after = g.census()
@@ -204,7 +278,7 @@ def test_captured_decoder_advances_position_on_the_device(orc, dims, steps, q4):
     pos = start + steps
     want_tok, want_logits = om.step(tok, pos)            # host-position step on the same caches
     got_tok, got_logits = g.step(tok, pos, want_logits=True)
-    assert maxrel(got_logits, want_logits) < 2e-3
+    check_logits(got_logits, want_logits, BAR, "host-position step after the replays", FRAC)
     assert got_tok == want_tok or _near_tie(want_logits)
     g.close(); om.close()
 
@@ -242,7 +316,7 @@ def test_greedy_loop_on_the_device(orc, dims, n, q4):
     g.greedy_sync_host_pos()
     want_tok, want_logits = om.step(fed, start + n)
     got_tok, got_logits = g.step(fed, start + n, want_logits=True)
-    assert maxrel(got_logits, want_logits) < 2e-3
+    check_logits(got_logits, want_logits, BAR, "host-position step after the loop", FRAC)
     # the cache bound lives in the loop: it stops queueing at max_ctx
     left = dims["max_ctx"] - (start + n)
     assert g.greedy_run(left + 5) == left
@@ -269,6 +343,6 @@ def test_token_ids_outside_the_vocabulary_are_declined(orc):
             g.greedy_init(bad, 0)
     want_tok, want_logits = om.step(7, 0)
     got_tok, got_logits = g.step(7, 0, want_logits=True)
-    assert maxrel(got_logits, want_logits) < 2e-3
+    check_logits(got_logits, want_logits, BAR, "step after the refusals", FRAC)
     assert got_tok == want_tok or _near_tie(want_logits)
     g.close(); om.close()
