@@ -81,6 +81,7 @@ SIGNATURES = {
     "tlhip_gemm_bf16_nt_swiglu": (cint, [P, P, P, i64, i64, i64]),
     "tlhip_gemm_bf16_nt_parts": (cint, [P, P, P, i64, i64, i64, i64, P]),
     "tlhip_gemm_f16w_bytes": (i64, [i64, i64, cint]),
+    "tlhip_gemm_f16w_exps_bytes": (i64, [i64, cint]),
     "tlhip_gemm_f16w_prepare": (cint, [P, i64, i64, cint, P, P]),
     "tlhip_gemm_f16w_nt": (cint, [P, P, P, P, i64, i64, i64]),
     "tlhip_gemm_f16w_nt_parts": (cint, [P, P, P, P, i64, i64, i64, i64, P]),
@@ -121,6 +122,7 @@ SIGNATURES = {
     "tlhip_tune_reset": (cint, []),
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
+    "tlhip_alloc_calls": (cint, [C.POINTER(u64)]),
     "tlhip_warm_fork": (cint, [P, P, cint, cint, cint]),
     "tlhip_warm_join": (cint, []),
 }
@@ -347,7 +349,7 @@ class TlHip:
         if nbytes <= 0:
             raise ValueError("gemm_f16w_prepare: need positive N, K and K % 32 == 0")
         image = self.empty_bytes(nbytes)
-        exps = self.empty_bytes((2 * N if gated else N))
+        exps = self.empty_bytes(self.c.tlhip_gemm_f16w_exps_bytes(N, int(gated)))
         self._chk(self.c.tlhip_gemm_f16w_prepare(W.ptr, N, K, int(gated), image.ptr, exps.ptr))
         return image, exps
 
@@ -373,6 +375,12 @@ class TlHip:
 
     def merge_heads(self, src, dst, T, H, D):
         self._chk(self.c.tlhip_merge_heads(src.ptr, dst.ptr, T, H, D))
+
+    def alloc_calls(self):
+        """Allocation and release calls the library has made so far (device and pinned host)."""
+        n = u64(0)
+        self._chk(self.c.tlhip_alloc_calls(C.byref(n)))
+        return int(n.value)
 
     def bench_copy(self, dst, src, nbytes, blocks=0):
         self._chk(self.c.tlhip_bench_copy(dst.ptr, src.ptr, nbytes, blocks))

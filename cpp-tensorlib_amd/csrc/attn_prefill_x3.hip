@@ -113,13 +113,20 @@ __device__ __forceinline__ void split3x8(const float (&x)[8], uint4& p1, uint4& 
 // a first term - three MFMAs where the bf16 planes need six.
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+// what is left after the first term, 0 where that is inf - inf (an infinite operand): a NaN second
+// term would turn the infinity an fp32 product gives there into NaN
+__device__ __forceinline__ f32x2 rest_or_zero(f32x2 d) {
+  d.x = d.x == d.x ? d.x : 0.f;
+  d.y = d.y == d.y ? d.y : 0.f;
+  return d;
+}
 __device__ __forceinline__ void split2x8_f16(const float (&x)[8], float s, uint4& p1, uint4& p2) {
   uint32_t a[4], b[4];
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     const f32x2 v = {x[2 * j] * s, x[2 * j + 1] * s};
     const f16x2 h = __builtin_convertvector(v, f16x2);
-    const f16x2 l = __builtin_convertvector(v - __builtin_convertvector(h, f32x2), f16x2);
+    const f16x2 l = __builtin_convertvector(rest_or_zero(v - __builtin_convertvector(h, f32x2)), f16x2);
     a[j] = __builtin_bit_cast(uint32_t, h);
     b[j] = __builtin_bit_cast(uint32_t, l);
   }

@@ -38,6 +38,7 @@ struct Context {
   int* argmax_dev = nullptr;      // one int32 result slot
   int* argmax_host = nullptr;     // pinned landing slot for the 4-byte result
   uint64_t census[TLHIP_C_COUNT] = {};
+  uint64_t alloc_calls = 0;       // hipMalloc / hipFree / hipHostMalloc / hipHostFree calls the library has made
   // int4 GEMV launch-shape override (tlhip_tune_gemv_q4)
   int tune_q4_rows = 0, tune_q4_kw = 0, tune_q4_bpc = 0, tune_q4_nw = 0, tune_q4_lpr = 0;
   int tune_cols_max_splits = 0;   // [K,N] GEMV K-split bound (tlhip_tune_gemv_cols), 0 = automatic

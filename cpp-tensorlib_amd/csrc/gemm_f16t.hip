@@ -78,13 +78,67 @@ __global__ __launch_bounds__(256) void w_image_kernel(const uint16_t* __restrict
   }
 }
 
+// The exponents buffer a preparation fills, `exps`: [pad] int8 row exponents, [pad] uint16 counts,
+// then the weight's own address and depth (pad = rows rounded up to 16). The count of a row is the
+// number of its nonzero elements that, times 2^ew[row], lie below 2^-17 - their eight significant
+// bits no longer fit above the f16 subnormal step of 2^-24, so the image holds them with an absolute
+// error of up to 2^-25 - or 0xffff for a row that holds an infinity or a NaN. The products weigh the
+// counts against the scale of each result and work out from W itself, exactly, the results in which
+// those errors could show; that is why the buffer remembers where W is.
+struct WHeader { const uint16_t* W; int64_t K; };
+__host__ __device__ inline int64_t exps_pad(int64_t rows) { return (rows + 15) & ~int64_t(15); }
+constexpr uint32_t kWSmallMax = 0xffffu;
+
+__global__ __launch_bounds__(256) void w_range_kernel(const uint16_t* __restrict__ W, const int8_t* __restrict__ ew,
+                                                      int K, uint16_t* __restrict__ counts, WHeader* __restrict__ hdr) {
+  __shared__ uint32_t cnt[4], inf[4];
+  const uint4* row = reinterpret_cast<const uint4*>(W + (size_t)blockIdx.x * K);
+  const int lim = 127 - 17 - (int)ew[blockIdx.x];      // biased exponent below which an element is too small
+  uint32_t small = 0;
+  bool nonfinite = false;
+  for (int i = threadIdx.x; i < K / 8; i += 256) {
+    const uint4 v = row[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint32_t m = (w[j] >> (16 * h)) & 0x7fffu;
+        const int field = (int)(m >> 7);
+        small += (m != 0u && field < lim) ? 1u : 0u;
+        nonfinite |= field == 255;
+      }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) small += (uint32_t)__shfl_xor((int)small, d);
+  const bool anyinf = __any(nonfinite);
+  if ((threadIdx.x & 63) == 0) { cnt[threadIdx.x >> 6] = small; inf[threadIdx.x >> 6] = anyinf ? 1u : 0u; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    small = cnt[0] + cnt[1] + cnt[2] + cnt[3];
+    if (small > kWSmallMax - 1) small = kWSmallMax - 1;
+    if (inf[0] | inf[1] | inf[2] | inf[3]) small = kWSmallMax;
+    counts[blockIdx.x] = (uint16_t)small;
+    if (blockIdx.x == 0) { hdr->W = W; hdr->K = K; }
+  }
+}
+
 // One block per row of the activation images (rows past M are zero rows): the row's largest
-// magnitude and from it ea[m], then its two f16 terms into the slab images - one read of A.
+// magnitude and from it the exponent e, then its two f16 terms into the slab images - one read of A.
 // The row stays in registers between the two steps: up to kRowRegs float4s per thread.
+// ea[m] = (e & 0xff) | (n << 8). n bounds the number of the row's nonzero elements that, scaled, lie
+// below 2^-10 (more than 2^24 below the row's largest): their second term is an f16 subnormal with
+// fewer than three bits left, so they are carried with an ABSOLUTE error of up to 2^-25 each (scaled)
+// instead of a relative one. The bound is K as soon as the row's smallest nonzero magnitude is that
+// small (a minimum costs less per element than a count, and this pass is bound by its memory
+// traffic only just), 0 otherwise. The GEMM weighs n against the scale of each result and works
+// out exactly the results for which those errors could show (gemm_f16t_kernel's epilogue). A row
+// that holds an infinity or a NaN gets the largest n: all of its results are worked out exactly.
 constexpr int kRowRegs = 32;            // K <= 256 * 4 * 32 = 32768
+constexpr uint32_t kSmallMax = 0x7fffffu;
 __global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ A, int* __restrict__ ea,
                                                       char* __restrict__ img, int M, int K) {
-  __shared__ uint32_t part[4];
+  __shared__ uint32_t part[4], cnt[4];
   const int gm = blockIdx.x, t = threadIdx.x, nslab = K / kBK, k4 = K / 4;
   const int tm = gm / kTile, row = gm % kTile;
   typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -109,20 +163,33 @@ __global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ 
   __syncthreads();
   mx = max(max(part[0], part[1]), max(part[2], part[3]));
   const int e = row_exponent((int)(mx >> 23), mx == 0);
-  if (t == 0 && gm < M) ea[gm] = e;
   const float s = pow2f(e);
   char* dst = img + (size_t)tm * nslab * kAImage;
+  uint32_t least = 0xffffffffu;                    // smallest nonzero magnitude's bits, minus one
 #pragma unroll
   for (int i = 0; i < kRowRegs; i++) {
     const int q = t + 256 * i;               // float4 q of the row: slab q / 8, 8-byte piece q % 8 of its 64 bytes
     if (q >= k4) break;
+    const f32x4 x = v[i] * s;
+#pragma unroll
+    for (int j = 0; j < 4; j++) least = min(least, (__float_as_uint(x[j]) & 0x7fffffffu) - 1u);   // 0 wraps to the top
     uint32_t h01, l01, h23, l23;
-    split2_f16(v[i][0] * s, v[i][1] * s, h01, l01);
-    split2_f16(v[i][2] * s, v[i][3] * s, h23, l23);
+    split2_f16(x[0], x[1], h01, l01);
+    split2_f16(x[2], x[3], h23, l23);
     const int c4 = q & 7;
     char* o = dst + (size_t)(q >> 3) * kAImage + image_off(row, c4 >> 1) + (c4 & 1) * 8;
     *reinterpret_cast<uint2*>(o) = make_uint2(h01, h23);
     *reinterpret_cast<uint2*>(o + kPlaneBytes) = make_uint2(l01, l23);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) least = min(least, (uint32_t)__shfl_xor((int)least, d));
+  if ((t & 63) == 0) cnt[t >> 6] = least;
+  __syncthreads();
+  if (t == 0 && gm < M) {
+    least = min(min(cnt[0], cnt[1]), min(cnt[2], cnt[3]));
+    uint32_t small = least < 0x3a800000u - 1u ? (uint32_t)K : 0u;          // 0 < |x| < 2^-10 somewhere
+    if (mx >= 0x7f800000u) small = kSmallMax;
+    ea[gm] = (e & 0xff) | (int)(small << 8);
   }
 }
 
@@ -141,7 +208,8 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
                                                            float* __restrict__ C, int M, int N, int nslab,
                                                            int part_slabs, int ldc, int tn0, int ff,
                                                            const int* __restrict__ ea,
-                                                           const int8_t* __restrict__ ew) {
+                                                           const int8_t* __restrict__ ew, int wpad,
+                                                           const float* __restrict__ A) {
   constexpr int BM = 128 * TM;
   constexpr int kAPlane = BM * kRowBytes;            // one plane of this block's rows in a stage
   constexpr int kStage = 2 * kAPlane + kWImage;
@@ -333,12 +401,77 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
     }
   };
   typedef float f32x4 __attribute__((ext_vector_type(4)));
+  // Where small elements were counted - in a row of A (a_image_kernel) or in a row of W
+  // (w_range_kernel) - their absolute errors add up to at most n 2^-10 in the units of acc, i.e.
+  // n 2^-10 2^-(ea + ew) in the result's. After the tile has been stored, a result for which that
+  // could reach a quarter of the absolute tolerance of 1e-5 (and every result of a row that is not
+  // finite) is worked out again from the operands themselves, the f32 activations and the bf16
+  // weight - an fp32 FMA chain over this block's K range in k order, the arithmetic of the
+  // reference's loop (tensorlib_cuda.cu:509-519) - and stored over the first one by the lane that
+  // stored that. Ordinary operands never get here: it takes an element 2^24 (of W: 2^31) below its
+  // row's largest AND a row-times-column scale above 2^14. The pass is per lane and serial; the
+  // kernel's time is not its concern.
+  const uint16_t* wcount = reinterpret_cast<const uint16_t*>(ew + wpad);
+  const WHeader* whdr = reinterpret_cast<const WHeader*>(ew + 3 * (size_t)wpad);
+  auto again = [&](bool gated_out) {
+    bool wsome = false;                 // does any of this wavefront's 128 columns carry a count?
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const int r = weight_row(GU, tn, wn * 128 + lane * 2 + e, nlim, ff);
+      wsome |= r >= 0 && wcount[r] != 0;
+    }
+    wsome = __any(wsome);
+#pragma unroll 1
+    for (int i = 0; i < TM; i++) {
+      const int gm = tm * BM + wm * 32 * TM + i * 32 + (lane & 31);
+      const int raw = gm < M ? ea[gm] : 0;
+      const uint32_t nsm = (uint32_t)raw >> 8;
+      if (!wsome && !__any(nsm != 0u)) continue;      // the ordinary case: nothing to weigh
+      if (gm >= M) continue;
+      const int em = (int)(int8_t)(raw & 0xff);
+      const int64_t K = whdr->K;
+      const float* arow = A + (size_t)gm * K + (size_t)sbeg * kBK;
+      auto needs = [&](int r) {
+        const uint32_t nw = wcount[r];
+        return (nsm | nw) != 0u && (nsm == kSmallMax || nw == kWSmallMax ||
+                                    ldexpf((float)(nsm + nw), -(em + (int)ew[r])) > 0x1p-8f);
+      };
+      auto chain = [&](int r) {         // row gm of A against row r of W over this block's K range
+        const uint16_t* wrow = whdr->W + (size_t)r * K + (size_t)sbeg * kBK;
+        float x = 0.f;
+#pragma unroll 1
+        for (int k = 0; k < ns * kBK; k += 2) {
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(wrow + k);
+          x = fmaf(arow[k], bf16_lo(w), x);
+          x = fmaf(arow[k + 1], bf16_hi(w), x);
+        }
+        return x;
+      };
+#pragma unroll 1
+      for (int idx = 0; idx < (gated_out ? 32 : 64); idx++) {
+        const int j = idx >> 4, v = idx & 15;
+        const int c = wn * 128 + j * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (gated_out) {
+          const int f = ltn * 128 + wn * 64 + j * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const int rg = weight_row(GU, tn, c, nlim, ff), ru = weight_row(GU, tn, c + 64, nlim, ff);
+          if (f >= N || rg < 0 || ru < 0 || !(needs(rg) || needs(ru))) continue;
+          const float gt = chain(rg), sg = 1.0f / (1.0f + expf(-gt));
+          C[(size_t)gm * ldc + f] = (gt * sg) * chain(ru);
+        } else {
+          const int gn = ltn * kTile + c;
+          const int r = weight_row(GU, tn, c, nlim, ff);
+          if ((!GU && gn >= N) || r < 0 || !needs(r)) continue;
+          C[(size_t)gm * ldc + gn] = chain(r);
+        }
+      }
+    }
+  };
   if (GU && gridDim.y == 1) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const int gm = tm * BM + wm * 32 * TM + i * 32 + (lane & 31);
       if (gm >= M) continue;
-      const int em = ea[gm];
+      const int em = (int)(int8_t)(ea[gm] & 0xff);
 #pragma unroll
       for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -365,6 +498,7 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
           }
         }
     }
+    again(true);
     TLHIP_MARK(6);
     return;
   }
@@ -372,7 +506,7 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
   for (int i = 0; i < TM; i++) {
     const int gm = tm * BM + wm * 32 * TM + i * 32 + (lane & 31);
     if (gm >= M) continue;
-    const int em = ea[gm];
+    const int em = (int)(int8_t)(ea[gm] & 0xff);
 #pragma unroll
     for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -395,6 +529,7 @@ __global__ __launch_bounds__(512, 1) void gemm_f16t_kernel(const char* __restric
         }
       }
   }
+  again(false);
   TLHIP_MARK(6);
 }
 
@@ -497,16 +632,20 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
       return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_nt: too many tiles for one grid");
     const dim3 grid((unsigned)nblk, (unsigned)S);
     auto launch = [&](auto fn) -> hipError_t {
-      // more than 64 KB of LDS per block has to be asked for once per kernel (and device)
-      static int asked_on[2] = {-1, -1};             // per instantiation of this lambda: [tile height - 1]
-      if (asked_on[P.tmh - 1] != c.device) {
+      // more than 64 KB of LDS per block has to be asked for once per kernel (and device); the
+      // four kernels share this one lambda instantiation (same function-pointer type), so the
+      // note of who has asked is kept per kernel: [gated][tile height - 1]
+      static int asked[2][2] = {{-1, -1}, {-1, -1}};
+      int& asked_on_ = asked[gu ? 1 : 0][P.tmh - 1];
+      if (asked_on_ != c.device) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)((size_t)f16t::kRing * (2 * 128 * P.tmh * f16t::kRowBytes + f16t::kWImage)));
         if (e != hipSuccess) return e;
-        asked_on[P.tmh - 1] = c.device;
+        asked_on_ = c.device;
       }
       fn<<<grid, dim3(512), lds, c.stream>>>(aimg, static_cast<const char*>(image), dst, (int)M, (int)pn, (int)nslab,
-                                             part_slabs, ldc, (int)P.tn0, (int)N, ea, static_cast<const int8_t*>(exps));
+                                             part_slabs, ldc, (int)P.tn0, (int)N, ea, static_cast<const int8_t*>(exps),
+                                             (int)f16t::exps_pad(gu ? 2 * N : N), pa);
       return hipSuccess;
     };
     const hipError_t e = P.tmh == 2 ? (gu ? launch(f16t::gemm_f16t_kernel<2, true>) : launch(f16t::gemm_f16t_kernel<2, false>))
@@ -534,6 +673,7 @@ extern "C" {
 
 int64_t tlhip_gemm_f16w_bytes(int64_t N, int64_t K, int gated) {
   if (N <= 0 || K <= 0 || (K % f16t::kBK) != 0) return 0;
+  if (K > 256 * 4 * f16t::kRowRegs) return 0;    // deeper than the products over an image go: no image
   const int64_t tn = cdiv64(N, gated ? 128 : f16t::kTile);
   return tn * (K / f16t::kBK) * f16t::kWImage;
 }
@@ -544,19 +684,27 @@ int tlhip_gemm_f16w_prepare(const void* W, int64_t N, int64_t K, int gated, void
   const int64_t rows = gated ? 2 * N : N;
   if (N <= 0 || K <= 0 || (K % f16t::kBK) != 0 || rows > 0x7fffffff || K > 0x3fffffff)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_prepare: need positive N, K and K %% 32 == 0");
-  if (!aligned16(W) || !aligned16(image))
-    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_prepare: weight and image must be 16-byte aligned");
+  if (!aligned16(W) || !aligned16(image) || !aligned16(exps))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_prepare: weight, image and exps must be 16-byte aligned");
   Context& c = ctx();
   const uint16_t* pw = static_cast<const uint16_t*>(W);
   int8_t* pe = static_cast<int8_t*>(exps);
-  row_exponent_bf16_kernel<<<dim3((unsigned)rows), dim3(256), 0, c.stream>>>(pw, (int)K, pe);
   const int64_t tn = cdiv64(N, gated ? 128 : f16t::kTile), nslab = K / f16t::kBK;
   if (tn > 0x7fffffff || nslab > 65535)
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemm_f16w_prepare: weight too large for one grid");
+  const int64_t pad = f16t::exps_pad(rows);
+  row_exponent_bf16_kernel<<<dim3((unsigned)rows), dim3(256), 0, c.stream>>>(pw, (int)K, pe);
+  f16t::w_range_kernel<<<dim3((unsigned)rows), dim3(256), 0, c.stream>>>(
+      pw, pe, (int)K, reinterpret_cast<uint16_t*>(pe + pad), reinterpret_cast<f16t::WHeader*>(pe + 3 * pad));
   f16t::w_image_kernel<<<dim3((unsigned)tn, (unsigned)nslab), dim3(256), 0, c.stream>>>(
       pw, pe, static_cast<char*>(image), (int)N, (int)K, (int)N, gated ? 1 : 0);
   const hipError_t e = hipGetLastError();   // a preparation is not a product: not in the census
   return e == hipSuccess ? TLHIP_OK : hip_fail(e, "kernel launch");
+}
+
+int64_t tlhip_gemm_f16w_exps_bytes(int64_t N, int gated) {
+  if (N <= 0) return 0;
+  return 3 * f16t::exps_pad(gated ? 2 * N : N) + (int64_t)sizeof(f16t::WHeader);
 }
 
 int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N,

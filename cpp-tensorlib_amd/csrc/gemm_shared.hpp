@@ -27,11 +27,23 @@ __device__ __forceinline__ int row_exponent(int field, bool all_zero) {
 }
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // e in [-126, 127]
 
-// two scaled floats -> their f16 terms, both round-to-nearest; x - hi is exact in fp32
+// What is left of x after its first f16 term; 0 where that is not a number: an infinite x has an
+// infinite first term and inf - inf, and a NaN second term would turn the +-inf that an fp32
+// product chain gives there into NaN (a NaN x stays NaN through its first term).
+__device__ __forceinline__ f32x2 rest_or_zero(f32x2 d) {
+  d.x = d.x == d.x ? d.x : 0.f;
+  d.y = d.y == d.y ? d.y : 0.f;
+  return d;
+}
+// two scaled floats -> their f16 terms, both round-to-nearest; x - hi is exact in fp32.
+// GUARD = false leaves out the two instructions per element that keep an infinity an infinity
+// (for a loop that is bound by its vector instructions; an infinite x then gives NaN terms).
+template <bool GUARD = true>
 __device__ __forceinline__ void split2_f16(float x0, float x1, uint32_t& hi, uint32_t& lo) {
   const f32x2 x = {x0, x1};
   const f16x2 h = __builtin_convertvector(x, f16x2);
-  const f16x2 l = __builtin_convertvector(x - __builtin_convertvector(h, f32x2), f16x2);
+  const f32x2 rest = x - __builtin_convertvector(h, f32x2);
+  const f16x2 l = __builtin_convertvector(GUARD ? rest_or_zero(rest) : rest, f16x2);
   hi = __builtin_bit_cast(uint32_t, h);
   lo = __builtin_bit_cast(uint32_t, l);
 }

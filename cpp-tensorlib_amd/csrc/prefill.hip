@@ -224,8 +224,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void gemm_bf16_nt_kernel(const flo
       if (H) {
         uint32_t h01, l01, h23, l23;
         const float s = sa[H ? i : 0];
-        split2_f16(ra[i].x * s, ra[i].y * s, h01, l01);
-        split2_f16(ra[i].z * s, ra[i].w * s, h23, l23);
+        split2_f16<false>(ra[i].x * s, ra[i].y * s, h01, l01);   // every block cuts its rows again, slab by slab:
+        split2_f16<false>(ra[i].z * s, ra[i].w * s, h23, l23);   // the loop is bound by these instructions
         const int o = lds_off(row, c4 >> 1) + (c4 & 1) * 4;
         *reinterpret_cast<uint2*>(&As[0][o]) = make_uint2(h01, h23);
         *reinterpret_cast<uint2*>(&As[1][o]) = make_uint2(l01, l23);

@@ -34,11 +34,12 @@ void* scratch(size_t bytes) {
   if (c.scratch) {
     (void)hipStreamSynchronize(c.stream);
     if (c.graphs_recorded > 0) c.retired_scratch.push_back(c.scratch);  // a graph may still point at it
-    else (void)hipFree(c.scratch);
+    else { (void)hipFree(c.scratch); c.alloc_calls++; }
     c.scratch = nullptr;
     c.scratch_bytes = 0;
   }
   size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+  c.alloc_calls++;
   if (hipMalloc(&c.scratch, want) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
@@ -155,6 +156,9 @@ int tlhip_init(int device) {
   Context& c = ctx();
   if (c.ready) {
     if (device != c.device) return fail(TLHIP_EINVAL, "already initialised on device %d", c.device);
+    // launch-shape overrides are process-wide and sticky: a client that initialises the library
+    // (again) starts from the built-in choices, whatever an earlier client of the process left
+    (void)tlhip_tune_reset();
     return TLHIP_OK;
   }
   int count = 0;
@@ -195,6 +199,7 @@ int tlhip_malloc(void** dptr, size_t bytes) {
   TLHIP_REQUIRE_READY();
   if (!dptr) return fail(TLHIP_EINVAL, "tlhip_malloc: null out pointer");
   *dptr = nullptr;
+  ctx().alloc_calls++;
   hipError_t e = hipMalloc(dptr, bytes ? bytes : 4);
   if (e != hipSuccess) {
     (void)hipGetLastError();
@@ -206,6 +211,7 @@ int tlhip_malloc(void** dptr, size_t bytes) {
 int tlhip_free(void* dptr) {
   if (!dptr) return TLHIP_OK;
   TLHIP_REQUIRE_READY();
+  ctx().alloc_calls++;
   hipError_t e = hipFree(dptr);
   return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipFree");
 }
@@ -214,6 +220,7 @@ int tlhip_host_alloc(void** hptr, size_t bytes) {
   TLHIP_REQUIRE_READY();
   if (!hptr) return fail(TLHIP_EINVAL, "tlhip_host_alloc: null out pointer");
   *hptr = nullptr;
+  ctx().alloc_calls++;
   hipError_t e = hipHostMalloc(hptr, bytes ? bytes : 4, hipHostMallocDefault);
   if (e != hipSuccess) {
     (void)hipGetLastError();
@@ -225,6 +232,7 @@ int tlhip_host_alloc(void** hptr, size_t bytes) {
 int tlhip_host_free(void* hptr) {
   if (!hptr) return TLHIP_OK;
   TLHIP_REQUIRE_READY();
+  ctx().alloc_calls++;
   hipError_t e = hipHostFree(hptr);
   return e == hipSuccess ? TLHIP_OK : hip_fail(e, "hipHostFree");
 }
@@ -405,6 +413,12 @@ int tlhip_census(uint64_t* counts, int n) {
   if (!counts || n < 0) return fail(TLHIP_EINVAL, "tlhip_census: bad arguments");
   int m = n < TLHIP_C_COUNT ? n : (int)TLHIP_C_COUNT;
   for (int i = 0; i < m; i++) counts[i] = ctx().census[i];
+  return TLHIP_OK;
+}
+
+int tlhip_alloc_calls(uint64_t* calls) {
+  if (!calls) return fail(TLHIP_EINVAL, "tlhip_alloc_calls: null out pointer");
+  *calls = ctx().alloc_calls;
   return TLHIP_OK;
 }
 

@@ -113,6 +113,7 @@ struct api {
                            int64_t) = nullptr;
   int (*gemm_bf16_nt_swiglu)(const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int64_t (*gemm_f16w_bytes)(int64_t, int64_t, int) = nullptr;
+  int64_t (*gemm_f16w_exps_bytes)(int64_t, int) = nullptr;
   int (*gemm_f16w_prepare)(const void*, int64_t, int64_t, int, void*, void*) = nullptr;
   int (*gemm_f16w_nt)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t) = nullptr;
   int (*gemm_f16w_nt_parts)(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int64_t,
@@ -195,6 +196,10 @@ struct extent {
     void* exps = nullptr;
   };
   std::vector<prepared> derived;
+  // (offset, rows, depth, gated) of weights whose preparation failed (no memory, or the library
+  // refused the product): not tried again until the extent's device bytes change.
+  struct unprepared { size_t off; int64_t n, k; bool gated; };
+  std::vector<unprepared> refused;
 };
 
 // The extents in use, ordered by base address so that an address INSIDE one (q4 scales at
@@ -246,6 +251,9 @@ struct context {
   // must fetch, not trust the copy it made after the previous one.
   std::vector<uintptr_t> capture_writes;
   std::unordered_map<void*, std::vector<uintptr_t>> graph_writes;
+  // Images dropped while a capture is open: freeing synchronises the device, which a capture
+  // forbids, so they are freed when the capture ends.
+  std::vector<void*> deferred_free;
   std::string why;  // why the backend is unavailable (diagnostics only)
   // Prompt-chunk products over bf16 weights run on the library's prepared f16 form of the weight
   // (a second copy of it, made on first use). TENSORLIB_HIP_PROMPT_F16=0 keeps them on the bf16 rows.
@@ -305,7 +313,8 @@ struct context {
               bind(f.gemm_bf16_nt, "tlhip_gemm_bf16_nt") &&
               bind(f.gemm_bf16_nt_parts, "tlhip_gemm_bf16_nt_parts") &&
               bind(f.gemm_bf16_nt_swiglu, "tlhip_gemm_bf16_nt_swiglu") &&
-              bind(f.gemm_f16w_bytes, "tlhip_gemm_f16w_bytes") && bind(f.gemm_f16w_prepare, "tlhip_gemm_f16w_prepare") &&
+              bind(f.gemm_f16w_bytes, "tlhip_gemm_f16w_bytes") && bind(f.gemm_f16w_exps_bytes, "tlhip_gemm_f16w_exps_bytes") &&
+              bind(f.gemm_f16w_prepare, "tlhip_gemm_f16w_prepare") &&
               bind(f.gemm_f16w_nt, "tlhip_gemm_f16w_nt") && bind(f.gemm_f16w_nt_parts, "tlhip_gemm_f16w_nt_parts") &&
               bind(f.gemm_f16w_nt_swiglu, "tlhip_gemm_f16w_nt_swiglu") &&
               bind(f.gemm_q4_nt, "tlhip_gemm_q4_nt") && bind(f.gemm_q4_nt_parts, "tlhip_gemm_q4_nt_parts") &&
@@ -378,12 +387,39 @@ struct context {
   // The extent's device bytes are changing: what was derived from them goes. (free_ drains the
   // device first, so a queued product that still reads an image finishes with it.)
   void forget_derived(extent& e) {
-    for (auto& d : e.derived) f.free_(d.image);
+    for (auto& d : e.derived) {
+      if (capturing) deferred_free.push_back(d.image);
+      else f.free_(d.image);
+    }
     e.derived.clear();
+    e.refused.clear();
+  }
+  void free_deferred() {
+    for (void* p : deferred_free) f.free_(p);
+    deferred_free.clear();
+  }
+  // The prepared product over `d` was refused by the library: drop the image and do not prepare
+  // this weight again (the caller runs the product on the bf16 rows).
+  void refuse_prepared(void* B, const extent::prepared* d) {
+    extent* e = buffers.containing(B);
+    if (!e) return;
+    for (size_t i = 0; i < e->derived.size(); i++)
+      if (&e->derived[i] == d) {
+        e->refused.push_back({d->off, d->n, d->k, d->gated});
+        if (capturing) deferred_free.push_back(d->image);
+        else f.free_(d->image);
+        e->derived.erase(e->derived.begin() + (long)i);
+        return;
+      }
   }
   // The prepared form of the bf16 weight B [n, k] (gated: [2n, k], gate rows | up rows), made now
   // if this is its first prompt-chunk product. nullptr: not a managed buffer, not a shape the
-  // prepared products take, no memory, or a capture is open - the caller uses the bf16 rows.
+  // prepared products take, no memory (remembered: not tried again until the buffer changes), or
+  // a capture is open - the caller uses the bf16 rows.
+  // Cost: the image is a SECOND copy of the weight (2 bytes per element plus one byte per row),
+  // held until the extent's device bytes can change. The pointer returned points into the
+  // extent's list and is valid only until the next call that prepares or drops a weight of the
+  // same extent: use it for the one product at hand, do not keep it.
   const extent::prepared* prepared_weight(void* B, int64_t n, int64_t k, bool gated) {
     if (!prompt_f16 || capturing) return nullptr;
     extent* e = buffers.containing(B);
@@ -391,14 +427,20 @@ struct context {
     const size_t off = static_cast<size_t>(static_cast<char*>(B) - e->base);
     for (const auto& d : e->derived)
       if (d.off == off && d.n == n && d.k == k && d.gated == gated) return &d;
+    for (const auto& r : e->refused)
+      if (r.off == off && r.n == n && r.k == k && r.gated == gated) return nullptr;
     const int64_t rows = gated ? 2 * n : n, bytes = f.gemm_f16w_bytes(n, k, gated ? 1 : 0);
     if (bytes <= 0 || off + static_cast<size_t>(rows * k * 2) > e->size) return nullptr;
     extent::prepared d;
     d.off = off; d.n = n; d.k = k; d.gated = gated;
-    if (f.malloc_(&d.image, static_cast<size_t>(bytes + ((rows + 15) & ~int64_t(15)))) != 0) return nullptr;
+    if (f.malloc_(&d.image, static_cast<size_t>(bytes + f.gemm_f16w_exps_bytes(n, gated ? 1 : 0))) != 0) {
+      e->refused.push_back({off, n, k, gated});
+      return nullptr;
+    }
     d.exps = static_cast<char*>(d.image) + bytes;
     if (f.gemm_f16w_prepare(B, n, k, gated ? 1 : 0, d.image, d.exps) != 0) {
       f.free_(d.image);
+      e->refused.push_back({off, n, k, gated});
       return nullptr;
     }
     pending = true;
@@ -428,6 +470,8 @@ class launch {
   void writes(P... p) { (c_.claim_device(p), ...); }
   // see context::prepared_weight; call after reads() has brought the weight up to date
   const extent::prepared* prepared(void* B, int64_t n, int64_t k, bool gated) { return c_.prepared_weight(B, n, k, gated); }
+  // the library refused the product over the prepared form: the caller goes on to the bf16 rows
+  void refused(void* B, const extent::prepared* p) { c_.refuse_prepared(B, p); }
   bool sent(int rc) {
     if (rc != 0) return false;   // declined or failed: the caller falls back
     c_.pending = true;
@@ -554,7 +598,15 @@ inline void upload(void* native, const float* src, int64_t n) {
 inline bool upload_raw(void* dst_dev, const void* src_host, int64_t bytes) {
   auto& c = context::get();
   if (!c.ready || !dst_dev || !src_host || bytes < 0) return false;
-  return bytes == 0 || c.f.memcpy_h2d(dst_dev, src_host, (size_t)bytes) == 0;
+  if (bytes == 0) return true;
+  if (extent* e = c.buffers.containing(dst_dev)) {
+    // a managed buffer: bring a staging-live one to the device first (the copy may cover only part
+    // of it), then the device half is the current one and what was derived from it is stale
+    if (e->live == extent::side::staging) c.push(*e, e->size);
+    c.forget_derived(*e);
+    e->live = extent::side::device;
+  }
+  return c.f.memcpy_h2d(dst_dev, src_host, (size_t)bytes) == 0;
 }
 
 // Blocking D2H from a device address (which may lie inside a managed buffer) into any host
@@ -679,7 +731,10 @@ inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int6
   L.reads(a, B);
   L.writes(out);
   if (prompt_product_is_large(m, n, k))   // on the weight's prepared f16 form where there is one
-    if (const auto* p = L.prepared(B, n, k, false)) return L.sent(L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k));
+    if (const auto* p = L.prepared(B, n, k, false)) {
+      if (L.sent(L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k))) return true;
+      L.refused(B, p);                    // the bf16 rows serve what the prepared product declined
+    }
   return L.sent(L.lib.gemm_bf16_nt(a, B, out, m, n, k));
 }
 
@@ -690,7 +745,10 @@ inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t 
   L.reads(a, B);
   L.writes(act);
   if (prompt_product_is_large(m, 2 * ff, k))
-    if (const auto* p = L.prepared(B, ff, k, true)) return L.sent(L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k));
+    if (const auto* p = L.prepared(B, ff, k, true)) {
+      if (L.sent(L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k))) return true;
+      L.refused(B, p);
+    }
   return L.sent(L.lib.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
 }
 
@@ -729,8 +787,10 @@ inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_byte
   L.reads(a, B);
   L.writes(parts);
   if (prompt_product_is_large(m, n, k))
-    if (const auto* p = L.prepared(B, n, k, false))
-      return L.sent(L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts));
+    if (const auto* p = L.prepared(B, n, k, false)) {
+      if (L.sent(L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts))) return true;
+      L.refused(B, p);
+    }
   return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
 }
 
@@ -1209,6 +1269,7 @@ inline void* capture_end() {
   int rc = c.f.graph_end(&g);
   c.capturing = false;
   c.pending = false;  // recorded launches did not run
+  c.free_deferred();
   if (rc != 0 || !g) return nullptr;
   std::sort(c.capture_writes.begin(), c.capture_writes.end());
   c.capture_writes.erase(std::unique(c.capture_writes.begin(), c.capture_writes.end()),
@@ -1225,7 +1286,10 @@ inline bool graph_launch(void* g) {
   auto it = c.graph_writes.find(g);
   if (it != c.graph_writes.end())
     for (uintptr_t base : it->second)
-      if (extent* e = c.buffers.at_base(base)) e->live = extent::side::device;
+      if (extent* e = c.buffers.at_base(base)) {
+        c.forget_derived(*e);        // a replay rewrites the bytes an image was made from
+        e->live = extent::side::device;
+      }
   return true;
 }
 inline void graph_destroy(void* g) {

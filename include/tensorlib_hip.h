@@ -359,21 +359,33 @@ int tlhip_gemm_bf16_nt_swiglu(const void* A, const void* W, void* act, int64_t M
 /* The same three products over a PREPARED weight, for a harness that owns its weights (no reference
  * counterpart: gemm_bf16_nt of cuda.h:787-841 takes the weight alone). tlhip_gemm_f16w_prepare, once
  * when the weight is loaded, writes
- *   exps[r] (int8, one per row of W) = 14 - floor(log2(max_k |W[r][k]|)), what brings the row's
- *     largest magnitude into [2^14, 2^15) (0 for a row of zeros), and
- *   image (tlhip_gemm_f16w_bytes(N, K, gated) bytes) = every weight times 2^exps[r] as f16, laid out
- *     slab by slab (256 rows x 32 k, 16 KB) in the order the kernel's LDS reads expect. A bf16
- *     weight has 8 significant bits and an f16 holds 11, so each weight is exact unless it lies more
- *     than 2^29 below its row's largest (then its absolute error is below 2^-40 of that).
+ *   exps (tlhip_gemm_f16w_exps_bytes(N, gated) bytes, 16-byte aligned): per row of W the int8
+ *     exponent 14 - floor(log2(max_k |W[r][k]|)), what brings the row's largest magnitude into
+ *     [2^14, 2^15) (0 for a row of zeros); per row the count of its nonzero weights that lie more than
+ *     2^31 below the row's largest (0xffff: the row holds an infinity or a NaN); and W's own address, and
+ *   image (tlhip_gemm_f16w_bytes(N, K, gated) bytes; 0 = no image for this shape, K > 32768 included)
+ *     = every weight times 2^exponent as f16, laid out slab by slab (256 rows x 32 k, 16 KB) in the
+ *     order the kernel's LDS reads expect. A bf16 weight has 8 significant bits and an f16 holds 11,
+ *     so each weight is exact unless it is one of the counted ones (then its absolute error is below
+ *     2^-40 of the row's largest).
  * gated != 0: W = [gate rows | up rows], [2*N, K], N = features (the operand of
  * tlhip_gemm_bf16_nt_swiglu); the image then serves tlhip_gemm_f16w_nt_swiglu only, a plain image
  * the other two. K % 32 == 0.
  * The products cut every activation row, scaled the same way, into two f16 terms, both rounded to
  * nearest (2^-24 relative), and run two matrix-core products per weight instead of three, fp32
  * sums, the result scaled back exactly: the error is that of one fp32 rounding per product, as in
- * tlhip_gemm_bf16_nt, which these agree with to fp32 summation order. The image replaces W for
- * prompt chunks; the decode GEMV still reads the bf16 weight. */
+ * tlhip_gemm_bf16_nt, which these agree with to fp32 summation order. An activation more than 2^24
+ * below its row's largest (like a counted weight) is carried with an absolute error only; the
+ * products count those too and work out again, from A and W themselves with the fp32 FMA chain of
+ * tensorlib_cuda.cu:509-519, every result in which such errors could reach a quarter of an absolute
+ * tolerance of 1e-5, and every result of a row of A or W that holds an infinity or a NaN (which then
+ * comes out as that chain leaves it). So the results meet allclose(rtol 1e-4, atol 1e-5) against
+ * the fp32 chain whatever the spread of the operands; ordinary operands never take that path.
+ * The image and exps are DERIVED from W and exps refers to it: W must stay allocated and unchanged
+ * while they are in use (the decode GEMV keeps reading the bf16 weight anyway), and they must be
+ * prepared again when W changes. */
 int64_t tlhip_gemm_f16w_bytes(int64_t N, int64_t K, int gated);
+int64_t tlhip_gemm_f16w_exps_bytes(int64_t N, int gated);
 int tlhip_gemm_f16w_prepare(const void* W, int64_t N, int64_t K, int gated, void* image, void* exps);
 int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N,
                        int64_t K);
@@ -386,7 +398,11 @@ int tlhip_gemm_f16w_nt_swiglu(const void* A, const void* image, const void* exps
  * sum over groups of scale * (A . q) with exact products on the matrix pipe, fp32 sums - the decode
  * GEMV's arithmetic, M rows at a time. No reference counterpart: the reference feeds prompts to
  * an int4 model one token at a time (qwen_model.h:419 gates its batched prefill on bf16 weights);
- * parity is against tlhip_gemv_q4 / the CPU path row by row. */
+ * parity is against tlhip_gemv_q4 / the CPU path row by row. For M > 64 the activations enter as two
+ * f16 terms of each row scaled by a power of two (nibbles are exact in f16): an activation more than
+ * 2^24 below its row's largest keeps an absolute, not a relative, error (2^-39.5 of that largest),
+ * and a row that holds an infinity comes out as NaN where the decode GEMV gives +-inf - parity
+ * unpinned for such rows (no reference test feeds them); tlhip_gemv_q4 row by row is exact there. */
 int tlhip_gemm_q4_nt(const void* A, const void* qw, const void* scales, void* C, int64_t M, int64_t N,
                      int64_t K, int64_t group);
 int tlhip_gemm_q4_nt_parts(const void* A, const void* qw, const void* scales, void* parts,

@@ -22,6 +22,12 @@ extern "C" {
 int tlhip_bench_copy(void* dst, const void* src, size_t bytes, int blocks);
 int tlhip_bench_read(const void* src, size_t bytes, void* sink4, int blocks);
 
+/* How many device / pinned-host allocation and release calls (hipMalloc, hipFree, hipHostMalloc,
+ * hipHostFree) the library has made since it was loaded: its own scratch growth and the
+ * tlhip_malloc / tlhip_free / tlhip_host_* calls of its users. A caller that must not allocate
+ * (tlhip_attn_decode_static) can be checked against it. */
+int tlhip_alloc_calls(uint64_t* calls);
+
 /* ---- weight warm-up on a second stream ---------------------------------------------------
  * tlhip_warm_fork: up to four byte ranges (16-byte aligned) are read once, in the order given, by
  * `blocks` blocks of 256 threads (<= 0: 32) on a second stream of the same priority that starts

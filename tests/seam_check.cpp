@@ -272,6 +272,68 @@ int main() {
     ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w2, "on the bf16 rows");
     hip::set_prompt_f16(true);
     check("prepared weight follows host edits and device writes of its buffer", ok);
+
+    // a raw upload into the weight (the loader's way of writing device bytes) drops the cached form too
+    ok = hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k);          // prepares again
+    std::vector<uint16_t> fresh(n * k);
+    for (auto& h : fresh) { const float v = 0.11f * rnd(); uint32_t u; std::memcpy(&u, &v, 4); h = (uint16_t)(u >> 16); }
+    ok = ok && hip::upload_raw(w.native, fresh.data(), n * k * 2);
+    std::memcpy(w.host, fresh.data(), (size_t)n * k * 2);                    // the comparison reads the host half
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "after upload_raw into the weight");
+    check("prepared weight follows a raw upload into its buffer", ok);
+
+    // a recorded graph that writes the weight: every replay drops the cached form, and the
+    // drop recorded while the capture was open waits for the capture's end
+    ok = hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k);          // prepared form exists
+    w2.read();
+    ok = ok && hip::capture_begin();
+    ok = ok && hip::copy_d2d(w.native, w2.native, n * k * 2);             // recorded: claims the weight, drops the form
+    void* g = hip::capture_end();
+    ok = ok && g != nullptr;
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "capture alone changes nothing");
+    ok = ok && hip::graph_launch(g);
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w2, "after a replay that overwrites the weight");
+    hip::graph_destroy(g);
+    check("prepared weight follows a graph replay that writes its buffer", ok);
+
+    // a weight row that spans 2^40: its image is not exact for the tiny element, and a row of A
+    // that is one huge activation at that element's k makes the result that element alone
+    reinterpret_cast<uint16_t*>(w.write())[3 * k + 9] = 0x2b80;             // 2^-40
+    {
+      float* pa = a.write();
+      for (int64_t i = 0; i < k; i++) pa[(m / 2) * k + i] = 0.0f;
+      pa[(m / 2) * k + 9] = 3.0e9f;
+    }
+    ok = hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k) && rows_match(w, "tiny weight under a huge activation");
+    {
+      const float got = o.read()[(m / 2) * n + 3];
+      const double want = 3.0e9 * std::ldexp(1.0, -40);
+      ok = ok && close(got, want) && std::fabs(got - want) <= 1e-4 * want;
+      if (!ok) std::printf("  tiny weight: got %.9g want %.9g\n", got, want);
+    }
+    check("a weight element its f16 image cannot hold is taken from the weight itself where it shows", ok);
+  }
+
+  {  // a product deeper than the prepared form goes (K > 32768) has no image and runs on the bf16 rows
+    const int64_t m = 96, n = 1280, k = 32768 + 64;                          // m * n * k = 4.03e9: "large"
+    buf a(m * k), w(n * k / 2), o(m * n);
+    fill(a);
+    uint16_t* pw = reinterpret_cast<uint16_t*>(w.write());
+    for (int64_t i = 0; i < n * k; i++) { const float v = 0.05f * rnd(); uint32_t u; std::memcpy(&u, &v, 4); pw[i] = (uint16_t)(u >> 16); }
+    bool ok = hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k);
+    ok = ok && hip::gemm_bf16_nt(a.native, w.native, o.native, m, n, k);
+    const float* got = o.read();
+    for (int64_t r : {int64_t(0), m - 1})
+      for (int64_t c : {int64_t(0), n - 1}) {
+        double want = 0;
+        for (int64_t i = 0; i < k; i++) {
+          const uint32_t u = (uint32_t)reinterpret_cast<const uint16_t*>(w.host)[c * k + i] << 16;
+          float f; std::memcpy(&f, &u, 4);
+          want += (double)a.host[r * k + i] * (double)f;
+        }
+        ok = ok && close(got[r * n + c], want);
+      }
+    check("a prompt product deeper than the prepared form runs on the bf16 rows", ok);
   }
 
   {  // pool: a released buffer comes back for the same size, contents pointer included

@@ -135,17 +135,41 @@ def test_gemm_f16w_random_shapes_exact(lib, orc):
         P.free()
 
 
+def _same_as_fp32_chain(got, want, A=None, Ww=None):
+    """allclose(1e-4, 1e-5) against the oracle's fp32 chain where that is finite; the same infinity
+    or a NaN where it is not. Two fp32 evaluations of a sum whose terms cancel can differ by more than
+    rtol of the (small) result without either being wrong: with the operands given (A f32, Ww the
+    widened weight), an element outside allclose passes only if it is within twice the oracle's own
+    distance from the float64 product - no worse an evaluation than the reference's chain, which is
+    itself off by more than the tolerance there. Returns (ok, worst element in tolerances, elements
+    judged against float64 that way)."""
+    fin = np.isfinite(want)
+    with np.errstate(over="ignore", invalid="ignore"):
+        units = np.where(fin, np.abs(got.astype(np.float64) - want) / (ATOL + RTOL * np.abs(want.astype(np.float64))), 0.0)
+    units = np.nan_to_num(units, nan=np.inf)
+    out = fin & (units > 1.0)
+    by_bound = 0
+    if out.any() and A is not None:
+        a64, w64 = A.astype(np.float64), Ww.astype(np.float64)
+        with np.errstate(over="ignore", invalid="ignore"):
+            truth = a64 @ w64.T
+        with np.errstate(over="ignore", invalid="ignore"):
+            excused = out & (np.abs(got - truth) <= 2.0 * np.abs(want - truth))
+        by_bound = int(excused.sum())
+        out = out & ~excused
+    same_inf = np.array_equal(np.isnan(want), np.isnan(got)) and np.array_equal(want[np.isinf(want)], got[np.isinf(want)])
+    return (not out.any()) and same_inf, float(units.max()) if units.size else 0.0, by_bound
+
+
 def test_gemm_f16w_wide_ranges(lib, orc):
-    """Rows whose magnitudes are far apart, in A and in W, against float64. The scaling is per row,
-    so a row of 1e-30 or 1e+20 is as accurate as a row of ones. Bound per result:
-      (K/8 + 4) 2^-24 sum_k |a w|      fp32 accumulation in K/16 steps per plane, at most one ulp of the
-                                       running sum each (the reference's own chain has K such steps),
-                                       plus the split's 2^-24 and the product's rounding;
-      2^-38 max|a_row| sum_k |w|       inside a row, an activation more than 2^23 below the row's
-                                       largest keeps an absolute error of 2^-39.5 of that largest
-                                       (its second f16 term is a subnormal);
-      2^-39 sum_k |a| max|w_row|       a weight more than 2^29 below its row's largest likewise.
-    Results below the f32 normal range are not compared."""
+    """Rows whose magnitudes are far apart, in A and between the rows of W: EVERY row against the
+    oracle's fp32 product at allclose(1e-4, 1e-5), the adversarial ones included. The scaling is per
+    row, so a row of 1e-30 or 1e+20 is as accurate as a row of ones. Inside a row, an activation more
+    than 2^24 below the row's largest is carried with an absolute error only; rows 6, 8 and 9 are
+    built so that this would show - an outlier 10^7 to 10^8 above the rest that meets zero or tiny
+    weights, so that the results are made of the small elements alone - and the kernel has to notice
+    and work those results out with the reference's fp32 chain. Rows with an infinity or a NaN come
+    out as the reference's chain leaves them (+-inf, NaN where inf meets a zero weight)."""
     M, N, K = 260, 516, 512
     rng = np.random.default_rng(31)
     A = rng.standard_normal((M, K)).astype(np.float32)
@@ -153,30 +177,86 @@ def test_gemm_f16w_wide_ranges(lib, orc):
     A[3] *= np.float32(1e20); A[4] *= np.float32(1e-30); A[5] = 0.0
     A[6, 17] = 3e7                      # one outlier 10^7 times the rest of its row
     A[7] *= np.exp2(rng.integers(-12, 12, K)).astype(np.float32)   # 2^24 between elements of a row
+    A[8, 5] = 1e8                       # an outlier that meets only zero weights (column 5 of W below)
+    A[9, 5] = -4e9; A[9] *= np.float32(1e-3)
+    A[10, 3] = np.inf
+    A[11, 7] = np.nan
+    A[12, 3] = np.inf; A[12, 9] = -np.inf
     Wf[2] *= np.float32(1e-20); Wf[3] *= np.float32(1e15); Wf[4] = 0.0
-    Wf[5] *= np.exp2(rng.integers(-14, 14, K)).astype(np.float32)
+    Wf[5] *= np.exp2(rng.integers(-6, 6, K)).astype(np.float32)
     Wf[6, 100] = 5e4
+    Wf[:, 5] = 0.0
+    Wf[7:40, 17] *= np.float32(1e-6)    # the outlier of row 6 meets tiny weights in these columns
     Wb = orc.to_bf16(Wf).reshape(N, K)
-    Ww = orc.bf16_widen(Wb).reshape(N, K).astype(np.float64)
+    Ww = orc.bf16_widen(Wb).reshape(N, K)
     P = Prepared(lib, Wb)
-    got = P.product(A).astype(np.float64)
-    a64 = A.astype(np.float64)
+    got = P.product(A)
     with np.errstate(over="ignore", invalid="ignore"):
-        want = a64 @ Ww.T
-        bound = ((K / 8 + 4) * 2.0 ** -24 * (np.abs(a64) @ np.abs(Ww).T)
-                 + 2.0 ** -38 * np.abs(a64).max(axis=1)[:, None] * np.abs(Ww).sum(axis=1)[None, :]
-                 + 2.0 ** -39 * np.abs(a64).sum(axis=1)[:, None] * np.abs(Ww).max(axis=1)[None, :])
-    ok = np.isfinite(want) & (np.abs(want) < 3e38) & ((np.abs(want) > 1e-37) | (want == 0.0))
-    assert np.all(np.isfinite(got[ok]))
-    err = np.abs(got - want)
-    assert np.all(err[ok] <= bound[ok]), float((err[ok] / (bound[ok] + 1e-300)).max())
-    print("   worst error / bound: %.3f" % float((err[ok] / (bound[ok] + 1e-300)).max()), flush=True)
-    assert np.all(got[5] == 0.0) and np.all(got[:, 4] == 0.0)
-    # and the plain rows meet the GEMM's tolerance against the oracle
-    plain = [0, 1, 2, 100, 259]
-    w2 = orc.gemm_bf16_nt(np.ascontiguousarray(A[plain]), Wb)
-    cols = np.array([c for c in range(N) if c not in (2, 3, 4, 5, 6)])
-    assert allclose(got[plain][:, cols].astype(np.float32), w2[:, cols], RTOL, ATOL)
+        want = orc.gemm_bf16_nt(A, Wb)
+    for r in range(14):
+        ok, worst, nb = _same_as_fp32_chain(got[r:r + 1], want[r:r + 1], A[r:r + 1], Ww)
+        print("   row %2d: worst %.3f tolerances, %d elements judged against float64%s"
+              % (r, worst, nb, "" if np.all(np.isfinite(want[r])) else "  (not finite in the reference)"), flush=True)
+        assert ok, (r, worst)
+    ok, worst, nb = _same_as_fp32_chain(got, want, A, Ww)
+    assert ok and nb <= 8, (worst, nb)
+    assert np.all(got[5] == 0.0) and np.all(got[:13, 4][np.isfinite(want[:13, 4])] == 0.0)
+    # the same rows through the gated product and through K-split parts
+    P.free()
+
+
+def test_gemm_f16w_wide_ranges_under_a_k_split_and_gated(lib, orc):
+    """The same kind of rows where the product is split over K (each part works out its own K range
+    exactly) and through the gated epilogue."""
+    M, ff, K = 130, 256, 1024
+    rng = np.random.default_rng(33)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    A[2, 700] = 2e8
+    A[3, 5] = np.inf
+    Wf = (rng.standard_normal((2 * ff, K)) * 0.02).astype(np.float32)
+    Wf[:, 700] = 0.0
+    Wb = orc.to_bf16(Wf).reshape(2 * ff, K)
+    with np.errstate(over="ignore", invalid="ignore"):
+        both = orc.gemm_bf16_nt(A, Wb)
+    Pp = Prepared(lib, Wb)                         # plain: [M, 2 ff], few tiles -> K split
+    got = Pp.product(A)
+    ok, worst, nb = _same_as_fp32_chain(got, both, A, orc.bf16_widen(Wb).reshape(2 * ff, K))
+    assert ok and nb <= 4, (worst, nb)
+    Pp.free()
+    Pg = Prepared(lib, Wb, gated=True)
+    got = Pg.product(A)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = orc.swiglu(np.ascontiguousarray(both[:, :ff]), np.ascontiguousarray(both[:, ff:]))
+    fin = np.isfinite(want)
+    assert np.all(np.abs(got[fin] - want[fin]) <= 2e-5 + 2e-4 * np.abs(want[fin])), "gated rows"
+    assert np.array_equal(np.isnan(got[3]), np.isnan(want[3]))
+    Pg.free()
+
+
+def test_gemm_f16w_weights_the_image_cannot_hold(lib, orc):
+    """Weight rows whose nonzero elements span more than 2^31, or that hold an infinity: the f16 image
+    is not exact there, the preparation counts such elements per row, and the products work out from
+    W itself the results in which that could show. Here it does show: row 3 of A is a single huge
+    activation at the k of a tiny weight, so the results of that row ARE those tiny weights."""
+    M, N, K = 70, 96, 128
+    rng = np.random.default_rng(35)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    Wf = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    Wf[3] *= np.float32(1e-25); Wf[4] *= np.float32(1e20)       # rows may differ by any factor
+    Wf[7, 11] = 1e-12                  # 2^-34 of its row's largest
+    Wf[8, 11] = -3e-13
+    Wf[9, 1] = np.inf
+    A[3] = 0.0; A[3, 11] = 2e9         # picks out column 11 of W
+    A[5, 11] = 1e7
+    Wb = orc.to_bf16(Wf).reshape(N, K)
+    P = Prepared(lib, Wb)
+    got = P.product(A)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = orc.gemm_bf16_nt(A, Wb)
+    ok, worst, nb = _same_as_fp32_chain(got, want, A, orc.bf16_widen(Wb).reshape(N, K))
+    assert ok and nb == 0, (worst, nb)
+    assert want[3, 7] != 0.0 and abs(got[3, 7] - want[3, 7]) <= 1e-4 * abs(want[3, 7])     # 2e9 * 1e-12, from W itself
+    assert np.all(np.isinf(got[:, 9]) | np.isnan(got[:, 9]))
     P.free()
 
 
@@ -286,7 +366,9 @@ def test_gemm_f16w_declines(lib):
     """K must be whole slabs of 32 and at most 32768; nulls and misaligned operands are refused;
     the library stays usable."""
     a, w, c = lib.empty((8, 40)), lib.empty_bytes(64 * 40 * 2), lib.empty((8, 64))
-    img, ex = lib.empty_bytes(1 << 16), lib.empty_bytes(64)
+    img, ex = lib.empty_bytes(1 << 16), lib.empty_bytes(lib.c.tlhip_gemm_f16w_exps_bytes(64, 0))
+    assert lib.c.tlhip_gemm_f16w_exps_bytes(64, 0) == 3 * 64 + 16 and lib.c.tlhip_gemm_f16w_exps_bytes(70, 1) == 3 * 144 + 16
+    assert lib.c.tlhip_gemm_f16w_bytes(64, 32800, 0) == 0 and lib.c.tlhip_gemm_f16w_bytes(64, 32768 + 32, 0) == 0   # deeper than the products go
     assert lib.c.tlhip_gemm_f16w_bytes(64, 40, 0) == 0
     assert lib.c.tlhip_gemm_f16w_bytes(64, 64, 0) == 2 * 16384          # one column tile, two slabs
     assert lib.c.tlhip_gemm_f16w_bytes(130, 64, 1) == 2 * 2 * 16384     # gated: 128 features per tile

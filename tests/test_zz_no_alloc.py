@@ -2,7 +2,10 @@
 split partials live in a fixed 1 MiB array inside the library), gives the results of
 tlhip_attn_decode bit for bit - same kernels, same launch plan - and against the oracle within
 the bar of BASELINE (allclose rtol 1e-4 / atol 1e-5). Two calls in a row share the array, the
-second on a smaller input; a shape whose partials exceed the array is refused."""
+second on a smaller input; a shape whose partials exceed the array is refused. That the calls
+allocate nothing is checked twice: the library's count of allocation and release calls does not
+move across them, and they run inside a graph capture, where the library's growable scratch
+refuses to grow, with every replay of the graph equal to the eager result."""
 import numpy as np
 import pytest
 
@@ -32,9 +35,12 @@ def test_static_entry_equals_attn_decode_on_two_calls_in_a_row(lib, orc):
                      lib.to_device(np.full((Hq, D), np.nan, np.float32)), lib.empty((Hq, D))))
     lib.sync()
     # the calls under test, back to back on the library's stream
+    allocs = lib.alloc_calls()
     for (Hq, Hkv, ctx, kv_max, D, _), (q, K, V, dq, dk, dv, do, _ref) in zip(cases, bufs):
         print("case attn_decode_static", Hq, Hkv, ctx, D, flush=True)
         lib.attn_decode_static(dq, dk, dv, do, Hq, Hkv, ctx, kv_max, D, float(1.0 / np.sqrt(D)))
+    lib.sync()
+    assert lib.alloc_calls() == allocs, "the static entry point allocated or released memory"
     for (Hq, Hkv, ctx, kv_max, D, _), (q, K, V, dq, dk, dv, do, dref) in zip(cases, bufs):
         scale = float(1.0 / np.sqrt(D))
         lib.attn_decode(dq, dk, dv, dref, Hq, Hkv, ctx, kv_max, D, scale)
@@ -51,6 +57,32 @@ def test_static_entry_equals_attn_decode_on_two_calls_in_a_row(lib, orc):
     for b in bufs:
         for d in b[3:]:
             d.free()
+
+
+def test_static_entry_inside_a_graph_capture(lib, orc):
+    """The 7B decode shape recorded into a graph (where growing the library's scratch is refused, so
+    a fallback to it would fail the call) and replayed three times with eager work and syncs in
+    between: every replay equals the eager call bit for bit, and nothing was allocated."""
+    Hq, Hkv, ctx, kv_max, D = 28, 4, 4096, 4352, 128
+    q, K, V = _inputs(orc, Hq, Hkv, ctx, kv_max, D, 51)
+    dq, dk, dv = lib.to_device(q), lib.to_device(K), lib.to_device(V)
+    do, dref = lib.empty((Hq, D)), lib.empty((Hq, D))
+    scale = float(1.0 / np.sqrt(D))
+    lib.attn_decode_static(dq, dk, dv, dref, Hq, Hkv, ctx, kv_max, D, scale)
+    ref = dref.numpy()
+    allocs = lib.alloc_calls()
+    lib.graph_begin()
+    lib.attn_decode_static(dq, dk, dv, do, Hq, Hkv, ctx, kv_max, D, scale)
+    g = lib.graph_end()
+    assert lib.alloc_calls() == allocs
+    nan = np.full((Hq, D), np.nan, np.float32)
+    for i in range(3):
+        do.upload(nan)                      # eager work and a sync between the replays
+        lib.graph_launch(g)
+        assert np.array_equal(do.numpy(), ref), i
+    lib.graph_destroy(g)
+    for d in (dq, dk, dv, do, dref):
+        d.free()
 
 
 def test_static_entry_bf16_cache(lib, orc):
