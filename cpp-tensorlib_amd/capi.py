@@ -123,6 +123,7 @@ SIGNATURES = {
     "tlhip_bench_copy": (cint, [P, P, sz, cint]),
     "tlhip_bench_read": (cint, [P, sz, P, cint]),
     "tlhip_alloc_calls": (cint, [C.POINTER(u64)]),
+    "tlhip_tune_attn_decode": (cint, [cint]),
     "tlhip_warm_fork": (cint, [P, P, cint, cint, cint]),
     "tlhip_warm_join": (cint, []),
 }
@@ -500,6 +501,10 @@ class TlHip:
     def tune_attn_prefill(self, kernel):
         """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes, 4: f16 terms."""
         self._chk(self.c.tlhip_tune_attn_prefill(int(kernel)))
+
+    def tune_attn_decode(self, kernel):
+        """0: built-in choice, 1: the key-slot decode attention kernel for every shape."""
+        self._chk(self.c.tlhip_tune_attn_decode(int(kernel)))
 
     def tune_gemm_planes(self, planes):
         """3: the int4 prompt GEMMs cut activations into three bf16 terms; 0: built-in choice (two f16)."""

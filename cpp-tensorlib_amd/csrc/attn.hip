@@ -642,6 +642,328 @@ __global__ __launch_bounds__(1024) void attn_combine_kernel(const float* __restr
   }
 }
 
+// ---- decode attention for a GQA group: one block per (kv head, split), one wavefront per head ----
+//
+// At the decode sizes of a GQA model (7 query heads per kv head, a few thousand keys) a step is
+// not bound by bandwidth but by two other things: how many load instructions a CU has to issue
+// (about one 1 KB instruction per 10 ns while misses are outstanding) and how long each
+// wavefront's own instruction stream is. The kernel above lets two blocks fetch the K/V rows of a
+// kv head (one per half of the head group) and pays the per-head costs - the softmax update, the
+// sums over key slots at the end - once per head AND wavefront, then merges the wavefronts of a
+// block through LDS. Here:
+//   * a block owns a (kv head, split) pair and ALL of the group's query heads: a 64-key tile of K
+//     and of V is copied global -> LDS once per CU, without passing through registers
+//     (global_load_lds, 1 KB of whole rows per instruction, requested before anything else);
+//   * wavefront h of the block serves query head h over the whole tile, so the running softmax
+//     state of a (head, split) lives in ONE wavefront: nothing is merged inside the block, and the
+//     per-head costs are paid once per head; the last wavefront serves no head: it copies, and in
+//     the fused form it makes the step's new key/value row;
+//   * scores: lane = key. A lane walks its key's row in LDS 16 bytes at a time against the query
+//     row, which every lane reads from the same LDS address (a broadcast): 4 FMAs per two LDS
+//     reads and no cross-lane step at all. The row's 16-byte chunks are stored XOR-swizzled by the
+//     key number (chunk j of key k at position j ^ (k mod CH)) - the copy chooses which global
+//     chunk each lane fetches, so this costs nothing - which spreads the 64 lanes' reads, 512 bytes
+//     apart, over all banks;
+//   * the softmax maximum and sum are plain wavefront reductions over the 64 keys;
+//   * P.V: lane = (key group, 4 output columns): CH = D/4 lanes cover a V row (a contiguous,
+//     conflict-free LDS read), the 64/CH key groups take KPG = CH keys each, probabilities are
+//     read from a per-head LDS line (the lanes of a group read the same address), and the key
+//     groups are added up at the very end with one or two register swaps per column.
+// Tiles are dealt round-robin over the splits (tile t to split t mod S); a block whose split holds
+// several tiles (long contexts, or a context past what the planned grid covers at one tile each)
+// copies the next tile into a second LDS stage while it works on the current one. The deal does
+// not depend on the live context, so a grid planned for the cache capacity (position on the
+// device) and one planned for the live context give the same bits: splits without keys write
+// neutral partials, which add exact zeros in the combine.
+// QKV: as in the kernel above, the raw [q | k | v] projection comes in; the block's query rows get
+// their bias and rotation on the way into LDS, and the block whose tile holds the step's position
+// forms the new key/value row (same arithmetic as the stand-alone epilogue, so cache rows are
+// bit-identical), stores it into the cache and uses it from LDS in place of the stale cache row.
+namespace gqa {
+
+constexpr int kKeys = 64;   // keys per tile: the lanes of a wavefront
+
+template <int D> struct Geo {
+  static constexpr int CH = D / 4;               // 16-byte chunks per row
+  static constexpr int RB = D * 4;               // bytes per row
+  static constexpr int KG = 64 / CH;             // key groups of the P.V pass
+  static constexpr int TILE = kKeys * RB;        // bytes of a tile's K (or V) rows
+  static constexpr int RPI = 1024 / RB;          // rows per 1 KB copy
+  static constexpr int COPIES = 2 * kKeys / RPI; // 1 KB copies per tile (K and V)
+};
+
+template <int D> inline size_t lds_bytes(int group, int stages) {
+  return (size_t)stages * 2 * Geo<D>::TILE + (size_t)(2 * D + 2 * group * D + D + group * 64) * sizeof(float);
+}
+
+template <int D, int GRP, bool QKV>
+__global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
+    const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
+    float* __restrict__ out, float* __restrict__ part_m, float* __restrict__ part_l,
+    float* __restrict__ part_acc, int ctx, int64_t kv_stride, float scale, int S,
+    const uint32_t* __restrict__ dpos, QkvFuse fz, int kv_rows, int n_kv_heads, int stages) {
+  using Gm = Geo<D>;
+  constexpr int CH = Gm::CH, RB = Gm::RB, KG = Gm::KG, TILE = Gm::TILE, RPI = Gm::RPI;
+  constexpr int NW = GRP + 1;
+  constexpr int CPW = (Gm::COPIES / 2 + NW - 1) / NW;        // 1 KB copies per wavefront and tile, of K and again of V
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int lane = threadIdx.x & 63, tq = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kvh = blockIdx.x % n_kv_heads, split = blockIdx.x / n_kv_heads;
+  char* extra = smem + (size_t)stages * 2 * TILE;
+  float* newk = reinterpret_cast<float*>(extra);             // the step's own key / value row (QKV)
+  float* newv = newk + D;
+  float* qs = newv + D;                                      // QKV: the query rows with bias, not yet rotated
+  float* qrot = qs + GRP * D;                                // the query rows the scores use
+  float* tabs = qrot + GRP * D;                              // QKV: (cos, sin) pairs of the step
+  float* pb = tabs + D;                                      // [GRP][64] probabilities of the current tile
+  const float* Kh = K + (size_t)kvh * kv_stride;
+  const float* Vh = V + (size_t)kvh * kv_stride;
+
+  // A block barrier without the fence __syncthreads() carries: that fence waits for every copy
+  // in flight (they write LDS). What has to be complete is waited for by count instead.
+  auto barrier = [] {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  // this wavefront's copies of tile t into `stage`: rows past the cache's capacity are clamped
+  // (mapped memory whatever it holds; such keys are masked where they are used)
+  // (all of a wavefront's K copies go out before its V copies: loads land in order, so the scores
+  // can start when "all but my CPW youngest" have landed)
+  auto copy_tile = [&](int t, char* stage) {
+#pragma unroll
+    for (int half = 0; half < 2; half++)
+#pragma unroll
+      for (int i = 0; i < CPW; i++) {
+        const int rp = min(wave + i * NW, Gm::COPIES / 2 - 1);   // (a spare slot repeats the last copy)
+        const int r = rp * RPI + lane / CH;                      // row of the tile
+        const int j = (lane % CH) ^ (r & (CH - 1));              // the chunk that belongs at this lane's position
+        const int key = min(t * kKeys + r, kv_rows - 1);
+        const float* src = (half ? Vh : Kh) + (size_t)key * D + j * 4;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(stage + half * TILE + rp * 1024),
+                                         16, 0, 0);
+      }
+  };
+
+  // ---- requests, oldest first: the query rows (a few), then the first tile -----------------------
+  TLHIP_MARK(0);
+  constexpr int QT = GRP * CH;                               // float4s of the block's query rows
+  float4 q_own = make_float4(0.f, 0.f, 0.f, 0.f), q_bias = q_own;
+  if (tq < QT) {
+    const size_t r = ((size_t)kvh * GRP + tq / CH) * D + (tq % CH) * 4;
+    q_own = *reinterpret_cast<const float4*>(q + r);
+    if (QKV && fz.bq) q_bias = *reinterpret_cast<const float4*>(fz.bq + r);
+  } else if (QKV && tq < QT + D / 4) {
+    q_own = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(fz.table) + (tq - QT) * 4);
+  }
+  // QKV: what the step's own key/value row is made of, requested now by the wavefront that serves
+  // no head (in every block: which block needs it depends on the position, which may live on the
+  // device and is not known yet)
+  float4 nk_own = q_own, nk_oth = q_own, nv_own = q_own, nt0 = q_own, nt1 = q_own;
+  const int nd0 = (lane % CH) * 4;
+  const bool nlo = nd0 < D / 2;
+  if (QKV && wave == GRP) {
+    const int Hq = n_kv_heads * GRP;
+    const float* kraw = q + (size_t)(Hq + kvh) * D;
+    const float* vraw = q + (size_t)(Hq + n_kv_heads + kvh) * D;
+    const int j0 = nlo ? nd0 : nd0 - D / 2;
+    nk_own = load_biased4(kraw, fz.bk ? fz.bk + (size_t)kvh * D : nullptr, nd0);
+    nk_oth = load_biased4(kraw, fz.bk ? fz.bk + (size_t)kvh * D : nullptr, nlo ? nd0 + D / 2 : nd0 - D / 2);
+    nv_own = load_biased4(vraw, fz.bv ? fz.bv + (size_t)kvh * D : nullptr, nd0);
+    nt0 = *reinterpret_cast<const float4*>(fz.table + j0);
+    nt1 = *reinterpret_cast<const float4*>(fz.table + j0 + 2);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  copy_tile(split, smem);
+  __builtin_amdgcn_sched_barrier(0);
+  TLHIP_MARK(7);
+
+  // ---- the position, the live context, who makes the new row -------------------------------------
+  int64_t new_pos = 0;
+  bool has_new = false;
+  if constexpr (QKV) {
+    new_pos = dpos ? (int64_t)*dpos : (int64_t)ctx - 1;
+    has_new = new_pos < fz.kv_max;
+    ctx = (int)min(new_pos, fz.kv_max) + (has_new ? 1 : 0);  // keys [0, pos) of the cache and the new one
+  } else if (dpos) {
+    ctx = min(ctx, (int)*dpos + 1);
+  }
+  const int newt = (int)(new_pos / kKeys), newj = (int)(new_pos % kKeys);
+  const bool owner = QKV && has_new && newt % S == split;    // this block's tiles include the step's position
+
+  // ---- query rows into LDS (the copies stay in flight: wait for what is older than them) ----------
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * CPW) : "memory");
+  if (tq < QT) {
+    if constexpr (QKV) {
+      q_own.x += q_bias.x; q_own.y += q_bias.y; q_own.z += q_bias.z; q_own.w += q_bias.w;
+      *reinterpret_cast<float4*>(qs + (tq / CH) * D + (tq % CH) * 4) = q_own;
+    } else {
+      *reinterpret_cast<float4*>(qrot + (tq / CH) * D + (tq % CH) * 4) = q_own;
+    }
+  } else if (QKV && tq < QT + D / 4) {
+    *reinterpret_cast<float4*>(tabs + (tq - QT) * 4) = q_own;
+  }
+  if constexpr (QKV) {
+    barrier();
+    if (tq < QT) {
+      const int g = tq / CH, d0 = (tq % CH) * 4;
+      const bool lo = d0 < D / 2;
+      const int j0 = lo ? d0 : d0 - D / 2;
+      const float4 own = *reinterpret_cast<const float4*>(qs + g * D + d0);
+      const float4 oth = *reinterpret_cast<const float4*>(qs + g * D + (lo ? d0 + D / 2 : d0 - D / 2));
+      const float4 t0 = *reinterpret_cast<const float4*>(tabs + 2 * j0);        // (c0, s0, c1, s1)
+      const float4 t1 = *reinterpret_cast<const float4*>(tabs + 2 * j0 + 4);    // (c2, s2, c3, s3)
+      *reinterpret_cast<float4*>(qrot + g * D + d0) = rope4_pair(own, oth, t0, t1, lo);
+    }
+    // the step's own key/value row: formed by the wavefront that serves no head, kept in LDS for
+    // this block's scores and stored into the cache (rows of other tiles belong to other blocks)
+    if (owner && wave == GRP && lane < CH) {
+      float* krow = static_cast<float*>(fz.Kw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
+      float* vrow = static_cast<float*>(fz.Vw) + (size_t)kvh * kv_stride + (size_t)new_pos * D;
+      const float4 kr = rope4_pair(nk_own, nk_oth, nt0, nt1, nlo);
+      *reinterpret_cast<float4*>(krow + nd0) = kr;
+      *reinterpret_cast<float4*>(vrow + nd0) = nv_own;
+      *reinterpret_cast<float4*>(newk + nd0) = kr;
+      *reinterpret_cast<float4*>(newv + nd0) = nv_own;
+    }
+  }
+  TLHIP_MARK(1);
+
+  // ---- the tiles of this split ---------------------------------------------------------------------
+  const int h = wave;                                        // the query head this wavefront serves (wave GRP: none)
+  const int cg = lane % CH, kg = lane / CH;
+  float m = -INFINITY, l = 0.f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  int st = 0;
+  bool first = true;
+  // The first tile is used as it lands: its K rows (and the query rows, and the new row) are
+  // waited for, the scores and the softmax run while its V rows are still on their way. A later
+  // tile has landed whole by the time its turn comes (it was copied during the tile before it).
+  for (int t = split; t * kKeys < ctx; t += S) {
+    char* stage = smem + (size_t)st * 2 * TILE;
+    const int tn = t + S;
+    const bool more = tn * kKeys < ctx;
+    if (first) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CPW) : "memory");     // my K copies of the first tile
+      barrier();                                                     // ... and everyone's; query rows and the new row too
+      TLHIP_MARK(2);
+    }
+    if (more) copy_tile(tn, smem + (size_t)(st ^ 1) * 2 * TILE);   // (stages == 2 whenever a split holds two tiles)
+    const int nvalid = min(kKeys, ctx - t * kKeys);          // >= 1
+    const bool with_new = QKV && has_new && t == newt;       // key newj of this tile is the new row
+    const bool plain = nvalid == kKeys && !with_new;
+    if (h < GRP) {
+      // scores: lane = key
+      const bool mine_new = with_new && lane == newj;
+      const char* krow = mine_new ? reinterpret_cast<const char*>(newk) : stage + lane * RB;
+      const int swz = mine_new ? 0 : (lane & (CH - 1)) << 4;
+      const float* qh = qrot + h * D;
+      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+      for (int j = 0; j < CH; j += 4) {
+        const float4 k0 = *reinterpret_cast<const float4*>(krow + (((j + 0) << 4) ^ swz));
+        const float4 k1 = *reinterpret_cast<const float4*>(krow + (((j + 1) << 4) ^ swz));
+        const float4 k2 = *reinterpret_cast<const float4*>(krow + (((j + 2) << 4) ^ swz));
+        const float4 k3 = *reinterpret_cast<const float4*>(krow + (((j + 3) << 4) ^ swz));
+        const float4 q0 = *reinterpret_cast<const float4*>(qh + (j + 0) * 4);
+        const float4 q1 = *reinterpret_cast<const float4*>(qh + (j + 1) * 4);
+        const float4 q2 = *reinterpret_cast<const float4*>(qh + (j + 2) * 4);
+        const float4 q3 = *reinterpret_cast<const float4*>(qh + (j + 3) * 4);
+        s0 = fmaf(q0.x, k0.x, s0); s0 = fmaf(q0.y, k0.y, s0); s0 = fmaf(q0.z, k0.z, s0); s0 = fmaf(q0.w, k0.w, s0);
+        s1 = fmaf(q1.x, k1.x, s1); s1 = fmaf(q1.y, k1.y, s1); s1 = fmaf(q1.z, k1.z, s1); s1 = fmaf(q1.w, k1.w, s1);
+        s2 = fmaf(q2.x, k2.x, s2); s2 = fmaf(q2.y, k2.y, s2); s2 = fmaf(q2.z, k2.z, s2); s2 = fmaf(q2.w, k2.w, s2);
+        s3 = fmaf(q3.x, k3.x, s3); s3 = fmaf(q3.y, k3.y, s3); s3 = fmaf(q3.z, k3.z, s3); s3 = fmaf(q3.w, k3.w, s3);
+      }
+      const float sc = lane < nvalid ? ((s0 + s1) + (s2 + s3)) * scale : -INFINITY;
+      // online softmax over the tile's keys: m and l are the same in every lane
+      const float mnew = fmaxf(m, wave_max(sc));             // finite: the tile holds a live key
+      const float corr = __expf(m - mnew);                   // 0 on the first tile (m = -inf)
+      const float p = __expf(sc - mnew);                     // 0 for masked keys
+      l = fmaf(l, corr, wave_sum(p));
+      acc.x *= corr; acc.y *= corr; acc.z *= corr; acc.w *= corr;
+      m = mnew;
+      pb[h * 64 + lane] = p;
+      wave_lds_sync();
+      TLHIP_MARK(3);
+    }
+    if (first) {                                             // the first tile's V rows
+      if (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * CPW) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      barrier();
+      first = false;
+    }
+    if (h < GRP) {
+      // P.V: lane = (key group kg, columns 4 cg .. 4 cg + 3)
+      const char* vt = stage + TILE;
+      const float* ph = pb + h * 64 + kg * CH;
+      if (plain) {
+        const char* vb = vt + (size_t)kg * CH * RB;
+        const int c4 = cg << 4;
+#pragma unroll
+        for (int i = 0; i < CH; i += 4) {
+          const float4 p4 = *reinterpret_cast<const float4*>(ph + i);
+          const float pp[4] = {p4.x, p4.y, p4.z, p4.w};
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const float4 v = *reinterpret_cast<const float4*>(vb + (i + u) * RB + (c4 ^ ((i + u) << 4)));
+            acc.x = fmaf(pp[u], v.x, acc.x); acc.y = fmaf(pp[u], v.y, acc.y);
+            acc.z = fmaf(pp[u], v.z, acc.z); acc.w = fmaf(pp[u], v.w, acc.w);
+          }
+        }
+      } else {
+        // the tile at the end of the context, or the one that holds the new row: a masked key
+        // (weight 0) reads the last live row instead of its own, which may hold anything
+#pragma unroll 4
+        for (int i = 0; i < CH; i++) {
+          const int row = min(kg * CH + i, nvalid - 1);
+          const char* vrow = with_new && row == newj ? reinterpret_cast<const char*>(newv) + (cg << 4)
+                                                     : vt + row * RB + ((cg ^ (row & (CH - 1))) << 4);
+          const float4 v = *reinterpret_cast<const float4*>(vrow);
+          const float pp = ph[i];
+          acc.x = fmaf(pp, v.x, acc.x); acc.y = fmaf(pp, v.y, acc.y);
+          acc.z = fmaf(pp, v.z, acc.z); acc.w = fmaf(pp, v.w, acc.w);
+        }
+      }
+    }
+    if (more) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the next tile has landed (my copies) ...
+      barrier();                                             // ... everyone's; and this stage is free again
+    }
+    st ^= 1;
+  }
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // (a block without keys still has its copies in flight)
+  // ---- add up the key groups and store ----------------------------------------------------------------
+  TLHIP_MARK(4);
+  if (h < GRP) {
+    const auto across = [](float a) {
+      if (KG == 4) {
+        const LanePair p16 = swap16(a, a);
+        a = p16.first + p16.second;
+      }
+      const LanePair p32 = swap32(a, a);
+      return p32.first + p32.second;
+    };
+    acc.x = across(acc.x); acc.y = across(acc.y); acc.z = across(acc.z); acc.w = across(acc.w);
+    if (lane < CH) {
+      const size_t head = (size_t)kvh * GRP + h;
+      if (S == 1) {
+        // (divisions, as in the combine kernel: a grid with one split and one with more give the same bits)
+        *reinterpret_cast<float4*>(out + head * D + lane * 4) = make_float4(acc.x / l, acc.y / l, acc.z / l, acc.w / l);
+      } else {
+        const size_t ps = head * S + split;
+        *reinterpret_cast<float4*>(part_acc + ps * D + lane * 4) = acc;   // zeros, -inf, 0 where the split held no key
+        if (lane == 0) { part_m[ps] = m; part_l[ps] = l; }
+      }
+    }
+  }
+  TLHIP_MARK(6);
+}
+
+}  // namespace gqa
+
 struct AttnPlan { int G, gz, nw, TK, S, chunk; };
 
 // Split-KV plan. Work is cut into wave tiles of TK keys; the chip wants 4 to 8
@@ -701,6 +1023,83 @@ static size_t attn_partials_floats(int Hq, int S, int D) {
   return hs * 2 + hs * D;
 }
 
+// ---- the GQA kernel's plan and launch ----------------------------------------------------------
+// Which calls it serves: f32 caches, 3 to 8 query heads per kv head (one wavefront each).
+template <typename KT> static bool gqa_applies(int group) { return false; }
+template <> bool gqa_applies<float>(int group) { return group >= 3 && group <= 8; }
+
+// Splits: one tile each while there are CUs for them (a block per CU and kv head), never more
+// than the combine kernel sums in one pass (8 per column group; beyond that its summation order
+// would depend on the count). stages: 2 when a split holds more than one tile.
+struct GqaPlan { int S, stages; };
+static GqaPlan plan_gqa(int Hkv, int ctx, int cus, int D) {
+  const int tiles = (ctx + gqa::kKeys - 1) / gqa::kKeys;
+  int S = cus / Hkv;
+  if (S > 8 * (1024 / D)) S = 8 * (1024 / D);
+  if (S > tiles) S = tiles;
+  if (S < 1) S = 1;
+  return GqaPlan{S, (tiles + S - 1) / S > 1 ? 2 : 1};
+}
+
+static size_t attn_partials_floats(int Hq, int S, int D);
+
+template <int D>
+static int launch_gqa(const float* q, const float* K, const float* V, float* out, int Hq, int Hkv, int ctx,
+                      int64_t kv_max, float scale, const uint32_t* dpos, float* partials, size_t partials_bytes,
+                      const QkvFuse* fuse) {
+  Context& c = tlhip::ctx();
+  const int group = Hq / Hkv;
+  const GqaPlan p = plan_gqa(Hkv, ctx, c.cus, D);
+  const int S = p.S;
+  float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
+  if (S > 1) {
+    const size_t hs = (size_t)Hq * S;
+    const size_t need = attn_partials_floats(Hq, S, D) * sizeof(float);
+    float* base;
+    if (dpos || partials) {   // a buffer the caller named: never the library's growable scratch
+      if (!partials || partials_bytes < need)
+        return fail(TLHIP_EINVAL, "attention: %zu bytes of split partials needed, the buffer given holds %zu",
+                    need, partials_bytes);
+      base = partials;
+    } else {
+      base = static_cast<float*>(scratch(need));
+    }
+    if (!base) return fail(TLHIP_ENOMEM, "tlhip_attn_decode: no scratch for %d splits", S);
+    pm = base;
+    pl = pm + hs;
+    pacc = pl + hs;
+  }
+  const size_t lds = gqa::lds_bytes<D>(group, p.stages);
+  const dim3 grid((unsigned)(Hkv * S)), block(64 * (group + 1));
+  const int64_t kv_stride = kv_max * D;
+  const QkvFuse fz = fuse ? *fuse : QkvFuse{};
+  hipError_t e = hipSuccess;
+  auto go = [&](auto kernel) {
+    // more than 64 KB of LDS per block has to be asked for; asking is cheap next to a launch
+    if (lds > 64 * 1024)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+      hipLaunchKernelGGL(kernel, grid, block, lds, c.stream, q, K, V, out, pm, pl, pacc, ctx, kv_stride, scale, S, dpos,
+                         fz, (int)kv_max, Hkv, p.stages);
+  };
+#define TLHIP_GQA(GG) \
+  if (fuse) go(gqa::attn_gqa_kernel<D, GG, true>); else go(gqa::attn_gqa_kernel<D, GG, false>)
+  switch (group) {
+    case 3: TLHIP_GQA(3); break;
+    case 4: TLHIP_GQA(4); break;
+    case 5: TLHIP_GQA(5); break;
+    case 6: TLHIP_GQA(6); break;
+    case 7: TLHIP_GQA(7); break;
+    default: TLHIP_GQA(8); break;
+  }
+#undef TLHIP_GQA
+  if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
+  if (S > 1)
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(1024), (size_t)(S + 1024) * sizeof(float),
+                       c.stream, pm, pl, pacc, out, S, D);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
+}
+
 // dpos != nullptr: ctx is the cache CAPACITY the grid is planned for, the live
 // context is read from the device, and the split partials live in a buffer the
 // caller owns (a captured graph bakes the address in).
@@ -711,6 +1110,9 @@ static int launch_attn(const float* q, const KT* K, const KT* V, float* out, int
                        const QkvFuse* fuse = nullptr) {
   Context& c = tlhip::ctx();
   const int group = Hq / Hkv;
+  if (gqa_applies<KT>(group) && c.tune_attn_decode != 1)
+    return launch_gqa<D>(q, reinterpret_cast<const float*>(K), reinterpret_cast<const float*>(V), out, Hq, Hkv, ctx,
+                         kv_max, scale, dpos, partials, partials_bytes, fuse);
   const AttnPlan p = plan_attn(Hkv, group, ctx, c.cus, dpos != nullptr);
   float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
   const int S = p.S;
@@ -845,7 +1247,8 @@ int tlhip_attn_decode_static(const void* q, const void* K, const void* V, void* 
     return fail(TLHIP_EINVAL, "tlhip_attn_decode_static: operands must be 16-byte aligned");
   const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads, cx = (int)ctx_len;
   // the same launch plan as tlhip_attn_decode; its split partials must fit the fixed array
-  const AttnPlan p = plan_attn(Hkv, Hq / Hkv, cx, c.cus, false);
+  AttnPlan p = plan_attn(Hkv, Hq / Hkv, cx, c.cus, false);
+  if (!kv_bf16 && gqa_applies<float>(Hq / Hkv) && c.tune_attn_decode != 1) p.S = plan_gqa(Hkv, cx, c.cus, (int)D).S;
   const size_t need = p.S > 1 ? attn_partials_floats(Hq, p.S, (int)D) * sizeof(float) : 0;
   if (need > fixed::kBytes)
     return fail(TLHIP_EUNSUPPORTED,
@@ -942,7 +1345,8 @@ int64_t tlhip_attn_partials_bytes(int64_t n_q_heads, int64_t n_kv_heads, int64_t
       kv_max > 0x3fffffff || (D != 64 && D != 128))
     return 0;
   const AttnPlan p = plan_attn((int)n_kv_heads, (int)(n_q_heads / n_kv_heads), (int)kv_max, ctx().cus, true);
-  return (int64_t)(attn_partials_floats((int)n_q_heads, p.S, (int)D) * sizeof(float)) + 16;
+  const GqaPlan g = plan_gqa((int)n_kv_heads, (int)kv_max, ctx().cus, (int)D);   // whichever kernel serves the cache type
+  return (int64_t)(attn_partials_floats((int)n_q_heads, p.S > g.S ? p.S : g.S, (int)D) * sizeof(float)) + 16;
 }
 
 int tlhip_attn_decode_dpos(const void* q, const void* K, const void* V, void* out, int64_t n_q_heads,

@@ -473,6 +473,7 @@ int tlhip_tune_reset(void) {
   c.tune_cols_max_splits = 0;
   c.tune_prefill_valu = 0;
   c.tune_gemm_planes = 0;
+  c.tune_attn_decode = 0;
   return TLHIP_OK;
 }
 
@@ -485,6 +486,13 @@ int tlhip_tune_attn_prefill(int valu_kernel) {
   TLHIP_REQUIRE_READY();
   if (valu_kernel < 0 || valu_kernel > 4) return fail(TLHIP_EINVAL, "tlhip_tune_attn_prefill: 0 (built-in choice) .. 4");
   ctx().tune_prefill_valu = valu_kernel;
+  return 0;
+}
+
+int tlhip_tune_attn_decode(int kernel) {
+  TLHIP_REQUIRE_READY();
+  if (kernel != 0 && kernel != 1) return fail(TLHIP_EINVAL, "tlhip_tune_attn_decode: 0 (built-in choice) or 1");
+  ctx().tune_attn_decode = kernel;
   return 0;
 }
 

@@ -53,6 +53,11 @@ int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int wa
  * 4 = the f16-term kernels (two f16 terms per operand, scaled per query row and per 32-key tile).
  * Same results within fp32 summation order; for A/B timing and tests. */
 int tlhip_tune_attn_prefill(int kernel);
+/* Which kernel serves decode attention: 0 = the built-in choice (for f32 caches with 3 to 8 query
+ * heads per kv head the kernel that gives every query head a wavefront over K/V tiles staged in
+ * LDS; otherwise the key-slot kernel), 1 = the key-slot kernel for every shape. Same results
+ * within fp32 summation order; for A/B timing and tests. */
+int tlhip_tune_attn_decode(int kernel);
 /* How the prompt GEMMs over an int4 weight (M > 64) cut the f32 activations: 0 = the built-in
  * choice (two f16 terms), 3 = three bf16 terms. Same results within fp32 summation order; for A/B
  * timing and tests. */

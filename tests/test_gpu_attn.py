@@ -34,12 +34,17 @@ def test_attn_config3(lib, orc, ctx):
 
 
 @pytest.mark.parametrize("D,Hq,Hkv", [(64, 14, 2), (128, 28, 4), (128, 4, 2), (64, 6, 2),
-                                      (128, 3, 1), (64, 16, 1), (128, 5, 5)])
-@pytest.mark.parametrize("ctx", [1, 2, 63, 64, 65, 255, 256, 257, 1000, 2047])
-def test_attn_gqa_and_split_boundaries(lib, orc, D, Hq, Hkv, ctx):
+                                      (128, 3, 1), (64, 16, 1), (128, 5, 5),
+                                      (128, 32, 8), (64, 10, 2), (128, 12, 2), (64, 16, 2)])   # groups of 4, 5, 6, 8
+@pytest.mark.parametrize("ctx", [1, 2, 63, 64, 65, 127, 128, 129, 255, 256, 257, 1000, 2047])
+@pytest.mark.parametrize("kernel", ["built-in", "key-slot"])
+def test_attn_gqa_and_split_boundaries(lib, orc, D, Hq, Hkv, ctx, kernel):
     """GQA head map h/group and the split/tile boundaries (check_attn64.cpp:65-66),
-    reading a cache prefix: kv_max > ctx, rows past ctx hold garbage that must not leak."""
-    print("case attn gqa", D, Hq, Hkv, ctx, flush=True)
+    reading a cache prefix: kv_max > ctx, rows past ctx hold garbage that must not leak.
+    kernel: the library's choice (groups of 3 to 8 heads over an f32 cache take the kernel that
+    stages 64-key tiles in LDS, one wavefront per head) or the key-slot kernel forced for every shape."""
+    print("case attn gqa", D, Hq, Hkv, ctx, kernel, flush=True)
+    lib.tune_attn_decode(1 if kernel == "key-slot" else 0)
     kv_max = ctx + 37
     q = orc.normal(Hq * D, 4 + ctx).reshape(Hq, D)
     K = orc.normal(Hkv * kv_max * D, 5 + ctx).reshape(Hkv, kv_max, D)
@@ -47,7 +52,10 @@ def test_attn_gqa_and_split_boundaries(lib, orc, D, Hq, Hkv, ctx):
     K[:, ctx:, :] = 1e30
     V[:, ctx:, :] = np.nan
     scale = 1.0 / np.sqrt(float(D))
-    got = _run(lib, q, K, V, ctx, scale)
+    try:
+        got = _run(lib, q, K, V, ctx, scale)
+    finally:
+        lib.tune_attn_decode(0)
     want = orc.attn_decode(q, K, V, scale, ctx=ctx)
     assert np.all(np.isfinite(got))
     assert allclose(got, want, RTOL, ATOL), maxrel(got, want)
@@ -109,6 +117,7 @@ def test_attn_decode_device_position(lib, orc, D, Hq, Hkv, kv_max):
     V = orc.normal(Hkv * kv_max * D, 92).reshape(Hkv, kv_max, D)
     scale = 1.0 / np.sqrt(float(D))
     dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, D))
+    dhost = lib.empty((Hq, D))
     nb = lib.attn_partials_bytes(Hq, Hkv, kv_max, D)
     assert nb > 0
     part = lib.empty_bytes(nb)
@@ -123,6 +132,10 @@ def test_attn_decode_device_position(lib, orc, D, Hq, Hkv, kv_max):
         want = orc.attn_decode(q, K, V, scale, ctx=pos + 1)
         assert np.all(np.isfinite(got)), pos
         assert allclose(got, want, RTOL, ATOL), (pos, maxrel(got, want))
+        # the host-position call plans its grid for the live context, this one for the capacity:
+        # the same bits all the same (check_attn64.cpp:94-103), splits without keys add exact zeros
+        lib.attn_decode(dq, dk, dv, dhost, Hq, Hkv, pos + 1, kv_max, D, scale)
+        assert np.array_equal(got, dhost.numpy()), pos
     # too small a partials buffer is refused, not overrun
     if nb > 64:
         small = lib.empty_bytes(32)
