@@ -829,11 +829,22 @@ __global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
       *reinterpret_cast<float4*>(newv + nd0) = nv_own;
     }
   }
-  TLHIP_MARK(1);
-
   // ---- the tiles of this split ---------------------------------------------------------------------
   const int h = wave;                                        // the query head this wavefront serves (wave GRP: none)
   const int cg = lane % CH, kg = lane / CH;
+  // While the tile is on its way: every lane of a head's wavefront takes the whole query row
+  // into registers (reads of one LDS address by all lanes). The scores then read LDS for the keys
+  // only - they are bound by the LDS pipe, and the query reads were half of its traffic. (Blocks
+  // of more than eight wavefronts leave a lane fewer registers than the row needs at head size
+  // 128; they read the row from LDS as they go.)
+  constexpr bool QREG = D == 64 || NW <= 8;
+  float4 qreg[QREG ? CH : 1];
+  barrier();                                                 // the rotated query rows (and the new row) are in LDS
+  if (QREG && h < GRP) {
+#pragma unroll
+    for (int j = 0; j < CH; j++) qreg[j] = *reinterpret_cast<const float4*>(qrot + h * D + j * 4);
+  }
+  TLHIP_MARK(1);
   float m = -INFINITY, l = 0.f;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   int st = 0;
@@ -847,6 +858,7 @@ __global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
     const bool more = tn * kKeys < ctx;
     if (first) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CPW) : "memory");     // my K copies of the first tile
+      TLHIP_MARK(5);
       barrier();                                                     // ... and everyone's; query rows and the new row too
       TLHIP_MARK(2);
     }
@@ -856,21 +868,23 @@ __global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
     const bool plain = nvalid == kKeys && !with_new;
     if (h < GRP) {
       // scores: lane = key
+      // (rows start at multiples of the row size, so "row + (chunk position)" is an XOR: one
+      // instruction per read for the swizzle and the address together)
       const bool mine_new = with_new && lane == newj;
-      const char* krow = mine_new ? reinterpret_cast<const char*>(newk) : stage + lane * RB;
-      const int swz = mine_new ? 0 : (lane & (CH - 1)) << 4;
+      const uint32_t kx = mine_new ? (uint32_t)(reinterpret_cast<const char*>(newk) - smem)
+                                   : ((uint32_t)(stage - smem) + lane * RB) ^ ((lane & (CH - 1)) << 4);
       const float* qh = qrot + h * D;
       float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
 #pragma unroll
       for (int j = 0; j < CH; j += 4) {
-        const float4 k0 = *reinterpret_cast<const float4*>(krow + (((j + 0) << 4) ^ swz));
-        const float4 k1 = *reinterpret_cast<const float4*>(krow + (((j + 1) << 4) ^ swz));
-        const float4 k2 = *reinterpret_cast<const float4*>(krow + (((j + 2) << 4) ^ swz));
-        const float4 k3 = *reinterpret_cast<const float4*>(krow + (((j + 3) << 4) ^ swz));
-        const float4 q0 = *reinterpret_cast<const float4*>(qh + (j + 0) * 4);
-        const float4 q1 = *reinterpret_cast<const float4*>(qh + (j + 1) * 4);
-        const float4 q2 = *reinterpret_cast<const float4*>(qh + (j + 2) * 4);
-        const float4 q3 = *reinterpret_cast<const float4*>(qh + (j + 3) * 4);
+        const float4 k0 = *reinterpret_cast<const float4*>(smem + (kx ^ ((j + 0) << 4)));
+        const float4 k1 = *reinterpret_cast<const float4*>(smem + (kx ^ ((j + 1) << 4)));
+        const float4 k2 = *reinterpret_cast<const float4*>(smem + (kx ^ ((j + 2) << 4)));
+        const float4 k3 = *reinterpret_cast<const float4*>(smem + (kx ^ ((j + 3) << 4)));
+        const float4 q0 = QREG ? qreg[QREG ? j + 0 : 0] : *reinterpret_cast<const float4*>(qh + (j + 0) * 4);
+        const float4 q1 = QREG ? qreg[QREG ? j + 1 : 0] : *reinterpret_cast<const float4*>(qh + (j + 1) * 4);
+        const float4 q2 = QREG ? qreg[QREG ? j + 2 : 0] : *reinterpret_cast<const float4*>(qh + (j + 2) * 4);
+        const float4 q3 = QREG ? qreg[QREG ? j + 3 : 0] : *reinterpret_cast<const float4*>(qh + (j + 3) * 4);
         s0 = fmaf(q0.x, k0.x, s0); s0 = fmaf(q0.y, k0.y, s0); s0 = fmaf(q0.z, k0.z, s0); s0 = fmaf(q0.w, k0.w, s0);
         s1 = fmaf(q1.x, k1.x, s1); s1 = fmaf(q1.y, k1.y, s1); s1 = fmaf(q1.z, k1.z, s1); s1 = fmaf(q1.w, k1.w, s1);
         s2 = fmaf(q2.x, k2.x, s2); s2 = fmaf(q2.y, k2.y, s2); s2 = fmaf(q2.z, k2.z, s2); s2 = fmaf(q2.w, k2.w, s2);
@@ -899,15 +913,14 @@ __global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
       const char* vt = stage + TILE;
       const float* ph = pb + h * 64 + kg * CH;
       if (plain) {
-        const char* vb = vt + (size_t)kg * CH * RB;
-        const int c4 = cg << 4;
+        const uint32_t vx = ((uint32_t)(vt - smem) + kg * CH * RB) ^ (cg << 4);   // the group's first row, this lane's chunk
 #pragma unroll
         for (int i = 0; i < CH; i += 4) {
           const float4 p4 = *reinterpret_cast<const float4*>(ph + i);
           const float pp[4] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
           for (int u = 0; u < 4; u++) {
-            const float4 v = *reinterpret_cast<const float4*>(vb + (i + u) * RB + (c4 ^ ((i + u) << 4)));
+            const float4 v = *reinterpret_cast<const float4*>(smem + (vx ^ ((i + u) << 4)) + (i + u) * RB);
             acc.x = fmaf(pp[u], v.x, acc.x); acc.y = fmaf(pp[u], v.y, acc.y);
             acc.z = fmaf(pp[u], v.z, acc.z); acc.w = fmaf(pp[u], v.w, acc.w);
           }
