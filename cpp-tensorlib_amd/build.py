@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libtensorlib_hip.so")
-SOURCES = ["runtime.hip", "gemv.hip", "elementwise.hip", "modelops.hip", "attn.hip", "attn_prefill_mfma.hip", "attn_prefill_x3.hip", "prefill.hip", "gemm_f16t.hip", "convert.hip", "sgemm.hip"]
+SOURCES = ["runtime.hip", "gemv.hip", "elementwise.hip", "modelops.hip", "attn.hip", "attn_prefill_mfma.hip", "attn_prefill_f16.hip", "prefill.hip", "gemm_f16t.hip", "convert.hip", "sgemm.hip"]
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 on this pool.
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -499,7 +499,7 @@ class TlHip:
                                                 1 if kv_bf16 else 0, pos0))
 
     def tune_attn_prefill(self, kernel):
-        """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 3: bf16 planes, 4: f16 terms."""
+        """0 / False: built-in choice, 1 / True: VALU kernel, 2: fp32 matrix pipe, 4: f16 terms."""
         self._chk(self.c.tlhip_tune_attn_prefill(int(kernel)))
 
     def tune_attn_decode(self, kernel):

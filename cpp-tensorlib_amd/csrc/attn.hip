@@ -1178,23 +1178,23 @@ template <int D, typename KT>
 int launch_prefill_mfma(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
                         int64_t kv_max, float scale, int pos0, int token_major);
 
-// attn_prefill_x3.hip
+// attn_prefill_f16.hip
 bool prefill_x3_applies(int D, int T, int pos0);
 template <int D, typename KT>
 int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
-                      int64_t kv_max, float scale, int pos0, int token_major, bool f16_terms);
+                      int64_t kv_max, float scale, int pos0, int token_major);
 
-// Three kernels serve causal prefill attention. Deep in a context the bf16-plane
-// kernels on the matrix cores; otherwise the fp32 matrix-pipe kernel; the VALU kernel that
-// shares its code with decode attention on request. tune_prefill: 0 = that choice, 1 = VALU,
-// 2 = fp32 matrix pipe, 3 = bf16 planes, 4 = f16 terms (what the choice takes deep in a context).
+// Three kernels serve causal prefill attention. Deep in a context the f16-term kernels on the
+// matrix cores; otherwise the fp32 matrix-pipe kernel; the VALU kernel that shares its code with
+// decode attention on request. tune_prefill: 0 = that choice, 1 = VALU, 2 = fp32 matrix pipe,
+// 4 = f16 terms (what the choice takes deep in a context).
 template <int D, typename KT>
 static int launch_prefill(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv,
                           int T, int64_t kv_max, float scale, int pos0, int token_major) {
   Context& c = tlhip::ctx();
   const int mode = c.tune_prefill_valu;
-  if (mode >= 3 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
-    const int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major, mode != 3);
+  if (mode == 4 || (mode == 0 && prefill_x3_applies(D, T, pos0))) {
+    const int rc = launch_prefill_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major);
     if (rc < 0) return rc;
     if (rc == 0) TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_PREFILL);
     if (mode != 0) return fail(TLHIP_ENOMEM, "tlhip_attn_prefill: no scratch for the key/value planes");

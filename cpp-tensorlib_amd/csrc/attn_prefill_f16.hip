@@ -1,50 +1,39 @@
-// Causal prefill attention on the bf16 matrix cores with fp32-level products
+// Causal prefill attention on the 16-bit matrix cores with fp32-level products
 // (tlhip_attn_prefill deep in a context, cuda.h:1165-1201).
 //
 //   out[h, p, :] = softmax_k( scale * q[h, p, :] . K[kv(h), k, :] ) . V[kv(h), k, :],  k <= pos0 + p
 //
-// The fp32 matrix instructions share the vector ALU's multipliers: a kernel built on them
-// runs its softmax and its products one after the other. v_mfma_f32_16x16x32_bf16 runs on the
-// matrix cores proper, 16 times faster and beside the vector ALU, but multiplies bf16. Every
-// f32 operand x is therefore cut into three bf16 planes x = x1 + x2 + x3 (each the
-// round-to-nearest bf16 of what the planes before it left; |x - x1 - x2 - x3| <= 2^-26 |x|),
-// and a product a.b is formed from the six plane pairs whose weight is at least 2^-16:
-//   a1b1 + (a1b2 + a2b1) + (a1b3 + a2b2 + a3b1)       dropped: a2b3, a3b2, a3b3, < 2^-23 |ab|
-// smallest first, accumulated in fp32 inside the MFMA. A cache that already holds bf16 needs one
-// plane for K and V and three products. Scores and outputs then differ from an fp32 loop by
-// what a different summation order would give.
-//
-// The f16 form (what the library picks; the bf16 planes remain selectable) does the same with TWO
-// f16 terms per operand, each rounded to nearest, and the three term pairs a1b1 + (a1b2 + a2b1);
-// a2b2 <= 2^-24 |ab| is dropped - three MFMAs per product instead of six, two instead of three
-// over a bf16 cache. f16 has 11 significant bits but a narrow exponent, so the operand is first
-// multiplied by a power of two that brings its block's largest magnitude into [2^14, 2^15): one
-// exponent per query row, one each for K and V per 32-key tile (kept beside the planes). Two
-// terms then carry 23 bits of a value whose magnitude is within 2^14 of its block's largest and
-// an absolute 2^-39 of that largest below. The Q and K exponents leave through the score scale;
-// P enters as p * 2^14 and the output accumulators move from one tile's V exponent to the next in
-// the multiplication that applies the softmax correction. It runs on v_mfma_f32_32x32x16_f16.
+// The fp32 matrix instructions share the vector ALU's multipliers: a kernel built on them runs
+// its softmax and its products one after the other. v_mfma_f32_32x32x16_f16 runs on the matrix
+// cores proper, 16 times faster and beside the vector ALU, but multiplies f16. Every f32 operand
+// is therefore cut into TWO f16 terms, each rounded to nearest, and a product a.b is formed from
+// the three term pairs that hold a first term, a1b1 + (a1b2 + a2b1), smallest first, accumulated
+// in fp32 inside the MFMA; a2b2 <= 2^-24 |ab|, an fp32 rounding, is dropped. (A cache that already
+// holds bf16 needs one term for K and V and two products.) f16 has 11 significant bits but a
+// narrow exponent, so an operand is first multiplied by a power of two that brings its block's
+// largest magnitude into [2^14, 2^15): one exponent per query row, one each for K and V per
+// 32-key tile (kept beside the terms). Two terms then carry 23 bits of a value whose magnitude is
+// within 2^14 of its block's largest and an absolute 2^-39 of that largest below. The Q and K
+// exponents leave through the score scale; P enters as p * 2^14 and the output accumulators move
+// from one tile's V exponent to the next in the multiplication that applies the softmax
+// correction. Scores and outputs then differ from an fp32 loop by what a different summation
+// order would give.
 //
 // Three kernels per call:
-//  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into planes (or terms),
-//     written as the exact register image of the MFMA operands, one 32-key tile after the other
-//     (bf16 form; the f16 form's images are described at the kernel):
-//       K image [plane][k-step][16-key half 0..1][lane][8]  = K[32t + 16h + l%16][32s + 8(l/16) + j]
-//       V image [plane][16-column tile][lane][8]            = V[32t + tile_key(l/16, j)][16d + l%16]
-//     so that the attention kernel copies a tile to LDS verbatim and every operand is one
-//     conflict-free 16-byte LDS read per lane. Keys at and past pos0 + T are written as zeros.
-//  2. attn_x3_kernel (bf16 planes) / attn_w32_kernel (f16 terms): a block serves ONE kv head and
-//     up to 7 wavefronts of 32 query rows each that all read the same K/V tiles: with
-//     grouped-query attention the query heads of the group (32 positions each), else consecutive
-//     runs of positions. The 32-key tiles of the block's causal range are dealt round-robin over
-//     `S` blocks (key splits); a tile is staged into LDS once per block (double buffered, one
-//     barrier per tile) by an eighth wavefront and read by every computing wavefront. Both
-//     products are formed transposed (S^T = K . Q^T, O^T = V^T . P^T): a lane's scores,
-//     probabilities and output columns all belong to one query row, so the softmax needs no
-//     exchange through LDS and P goes from the score registers - cut into planes - straight back
-//     into the matrix core. Per tile and wavefront (head size 128, f32 cache): 96 + 96 MFMAs of
-//     16x16x32 in the bf16 form, 24 + 24 of 32x32x16 (the work of 48 + 48) in the f16 form, and
-//     an online-softmax update on 16 scores per lane.
+//  1. kv_planes_kernel cuts the cache rows [0, pos0 + T) of every kv head into terms, written as
+//     the exact register image of the MFMA operands, one 32-key tile after the other (layouts at
+//     the kernel), so that the attention kernel copies a tile to LDS verbatim and every operand is
+//     one conflict-free 16-byte LDS read per lane. Keys at and past pos0 + T are written as zeros.
+//  2. attn_w32_kernel: a block serves ONE kv head and up to 7 wavefronts of 32 query rows each
+//     that all read the same K/V tiles: with grouped-query attention the query heads of the group
+//     (32 positions each), else consecutive runs of positions. The 32-key tiles of the block's
+//     causal range are dealt round-robin over `S` blocks (key splits); a tile is staged into LDS
+//     once per block (double buffered, one barrier per tile) by an eighth wavefront and read by
+//     every computing wavefront. Both products are formed transposed (S^T = K . Q^T,
+//     O^T = V^T . P^T): a lane's scores, probabilities and output columns all belong to one query
+//     row, so the softmax needs no exchange through LDS and P goes from the score registers - cut
+//     into terms - straight back into the matrix core. Per tile and wavefront (head size 128, f32
+//     cache): 24 + 24 MFMAs of 32x32x16 and an online-softmax update on 16 scores per lane.
 //     S == 1 writes the normalised rows; S > 1 leaves (max, sum, accumulator) per split and
 //  3. attn_x3_merge_kernel combines them in split order.
 #include "common.hpp"
@@ -53,19 +42,12 @@ namespace tlhip {
 
 namespace x3 {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a 16-byte unit in registers
 
 constexpr int kTile = 32;                    // keys per tile
-// 16-byte units of one K plane of a tile (D/32 k-steps x 2 key halves x 64 lanes) and of one V
-// plane (D/16 column tiles x 64 lanes): 4 D either way. Head sizes 64 and 128 are built.
-// The scores of a 32-key tile leave the two 16x16 MFMAs with lane (g = l/16, c = l%16) holding,
-// for query row c, the keys 16h + 4g + r (h = 0, 1; r = 0..3). Those 8 values, in the order
-// j = 4h + r, are the lane's 8 elements of the P.V reduction index, so the V image lists the keys
-// in the same order: element j of lane group g is key 16 (j / 4) + 4 g + j % 4 of the tile.
-__host__ __device__ constexpr int tile_key(int g, int j) { return 16 * (j >> 2) + 4 * g + (j & 3); }
-
+// 16-byte units of one K term of a tile (D/16 dim steps x 64 lanes) and of one V term (D/32 column
+// tiles x 2 key steps x 64 lanes): 4 D either way. Head sizes 64 and 128 are built.
 // The 32x32x16 MFMA leaves the scores of a 32-key tile with lane (g = l/32, c = l%32) holding, for
 // query row c, the keys 8a + 4g + b (a, b = 0..3) in accumulator register 4a + b. Registers
 // 8u .. 8u + 7 are the lane's 8 elements of key step u of P.V, so element j of lane half g in
@@ -76,41 +58,9 @@ template <int D> struct Img { static constexpr int kKUnits = (D / 32) * 2 * 64, 
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
-// Two floats -> three packed bf16 pairs (element 0 in the low half); hi + mid + lo reproduces x
-// to 2^-26 relative. The conversions are the hardware's packed round-to-nearest-even
-// (v_cvt_pk_bf16_f32); both remainders are exact in f32.
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// An operand, first multiplied by a power of two that brings it into the f16 range, is cut into
+// TWO f16 terms, both rounded to nearest (2^-24 relative while the second term is a normal f16).
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16x2(f32x2 v) {
-  union { bf16x2 b; uint32_t u; } t;
-  t.b = __builtin_convertvector(v, bf16x2);
-  return t.u;
-}
-__device__ __forceinline__ f32x2 widen_bf16x2(uint32_t u) {
-  return f32x2{__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u)};
-}
-__device__ __forceinline__ void split3x2(f32x2 x, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
-  hi = pack_bf16x2(x);
-  const f32x2 r1 = x - widen_bf16x2(hi);
-  mid = pack_bf16x2(r1);
-  const f32x2 r2 = r1 - widen_bf16x2(mid);
-  lo = pack_bf16x2(r2);
-}
-
-// 8 floats -> 8 bf16 per plane, packed as the MFMA wants them (element j in bits [16j, 16j+16) of the 128)
-__device__ __forceinline__ void split3x8(const float (&x)[8], uint4& p1, uint4& p2, uint4& p3) {
-  uint32_t a[4], b[4], c[4];
-#pragma unroll
-  for (int j = 0; j < 4; j++) split3x2(f32x2{x[2 * j], x[2 * j + 1]}, a[j], b[j], c[j]);
-  p1 = make_uint4(a[0], a[1], a[2], a[3]);
-  p2 = make_uint4(b[0], b[1], b[2], b[3]);
-  p3 = make_uint4(c[0], c[1], c[2], c[3]);
-}
-
-// The f16 form: an operand, first multiplied by a power of two that brings it
-// into the f16 range, is cut into TWO f16 terms, both rounded to nearest (2^-24 relative while
-// the second term is a normal f16), and a product is formed from the three term pairs that hold
-// a first term - three MFMAs where the bf16 planes need six.
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // what is left after the first term, 0 where that is inf - inf (an infinite operand): a NaN second
@@ -151,25 +101,21 @@ __device__ __forceinline__ int f16_exponent(uint32_t maxbits) {
   return maxbits == 0 ? 0 : max(-100, min(100, 14 - ((int)(maxbits >> 23) - 127)));
 }
 __device__ __forceinline__ float pow2i(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // e in [-126, 127]
-__device__ __forceinline__ f32x4 mma16(const u32x4 a, const u32x4 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
 __device__ __forceinline__ u32x4 as_u32x4(const uint4& u) { return u32x4{u.x, u.y, u.z, u.w}; }
 
 __device__ __forceinline__ float cache_elem(const float* p) { return *p; }
 __device__ __forceinline__ float cache_elem(const uint16_t* p) { return bf16_bits_to_f32(*p); }
 
-// ---- 1. planes ---------------------------------------------------------------------------
-// grid = (tiles, Hkv), block = 256. NP planes: bf16 form 3 for an f32 cache, 1 for a bf16 cache;
-// f16 form (F) 2 and 1.
+// ---- 1. terms ----------------------------------------------------------------------------
+// grid = (tiles, Hkv), block = 256. NP terms per element: 2 for an f32 cache, 1 for a bf16 cache.
 // planes: per (kv head, tile) a K image of NP * kKUnits uint4, then a V image of NP * kVUnits uint4.
-// F: K and V of a tile are scaled by 2^ek and 2^ev, one exponent each per tile (from the tile's
+// K and V of a tile are scaled by 2^ek and 2^ev, one exponent each per tile (from the tile's
 // largest magnitude), left in texp[(kv head * tiles + tile) * 2 + {0, 1}]; the attention kernel
 // folds them into its score scale and its running output scale.
-// and the operand images are those of the 32x32x16 MFMA:
+// The operand images are those of the 32x32x16 MFMA:
 //   K image [term][16-dim step s][lane][8]        = K[32t + l%32][16s + 8(l/32) + j]
 //   V image [term][32-column tile][key step u][lane][8] = V[32t + wide_key(u, l/32, j)][32d + l%32]
-template <typename KT, int NP, int D, bool F>
+template <typename KT, int NP, int D>
 __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K, const KT* __restrict__ V,
                                                         uint4* __restrict__ planes, int* __restrict__ texp,
                                                         int64_t kv_stride, int kend, int ntiles) {
@@ -187,9 +133,9 @@ __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K
   for (int i = 0; i < kPer; i++) {
     const int u = threadIdx.x + 256 * i;
     if (u < kKUnits) {
-      const int l = u & 63, half = (u >> 6) & 1, ks = u >> 7;
-      const int key = F ? t * kTile + (l & 31) : t * kTile + 16 * half + (l & 15);
-      const int dim = F ? 16 * (u >> 6) + 8 * (l >> 5) : 32 * ks + 8 * (l >> 4);
+      const int l = u & 63;
+      const int key = t * kTile + (l & 31);
+      const int dim = 16 * (u >> 6) + 8 * (l >> 5);
       const bool live = key < kend;
       const KT* src = Kh + (size_t)min(key, kend - 1) * kD + dim;
 #pragma unroll
@@ -197,52 +143,42 @@ __global__ __launch_bounds__(256) void kv_planes_kernel(const KT* __restrict__ K
 #pragma unroll
       for (int j = 0; j < 8; j++) mxk = max(mxk, __float_as_uint(x[i][j]) & 0x7fffffffu);
     } else {
-      const int v = u - kKUnits, l = v & 63, dt = v >> 6;
-      const int dim = F ? 32 * (v >> 7) + (l & 31) : 16 * dt + (l & 15);
+      const int v = u - kKUnits, l = v & 63;
+      const int dim = 32 * (v >> 7) + (l & 31);
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        const int key = t * kTile + (F ? wide_key((v >> 6) & 1, l >> 5, j) : tile_key(l >> 4, j));
+        const int key = t * kTile + wide_key((v >> 6) & 1, l >> 5, j);
         x[i][j] = key < kend ? cache_elem(Vh + (size_t)key * kD + dim) : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < 8; j++) mxv = max(mxv, __float_as_uint(x[i][j]) & 0x7fffffffu);
     }
   }
-  float sk = 1.0f, sv = 1.0f;
-  if (F) {
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-      mxk = max(mxk, (uint32_t)__shfl_xor((int)mxk, d));
-      mxv = max(mxv, (uint32_t)__shfl_xor((int)mxv, d));
-    }
-    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = mxk; red[1][threadIdx.x >> 6] = mxv; }
-    __syncthreads();
-    mxk = max(max(red[0][0], red[0][1]), max(red[0][2], red[0][3]));
-    mxv = max(max(red[1][0], red[1][1]), max(red[1][2], red[1][3]));
-    const int ek = f16_exponent(mxk), ev = f16_exponent(mxv);
-    if (threadIdx.x == 0) {
-      texp[((size_t)kvh * ntiles + t) * 2] = ek;
-      texp[((size_t)kvh * ntiles + t) * 2 + 1] = ev;
-    }
-    sk = pow2i(ek);
-    sv = pow2i(ev);
+  for (int d = 32; d >= 1; d >>= 1) {
+    mxk = max(mxk, (uint32_t)__shfl_xor((int)mxk, d));
+    mxv = max(mxv, (uint32_t)__shfl_xor((int)mxv, d));
   }
+  if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = mxk; red[1][threadIdx.x >> 6] = mxv; }
+  __syncthreads();
+  mxk = max(max(red[0][0], red[0][1]), max(red[0][2], red[0][3]));
+  mxv = max(max(red[1][0], red[1][1]), max(red[1][2], red[1][3]));
+  const int ek = f16_exponent(mxk), ev = f16_exponent(mxv);
+  if (threadIdx.x == 0) {
+    texp[((size_t)kvh * ntiles + t) * 2] = ek;
+    texp[((size_t)kvh * ntiles + t) * 2 + 1] = ev;
+  }
+  const float sk = pow2i(ek), sv = pow2i(ev);
 #pragma unroll
   for (int i = 0; i < kPer; i++) {
     const int u = threadIdx.x + 256 * i;
     const bool isk = u < kKUnits;
     uint4* dst = isk ? img + u : img + NP * kKUnits + (u - kKUnits);
     const int plane_stride = isk ? kKUnits : kVUnits;
-    uint4 p1, p2, p3;
-    if (F) {
-      split2x8_f16(x[i], isk ? sk : sv, p1, p2);
-      dst[0] = p1;
-      if (NP == 2) dst[plane_stride] = p2;
-    } else {
-      split3x8(x[i], p1, p2, p3);
-      dst[0] = p1;
-      if (NP == 3) { dst[plane_stride] = p2; dst[2 * plane_stride] = p3; }
-    }
+    uint4 p1, p2;
+    split2x8_f16(x[i], isk ? sk : sv, p1, p2);
+    dst[0] = p1;
+    if (NP == 2) dst[plane_stride] = p2;
   }
 }
 
@@ -276,290 +212,8 @@ constexpr int kRT = 2;          // 16-row tiles per computing wavefront
 constexpr int kF16Weight = 1;   // f16 form: term pairs (a, b) with a + b <= this; 1 leaves out lo x lo, <= 2^-24 |a b|
 constexpr int kCompute = 7;     // computing wavefronts per block
 
-template <int NP, int D>
-__global__ __launch_bounds__(512, 1) void attn_x3_kernel(const float* __restrict__ q, const uint4* __restrict__ planes,
-                                                          float* __restrict__ out, float* __restrict__ part_o,
-                                                          float* __restrict__ part_ml, float scale, const Geometry g) {
-  constexpr int QP = 3;                                       // planes of Q and of P
-  constexpr int kW = 2;                                       // products keep the plane pairs (a, b) with a + b <= this
-  constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
-  constexpr int kKS = D / 32, kDT = D / 16;                   // k-steps of Q.K^T, column tiles of P.V
-  constexpr int kKImg = NP * kKUnits, kVImg = NP * kVUnits;   // 16-byte units of a tile's K and V images
-  constexpr int kImg = kKImg + kVImg;
-  constexpr int kCopyK = kKImg / 64, kCopyV = kVImg / 64;     // units a lane of the copying wavefront moves per tile
-  extern __shared__ u32x4 lds4[];                             // K images [2], V images [2]
-  u32x4* kbuf = lds4;
-  u32x4* vbuf = lds4 + 2 * kKImg;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l15 = lane & 15, lq = lane >> 4;
-  const int kvh = blockIdx.x / g.head_chunks, hc = blockIdx.x - kvh * g.head_chunks;
-  const int nblk = gridDim.y;
-  const int pblock = nblk - 1 - (int)blockIdx.y;          // longest causal ranges first
-  const int split = blockIdx.z;
-  // causal range of the block: tiles up to its last row's limit, dealt round-robin over the splits
-  const int blk_last = min((pblock + 1) * g.np * (16 * kRT), g.T) - 1;
-  const int nkt_blk = (g.pos0 + blk_last) / kTile + 1;
-  const int n = nkt_blk > split ? (nkt_blk - split + g.S - 1) / g.S : 0;   // this block's tiles: split, split + S, ...
-  const auto tile_of = [&](int i) { return split + i * g.S; };
-  const u32x4* img0 = reinterpret_cast<const u32x4*>(planes) + (size_t)kvh * g.ntiles * kImg;
-
-  if (wave == kCompute) {
-    // ---- the copying wavefront (branch-free: tiles past the range are clamped, parked, never read) ----
-    // Interval i needs K of tile i and V of tile i-1. What the interval AFTER it needs - K of
-    // tile i+1, V of tile i - is in registers when interval i begins (requested one interval
-    // earlier) and is parked first thing: those buffers were last read in interval i-1, which
-    // every wavefront has left. The requests for the interval after that go out right behind
-    // and have a whole interval to arrive.
-    u32x4 stk[kCopyK], stv[kCopyV];
-    const auto request = [&](int ik, int iv) {
-      const u32x4* srck = img0 + (size_t)min(tile_of(ik), g.ntiles - 1) * kImg;
-      const u32x4* srcv = img0 + (size_t)min(tile_of(iv), g.ntiles - 1) * kImg + kKImg;
-#pragma unroll
-      for (int c = 0; c < kCopyK; c++) stk[c] = srck[lane + 64 * c];
-#pragma unroll
-      for (int c = 0; c < kCopyV; c++) stv[c] = srcv[lane + 64 * c];
-    };
-    request(0, 0);
-#pragma unroll
-    for (int c = 0; c < kCopyK; c++) kbuf[lane + 64 * c] = stk[c];
-    request(1, 0);
-    __syncthreads();
-    for (int i = 0; i <= n; i++) {
-#pragma unroll
-      for (int c = 0; c < kCopyK; c++) kbuf[((i + 1) & 1) * kKImg + lane + 64 * c] = stk[c];
-#pragma unroll
-      for (int c = 0; c < kCopyV; c++) vbuf[(i & 1) * kVImg + lane + 64 * c] = stv[c];
-      request(i + 2, i + 1);
-      __syncthreads();
-    }
-    return;
-  }
-
-  const int hh = wave % g.nh, pt = wave / g.nh;
-  const int hloc = hc * g.nh + hh;                        // head inside the group
-  const int p_first = (pblock * g.np + pt) * (16 * kRT);  // this wavefront's first query position
-  const bool active = pt < g.np && hloc < g.group && p_first < g.T;
-  const bool late = wave >= 4;                            // softmax before the matrix phase
-  const int h = kvh * g.group + min(hloc, g.group - 1);
-  const int my_last_key = g.pos0 + min(p_first + 16 * kRT - 1, g.T - 1);
-  const int kend = g.pos0 + g.T;
-
-  // Both products are formed transposed, S^T = K . Q^T and O^T = V^T . P^T, so that a lane's
-  // results all belong to ONE query row (row l%16 of each of the wavefront's two 16-row tiles):
-  // its 8 scores of a tile are 8 keys of that row, they stay in the lane through the softmax,
-  // become - cut into planes - the lane's B operand of P.V as they are, and the output
-  // accumulators they feed hold 4 columns of the same row. No exchange through LDS, one
-  // running maximum and one running sum per lane and tile; a row's keys are spread over the 4
-  // lanes c, c+16, c+32, c+48, which meet in two register swaps.
-
-  // ---- the wavefront's query rows as operand planes: row l%16 of each tile, dims 32s + 8(l/16) + j ----
-  uint4 qa[kRT][QP][kKS];
-#pragma unroll
-  for (int rt = 0; rt < kRT; rt++) {
-    const float* qrow = q + ((size_t)h * g.T + min(p_first + 16 * rt + l15, g.T - 1)) * kD;
-    float x[kKS][8];
-#pragma unroll
-    for (int ks = 0; ks < kKS; ks++) {
-      const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq);
-      const float4 b = *reinterpret_cast<const float4*>(qrow + 32 * ks + 8 * lq + 4);
-      x[ks][0] = a.x; x[ks][1] = a.y; x[ks][2] = a.z; x[ks][3] = a.w;
-      x[ks][4] = b.x; x[ks][5] = b.y; x[ks][6] = b.z; x[ks][7] = b.w;
-      if (scale < 0.f) {   // the sign of the scale goes into Q: the softmax below multiplies by |scale|
-#pragma unroll
-        for (int j = 0; j < 8; j++) x[ks][j] = -x[ks][j];
-      }
-      split3x8(x[ks], qa[rt][0][ks], qa[rt][1][ks], qa[rt][2][ks]);
-    }
-  }
-
-  f32x4 o[kRT][kDT];                  // O^T: columns 16 dt + 4(l/16) + r of row l%16
-  float mrow[kRT], lrow[kRT];         // row l%16: running maximum; this lane's share of the running sum
-  f32x4 s[kRT][2];                    // S^T of the tile whose softmax is pending: keys 16 h + 4(l/16) + r
-  uint4 pa3[kRT][QP];                 // P planes of the tile whose P.V is pending
-#pragma unroll
-  for (int rt = 0; rt < kRT; rt++) {
-#pragma unroll
-    for (int dt = 0; dt < kDT; dt++) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    mrow[rt] = -INFINITY;
-    lrow[rt] = 0.f;
-    s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int pl = 0; pl < QP; pl++) pa3[rt][pl] = make_uint4(0, 0, 0, 0);
-  }
-
-  // the vector phase of tile number i: masks, running maximum and sum, rescale of the output
-  // accumulators, P cut into planes. Scores are taken to base-2 units (score * |scale| * log2 e) in
-  // the same fused multiply-add that subtracts the running maximum; mrow is kept in those units.
-  const float ascale = fabsf(scale) * 1.44269504088896341f;
-  const auto softmax_tile = [&](int i) {
-    const int kt = tile_of(i);
-    // only a tile that reaches past the first row's causal limit (or the chunk's last key) needs masks
-    const bool masked = (kt + 1) * kTile - 1 > min(g.pos0 + p_first, kend - 1);   // (uniform for the wavefront)
-#pragma unroll
-    for (int rt = 0; rt < kRT; rt++) {
-      float v[8], mx;
-      if (masked) {
-        const int limit = min(g.pos0 + p_first + 16 * rt + l15, kend - 1);   // last key the row sees
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = kt * kTile + tile_key(lq, j) <= limit ? s[rt][j >> 2][j & 3] * ascale : -INFINITY;
-        mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = s[rt][j >> 2][j & 3];
-        mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7]))) * ascale;   // ascale >= 0
-      }
-      LanePair e = swap16(mx, mx);
-      mx = fmaxf(e.first, e.second);
-      e = swap32(mx, mx);
-      mx = fmaxf(e.first, e.second);               // over the row's 32 keys
-      const float mnew = fmaxf(mrow[rt], mx);
-      const float mref = mnew == -INFINITY ? 0.f : mnew;
-      const float corr = __builtin_amdgcn_exp2f(mrow[rt] - mref);
-      float p[8];
-      if (masked) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) p[j] = __builtin_amdgcn_exp2f(v[j] - mref);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) p[j] = __builtin_amdgcn_exp2f(fmaf(v[j], ascale, -mref));
-      }
-      const float psum = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-      lrow[rt] = fmaf(lrow[rt], corr, psum);
-      mrow[rt] = mnew;
-      // deep in a context the running maximum of a row seldom moves: skip the 64 multiplications
-      // when no row of the tile needs them
-      if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
-#pragma unroll
-        for (int dt = 0; dt < kDT; dt++) {
-          o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
-        }
-      }
-      split3x8(p, pa3[rt][0], pa3[rt][1], pa3[rt][2]);
-    }
-  };
-  const auto mine = [&](int i) { return active && i >= 0 && i < n && tile_of(i) * kTile <= my_last_key; };
-
-#ifdef TLHIP_TRACE
-  unsigned long long ph[4] = {0, 0, 0, 0}, tc;
-  TLHIP_MARK(0);
-#define TLHIP_X3_T0() tc = __builtin_readcyclecounter()
-#define TLHIP_X3_T(k) do { const unsigned long long n_ = __builtin_readcyclecounter(); ph[k] += n_ - tc; tc = n_; } while (0)
-#else
-#define TLHIP_X3_T0()
-#define TLHIP_X3_T(k)
-#endif
-  __syncthreads();   // K of tile 0 is in LDS
-  TLHIP_X3_T0();
-  for (int i = 0; i <= n; i++) {   // interval n drains: P.V of the last tile (and, for the late half, its softmax)
-    if (late && mine(i - 1)) softmax_tile(i - 1);
-    TLHIP_X3_T(0);
-    // ---- matrix phase; plane pairs (a, b) with a + b <= 2, smallest products first ----
-    if (mine(i - 1)) {   // O^T[D x 32 rows] += V^T[D x 32 keys] . P^T[32 keys x 32 rows] of tile i-1, 16-column tiles
-      const u32x4* vimg = vbuf + ((i - 1) & 1) * kVImg;
-      // two column tiles at a time: four independent accumulators take turns, so that an MFMA
-      // never waits for the result of the one issued just before it
-#pragma unroll
-      for (int dt = 0; dt < kDT; dt += 2) {
-        u32x4 vb[2][NP];
-#pragma unroll
-        for (int d2 = 0; d2 < 2; d2++)
-#pragma unroll
-          for (int p = 0; p < NP; p++) vb[d2][p] = vimg[p * kVUnits + (dt + d2) * 64 + lane];
-#pragma unroll
-        for (int w = kW; w >= 0; w--)
-#pragma unroll
-          for (int pb = NP - 1; pb >= 0; pb--) {
-            const int pa = w - pb;
-            if (pa >= 0 && pa < QP) {
-#pragma unroll
-              for (int d2 = 0; d2 < 2; d2++)
-#pragma unroll
-                for (int rt = 0; rt < kRT; rt++)
-                  o[rt][dt + d2] = mma16(vb[d2][pb], as_u32x4(pa3[rt][pa]), o[rt][dt + d2]);
-            }
-          }
-      }
-    }
-    if (mine(i)) {       // S^T[32 keys x 32 rows] of tile i as 16 x 16 tiles
-      const u32x4* kimg = kbuf + (i & 1) * kKImg;
-#pragma unroll
-      for (int rt = 0; rt < kRT; rt++) s[rt][0] = s[rt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < kKS; ks++) {
-        u32x4 kb[2][NP];
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++)
-#pragma unroll
-          for (int p = 0; p < NP; p++) kb[hf][p] = kimg[p * kKUnits + (ks * 2 + hf) * 64 + lane];
-#pragma unroll
-        for (int w = kW; w >= 0; w--)
-#pragma unroll
-          for (int pb = NP - 1; pb >= 0; pb--) {
-            const int pa = w - pb;
-            if (pa >= 0 && pa < QP) {
-#pragma unroll
-              for (int hf = 0; hf < 2; hf++)
-#pragma unroll
-                for (int rt = 0; rt < kRT; rt++)
-                  s[rt][hf] = mma16(kb[hf][pb], as_u32x4(qa[rt][pa][ks]), s[rt][hf]);
-            }
-          }
-      }
-    }
-    TLHIP_X3_T(1);
-    if (!late && mine(i)) softmax_tile(i);
-    TLHIP_X3_T(0);
-    __syncthreads();
-    TLHIP_X3_T(2);
-  }
-#ifdef TLHIP_TRACE
-  {
-    const unsigned b = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-    if (lane == 0 && b < kTraceBlocks) {
-      unsigned long long* gt = &g_trace[(b * kTraceWaves + wave) * kTraceSlots];
-      gt[1] = ph[0]; gt[2] = ph[1]; gt[3] = ph[2]; gt[4] = n + 1;
-    }
-  }
-  TLHIP_MARK(6);
-#endif
-#undef TLHIP_X3_T0
-#undef TLHIP_X3_T
-
-  // ---- rows complete for this split: the row's sum over its 4 lanes, store 4 columns per lane and tile ----
-  if (!active) return;
-#pragma unroll
-  for (int rt = 0; rt < kRT; rt++) {
-    const int p = p_first + 16 * rt + l15;
-    LanePair e = swap16(lrow[rt], lrow[rt]);
-    float lsum = e.first + e.second;
-    e = swap32(lsum, lsum);
-    lsum = e.first + e.second;
-    if (p >= g.T) continue;
-    if (g.S == 1) {
-      const float inv = 1.0f / lsum;
-      float* op = out + (size_t)h * g.o_head + (size_t)p * g.o_row + 4 * lq;
-#pragma unroll
-      for (int dt = 0; dt < kDT; dt++)
-        *reinterpret_cast<float4*>(op + 16 * dt) =
-            make_float4(o[rt][dt][0] * inv, o[rt][dt][1] * inv, o[rt][dt][2] * inv, o[rt][dt][3] * inv);
-    } else {
-      const size_t row = (size_t)h * g.T + p, rows = (size_t)g.rows;   // row number in [Hq * T)
-      float* po = part_o + ((size_t)split * rows + row) * kD + 4 * lq;
-#pragma unroll
-      for (int dt = 0; dt < kDT; dt++)
-        *reinterpret_cast<float4*>(po + 16 * dt) = make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
-      if (lq == 0) {
-        part_ml[((size_t)split * rows + row) * 2] = mrow[rt];
-        part_ml[((size_t)split * rows + row) * 2 + 1] = lsum;
-      }
-    }
-  }
-}
-
-// ---- 2b. attention on 32x32x16 MFMAs (f16 terms) ------------------------------------------
-// The same block, loop and phases as attn_x3_kernel<.., true>; a computing wavefront's 32 query
-// rows are ONE 32-column tile of both transposed products:
+// ---- 2. attention on 32x32x16 MFMAs (f16 terms) -------------------------------------------
+// A computing wavefront's 32 query rows are ONE 32-column tile of both transposed products:
 //   S^T[32 keys x 32 rows] = K[32 keys x D] . Q^T      D/16 steps, A = K image, B = the row's Q terms
 //   O^T[D x 32 rows]      += V^T[D x 32 keys] . P^T    D/32 column tiles x 2 key steps
 // Lane (g = l/32, c = l%32) holds, for query row c, 16 scores of a tile (keys 8a + 4g + b) and,
@@ -598,7 +252,7 @@ __global__ __launch_bounds__(512, 1) void attn_w32_kernel(const float* __restric
   const u32x4* img0 = reinterpret_cast<const u32x4*>(planes) + (size_t)kvh * g.ntiles * kImg;
   const int* texp0 = texp + (size_t)kvh * g.ntiles * 2;
 
-  if (wave == kCompute) {   // the copying wavefront, as in attn_x3_kernel
+  if (wave == kCompute) {   // the copying wavefront
     u32x4 stk[kCopyK], stv[kCopyV];
     const auto request = [&](int ik, int iv) {
       const u32x4* srck = img0 + (size_t)min(tile_of(ik), g.ntiles - 1) * kImg;
@@ -903,11 +557,11 @@ bool prefill_x3_applies(int D, int T, int pos0) {
 
 // Launches the three kernels. Returns 0 when launched, a negative status on failure, 1 when the
 // scratch for the planes could not be had (the caller then uses the fp32 matrix-pipe kernel).
-template <int D, typename KT, bool F>   // F: two f16 terms on 32x32x16 tiles; else three bf16 planes on 16x16x32 tiles
+template <int D, typename KT>
 static int launch_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
                      int64_t kv_max, float scale, int pos0, int token_major) {
   using namespace x3;
-  constexpr int NP = sizeof(KT) == 4 ? (F ? 2 : 3) : 1;
+  constexpr int NP = sizeof(KT) == 4 ? 2 : 1;
   constexpr int kD = D, kKUnits = Img<D>::kKUnits, kVUnits = Img<D>::kVUnits;
   Context& c = ctx();
   Geometry g{};
@@ -945,18 +599,13 @@ static int launch_x3(const float* q, const KT* K, const KT* V, float* out, int H
   int* texp = reinterpret_cast<int*>(buf + plane_bytes + part_o_bytes + part_ml_bytes);
   const size_t lds = 2 * kImgBytes;
   if (lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_prefill: not enough LDS");
-  const void* fn = nullptr;
-  if constexpr (F) fn = reinterpret_cast<const void*>(attn_w32_kernel<NP, D>);
-  else fn = reinterpret_cast<const void*>(attn_x3_kernel<NP, D>);
+  const void* fn = reinterpret_cast<const void*>(attn_w32_kernel<NP, D>);
   hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  hipLaunchKernelGGL((kv_planes_kernel<KT, NP, D, F>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes, texp,
+  hipLaunchKernelGGL((kv_planes_kernel<KT, NP, D>), dim3(g.ntiles, Hkv), dim3(256), 0, c.stream, K, V, planes, texp,
                      kv_max * (int64_t)kD, kend, g.ntiles);
   const dim3 grid(Hkv * g.head_chunks, pblocks, S);
-  if constexpr (F)
-    hipLaunchKernelGGL((attn_w32_kernel<NP, D>), grid, dim3(512), lds, c.stream, q, planes, texp, out, part_o, part_ml, scale, g);
-  else
-    hipLaunchKernelGGL((attn_x3_kernel<NP, D>), grid, dim3(512), lds, c.stream, q, planes, out, part_o, part_ml, scale, g);
+  hipLaunchKernelGGL((attn_w32_kernel<NP, D>), grid, dim3(512), lds, c.stream, q, planes, texp, out, part_o, part_ml, scale, g);
   if (S > 1) {
     const int64_t threads = (int64_t)rows * (kD / 4);
     hipLaunchKernelGGL(attn_x3_merge_kernel<D>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c.stream, part_o,
@@ -965,17 +614,15 @@ static int launch_x3(const float* q, const KT* K, const KT* V, float* out, int H
   return 0;
 }
 
-// f16_terms: two f16 terms per operand on 32x32x16 tiles; else three bf16 planes on 16x16x32 tiles
 template <int D, typename KT>
 int launch_prefill_x3(const float* q, const KT* K, const KT* V, float* out, int Hq, int Hkv, int T,
-                      int64_t kv_max, float scale, int pos0, int token_major, bool f16_terms) {
-  return f16_terms ? launch_x3<D, KT, true>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major)
-                   : launch_x3<D, KT, false>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major);
+                      int64_t kv_max, float scale, int pos0, int token_major) {
+  return launch_x3<D, KT>(q, K, V, out, Hq, Hkv, T, kv_max, scale, pos0, token_major);
 }
 
-template int launch_prefill_x3<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int, bool);
-template int launch_prefill_x3<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int, bool);
-template int launch_prefill_x3<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int, bool);
-template int launch_prefill_x3<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int, bool);
+template int launch_prefill_x3<128, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<128, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<64, float>(const float*, const float*, const float*, float*, int, int, int, int64_t, float, int, int);
+template int launch_prefill_x3<64, uint16_t>(const float*, const uint16_t*, const uint16_t*, float*, int, int, int, int64_t, float, int, int);
 
 }  // namespace tlhip

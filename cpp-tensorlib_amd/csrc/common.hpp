@@ -44,7 +44,7 @@ struct Context {
   int tune_cols_max_splits = 0;   // [K,N] GEMV K-split bound (tlhip_tune_gemv_cols), 0 = automatic
   int tune_gemm_planes = 0;       // tlhip_tune_gemm_planes: 0 = automatic, 3 = int4 prompt GEMMs on three bf16 planes of A
   int tune_attn_decode = 0;       // tlhip_tune_attn_decode: 0 = automatic, 1 = the key-slot kernel for every shape
-  int tune_prefill_valu = 0;      // tlhip_tune_attn_prefill: 0 = automatic, 1 = VALU kernel, 2 = fp32 matrix pipe, 3 = bf16 planes, 4 = f16 terms
+  int tune_prefill_valu = 0;      // tlhip_tune_attn_prefill: 0 = automatic, 1 = VALU kernel, 2 = fp32 matrix pipe, 4 = f16 terms
 };
 
 Context& ctx();

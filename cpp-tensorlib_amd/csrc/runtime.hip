@@ -484,7 +484,8 @@ int tlhip_tune_gemv_cols(int max_k_splits) {
 
 int tlhip_tune_attn_prefill(int valu_kernel) {
   TLHIP_REQUIRE_READY();
-  if (valu_kernel < 0 || valu_kernel > 4) return fail(TLHIP_EINVAL, "tlhip_tune_attn_prefill: 0 (built-in choice) .. 4");
+  if (valu_kernel < 0 || valu_kernel > 4 || valu_kernel == 3)
+    return fail(TLHIP_EINVAL, "tlhip_tune_attn_prefill: 0 (built-in choice), 1, 2 or 4");
   ctx().tune_prefill_valu = valu_kernel;
   return 0;
 }

@@ -49,8 +49,8 @@ int tlhip_tune_gemv_q4(int rows_per_wave, int k_waves, int blocks_per_cu, int wa
 /* Which kernel serves tlhip_attn_prefill: 0 = the built-in choice (the f16-term kernels on the
  * matrix cores from about 640 keys on at head size 128 and 1024 at head size 64, else the fp32
  * matrix pipe), 1 = the VALU kernel that shares its code with decode attention,
- * 2 = the fp32 matrix-pipe kernel, 3 = the bf16-plane kernels (three bf16 planes per operand),
- * 4 = the f16-term kernels (two f16 terms per operand, scaled per query row and per 32-key tile).
+ * 2 = the fp32 matrix-pipe kernel, 4 = the f16-term kernels (two f16 terms per operand, scaled per
+ * query row and per 32-key tile); 3 is not in use.
  * Same results within fp32 summation order; for A/B timing and tests. */
 int tlhip_tune_attn_prefill(int kernel);
 /* Which kernel serves decode attention: 0 = the built-in choice (for f32 caches with 3 to 8 query

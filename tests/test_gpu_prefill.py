@@ -347,13 +347,13 @@ def test_gemm_bf16_nt_declines(lib):
         b.free()
 
 
-KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "planes": 3, "f16terms": 4}
+KERNELS = {"auto": 0, "valu": 1, "fp32pipe": 2, "f16terms": 4}
 
 
 def _prefill(lib, q, K, V, scale, pos0, kv_bf16=False, kernel="auto"):
     """kernel (tlhip_tune_attn_prefill): the library's own choice, the VALU kernel, the fp32
-    matrix-pipe kernel, the bf16-plane kernels on the matrix cores, or their f16 form (two f16 terms
-    per operand; what the library's own choice takes deep in a context)."""
+    matrix-pipe kernel, or the f16-term kernels on the matrix cores (two f16 terms per operand; what
+    the library's own choice takes deep in a context)."""
     Hq, T, D = q.shape
     Hkv, kv_max, _ = K.shape
     dq, dk, dv, do = lib.to_device(q), lib.to_device(K), lib.to_device(V), lib.empty((Hq, T, D))
@@ -409,22 +409,21 @@ def _attn_f64(q, K, V, scale, pos0):
     return out
 
 
-@pytest.mark.parametrize("kernel", ["fp32pipe", "planes", "f16terms"])
+@pytest.mark.parametrize("kernel", ["fp32pipe", "f16terms"])
 @pytest.mark.parametrize("case", ["one_dominant_key", "equal_scores", "large_values", "tiny_values", "cancelling_values",
                                   "value_scale_by_tile"])
 def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
-    """Rows chosen against the bf16-plane products (three planes per operand, six plane pairs per
-    product: what is dropped is below 2^-23 of |a b|), the f16-term products (two terms per operand
-    scaled per query row and per 32-key tile, three term pairs) and the online softmax:
+    """Rows chosen against the f16-term products (two terms per operand, scaled per query row and
+    per 32-key tile, three term pairs: what is dropped is below 2^-24 of |a b|) and the online softmax:
       one_dominant_key    one key's score exceeds the others by ~40: the softmax is one-hot to
                           fp32 and the output must be that key's value row;
       equal_scores        every key of a row scores the same to 1e-6: the output is a plain mean,
                           where an error in the scores is not damped by a peaked softmax;
       large_values        |q|, |k|, |v| around 2^10 (scores around 1e5 before the maximum is
                           taken): plane residuals of large numbers;
-      tiny_values         values around 2^-40: the third plane is near the bottom of bf16's range;
+      tiny_values         values around 2^-40: far below f16's range before the per-tile scaling;
       cancelling_values   V alternates +-(1000 + small) so that the output is a small difference
-                          of large terms (tests the value planes and the fp32 accumulation);
+                          of large terms (tests the value terms and the fp32 accumulation);
       value_scale_by_tile every run of 32 keys has its V rows scaled by its own power of two between
                           2^-24 and 2^24 and its K rows by one between 2^-2 and 2^2 (the f16 form
                           scales K and V per 32-key tile and carries the output accumulators from
@@ -473,7 +472,7 @@ def test_attn_prefill_adversarial_rows(lib, orc, case, kernel):
     err, err_ref = np.abs(got - exact), np.abs(want - exact)
     # An fp32 score carries up to 2^-24 sum_i |q_i k_i| scale of rounding per product, and an error
     # d in a score is a relative error d in its probability: the bound grows with the largest
-    # sum_i |q_i k_i| scale of a row (its own dot products are what the planes must reproduce).
+    # sum_i |q_i k_i| scale of a row (its own dot products are what the terms must reproduce).
     absdot = np.einsum("htd,kd->htk", np.abs(q).astype(np.float64), np.abs(K[0]).astype(np.float64)).max(axis=2) * float(scale)
     bound = 2.0 ** -22 * (4.0 + absdot)[:, :, None] * mag + 1e-37
     print("   max err / bound: kernel %.3f, CPU oracle %.3f" % ((err / bound).max(), (err_ref / bound).max()), flush=True)
