@@ -109,6 +109,10 @@ SIGNATURES = {
     "tlhip_attn_decode_qkv": (cint, [P, P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, cint, P, i64]),
     "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
     "tlhip_token_advance": (cint, [P, P, P, i64]),
+    "tlhip_attn_parts_splits": (cint, [i64, i64, i64, i64, cint]),
+    "tlhip_attn_decode_qkv_parts": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, P, i64, P]),
+    "tlhip_gemv_q4_attn": (cint, [P, i64, i64, i64, P, P, P, i64, i64, i64]),
+    "tlhip_gemv_bf16_row_attn": (cint, [P, i64, i64, i64, P, P, i64, i64]),
     "tlhip_gemv_q4_swiglu": (cint, [P, P, P, P, i64, i64, i64]),
     "tlhip_gemv_bf16_row_swiglu": (cint, [P, P, P, i64, i64]),
     "tlhip_gemv_q4_rmsnorm": (cint, [P, P, P, P, P, P, P, i64, i64, i64, f32]),
@@ -431,6 +435,26 @@ class TlHip:
         self._chk(self.c.tlhip_attn_decode_qkv(
             qkv.ptr, opt(bq), opt(bk), opt(bv), Kc.ptr, Vc.ptr, out.ptr, Hq, Hkv, pos, opt(d_pos), kv_max,
             D, scale, table.ptr, int(kv_bf16), opt(partials), partials.nbytes if partials is not None else 0))
+
+    def attn_parts_splits(self, Hq, Hkv, plan_ctx, D, kv_bf16=False):
+        """Splits tlhip_attn_decode_qkv_parts would leave for a grid planned for plan_ctx keys; 0: shape not served."""
+        return int(self.c.tlhip_attn_parts_splits(Hq, Hkv, plan_ctx, D, int(kv_bf16)))
+
+    def attn_decode_qkv_parts(self, qkv, bq, bk, bv, Kc, Vc, Hq, Hkv, pos, kv_max, D, scale, table, partials,
+                              d_pos=None):
+        """The fused decode attention with the split merge left to gemv_*_attn; returns the number of splits."""
+        opt = lambda b: b.ptr if b is not None else None
+        n = C.c_int(0)
+        self._chk(self.c.tlhip_attn_decode_qkv_parts(
+            qkv.ptr, opt(bq), opt(bk), opt(bv), Kc.ptr, Vc.ptr, Hq, Hkv, pos, opt(d_pos), kv_max, D, scale,
+            table.ptr, partials.ptr, partials.nbytes, C.byref(n)))
+        return n.value
+
+    def gemv_q4_attn(self, parts, n_parts, heads, D, wq, y, N, K, group=32):
+        self._chk(self.c.tlhip_gemv_q4_attn(parts.ptr, n_parts, heads, D, wq.ptr, wq.ptr + N * K // 2, y.ptr, N, K, group))
+
+    def gemv_bf16_row_attn(self, parts, n_parts, heads, D, W, y, N, K):
+        self._chk(self.c.tlhip_gemv_bf16_row_attn(parts.ptr, n_parts, heads, D, W.ptr, y.ptr, N, K))
 
     # element types of the load-time converters
     T_F32, T_F16, T_BF16 = 0, 1, 2

@@ -962,7 +962,7 @@ __global__ __launch_bounds__(64 * (GRP + 1)) void attn_gqa_kernel(
     acc.x = across(acc.x); acc.y = across(acc.y); acc.z = across(acc.z); acc.w = across(acc.w);
     if (lane < CH) {
       const size_t head = (size_t)kvh * GRP + h;
-      if (S == 1) {
+      if (S == 1 && out) {
         // (divisions, as in the combine kernel: a grid with one split and one with more give the same bits)
         *reinterpret_cast<float4*>(out + head * D + lane * 4) = make_float4(acc.x / l, acc.y / l, acc.z / l, acc.w / l);
       } else {
@@ -1060,12 +1060,13 @@ template <int D>
 static int launch_gqa(const float* q, const float* K, const float* V, float* out, int Hq, int Hkv, int ctx,
                       int64_t kv_max, float scale, const uint32_t* dpos, float* partials, size_t partials_bytes,
                       const QkvFuse* fuse) {
+  // out == nullptr: the partials are the result (also of a single split); whoever reads them merges
   Context& c = tlhip::ctx();
   const int group = Hq / Hkv;
   const GqaPlan p = plan_gqa(Hkv, ctx, c.cus, D);
   const int S = p.S;
   float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
-  if (S > 1) {
+  if (S > 1 || !out) {
     const size_t hs = (size_t)Hq * S;
     const size_t need = attn_partials_floats(Hq, S, D) * sizeof(float);
     float* base;
@@ -1107,7 +1108,7 @@ static int launch_gqa(const float* q, const float* K, const float* V, float* out
   }
 #undef TLHIP_GQA
   if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(LDS)");
-  if (S > 1)
+  if (S > 1 && out)
     hipLaunchKernelGGL(attn_combine_kernel, dim3(Hq), dim3(1024), (size_t)(S + 1024) * sizeof(float),
                        c.stream, pm, pl, pacc, out, S, D);
   TLHIP_CHECK_LAUNCH(TLHIP_C_ATTN_DECODE);
@@ -1432,6 +1433,62 @@ int tlhip_attn_decode_qkv(const void* qkv, const void* bq, const void* bk, const
                   : launch_attn<64, float>(pq, pk, pv, po, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz);
   }
   if (rc == TLHIP_OK) {
+    ctx().census[TLHIP_C_ROPE]++;
+    ctx().census[TLHIP_C_KV_APPEND]++;
+  }
+  return rc;
+}
+
+// Splits whose partials a GEMV's staging pass merges in the summation order of the merge kernel:
+// one per column group of that kernel (1024 / D), 16 at most.
+static int parts_limit(int64_t D) { return D == 64 ? 16 : 8; }
+
+int tlhip_attn_parts_splits(int64_t n_q_heads, int64_t n_kv_heads, int64_t plan_ctx, int64_t D, int kv_bf16) {
+  if (!ctx().ready || kv_bf16 || (D != 64 && D != 128) || n_kv_heads <= 0 || n_kv_heads > 65535 || n_q_heads <= 0 ||
+      n_q_heads % n_kv_heads != 0 || plan_ctx <= 0 || plan_ctx > 0x3fffffff)
+    return 0;
+  if (!gqa_applies<float>((int)(n_q_heads / n_kv_heads)) || ctx().tune_attn_decode == 1) return 0;
+  if ((n_q_heads & 1) != 0) return 0;   // the accumulators follow 2 * heads * splits floats and are read 16 bytes at a time
+  const int S = plan_gqa((int)n_kv_heads, (int)plan_ctx, ctx().cus, (int)D).S;
+  return S <= parts_limit(D) ? S : 0;
+}
+
+int tlhip_attn_decode_qkv_parts(const void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                                void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t pos,
+                                const void* d_pos, int64_t kv_max, int64_t D, float scale,
+                                const void* table, void* partials, int64_t partials_bytes, int* n_parts) {
+  TLHIP_REQUIRE_READY();
+  if (!qkv || !Kc || !Vc || !table || !partials || !n_parts)
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv_parts: null pointer");
+  if (D != 64 && D != 128) return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv_parts: head_dim must be 64 or 128");
+  if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv_parts: Hq must be a positive multiple of Hkv");
+  if (kv_max <= 0 || kv_max > 0x3fffffff || n_kv_heads > 65535 || kv_max * D > ((int64_t)1 << 40))
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_attn_decode_qkv_parts: shape too large");
+  if (!d_pos && (pos < 0 || pos >= kv_max))
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv_parts: need 0 <= pos < kv_max");
+  if (!aligned16(qkv) || !aligned16(Kc) || !aligned16(Vc) || !aligned16(table) || (bq && !aligned16(bq)) ||
+      (bk && !aligned16(bk)) || (bv && !aligned16(bv)) || !aligned16(partials))
+    return fail(TLHIP_EINVAL, "tlhip_attn_decode_qkv_parts: operands must be 16-byte aligned");
+  const int cx = d_pos ? (int)kv_max : (int)pos + 1;   // the grid is planned for this many keys
+  const int S = tlhip_attn_parts_splits(n_q_heads, n_kv_heads, cx, D, 0);
+  if (S <= 0)
+    return fail(TLHIP_EUNSUPPORTED,
+                "tlhip_attn_decode_qkv_parts: f32 cache, 3 to 8 query heads per kv head, an even head count and a "
+                "context of at most %d splits (ask tlhip_attn_parts_splits)", parts_limit(D));
+  const QkvFuse fz{static_cast<const float*>(bq), static_cast<const float*>(bk),
+                   static_cast<const float*>(bv), static_cast<const float2*>(table), Kc, Vc, kv_max};
+  const float* pq = static_cast<const float*>(qkv);
+  const uint32_t* dp = static_cast<const uint32_t*>(d_pos);
+  const size_t pb = partials_bytes > 0 ? (size_t)partials_bytes : 0;
+  const int Hq = (int)n_q_heads, Hkv = (int)n_kv_heads;
+  const float* pk = static_cast<const float*>(Kc);
+  const float* pv = static_cast<const float*>(Vc);
+  float* pp = static_cast<float*>(partials);
+  const int rc = D == 128 ? launch_gqa<128>(pq, pk, pv, nullptr, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz)
+                          : launch_gqa<64>(pq, pk, pv, nullptr, Hq, Hkv, cx, kv_max, scale, dp, pp, pb, &fz);
+  if (rc == TLHIP_OK) {
+    *n_parts = S;
     ctx().census[TLHIP_C_ROPE]++;
     ctx().census[TLHIP_C_KV_APPEND]++;
   }

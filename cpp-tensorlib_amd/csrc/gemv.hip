@@ -92,6 +92,8 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   float* xsum = reinterpret_cast<float*>(smem4 + (size_t)chunks * J * XS);  // [chunks*LPR], int4 only
   float* red = xsum + (Fmt::kScaled ? chunks * LPR : 0);   // [nw * QN * 8] K-split partials
   float* nsum = red + nw * QN * 8;                          // [16] per-wavefront sums of squares (norm producer)
+  float* fw = nsum + 16;                                    // [heads * 8] split weights (attention-merge producer)
+  float* fL = fw + (PRO == kAttnMerge ? pro.heads * kMergeMax : 0);   // [heads] the heads' sums
 
   const int kw = wave % KW;          // which K split this wavefront takes
   const int wn = wave / KW;          // which row group of the block tile
@@ -114,13 +116,28 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   // threads), 8 per thread in the norm form, whose vector is the hidden size (registers)
   constexpr int PL = PRO == kRmsnorm ? 2 : 5;
   float4 px[PL], pa[PL], pn[PL];
+  // attention-merge producer: this thread's first float4 of the first kPre splits' accumulators, and
+  // the (head, split) pair whose maximum and sum it weighs
+  constexpr int kPre = 8;
+  float4 pre[kPre];
+  float pre_m = -INFINITY, pre_l = 0.f;
+  if constexpr (PRO == kAttnMerge) {
+    const int S = pro.S, D4 = pro.D >> 2;
+    const int i = min(tid, n4 - 1), h = i / D4;
+    const float4* pacc = reinterpret_cast<const float4*>(x + 2 * pro.heads * S) + (size_t)h * S * D4 + (i - h * D4);
+#pragma unroll
+    for (int sp = 0; sp < kPre; sp++)
+      if (sp < S) pre[sp] = pacc[(size_t)sp * D4];
+    const int hh = tid / kMergeMax, sp = tid % kMergeMax;
+    if (hh < pro.heads && sp < S) { pre_m = x[hh * S + sp]; pre_l = x[pro.heads * S + hh * S + sp]; }
+  }
   {
     const float4* aux4 = PRO == kSwiglu ? x4 + n4 : (d4 ? d4 : x4);   // up half, or delta (x when none: ignored)
 #pragma unroll
     for (int k = 0; k < PL; k++) {
       const int i = min(tid + k * (int)blockDim.x, n4 - 1);
-      px[k] = x4[i];
-      if (PRO != kPlain) pa[k] = aux4[i];
+      if (PRO != kAttnMerge) px[k] = x4[i];
+      if (PRO != kPlain && PRO != kAttnMerge) pa[k] = aux4[i];
       if (PRO == kRmsnorm) pn[k] = reinterpret_cast<const float4*>(pro.norm_w)[i];
     }
   }
@@ -143,6 +160,35 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
   load_item(frag[0], 0);
   TLHIP_MARK(1);
 
+  if constexpr (PRO == kAttnMerge) {
+    // The splits' weights e^(m_s - M) and each head's sum, once per block into LDS: sixteen adjacent
+    // lanes hold the (up to) sixteen splits of a head. Sums in the order of attn_combine_kernel's
+    // wavefront sum over its first sixteen lanes: partners 8, 4, 2 and 1 lanes away in turn.
+    const int S = pro.S, hs = pro.heads * S;
+    const int nl = (pro.heads * kMergeMax + 63) & ~63;
+    for (int e = tid; e < nl; e += blockDim.x) {
+      const int h = e / kMergeMax, sp = e % kMergeMax;
+      const bool live = h < pro.heads && sp < S;
+      const float m = e == tid ? pre_m : (live ? x[h * S + sp] : -INFINITY);
+      const float l = e == tid ? pre_l : (live ? x[hs + h * S + sp] : 0.f);
+      float M = fmaxf(m, __shfl_xor(m, 8, kWave));
+      M = fmaxf(M, __shfl_xor(M, 4, kWave));
+      M = fmaxf(M, __shfl_xor(M, 2, kWave));
+      M = fmaxf(M, __shfl_xor(M, 1, kWave));
+      const float w = live ? __expf(m - M) : 0.f;
+      float t = mul_rn(l, w);   // (a product left to the compiler could fuse with the first sum)
+      t = add_rn(t, __shfl_xor(t, 8, kWave));
+      t += __shfl_xor(t, 4, kWave);
+      t += __shfl_xor(t, 2, kWave);
+      t += __shfl_xor(t, 1, kWave);
+      if (h < pro.heads) {
+        fw[e] = w;
+        if (sp == 0) fL[h] = t;
+      }
+    }
+    __syncthreads();
+  }
+
   {  // stage x (K = upr*E floats) into the interleaved layout, one pass:
      // thread i owns float4 i; the J threads of a unit are adjacent lanes, so the
      // unit's sum(x) is a J-lane shuffle reduction (J is 8 or 2, both divide 64).
@@ -150,6 +196,23 @@ __global__ __launch_bounds__(R >= 8 ? 512 : 1024) void gemv_rows_kernel(
     // float4 number k of this thread before the norm: x (+ delta), or swiglu(gate, up);
     // nv receives its norm weights. The first PL come from the registers requested above.
     const auto raw = [&](int k, int i, float4& nv) -> float4 {
+      if constexpr (PRO == kAttnMerge) {
+        const int D4 = pro.D >> 2, h = i / D4, d4i = i - h * D4, S = pro.S;
+        const float4* pacc = reinterpret_cast<const float4*>(x + 2 * pro.heads * S) + (size_t)h * S * D4 + d4i;
+        const float* fh = fw + h * kMergeMax;
+        // split 0's product, then the others' added one by one: the merge kernel's order
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        const auto add = [&](float f, const float4 a, bool first) {
+          const float4 p = make_float4(mul_rn(f, a.x), mul_rn(f, a.y), mul_rn(f, a.z), mul_rn(f, a.w));
+          v = first ? p : make_float4(add_rn(v.x, p.x), add_rn(v.y, p.y), add_rn(v.z, p.z), add_rn(v.w, p.w));
+        };
+#pragma unroll
+        for (int sp = 0; sp < kPre; sp++)
+          if (sp < S) add(fh[sp], k == 0 ? pre[sp] : pacc[(size_t)sp * D4], sp == 0);
+        for (int sp = kPre; sp < S; sp++) add(fh[sp], pacc[(size_t)sp * D4], false);
+        const float L = fL[h];
+        return make_float4(v.x / L, v.y / L, v.z / L, v.w / L);
+      }
       float4 v, aux;
       bool have = false;
 #pragma unroll
@@ -568,7 +631,7 @@ static auto pick_rows_fn(int R) -> void (*)(const float*, const uint4*, const fl
 template <typename Fmt, int PRO = kPlain, int EPI = kStore>
 static int launch_rows(const float* x, const void* W, const float* scales, float* y, int64_t N,
                        int64_t K, int census_id, const RowTune tn = RowTune{0, 0, 0, 0, 0},
-                       const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
+                       const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f, 0, 0, 0}) {
   Context& c = ctx();
   const int upr = (int)(K / Fmt::E);
   if (upr >= (1 << 24)) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large");
@@ -588,6 +651,7 @@ static int launch_rows(const float* x, const void* W, const float* scales, float
       if (cfg.nw / cfg.KW >= 2 && cfg.nw > 4) two.nw = cfg.nw / 2;   // keeps the rows of a block tile
       cfg = pick_rows_cfg(n, upr, Fmt::E, c.cus, c.lds_per_cu, two);
     }
+    if (PRO == kAttnMerge) cfg.lds += (size_t)pro.heads * (kMergeMax + 1) * sizeof(float);
     if (cfg.lds > (size_t)c.lds_per_cu) return fail(TLHIP_EUNSUPPORTED, "gemv: K too large for the LDS-staged kernel");
     const int rows_per_tile = (cfg.nw / cfg.KW) * (64 / cfg.lpr) * cfg.R;
     const int ntiles = (int)((n + rows_per_tile - 1) / rows_per_tile);
@@ -644,7 +708,7 @@ static RowTune q4_tune(const Context& c) {
 // int4, group 32, through the row kernel.
 template <int PRO, int EPI>
 static int launch_q4(const float* x, const void* W, const float* scales, float* y, int64_t N, int64_t K,
-                     const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f}) {
+                     const Producer pro = Producer{nullptr, nullptr, nullptr, 0.f, 0, 0, 0}) {
   return launch_rows<FmtQ4, PRO, EPI>(x, W, scales, y, N, K, TLHIP_C_GEMV_Q4, q4_tune(ctx()), pro);
 }
 
@@ -694,6 +758,45 @@ int tlhip_gemv_bf16_row(const void* a, const void* W, void* y, int64_t n, int64_
     return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row: K too large for the LDS-staged kernel");
   return launch_rows<FmtBf16>(static_cast<const float*>(a), W, nullptr, static_cast<float*>(y), n, k,
                               TLHIP_C_GEMV_BF16_ROW);
+}
+
+static int check_attn_merge(const void* parts, int64_t n_parts, int64_t heads, int64_t D, int64_t K, const char* who) {
+  if (!parts || !aligned16(parts)) return fail(TLHIP_EINVAL, "%s: partials pointer null or not 16-byte aligned", who);
+  if (heads <= 0 || heads > 4096 || (D != 64 && D != 128) || heads * D != K)
+    return fail(TLHIP_EINVAL, "%s: K must be heads x head_dim, head_dim 64 or 128", who);
+  // as many splits as the merge kernel sums one after the other: one per column group of its 1024 threads
+  const int64_t most = D == 64 ? kMergeMax : kMergeMax / 2;
+  if (n_parts < 1 || n_parts > most) return fail(TLHIP_EUNSUPPORTED, "%s: 1 to %d split partials", who, (int)most);
+  if (((2 * heads * n_parts) % 4) != 0) return fail(TLHIP_EUNSUPPORTED, "%s: heads x splits must be even", who);
+  return 0;
+}
+
+int tlhip_gemv_q4_attn(const void* parts, int64_t n_parts, int64_t heads, int64_t head_dim, const void* qw,
+                       const void* scales, void* y, int64_t N, int64_t K, int64_t group) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(parts, qw, y, N, K, "tlhip_gemv_q4_attn")) return rc;
+  if (int rc = check_attn_merge(parts, n_parts, heads, head_dim, K, "tlhip_gemv_q4_attn")) return rc;
+  if (!scales || group != 32 || !aligned16(qw)) return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_q4_attn: group 32, aligned weights");
+  const size_t xbytes = (size_t)((K / 32 + 63) / 64) * 66 * 32 * 4;
+  if (xbytes + 2048 + (size_t)heads * 68 > (size_t)ctx().lds_per_cu)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_q4_attn: K too large for the LDS-staged kernel");
+  Producer pro{nullptr, nullptr, nullptr, 0.f, (int)n_parts, (int)heads, (int)head_dim};
+  return launch_q4<kAttnMerge, kStore>(static_cast<const float*>(parts), qw, static_cast<const float*>(scales),
+                                       static_cast<float*>(y), N, K, pro);
+}
+
+int tlhip_gemv_bf16_row_attn(const void* parts, int64_t n_parts, int64_t heads, int64_t head_dim, const void* W,
+                             void* y, int64_t n, int64_t k) {
+  TLHIP_REQUIRE_READY();
+  if (int rc = check_gemv_args(parts, W, y, n, k, "tlhip_gemv_bf16_row_attn")) return rc;
+  if (int rc = check_attn_merge(parts, n_parts, heads, head_dim, k, "tlhip_gemv_bf16_row_attn")) return rc;
+  if (!aligned16(W)) return fail(TLHIP_EINVAL, "tlhip_gemv_bf16_row_attn: weight pointer not 16-byte aligned");
+  const size_t xbytes = (size_t)((k / 8 + 63) / 64) * 72 * 8 * 4;
+  if (xbytes + 2048 + (size_t)heads * 68 > (size_t)ctx().lds_per_cu)
+    return fail(TLHIP_EUNSUPPORTED, "tlhip_gemv_bf16_row_attn: K too large for the LDS-staged kernel");
+  Producer pro{nullptr, nullptr, nullptr, 0.f, (int)n_parts, (int)heads, (int)head_dim};
+  return launch_rows<FmtBf16, kAttnMerge>(static_cast<const float*>(parts), W, nullptr, static_cast<float*>(y), n, k,
+                                          TLHIP_C_GEMV_BF16_ROW, RowTune{0, 0, 0, 0, 0}, pro);
 }
 
 int tlhip_gemv_f32(const void* a, const void* B, void* y, int64_t n, int64_t k) {

@@ -138,13 +138,19 @@ __device__ __forceinline__ float wave_sum_rows(float (&a)[R], int lane) {
 //   kRmsnorm: s = in (+ delta); x = (s * 1/sqrt(mean(s*s) + eps)) * norm_w   (array.h:2429-2433);
 //             block 0 also writes s to xout (the residual stream), which therefore
 //             must not alias in or delta: other blocks still read them.
+//   kAttnMerge: x is the decode attention's output, still in the split partials the attention
+//             kernel left (per head and split: running maximum m, sum l, accumulator acc[D]):
+//             x[h*D + d] = sum_s e^(m_s - M) acc_s[d] / sum_s e^(m_s - M) l_s, at most 16 splits,
+//             in the summation order of the stand-alone merge kernel (same bits). The merge's
+//             launch goes; what it read (a few KB per head) every block now reads from L2.
 // How a block leaves its results (EPI):
 //   kStore:  y[row] = dot.
 //   kGateUp: W is [gate rows | up rows] (N/2 each); a lane group owns R/2 gate rows and the
 //            matching up rows, and writes y[i] = (g*sigmoid(g))*u for i < N/2 - the gated
 //            activation in the GEMV that produces it, once per element, instead of in every
 //            block of the GEMV that consumes it.
-enum { kPlain = 0, kSwiglu = 1, kRmsnorm = 2 };
+enum { kPlain = 0, kSwiglu = 1, kRmsnorm = 2, kAttnMerge = 3 };
+constexpr int kMergeMax = 16;  // splits the kAttnMerge producer takes (its lanes per head)
 enum { kStore = 0, kGateUp = 1 };
 __device__ __forceinline__ float gated(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 struct Producer {
@@ -152,6 +158,8 @@ struct Producer {
   const float* norm_w;
   float* xout;
   float eps;
+  // kAttnMerge: x points at the partials [heads*S] m | [heads*S] l | [heads*S][D] acc
+  int S = 0, heads = 0, D = 0;
 };
 
 }  // namespace tlhip

@@ -167,6 +167,13 @@ struct api {
                                 void*, int64_t, int64_t, int64_t, float) = nullptr;
   int (*gemv_bf16_row_rmsnorm_gateup)(const void*, const void*, const void*, void*, const void*, void*,
                                       int64_t, int64_t, float) = nullptr;
+  int (*attn_parts_splits)(int64_t, int64_t, int64_t, int64_t, int) = nullptr;
+  int (*attn_decode_qkv_parts)(const void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
+                              int64_t, const void*, int64_t, int64_t, float, const void*, void*, int64_t,
+                              int*) = nullptr;
+  int (*gemv_q4_attn)(const void*, int64_t, int64_t, int64_t, const void*, const void*, void*, int64_t, int64_t,
+                      int64_t) = nullptr;
+  int (*gemv_bf16_row_attn)(const void*, int64_t, int64_t, int64_t, const void*, void*, int64_t, int64_t) = nullptr;
   int (*warm_fork)(const void* const*, const int64_t*, int, int, int) = nullptr;
   int (*warm_join)() = nullptr;
   int (*event_create)(void**) = nullptr;
@@ -343,7 +350,11 @@ struct context {
               bind(f.gemv_q4_rmsnorm, "tlhip_gemv_q4_rmsnorm") &&
               bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm") &&
               bind(f.gemv_q4_rmsnorm_gateup, "tlhip_gemv_q4_rmsnorm_gateup") &&
-              bind(f.gemv_bf16_row_rmsnorm_gateup, "tlhip_gemv_bf16_row_rmsnorm_gateup");
+              bind(f.gemv_bf16_row_rmsnorm_gateup, "tlhip_gemv_bf16_row_rmsnorm_gateup") &&
+              bind(f.attn_parts_splits, "tlhip_attn_parts_splits") &&
+              bind(f.attn_decode_qkv_parts, "tlhip_attn_decode_qkv_parts") &&
+              bind(f.gemv_q4_attn, "tlhip_gemv_q4_attn") &&
+              bind(f.gemv_bf16_row_attn, "tlhip_gemv_bf16_row_attn");
     if (!ok) return;
     bind(f.warm_fork, "tlhip_warm_fork") && bind(f.warm_join, "tlhip_warm_join");   // optional
     why.clear();
@@ -1097,6 +1108,31 @@ inline bool attn_decode_qkv(void* qkv, void* bq, void* bk, void* bv, void* Kc, v
                                               partials_bytes));
 }
 
+// attn_decode_qkv with the split merge left to the o-projection (gemv_*_attn): writes the cache row
+// and `partials` (n_parts splits, also when that is 1), no `out`. attn_parts_splits says whether a
+// shape is served (0: it is not) for a grid planned for plan_ctx keys.
+inline int attn_parts_splits(int64_t n_q_heads, int64_t n_kv_heads, int64_t plan_ctx, int64_t D, bool kv_bf16 = false) {
+  auto& c = context::get();
+  return c.ready ? c.f.attn_parts_splits(n_q_heads, n_kv_heads, plan_ctx, D, kv_bf16 ? 1 : 0) : 0;
+}
+inline bool attn_decode_qkv_parts(void* qkv, void* bq, void* bk, void* bv, void* Kc, void* Vc, int64_t n_q_heads,
+                                  int64_t n_kv_heads, int64_t pos, void* d_pos, int64_t kv_max, int64_t D,
+                                  float scale, void* table, void* partials, int64_t partials_bytes, int* n_parts) {
+  launch L;
+  if (!L.ok || (D != 128 && D != 64) || !table || !partials || !n_parts) return false;
+  if (n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0) return false;
+  if (!d_pos && (pos < 0 || pos >= kv_max)) return false;
+  L.reads(qkv);
+  if (bq) L.reads(bq);
+  if (bk) L.reads(bk);
+  if (bv) L.reads(bv);
+  if (d_pos) L.reads(d_pos);
+  L.reads(table);
+  L.writes(Kc, Vc, partials);
+  return L.sent(L.lib.attn_decode_qkv_parts(qkv, bq, bk, bv, Kc, Vc, n_q_heads, n_kv_heads, pos, d_pos, kv_max, D,
+                                            scale, table, partials, partials_bytes, n_parts));
+}
+
 // ---- load-time weight conversion on the device ---------------------------------------------
 // The file's element types as the converters number them.
 enum class elem : int { f32 = 0, f16 = 1, bf16 = 2 };
@@ -1178,6 +1214,23 @@ inline bool gemv_bf16_row_swiglu(void* gu, void* B, void* y, int64_t n, int64_t 
   L.reads(gu, B);
   L.writes(y);
   return L.sent(L.lib.gemv_bf16_row_swiglu(gu, B, y, n, k));
+}
+// y = W . (the decode attention's output merged from the n_parts split partials of attn_decode_qkv_parts)
+inline bool gemv_q4_attn(void* parts, int64_t n_parts, int64_t heads, int64_t head_dim, void* qw, void* scales,
+                         void* y, int64_t N, int64_t K, int64_t group) {
+  launch L;
+  if (!L.ok || group != 32 || (K % 32) != 0 || heads * head_dim != K) return false;
+  L.reads(parts, qw, scales);
+  L.writes(y);
+  return L.sent(L.lib.gemv_q4_attn(parts, n_parts, heads, head_dim, qw, scales, y, N, K, group));
+}
+inline bool gemv_bf16_row_attn(void* parts, int64_t n_parts, int64_t heads, int64_t head_dim, void* B, void* y,
+                               int64_t n, int64_t k) {
+  launch L;
+  if (!L.ok || (k % 8) != 0 || heads * head_dim != k) return false;
+  L.reads(parts, B);
+  L.writes(y);
+  return L.sent(L.lib.gemv_bf16_row_attn(parts, n_parts, heads, head_dim, B, y, n, k));
 }
 // s = x (+ delta); xout (optional, distinct from x and delta) receives s;
 // y = W . rmsnorm(s, norm_w, eps)
@@ -1352,6 +1405,16 @@ struct kv_cache {
     if (!d_pos && pos >= max_ctx) return false;
     if (!attn_decode_qkv(qkv, bq, bk, bv, K, V, out, n_q_heads, n_kv_heads, pos, d_pos, max_ctx, D,
                          scale, table, partials, partials_bytes, kv_bf16))
+      return false;
+    if (!d_pos) pos++;
+    return true;
+  }
+  // attn_qkv with the split merge left to the o-projection's GEMV (gemv_*_attn)
+  bool attn_qkv_parts(void* qkv, void* bq, void* bk, void* bv, int64_t n_q_heads, float scale, void* table,
+                      void* d_pos, void* partials, int64_t partials_bytes, int* n_parts) {
+    if (!d_pos && pos >= max_ctx) return false;
+    if (kv_bf16 || !attn_decode_qkv_parts(qkv, bq, bk, bv, K, V, n_q_heads, n_kv_heads, pos, d_pos, max_ctx, D, scale,
+                                          table, partials, partials_bytes, n_parts))
       return false;
     if (!d_pos) pos++;
     return true;

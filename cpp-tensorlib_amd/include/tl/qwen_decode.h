@@ -73,6 +73,14 @@ inline bool gemv(const linear& L, void* a, void* y) {
   return hip::gemv_bf16_row(a, L.w, y, L.N, L.K);
 }
 
+// y = W . (attention output merged from n_parts split partials)
+inline bool gemv_attn(const linear& L, void* parts, int n_parts, int64_t heads, int64_t head_dim, void* y) {
+  if (L.fmt == wfmt::q4)
+    return hip::gemv_q4_attn(parts, n_parts, heads, head_dim, L.w, static_cast<char*>(L.w) + L.N * L.K / 2, y, L.N,
+                             L.K, kQ4Group);
+  return hip::gemv_bf16_row_attn(parts, n_parts, heads, head_dim, L.w, y, L.N, L.K);
+}
+
 // Prompt-chunk products, T rows at a time: out[T, N] = a[T, K] . W^T for either weight format
 // (bf16 rows or int4); `_parts` leaves the K-split parts for the launch that consumes them,
 // `_swiglu` takes the fused [gate | up] weight and writes the gated activation [T, N / 2].
@@ -179,6 +187,9 @@ struct model {
   // GEMV that consumes them). false: the reference's call sequence, one launch per op.
   bool fused = true;
   bool fused_attn = true;   // within the fused path: q/k/v epilogue + append inside the attention launch
+  // within fused_attn: where the launch plan cuts the context into few splits (short contexts, small
+  // models), the o-projection's GEMV merges them while it stages its input: no merge launch
+  bool merge_in_oproj = true;
   bool fused_prefill = true;     // prompt chunks: one launch for split_heads + rope + kv_fill, attention writes token-major
   bool prompt_f16 = true;        // prompt chunks of bf16 weights on the backend's prepared f16 form of them (a second copy, made on first use)
   bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
@@ -274,7 +285,9 @@ inline bool init(model& M, const dims& d) {
   S.logitsb = hip::alloc(d.vocab * 4, &S.logits_host);
   for (auto& L : M.layers)
     if (!L.cache.init(d.n_kv_heads, d.max_ctx, d.head_dim)) return false;
-  return S.logitsb != nullptr && S.embedb != nullptr;
+  M.attn_partials_bytes = hip::attn_partials_bytes(d.n_q_heads, d.n_kv_heads, d.max_ctx, d.head_dim);
+  M.attn_partials = hip::alloc_device(M.attn_partials_bytes);
+  return S.logitsb != nullptr && S.embedb != nullptr && M.attn_partials != nullptr;
 }
 
 inline bool set_layer_q4(model& M, int64_t li, const layer_blobs& b) {
@@ -671,7 +684,7 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
   const int64_t E = d.hidden, QD = d.q_dim(), KD = d.kv_dim();
   bool ok = true;
   if (M.fused) {
-    // 5 launches per layer (+1 when attention splits the context):
+    // 5 launches per layer (+1 when attention splits the context and the o-projection does not merge):
     //   [norm -> qkv GEMV] , [q/k/v epilogue + append -> attention] , o-proj GEMV ,
     //   [residual + norm -> gate|up GEMV] , [swiglu -> down GEMV]
     // (fused_attn = false runs the q/k/v epilogue as a launch of its own)
@@ -681,6 +694,10 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
     void* din = nullptr;     // MLP output of the previous layer, not yet added
     if (!M.rope_tab) M.rope_tab = hip::alloc_device(d.head_dim * 4);
     ok &= M.rope_tab && hip::rope_table(M.rope_tab, d.head_dim, pos, d_pos, d.rope_base);
+    // the attention's splits merged by the o-projection: decided once per step from the launch plan
+    const bool merge = M.fused_attn && M.merge_in_oproj && M.attn_partials &&
+                       hip::attn_parts_splits(d.n_q_heads, d.n_kv_heads, d_pos ? M.layers[0].cache.max_ctx : pos + 1,
+                                              d.head_dim, M.layers[0].cache.kv_bf16) > 0;
     size_t marks = 0;
     auto mark = [&] { if (marks < M.prof_events.size()) ok &= hip::event_record(M.prof_events[marks++]); };
     for (int64_t l = 0; l < d.n_layers; l++) {
@@ -698,7 +715,12 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
       ok &= gemv_rmsnorm(L.wqkv, rin, din, L.an, S.res[0], S.qkvb, d.eps);
       warm(2); warm(3); warm(4);   // beside attention: everything / o-proj and gate|up / + down
       mark();
-      if (M.fused_attn) {
+      int n_parts = 0;
+      if (merge) {
+        if (!d_pos) L.cache.pos = pos;
+        ok &= L.cache.attn_qkv_parts(S.qkvb, L.bq, L.bk, L.bv, d.n_q_heads, scale, M.rope_tab, d_pos, M.attn_partials,
+                                     M.attn_partials_bytes, &n_parts);
+      } else if (M.fused_attn) {
         if (!d_pos) L.cache.pos = pos;
         ok &= L.cache.attn_qkv(S.qkvb, L.bq, L.bk, L.bv, S.ab, d.n_q_heads, scale, M.rope_tab, d_pos,
                                d_pos ? M.attn_partials : nullptr, d_pos ? M.attn_partials_bytes : 0);
@@ -712,7 +734,7 @@ inline bool run_layers(model& M, void* x0, int64_t pos, void* logits_out = nullp
         ok &= L.cache.attn(S.qkvb, S.ab, d.n_q_heads, scale);
       }
       mark();
-      ok &= gemv(L.wo, S.ab, S.hb);
+      ok &= merge ? gemv_attn(L.wo, M.attn_partials, n_parts, d.n_q_heads, d.head_dim, S.hb) : gemv(L.wo, S.ab, S.hb);
       mark();
       if (M.gateup_epilogue) {
         ok &= gemv_rmsnorm_gateup(L.wgu, S.res[0], S.hb, L.fn, S.res[1], S.mb, d.eps);

@@ -62,6 +62,7 @@ def _load():
             "tlq_set_warm": (None, [P, cint, cint, cint]),
             "tlq_profile_steps": (cint, [P, i64, i64, i64, C.POINTER(C.c_double)]),
             "tlq_set_fused_attn": (None, [P, cint]),
+            "tlq_set_merge_in_oproj": (None, [P, cint]),
             "tlq_set_gateup_epilogue": (None, [P, cint]),
             "tlq_set_fused_prefill": (None, [P, cint]),
             "tlq_set_prompt_f16": (None, [P, cint]),
@@ -352,6 +353,11 @@ class QwenGPU:
     def set_fused_attn(self, on):
         """Within the fused path: run the q/k/v epilogue inside the attention launch (default) or alone."""
         self.L.tlq_set_fused_attn(self.h, 1 if on else 0)
+
+    def set_merge_in_oproj(self, on):
+        """Within the fused attention: let the o-projection's GEMV merge the attention's splits where
+        the launch plan makes few of them (default), or always run the merge launch."""
+        self.L.tlq_set_merge_in_oproj(self.h, 1 if on else 0)
 
     def set_fused_prefill(self, on):
         """Prompt chunks: one launch for split_heads + rope + kv_fill and token-major attention output (default), or the reference's op sequence."""

@@ -274,6 +274,20 @@ int tlhip_attn_decode_qkv(const void* qkv, const void* bq, const void* bk, const
                           const void* d_pos, int64_t kv_max, int64_t D, float scale,
                           const void* table, int kv_bf16, void* partials, int64_t partials_bytes);
 
+/* The same step with the split merge left to the o-projection (tlhip_gemv_*_attn below): nothing
+ * is written but the cache row and `partials`, laid out [Hq*S] running maxima | [Hq*S] sums |
+ * [Hq*S][D] accumulators for the S = *n_parts splits of the context that the launch plan chose
+ * (also when S is 1). Served: f32 caches, 3 to 8 query heads per kv head, an even head count, and
+ * contexts (capacities, with d_pos) that the plan cuts into at most 1024 / D, and at most 16,
+ * splits - tlhip_attn_parts_splits tells (0: not served, call tlhip_attn_decode_qkv). `partials`
+ * is required: tlhip_attn_partials_bytes. For small models: their merge launch costs as much as
+ * a projection. */
+int tlhip_attn_parts_splits(int64_t n_q_heads, int64_t n_kv_heads, int64_t plan_ctx, int64_t D, int kv_bf16);
+int tlhip_attn_decode_qkv_parts(const void* qkv, const void* bq, const void* bk, const void* bv, void* Kc,
+                                void* Vc, int64_t n_q_heads, int64_t n_kv_heads, int64_t pos,
+                                const void* d_pos, int64_t kv_max, int64_t D, float scale,
+                                const void* table, void* partials, int64_t partials_bytes, int* n_parts);
+
 /* ---- device-resident greedy loop (no reference counterpart: the reference gathers the
  * embedding row on the host and reads every token back, qwen_model.h:530-535, 642-647) ----
  * out[hidden] f32 = widened row *d_token of a bf16 [vocab, hidden] table; d_token is a device
@@ -315,13 +329,21 @@ int tlhip_embed_gather_f16(const void* table, const void* d_token, void* out, in
  * The producer of x is evaluated by every block while it stages x, which removes a
  * launch and a memory round trip per fused pair. Arithmetic is that of the separate
  * entry points: tlhip_swiglu then tlhip_gemv_*, and tlhip_rmsnorm_res then
- * tlhip_gemv_*, as run_layers_ chains them (bench/cuda/qwen_model.h:717-737).
+ * tlhip_gemv_*, as run_layers_ chains them (bench/cuda/qwen_model.h:717-737); the split merge of
+ * tlhip_attn_decode_qkv then tlhip_gemv_*.
  * Row layouts only (int4 group 32, bf16 [N,K]); other shapes return
  * TLHIP_EUNSUPPORTED and the caller issues the two separate calls. */
 /* y = W . swiglu(gu), gu = [gate (K) | up (K)] f32 */
 int tlhip_gemv_q4_swiglu(const void* gu, const void* qw, const void* scales, void* y, int64_t N,
                          int64_t K, int64_t group);
 int tlhip_gemv_bf16_row_swiglu(const void* gu, const void* W, void* y, int64_t n, int64_t k);
+/* y = W . x, x[h*D + d] = sum_s e^(m_s - M) acc_s[d] / sum_s e^(m_s - M) l_s: the decode attention's
+ * output, merged from the n_parts split partials tlhip_attn_decode_qkv_parts left (its layout;
+ * K = heads * head_dim), bit for bit what tlhip_attn_decode_qkv writes to `out`. */
+int tlhip_gemv_q4_attn(const void* parts, int64_t n_parts, int64_t heads, int64_t head_dim, const void* qw,
+                       const void* scales, void* y, int64_t N, int64_t K, int64_t group);
+int tlhip_gemv_bf16_row_attn(const void* parts, int64_t n_parts, int64_t heads, int64_t head_dim,
+                             const void* W, void* y, int64_t n, int64_t k);
 /* s = x (+ delta when non-NULL); xout (when non-NULL) receives s; y = W . rmsnorm(s, norm_w, eps).
  * xout must not alias x or delta. */
 int tlhip_gemv_q4_rmsnorm(const void* x, const void* delta, const void* norm_w, void* xout,

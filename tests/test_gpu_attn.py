@@ -243,3 +243,103 @@ def test_attn_decode_qkv_fused_prologue(lib, orc, D, Hq, Hkv, kv_max, kv_bf16):
         lib.attn_decode_qkv(q2, dbq, dbk, dbv, K2, V2, o2, Hq, Hkv, kv_max, kv_max, D, scale, tab, kv_bf16=kv_bf16)
     for b in (q2, K2, V2, o2, dbq, dbk, dbv, tab, dpos, part):
         b.free()
+
+
+@pytest.mark.parametrize("fmt", ["q4", "bf16"])
+@pytest.mark.parametrize("D,Hq,Hkv,kv_max,E", [(64, 14, 2, 1024, 896), (128, 28, 4, 512, 256), (64, 16, 2, 640, 160),
+                                               (128, 6, 2, 300, 96)])
+def test_attn_splits_merged_by_the_o_projection(lib, orc, fmt, D, Hq, Hkv, kv_max, E):
+    """The fused decode attention leaving its split partials (1 to 16 of them) and the o-projection's
+    GEMV merging them while it stages its input, against the path with the merge launch: the same
+    cache rows and the same projection bit for bit, and both within the tolerance of the oracle's
+    attention followed by its GEMV. Position on the host and, where the capacity's plan is served,
+    on the device."""
+    base, scale = 1e6, 1.0 / np.sqrt(float(D))
+    n, QD = (Hq + 2 * Hkv) * D, Hq * D
+    K0 = orc.normal(Hkv * kv_max * D, 521).reshape(Hkv, kv_max, D)
+    V0 = orc.normal(Hkv * kv_max * D, 522).reshape(Hkv, kv_max, D)
+    bq, bk, bv = orc.normal(Hq * D, 523, 0, 0.5), orc.normal(Hkv * D, 524, 0, 0.5), orc.normal(Hkv * D, 525, 0, 0.5)
+    dbq, dbk, dbv = lib.to_device(bq), lib.to_device(bk), lib.to_device(bv)
+    if fmt == "q4":
+        wbuf = orc.to_q4(orc.normal(QD * E, 526, 0.0, 0.05).reshape(QD, E))
+        gemv_o = lambda x: orc.gemv_q4(x, wbuf, E, QD)
+    else:
+        wbuf = orc.to_bf16(orc.normal(E * QD, 527, 0.0, 0.05).reshape(E, QD))
+        gemv_o = lambda x: orc.gemv_bf16_row(x, wbuf)
+    dw = lib.to_device(wbuf)
+    tab, dpos = lib.empty(D), lib.to_device(np.zeros(1, np.uint32))
+    part = lib.empty_bytes(lib.attn_partials_bytes(Hq, Hkv, kv_max, D))
+    assert lib.attn_parts_splits(Hq, Hkv, kv_max, D, kv_bf16=True) == 0
+    seen = set()
+    positions = sorted(set([0, 1, 63, 64, 65, 127, 128, 191, 300, kv_max // 2, kv_max - 65, kv_max - 2, kv_max - 1]))
+    for pos in [p for p in positions if 0 <= p < kv_max]:
+        for on_device in (False, True):
+            S = lib.attn_parts_splits(Hq, Hkv, kv_max if on_device else pos + 1, D)
+            if S == 0:
+                continue
+            print("case attn parts", fmt, D, Hq, Hkv, kv_max, pos, on_device, S, flush=True)
+            qkv = orc.normal(n, 530 + pos)
+            q1, K1, V1, o1, y1 = lib.to_device(qkv), lib.to_device(K0), lib.to_device(V0), lib.empty((Hq, D)), lib.empty(E)
+            q2, K2, V2, y2 = lib.to_device(qkv), lib.to_device(K0), lib.to_device(V0), lib.empty(E)
+            part.upload(np.full(part.nbytes // 4, np.nan, np.float32).view(np.uint8))
+            if on_device:
+                dpos.upload(np.array([pos], np.uint32))
+                lib.rope_table(tab, D, 0, base, d_pos=dpos)
+                lib.attn_decode_qkv(q1, dbq, dbk, dbv, K1, V1, o1, Hq, Hkv, 0, kv_max, D, scale, tab, d_pos=dpos, partials=part)
+                got_S = lib.attn_decode_qkv_parts(q2, dbq, dbk, dbv, K2, V2, Hq, Hkv, 0, kv_max, D, scale, tab, part, d_pos=dpos)
+            else:
+                lib.rope_table(tab, D, pos, base)
+                lib.attn_decode_qkv(q1, dbq, dbk, dbv, K1, V1, o1, Hq, Hkv, pos, kv_max, D, scale, tab)
+                got_S = lib.attn_decode_qkv_parts(q2, dbq, dbk, dbv, K2, V2, Hq, Hkv, pos, kv_max, D, scale, tab, part)
+            assert got_S == S
+            seen.add(S)
+            if fmt == "q4":
+                lib.gemv_q4(o1, dw, y1, E, QD)
+                lib.gemv_q4_attn(part, S, Hq, D, dw, y2, E, QD)
+            else:
+                lib.gemv_bf16_row(o1, dw, y1, E, QD)
+                lib.gemv_bf16_row_attn(part, S, Hq, D, dw, y2, E, QD)
+            assert np.array_equal(K1.numpy(), K2.numpy()) and np.array_equal(V1.numpy(), V2.numpy()), pos
+            two, got = y1.numpy(), y2.numpy()
+            assert np.array_equal(two, got), (pos, S, maxrel(got, two))
+            qr = orc.rope(qkv[:QD].reshape(Hq, D), pos, base, bias=bq.reshape(Hq, D))
+            want = gemv_o(orc.attn_decode(qr, K2.numpy(), V2.numpy(), scale, ctx=pos + 1).reshape(QD))
+            assert allclose(got, want, RTOL, ATOL), (pos, S, maxrel(got, want))
+            for b in (q1, K1, V1, o1, y1, q2, K2, V2, y2):
+                b.free()
+    assert len(seen) >= 3, seen          # one split, a few, and the most the shape's plan makes
+    # refusals: more parts than the merge sums in order, a K that is not heads x head_dim
+    y = lib.empty(E)
+    with pytest.raises(Exception):
+        (lib.gemv_q4_attn if fmt == "q4" else lib.gemv_bf16_row_attn)(part, 17 if D == 64 else 9, Hq, D, dw, y, E, QD)
+    with pytest.raises(Exception):
+        (lib.gemv_q4_attn if fmt == "q4" else lib.gemv_bf16_row_attn)(part, 1, Hq - 1, D, dw, y, E, QD)
+    for b in (dbq, dbk, dbv, dw, tab, dpos, part, y):
+        b.free()
+
+
+@pytest.mark.parametrize("D,heads,S", [(64, 14, 16), (64, 14, 5), (128, 28, 8), (128, 2, 3), (64, 4, 1)])
+def test_gemv_attn_merge_of_made_up_partials(lib, orc, D, heads, S):
+    """The merge alone, on partials no attention produced: maxima spread over 60 units (weights down
+    to e^-60), splits that held no key (maximum -inf, sum 0, accumulator 0), against the formula
+    x[h,d] = sum_s e^(m_s - M) acc_s[d] / sum_s e^(m_s - M) l_s in float64, through an identity-like
+    bf16 weight so that y is x itself."""
+    rng = np.random.default_rng(D + heads + S)
+    m = rng.uniform(-30, 30, (heads, S)).astype(np.float32)
+    l = rng.uniform(0.5, 64, (heads, S)).astype(np.float32)
+    acc = (rng.standard_normal((heads, S, D)) * l[:, :, None]).astype(np.float32)
+    if S > 2:
+        dead = rng.integers(1, S, heads)                   # one empty split per head, never split 0
+        for h in range(heads):
+            m[h, dead[h]], l[h, dead[h]], acc[h, dead[h]] = -np.inf, 0.0, 0.0
+    K = heads * D
+    w64 = np.exp(m.astype(np.float64) - m.max(axis=1, keepdims=True))
+    want = ((w64[:, :, None] * acc).sum(axis=1) / (w64 * l).sum(axis=1)[:, None]).reshape(K).astype(np.float32)
+    eye = orc.to_bf16(np.eye(K, dtype=np.float32))
+    part = lib.to_device(np.concatenate([m.ravel(), l.ravel(), acc.ravel()]))
+    dw, y = lib.to_device(eye), lib.empty(K)
+    lib.gemv_bf16_row_attn(part, S, heads, D, dw, y, K, K)
+    got = y.numpy()
+    assert allclose(got, want, 1e-5, 1e-6), maxrel(got, want)
+    for b in (part, dw, y):
+        b.free()
