@@ -33,32 +33,52 @@ __device__ __forceinline__ float byte1(uint32_t v) { return (float)((v >> 8) & 0
 __device__ __forceinline__ float byte2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
 __device__ __forceinline__ float byte3(uint32_t v) { return (float)(v >> 24); }
 
+// acc + h * x in one instruction, h the low (HI = false) or high half of `pair` read as an f16.
+// A half that holds only mantissa bits is an f16 subnormal, value bits * 2^-24: four weight bits
+// masked out of a word need no conversion to become a number.
+template <bool HI>
+__device__ __forceinline__ float fma_half(uint32_t pair, float x, float acc) {
+  float d;
+  if constexpr (HI)
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(pair), "v"(x), "v"(acc));
+  else
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(d) : "v"(pair), "v"(x), "v"(acc));
+  return d;
+}
+
 struct FmtQ4 {
   static constexpr int E = 32;  // weights per 16-byte unit == one scale group
   static constexpr bool kScaled = true;
-  // staged form of (x_even, x_odd, x_even, x_odd)
+  // staged form of (x_even, x_odd, x_even, x_odd): the odd ones over 16 (exact), because their
+  // nibbles are read where they sit, four bits up
   static __device__ __forceinline__ float4 stage(const float4 v) {
-    const float o0 = v.y * 0.0625f, o1 = v.w * 0.0625f;
-    return make_float4(v.x - o0, o0, v.z - o1, o1);
+    return make_float4(v.x, v.y * 0.0625f, v.z, v.w * 0.0625f);
   }
-  // sum_k nib_k * x_k over the unit, x in staged form
+  // sum_k nib_k * x_k over the unit, x in staged form. A 32-bit word holds weights 8i .. 8i+7,
+  // byte j the pair (2j, 2j+1), even in the low nibble. Masked in place, the nibbles of bytes 0
+  // and 2 (and, from the word shifted down a byte, 1 and 3) are the two f16 halves of a
+  // register: five integer instructions and eight mixed-precision FMAs per eight weights. The
+  // products are nib * 2^-24 * x, exact scalings of what the CPU loop adds (array.h:735-737), and
+  // the factor comes off the unit's sum; only activations below 2^-120 lose bits to it.
   static __device__ __forceinline__ float dot(const uint4 w, const float4 (&x)[8]) {
     const uint32_t d[4] = {w.x, w.y, w.z, w.w};
     float a0 = 0.f, a1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const uint32_t full = d[i], lo = low_nibbles(full);
+      const uint32_t full = d[i], up = full >> 8;
+      const uint32_t e02 = full & 0x000f000fu, o02 = full & 0x00f000f0u;
+      const uint32_t e13 = up & 0x000f000fu, o13 = up & 0x00f000f0u;
       const float4 xa = x[2 * i], xb = x[2 * i + 1];
-      a0 = fmaf(byte0(lo), xa.x, a0);
-      a1 = fmaf(byte0(full), xa.y, a1);
-      a0 = fmaf(byte1(lo), xa.z, a0);
-      a1 = fmaf(byte1(full), xa.w, a1);
-      a0 = fmaf(byte2(lo), xb.x, a0);
-      a1 = fmaf(byte2(full), xb.y, a1);
-      a0 = fmaf(byte3(lo), xb.z, a0);
-      a1 = fmaf(byte3(full), xb.w, a1);
+      a0 = fma_half<false>(e02, xa.x, a0);
+      a1 = fma_half<false>(o02, xa.y, a1);
+      a0 = fma_half<false>(e13, xa.z, a0);
+      a1 = fma_half<false>(o13, xa.w, a1);
+      a0 = fma_half<true>(e02, xb.x, a0);
+      a1 = fma_half<true>(o02, xb.y, a1);
+      a0 = fma_half<true>(e13, xb.z, a0);
+      a1 = fma_half<true>(o13, xb.w, a1);
     }
-    return a0 + a1;
+    return (a0 + a1) * 16777216.0f;
   }
 };
 
