@@ -24,8 +24,8 @@ def _inputs(orc, Hq, Hkv, ctx, kv_max, D, seed):
 
 
 def test_static_entry_equals_attn_decode_on_two_calls_in_a_row(lib, orc):
-    """First the 7B decode shape at ctx 4096 (28 query heads over 4 kv heads, 32-way split:
-    466 KB of partials), then at once a smaller one (14 over 2 heads of 64, ctx 700), then a
+    """First the 7B decode shape at ctx 4096 (28 query heads over 4 kv heads, 64-way split:
+    932 KB of partials), then at once a smaller one (14 over 2 heads of 64, ctx 700), then a
     one-split call that uses no partials; each against tlhip_attn_decode and the oracle."""
     cases = [(28, 4, 4096, 4352, 128, 11), (14, 2, 700, 1024, 64, 21), (4, 4, 40, 64, 128, 31)]
     bufs = []
