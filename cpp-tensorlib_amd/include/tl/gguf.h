@@ -61,7 +61,7 @@ inline void ggml_block(ggml_type t, uint64_t& elems, uint64_t& bytes) {
       bytes = g.bytes;
       return;
     }
-  detail::fail("unknown ggml type " + std::to_string(static_cast<uint32_t>(t)));
+  detail::fail("tensor storage code " + std::to_string(static_cast<uint32_t>(t)) + " is not one this reader knows");
 }
 
 // One metadata value. Unsigned scalars and bool land in u, signed in i, floats in
@@ -83,7 +83,7 @@ struct metadata_value {
   const std::string& as_str() const { return expect(val_type::string), s; }
   std::vector<std::string> as_str_array() const {
     if (type != val_type::array || arr_elem_type != val_type::string)
-      detail::fail("value is not a string array");
+      detail::fail("asked for a list of strings, the value holds something else");
     std::vector<std::string> out;
     out.reserve(arr.size());
     for (const auto& e : arr) out.push_back(e.s);
@@ -98,14 +98,14 @@ struct metadata_value {
         break;
       default: break;
     }
-    detail::fail("value is not a non-negative integer");
+    detail::fail("asked for a count, the value is not an integer >= 0");
   }
 
  private:
   void expect(val_type want) const {
     if (type != want)
-      detail::fail("value type mismatch (have " + std::to_string(static_cast<uint32_t>(type)) +
-                   ", want " + std::to_string(static_cast<uint32_t>(want)) + ")");
+      detail::fail("the value has code " + std::to_string(static_cast<uint32_t>(type)) + ", asked for as code " +
+                   std::to_string(static_cast<uint32_t>(want)));
   }
 };
 
@@ -133,16 +133,16 @@ class model {
   // directory that points outside the file.
   explicit model(const std::string& path) {
     const int fd = ::open(path.c_str(), O_RDONLY | O_CLOEXEC);
-    if (fd < 0) detail::fail("cannot open " + path);
+    if (fd < 0) detail::fail("open() failed: " + path);
     struct stat st {};
     if (::fstat(fd, &st) != 0 || st.st_size <= 0) {
       ::close(fd);
-      detail::fail("cannot stat " + path);
+      detail::fail("fstat() failed: " + path);
     }
     bytes_ = static_cast<size_t>(st.st_size);
     void* m = ::mmap(nullptr, bytes_, PROT_READ, MAP_PRIVATE, fd, 0);
     ::close(fd);
-    if (m == MAP_FAILED) detail::fail("mmap failed for " + path);
+    if (m == MAP_FAILED) detail::fail("mmap() failed: " + path);
     base_ = static_cast<const uint8_t*>(m);
     // weights are walked once, front to back, by the uploader
     ::posix_madvise(m, bytes_, POSIX_MADV_SEQUENTIAL);
@@ -174,7 +174,7 @@ class model {
   bool has(const std::string& key) const { return kv_.find(key) != kv_.end(); }
   const metadata_value& kv(const std::string& key) const {
     const auto it = kv_.find(key);
-    if (it == kv_.end()) detail::fail("missing key " + key);
+    if (it == kv_.end()) detail::fail("no metadata key " + key);
     return it->second;
   }
   const std::unordered_map<std::string, metadata_value>& metadata() const { return kv_; }
@@ -190,7 +190,7 @@ class model {
     const uint8_t* base;
     size_t size, at = 0;
     const uint8_t* need(size_t n) {
-      if (n > size || at > size - n) detail::fail("truncated file (read past end)");
+      if (n > size || at > size - n) detail::fail("the file ends inside a field");
       const uint8_t* p = base + at;
       at += n;
       return p;
@@ -203,7 +203,7 @@ class model {
     }
     std::string str() {
       const uint64_t len = get<uint64_t>();
-      if (len > size) detail::fail("truncated file (read past end)");
+      if (len > size) detail::fail("the file ends inside a field");
       const uint8_t* p = need(static_cast<size_t>(len));
       return std::string(reinterpret_cast<const char*>(p), static_cast<size_t>(len));
     }
@@ -227,25 +227,25 @@ class model {
       case val_type::string: v.s = c.str(); break;
       case val_type::array: {
         v.arr_elem_type = static_cast<val_type>(c.get<uint32_t>());
-        if (v.arr_elem_type == val_type::array) detail::fail("nested arrays unsupported");
+        if (v.arr_elem_type == val_type::array) detail::fail("a list of lists in the metadata");
         const uint64_t count = c.get<uint64_t>();
         // every element takes at least one byte: a count beyond the file is a corrupt header
-        if (count > c.size) detail::fail("truncated file (read past end)");
+        if (count > c.size) detail::fail("the file ends inside a field");
         v.arr.reserve(static_cast<size_t>(count));
         for (uint64_t k = 0; k < count; k++) v.arr.push_back(value(c, v.arr_elem_type));
         break;
       }
       default:
-        detail::fail("unknown value type " + std::to_string(static_cast<uint32_t>(t)));
+        detail::fail("metadata value code " + std::to_string(static_cast<uint32_t>(t)) + " is not one this reader knows");
     }
     return v;
   }
 
   void parse() {
     cursor c{base_, bytes_};
-    if (c.get<uint32_t>() != 0x46554747u) detail::fail("bad magic (not a GGUF file)");   // "GGUF"
+    if (c.get<uint32_t>() != 0x46554747u) detail::fail("the first four bytes are not 'GGUF'");   // "GGUF"
     version_ = c.get<uint32_t>();
-    if (version_ != 3) detail::fail("unsupported version " + std::to_string(version_));
+    if (version_ != 3) detail::fail("format version " + std::to_string(version_) + " (version 3 is read)");
     const uint64_t n_tensors = c.get<uint64_t>();
     const uint64_t n_kv = c.get<uint64_t>();
     for (uint64_t k = 0; k < n_kv; k++) {
@@ -257,7 +257,7 @@ class model {
     if (al != kv_.end()) alignment_ = al->second.type == val_type::u32 ? al->second.as_u32() : al->second.u;
     if (alignment_ == 0) detail::fail("general.alignment is zero");
 
-    if (n_tensors > bytes_) detail::fail("truncated file (read past end)");
+    if (n_tensors > bytes_) detail::fail("the file ends inside a field");
     tensors_.reserve(static_cast<size_t>(n_tensors));
     for (uint64_t k = 0; k < n_tensors; k++) {
       tensor_info t;
@@ -276,7 +276,7 @@ class model {
     data_start_ = (c.at + alignment_ - 1) / alignment_ * alignment_;
     for (auto& t : tensors_) {
       if (t.rel_offset > bytes_ || data_start_ > bytes_ - t.rel_offset)
-        detail::fail("truncated file (read past end)");
+        detail::fail("the file ends inside a field");
       cursor probe{base_, bytes_, static_cast<size_t>(data_start_ + t.rel_offset)};
       t.data = probe.need(static_cast<size_t>(t.nbytes));
     }

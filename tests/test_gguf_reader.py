@@ -176,6 +176,6 @@ def test_hyperparameters_from_metadata(qwen, tmp_path):
     # a missing key is reported, not guessed
     W.write(path, [("general.architecture", W.STRING, "qwen2")], [])
     g = qwen.GgufFile(path)
-    with pytest.raises(RuntimeError, match="missing key"):
+    with pytest.raises(RuntimeError, match="no metadata key"):
         g.dims()
     g.close()

@@ -226,7 +226,7 @@ def test_vocabulary_without_a_byte_piece_is_reported(tmp_path, refimpl):
         mine.encode(b"xyz")
     # a file without tokenizer metadata is refused at construction
     W.write(path, [("general.architecture", W.STRING, "qwen2")], [])
-    with pytest.raises(RuntimeError, match="missing key"):
+    with pytest.raises(RuntimeError, match="no metadata key"):
         qwen.Tokenizer(path)
 
 
