@@ -109,6 +109,11 @@ SIGNATURES = {
     "tlhip_attn_decode_qkv": (cint, [P, P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, cint, P, i64]),
     "tlhip_embed_gather_bf16": (cint, [P, P, P, i64, i64]),
     "tlhip_token_advance": (cint, [P, P, P, i64]),
+    "tlhip_gemm_f16w_aimage_bytes": (i64, [i64, i64]),
+    "tlhip_rmsnorm_res_parts_aimage": (cint, [P, P, i64, P, P, P, i64, f32, i64, P]),
+    "tlhip_gemm_f16w_nt_aimage": (cint, [P, P, P, P, P, i64, i64, i64]),
+    "tlhip_gemm_f16w_nt_parts_aimage": (cint, [P, P, P, P, P, i64, i64, i64, i64, P]),
+    "tlhip_gemm_f16w_nt_swiglu_aimage": (cint, [P, P, P, P, P, i64, i64, i64]),
     "tlhip_attn_parts_splits": (cint, [i64, i64, i64, i64, cint]),
     "tlhip_attn_decode_qkv_parts": (cint, [P, P, P, P, P, P, i64, i64, i64, P, i64, i64, f32, P, P, i64, P]),
     "tlhip_gemv_q4_attn": (cint, [P, i64, i64, i64, P, P, P, i64, i64, i64]),
@@ -373,6 +378,26 @@ class TlHip:
     def rmsnorm_res_parts(self, x, parts, n_parts, w, xout, hout, n, eps, rows=1):
         self._chk(self.c.tlhip_rmsnorm_res_parts(x.ptr, parts.ptr, n_parts, w.ptr, xout.ptr, hout.ptr,
                                                  n, eps, rows))
+
+    def gemm_f16w_aimage_bytes(self, M, K):
+        return int(self.c.tlhip_gemm_f16w_aimage_bytes(M, K))
+
+    def rmsnorm_res_parts_aimage(self, x, parts, n_parts, w, xout, hout, n, eps, rows, aimage):
+        """rmsnorm_res_parts that also leaves hout's activation image (gemm_f16w_aimage_bytes(rows, n) bytes)."""
+        self._chk(self.c.tlhip_rmsnorm_res_parts_aimage(x.ptr, parts.ptr, n_parts, w.ptr, xout.ptr, hout.ptr,
+                                                        n, eps, rows, aimage.ptr))
+
+    def gemm_f16w_nt_aimage(self, A, aimage, image, exps, out, M, N, K):
+        self._chk(self.c.tlhip_gemm_f16w_nt_aimage(A.ptr, aimage.ptr, image.ptr, exps.ptr, out.ptr, M, N, K))
+
+    def gemm_f16w_nt_swiglu_aimage(self, A, aimage, image, exps, act, M, ff, K):
+        self._chk(self.c.tlhip_gemm_f16w_nt_swiglu_aimage(A.ptr, aimage.ptr, image.ptr, exps.ptr, act.ptr, M, ff, K))
+
+    def gemm_f16w_nt_parts_aimage(self, A, aimage, image, exps, parts, M, N, K):
+        n = C.c_int(0)
+        self._chk(self.c.tlhip_gemm_f16w_nt_parts_aimage(A.ptr, aimage.ptr, image.ptr, exps.ptr, parts.ptr,
+                                                         parts.nbytes, M, N, K, C.byref(n)))
+        return n.value
 
     def split_heads(self, src, bias, dst, T, ld, off, H, D):
         self._chk(self.c.tlhip_split_heads(src.ptr, bias.ptr if bias is not None else None, dst.ptr,

@@ -193,6 +193,111 @@ __global__ __launch_bounds__(256) void a_image_kernel(const float* __restrict__ 
   }
 }
 
+// The residual norm of a prompt chunk writing the activation image of its own output: what
+// rmsnorm_wide_kernel<true, RV> (modelops.hip) followed by a_image_kernel would leave - the same
+// arithmetic in the same order for s = x + parts, hout = (s / rms) w, and the same exponent, terms
+// and small-element mark for the row of hout, which is still in registers - in one launch and
+// without reading hout back. One block of 1024 threads per image row (rows past M are zero rows).
+// x and xout may be the same buffer (a thread writes only what it has read).
+template <int RV>
+__global__ __launch_bounds__(1024) void rmsnorm_aimage_kernel(const float* x, const float* __restrict__ delta,
+                                                              const float* __restrict__ w, float* xout,
+                                                              float* __restrict__ hout, int n, float eps, int S,
+                                                              size_t part_stride, int* __restrict__ ea,
+                                                              char* __restrict__ img, int M) {
+  __shared__ float red[16];
+  __shared__ uint32_t part[16], cnt[16];
+  const int gm = blockIdx.x, t = threadIdx.x, n4 = n >> 2, nslab = n / kBK;
+  const int tm = gm / kTile, row = gm % kTile;
+  float4 o[RV];
+#pragma unroll
+  for (int k = 0; k < RV; k++) o[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+  uint32_t mx = 0;
+  if (gm < M) {                                    // (the same for every thread of the block)
+    const size_t base = (size_t)gm * n;
+    const float4* x4 = reinterpret_cast<const float4*>(x + base);
+    const float4* d4 = reinterpret_cast<const float4*>(delta + base);
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4 v[RV], wv[RV];
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < RV; k++) {
+      const int i = t + k * 1024;
+      if (i < n4) {
+        v[k] = x4[i];
+        wv[k] = w4[i];
+        float4 d = d4[i];
+        for (int sidx = 1; sidx < S; sidx++) {     // K-split parts, ascending
+          const float4 e = d4[sidx * (part_stride >> 2) + i];
+          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+        }
+        v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < RV; k++) {
+      const int i = t + k * 1024;
+      if (i < n4) {
+        reinterpret_cast<float4*>(xout + base)[i] = v[k];
+        acc += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+      }
+    }
+    const float sum = block_sum<16>(acc, red);
+    const float inv = 1.0f / sqrtf(sum * (1.0f / (float)n) + eps);
+#pragma unroll
+    for (int k = 0; k < RV; k++) {
+      const int i = t + k * 1024;
+      if (i < n4) {
+        o[k].x = (v[k].x * inv) * wv[k].x; o[k].y = (v[k].y * inv) * wv[k].y;
+        o[k].z = (v[k].z * inv) * wv[k].z; o[k].w = (v[k].w * inv) * wv[k].w;
+        reinterpret_cast<float4*>(hout + base)[i] = o[k];
+        mx = max(mx, __float_as_uint(o[k].x) & 0x7fffffffu);
+        mx = max(mx, __float_as_uint(o[k].y) & 0x7fffffffu);
+        mx = max(mx, __float_as_uint(o[k].z) & 0x7fffffffu);
+        mx = max(mx, __float_as_uint(o[k].w) & 0x7fffffffu);
+      }
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, d));
+  if ((t & 63) == 0) part[t >> 6] = mx;
+  __syncthreads();
+  mx = part[0];
+#pragma unroll
+  for (int k = 1; k < 16; k++) mx = max(mx, part[k]);
+  const int e = row_exponent((int)(mx >> 23), mx == 0);
+  const float sc = pow2f(e);
+  char* dst = img + (size_t)tm * nslab * kAImage;
+  uint32_t least = 0xffffffffu;                    // smallest nonzero magnitude's bits, minus one
+#pragma unroll
+  for (int k = 0; k < RV; k++) {
+    const int q = t + k * 1024;                    // float4 q of the row: slab q / 8, 8-byte piece q % 8 of its 64 bytes
+    if (q < n4) {
+      const float xs[4] = {o[k].x * sc, o[k].y * sc, o[k].z * sc, o[k].w * sc};
+#pragma unroll
+      for (int j = 0; j < 4; j++) least = min(least, (__float_as_uint(xs[j]) & 0x7fffffffu) - 1u);   // 0 wraps to the top
+      uint32_t h01, l01, h23, l23;
+      split2_f16(xs[0], xs[1], h01, l01);
+      split2_f16(xs[2], xs[3], h23, l23);
+      const int c4 = q & 7;
+      char* op = dst + (size_t)(q >> 3) * kAImage + image_off(row, c4 >> 1) + (c4 & 1) * 8;
+      *reinterpret_cast<uint2*>(op) = make_uint2(h01, h23);
+      *reinterpret_cast<uint2*>(op + kPlaneBytes) = make_uint2(l01, l23);
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) least = min(least, (uint32_t)__shfl_xor((int)least, d));
+  if ((t & 63) == 0) cnt[t >> 6] = least;
+  __syncthreads();
+  if (t == 0 && gm < M) {
+    least = cnt[0];
+    for (int k = 1; k < 16; k++) least = min(least, cnt[k]);
+    uint32_t small = least < 0x3a800000u - 1u ? (uint32_t)n : 0u;          // 0 < |x| < 2^-10 somewhere
+    if (mx >= 0x7f800000u) small = kSmallMax;
+    ea[gm] = (e & 0xff) | (int)(small << 8);
+  }
+}
+
 // Grid: x = tiles (row tiles fastest, one contiguous run of tiles per XCD), y = K-split parts of
 // `part_slabs` slabs each; part y goes to C + y * M * ldc. N = columns of this launch (gated:
 // features), tn0 = first column tile (the launch may cover a column range of the weight).
@@ -543,8 +648,9 @@ namespace {
 int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // plain: C[M][N]; parts (S_out != nullptr): C is the caller's [S][M][N]; gated: N = features, C[M][N] the activation
+// aimg_in: the activation image of A made before (tlhip_rmsnorm_res_parts_aimage), or nullptr: made here
 int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, int64_t M, int64_t N, int64_t K,
-                   size_t parts_bytes, int* S_out, bool gu) {
+                   size_t parts_bytes, int* S_out, bool gu, const void* aimg_in = nullptr) {
   TLHIP_REQUIRE_READY();
   const bool want_parts = S_out != nullptr;
   if (!A || !image || !exps || !C) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt: null pointer");
@@ -603,10 +709,17 @@ int gemm_f16w_impl(const void* A, const void* image, const void* exps, void* C, 
       }
   char* sbase = static_cast<char*>(scratch(ea_bytes + aimg_bytes + parts_need));
   if (!sbase) return fail(TLHIP_ENOMEM, "tlhip_gemm_f16w_nt: no scratch for the activation planes and K-split parts");
-  int* ea = reinterpret_cast<int*>(sbase);
-  char* aimg = sbase + ea_bytes;
+  const int* ea = reinterpret_cast<const int*>(sbase);
+  const char* aimg = sbase + ea_bytes;
   const float* pa = static_cast<const float*>(A);
-  f16t::a_image_kernel<<<dim3((unsigned)(timg * f16t::kTile)), dim3(256), 0, c.stream>>>(pa, ea, aimg, (int)M, (int)K);
+  if (aimg_in) {
+    if (!aligned16(aimg_in)) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt: activation image not 16-byte aligned");
+    ea = static_cast<const int*>(aimg_in);
+    aimg = static_cast<const char*>(aimg_in) + ea_bytes;
+  } else {
+    f16t::a_image_kernel<<<dim3((unsigned)(timg * f16t::kTile)), dim3(256), 0, c.stream>>>(
+        pa, reinterpret_cast<int*>(sbase), sbase + ea_bytes, (int)M, (int)K);
+  }
   float* pc = static_cast<float*>(C);
   for (int pi = 0; pi < npieces; pi++) {
     const Piece& P = pieces[pi];
@@ -715,6 +828,63 @@ int tlhip_gemm_f16w_nt(const void* A, const void* image, const void* exps, void*
 int tlhip_gemm_f16w_nt_swiglu(const void* A, const void* image, const void* exps, void* act, int64_t M,
                               int64_t ff, int64_t K) {
   return gemm_f16w_impl(A, image, exps, act, M, ff, K, 0, nullptr, true);
+}
+
+int64_t tlhip_gemm_f16w_aimage_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || (K % f16t::kBK) != 0 || K > 256 * 4 * f16t::kRowRegs || M > 0x3fffffff) return 0;
+  const int64_t ea_bytes = (M * (int64_t)sizeof(int) + 1023) & ~(int64_t)1023;
+  return ea_bytes + cdiv64(M, f16t::kTile) * (K / f16t::kBK) * f16t::kAImage;
+}
+
+int tlhip_rmsnorm_res_parts_aimage(const void* x, const void* parts, int64_t S, const void* w, void* xout,
+                                   void* hout, int64_t n, float eps, int64_t rows, void* aimage) {
+  TLHIP_REQUIRE_READY();
+  if (!x || !parts || !w || !xout || !hout || !aimage)
+    return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res_parts_aimage: null pointer");
+  if (n <= 0 || rows <= 0 || rows > 0x3fffffff || S <= 0 || S > 64 || (n % f16t::kBK) != 0 || n > 8192)
+    return fail(TLHIP_EUNSUPPORTED,
+                "tlhip_rmsnorm_res_parts_aimage: need positive rows, 1 <= S <= 64, n %% 32 == 0 and n <= 8192");
+  if (!aligned16(x) || !aligned16(parts) || !aligned16(xout) || !aligned16(w) || !aligned16(hout) || !aligned16(aimage))
+    return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res_parts_aimage: misaligned");
+  if (xout == parts) return fail(TLHIP_EINVAL, "tlhip_rmsnorm_res_parts_aimage: xout must not alias the parts");
+  const int64_t timg = cdiv64(rows, f16t::kTile);
+  if (timg * f16t::kTile > 0x7fffffff) return fail(TLHIP_EUNSUPPORTED, "tlhip_rmsnorm_res_parts_aimage: too many rows");
+  const size_t ea_bytes = ((size_t)rows * sizeof(int) + 1023) & ~(size_t)1023;
+  int* ea = static_cast<int*>(aimage);
+  char* img = static_cast<char*>(aimage) + ea_bytes;
+  const dim3 grid((unsigned)(timg * f16t::kTile)), block(1024);
+  const size_t ps = (size_t)(rows * n);
+  hipStream_t st = ctx().stream;
+  if (n <= 4096)
+    f16t::rmsnorm_aimage_kernel<1><<<grid, block, 0, st>>>(static_cast<const float*>(x), static_cast<const float*>(parts),
+                                                         static_cast<const float*>(w), static_cast<float*>(xout),
+                                                         static_cast<float*>(hout), (int)n, eps, (int)S, ps, ea, img, (int)rows);
+  else
+    f16t::rmsnorm_aimage_kernel<2><<<grid, block, 0, st>>>(static_cast<const float*>(x), static_cast<const float*>(parts),
+                                                         static_cast<const float*>(w), static_cast<float*>(xout),
+                                                         static_cast<float*>(hout), (int)n, eps, (int)S, ps, ea, img, (int)rows);
+  TLHIP_CHECK_LAUNCH(TLHIP_C_RMSNORM_RES);
+}
+
+int tlhip_gemm_f16w_nt_aimage(const void* A, const void* aimage, const void* image, const void* exps, void* C,
+                              int64_t M, int64_t N, int64_t K) {
+  if (!aimage) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_aimage: null activation image");
+  return gemm_f16w_impl(A, image, exps, C, M, N, K, 0, nullptr, false, aimage);
+}
+
+int tlhip_gemm_f16w_nt_swiglu_aimage(const void* A, const void* aimage, const void* image, const void* exps,
+                                     void* act, int64_t M, int64_t ff, int64_t K) {
+  if (!aimage) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_swiglu_aimage: null activation image");
+  return gemm_f16w_impl(A, image, exps, act, M, ff, K, 0, nullptr, true, aimage);
+}
+
+int tlhip_gemm_f16w_nt_parts_aimage(const void* A, const void* aimage, const void* image, const void* exps,
+                                    void* parts, int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int* n_parts) {
+  if (!n_parts || !aimage) return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_parts_aimage: null n_parts or activation image");
+  if (M > 0 && N > 0 && parts_bytes < (int64_t)(M * N * sizeof(float)))
+    return fail(TLHIP_EINVAL, "tlhip_gemm_f16w_nt_parts_aimage: the buffer must hold at least one [M, N] part");
+  *n_parts = 0;
+  return gemm_f16w_impl(A, image, exps, parts, M, N, K, (size_t)parts_bytes, n_parts, false, aimage);
 }
 
 int tlhip_gemm_f16w_nt_parts(const void* A, const void* image, const void* exps, void* parts,

@@ -301,6 +301,7 @@ void tlq_greedy_sync_host_pos(void* hv) {
 
 void tlq_set_fused(void* hv, int on) { static_cast<handle*>(hv)->M.fused = on != 0; }
 void tlq_set_fused_attn(void* hv, int on) { static_cast<handle*>(hv)->M.fused_attn = on != 0; }
+void tlq_set_norm_images(void* hv, int on) { static_cast<handle*>(hv)->M.norm_images = on != 0; }
 void tlq_set_merge_in_oproj(void* hv, int on) { static_cast<handle*>(hv)->M.merge_in_oproj = on != 0; }
 void tlq_set_fused_prefill(void* hv, int on) { static_cast<handle*>(hv)->M.fused_prefill = on != 0; }
 // prompt chunks of bf16 weights on their prepared f16 images (default) or on the bf16 rows

@@ -167,6 +167,15 @@ struct api {
                                 void*, int64_t, int64_t, int64_t, float) = nullptr;
   int (*gemv_bf16_row_rmsnorm_gateup)(const void*, const void*, const void*, void*, const void*, void*,
                                       int64_t, int64_t, float) = nullptr;
+  int64_t (*gemm_f16w_aimage_bytes)(int64_t, int64_t) = nullptr;
+  int (*rmsnorm_res_parts_aimage)(const void*, const void*, int64_t, const void*, void*, void*, int64_t, float,
+                                  int64_t, void*) = nullptr;
+  int (*gemm_f16w_nt_aimage)(const void*, const void*, const void*, const void*, void*, int64_t, int64_t,
+                             int64_t) = nullptr;
+  int (*gemm_f16w_nt_parts_aimage)(const void*, const void*, const void*, const void*, void*, int64_t, int64_t,
+                                   int64_t, int64_t, int*) = nullptr;
+  int (*gemm_f16w_nt_swiglu_aimage)(const void*, const void*, const void*, const void*, void*, int64_t, int64_t,
+                                    int64_t) = nullptr;
   int (*attn_parts_splits)(int64_t, int64_t, int64_t, int64_t, int) = nullptr;
   int (*attn_decode_qkv_parts)(const void*, const void*, const void*, const void*, void*, void*, int64_t, int64_t,
                               int64_t, const void*, int64_t, int64_t, float, const void*, void*, int64_t,
@@ -207,6 +216,18 @@ struct extent {
   // refused the product): not tried again until the extent's device bytes change.
   struct unprepared { size_t off; int64_t n, k; bool gated; };
   std::vector<unprepared> refused;
+  // The activation image of `rows` f32 rows of `k` at offset `off` of this extent (row exponents
+  // and two f16 terms, the operand form of the prompt products over a prepared weight), written
+  // by the launch that produced the rows. `valid` ends as soon as the extent's device bytes can
+  // change; the allocation stays with the extent for the next producer (a layer's norm output is
+  // the same buffer every layer) and goes when the extent is released.
+  struct act_image {
+    void* buf = nullptr;
+    size_t bytes = 0, off = 0;
+    int64_t rows = 0, k = 0;
+    bool valid = false;
+  };
+  act_image act;
 };
 
 // The extents in use, ordered by base address so that an address INSIDE one (q4 scales at
@@ -351,6 +372,11 @@ struct context {
               bind(f.gemv_bf16_row_rmsnorm, "tlhip_gemv_bf16_row_rmsnorm") &&
               bind(f.gemv_q4_rmsnorm_gateup, "tlhip_gemv_q4_rmsnorm_gateup") &&
               bind(f.gemv_bf16_row_rmsnorm_gateup, "tlhip_gemv_bf16_row_rmsnorm_gateup") &&
+              bind(f.gemm_f16w_aimage_bytes, "tlhip_gemm_f16w_aimage_bytes") &&
+              bind(f.rmsnorm_res_parts_aimage, "tlhip_rmsnorm_res_parts_aimage") &&
+              bind(f.gemm_f16w_nt_aimage, "tlhip_gemm_f16w_nt_aimage") &&
+              bind(f.gemm_f16w_nt_parts_aimage, "tlhip_gemm_f16w_nt_parts_aimage") &&
+              bind(f.gemm_f16w_nt_swiglu_aimage, "tlhip_gemm_f16w_nt_swiglu_aimage") &&
               bind(f.attn_parts_splits, "tlhip_attn_parts_splits") &&
               bind(f.attn_decode_qkv_parts, "tlhip_attn_decode_qkv_parts") &&
               bind(f.gemv_q4_attn, "tlhip_gemv_q4_attn") &&
@@ -404,6 +430,48 @@ struct context {
     }
     e.derived.clear();
     e.refused.clear();
+    e.act.valid = false;
+  }
+  // Room for the activation image of the `rows` rows of `k` at `p` that a launch is about to
+  // write, kept with p's extent (allocated on first use, reused afterwards). nullptr: not a
+  // managed buffer, not a shape that has an image, a capture is open, or no memory.
+  void* act_image_room(void* p, int64_t rows, int64_t k) {
+    if (!prompt_f16 || capturing) return nullptr;
+    extent* e = buffers.containing(p);
+    if (!e) return nullptr;
+    const int64_t bytes = f.gemm_f16w_aimage_bytes(rows, k);
+    const size_t off = static_cast<size_t>(static_cast<char*>(p) - e->base);
+    if (bytes <= 0 || off + static_cast<size_t>(rows * k * 4) > e->size) return nullptr;
+    extent::act_image& a = e->act;
+    a.valid = false;
+    if (a.bytes < static_cast<size_t>(bytes)) {
+      if (a.buf) f.free_(a.buf);
+      a.buf = nullptr;
+      a.bytes = 0;
+      if (f.malloc_(&a.buf, static_cast<size_t>(bytes)) != 0) { a.buf = nullptr; return nullptr; }
+      a.bytes = static_cast<size_t>(bytes);
+    }
+    a.off = off; a.rows = rows; a.k = k;
+    return a.buf;
+  }
+  void act_image_made(void* p) {
+    if (extent* e = buffers.containing(p)) e->act.valid = e->act.buf != nullptr;
+  }
+  // The image of exactly these rows, if the launch that wrote them left one and nothing has
+  // written the extent since.
+  const void* act_image_of(const void* p, int64_t rows, int64_t k) {
+    if (!prompt_f16) return nullptr;
+    extent* e = buffers.containing(p);
+    if (!e || !e->act.valid) return nullptr;
+    const size_t off = static_cast<size_t>(static_cast<const char*>(p) - e->base);
+    return e->act.off == off && e->act.rows == rows && e->act.k == k ? e->act.buf : nullptr;
+  }
+  void drop_act_image(extent& e) {
+    if (e.act.buf) {
+      if (capturing) deferred_free.push_back(e.act.buf);
+      else f.free_(e.act.buf);
+    }
+    e.act = extent::act_image{};
   }
   void free_deferred() {
     for (void* p : deferred_free) f.free_(p);
@@ -483,6 +551,10 @@ class launch {
   const extent::prepared* prepared(void* B, int64_t n, int64_t k, bool gated) { return c_.prepared_weight(B, n, k, gated); }
   // the library refused the product over the prepared form: the caller goes on to the bf16 rows
   void refused(void* B, const extent::prepared* p) { c_.refuse_prepared(B, p); }
+  // see context::act_image_room / act_image_made / act_image_of; room() after writes(), made() after a good launch
+  void* act_room(void* p, int64_t rows, int64_t k) { return c_.act_image_room(p, rows, k); }
+  void act_made(void* p) { c_.act_image_made(p); }
+  const void* act_of(const void* p, int64_t rows, int64_t k) { return c_.act_image_of(p, rows, k); }
   bool sent(int rc) {
     if (rc != 0) return false;   // declined or failed: the caller falls back
     c_.pending = true;
@@ -579,6 +651,7 @@ inline void release(void* buf, int64_t, float*) {
   extent e;
   c.buffers.leave(buf, e);
   c.forget_derived(e);
+  c.drop_act_image(e);
   if (e.staging) c.buffers.park(e);
   else c.f.free_(e.base);   // device-only extents are not kept for reuse
 }
@@ -743,7 +816,10 @@ inline bool gemm_bf16_nt(void* a, void* B, void* out, int64_t m, int64_t n, int6
   L.writes(out);
   if (prompt_product_is_large(m, n, k))   // on the weight's prepared f16 form where there is one
     if (const auto* p = L.prepared(B, n, k, false)) {
-      if (L.sent(L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k))) return true;
+      const void* ai = L.act_of(a, m, k);   // the activation image a's producer left, if any
+      if (L.sent(ai ? L.lib.gemm_f16w_nt_aimage(a, ai, p->image, p->exps, out, m, n, k)
+                    : L.lib.gemm_f16w_nt(a, p->image, p->exps, out, m, n, k)))
+        return true;
       L.refused(B, p);                    // the bf16 rows serve what the prepared product declined
     }
   return L.sent(L.lib.gemm_bf16_nt(a, B, out, m, n, k));
@@ -757,7 +833,10 @@ inline bool gemm_bf16_nt_swiglu(void* a, void* B, void* act, int64_t m, int64_t 
   L.writes(act);
   if (prompt_product_is_large(m, 2 * ff, k))
     if (const auto* p = L.prepared(B, ff, k, true)) {
-      if (L.sent(L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k))) return true;
+      const void* ai = L.act_of(a, m, k);
+      if (L.sent(ai ? L.lib.gemm_f16w_nt_swiglu_aimage(a, ai, p->image, p->exps, act, m, ff, k)
+                    : L.lib.gemm_f16w_nt_swiglu(a, p->image, p->exps, act, m, ff, k)))
+        return true;
       L.refused(B, p);
     }
   return L.sent(L.lib.gemm_bf16_nt_swiglu(a, B, act, m, ff, k));
@@ -799,7 +878,10 @@ inline bool gemm_bf16_nt_parts(void* a, void* B, void* parts, int64_t parts_byte
   L.writes(parts);
   if (prompt_product_is_large(m, n, k))
     if (const auto* p = L.prepared(B, n, k, false)) {
-      if (L.sent(L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts))) return true;
+      const void* ai = L.act_of(a, m, k);
+      if (L.sent(ai ? L.lib.gemm_f16w_nt_parts_aimage(a, ai, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts)
+                    : L.lib.gemm_f16w_nt_parts(a, p->image, p->exps, parts, parts_bytes, m, n, k, n_parts)))
+        return true;
       L.refused(B, p);
     }
   return L.sent(L.lib.gemm_bf16_nt_parts(a, B, parts, parts_bytes, m, n, k, n_parts));
@@ -881,12 +963,22 @@ inline bool rmsnorm_res(void* x, void* delta, void* w, void* xout, void* hout, i
 }
 
 // rmsnorm_res with delta = parts[0] + ... + parts[n_parts-1], rows * n floats apart.
+// next_n: columns of the bf16 product that will consume hout (0: unknown or none). Where that
+// product will run over the weight's prepared form, the norm leaves hout's activation image with
+// hout's buffer and the product skips its own pass over hout (same bits either way).
 inline bool rmsnorm_res_parts(void* x, void* parts, int64_t n_parts, void* w, void* xout, void* hout,
-                              int64_t n, float eps, int64_t rows = 1) {
+                              int64_t n, float eps, int64_t rows = 1, int64_t next_n = 0) {
   launch L;
   if (!L.ok || n <= 0 || rows <= 0 || n_parts <= 0) return false;
   L.reads(x, parts, w);
   L.writes(xout, hout);
+  if (next_n > 0 && prompt_product_is_large(rows, next_n, n) && (n % 32) == 0 && n <= 8192)
+    if (void* room = L.act_room(hout, rows, n)) {
+      if (L.sent(L.lib.rmsnorm_res_parts_aimage(x, parts, n_parts, w, xout, hout, n, eps, rows, room))) {
+        L.act_made(hout);
+        return true;
+      }
+    }
   return L.sent(L.lib.rmsnorm_res_parts(x, parts, n_parts, w, xout, hout, n, eps, rows));
 }
 

@@ -191,6 +191,7 @@ struct model {
   // models), the o-projection's GEMV merges them while it stages its input: no merge launch
   bool merge_in_oproj = true;
   bool fused_prefill = true;     // prompt chunks: one launch for split_heads + rope + kv_fill, attention writes token-major
+  bool norm_images = true;       // prompt chunks: the residual norms leave the activation image of their output for the prepared-weight product that reads it
   bool prompt_f16 = true;        // prompt chunks of bf16 weights on the backend's prepared f16 form of them (a second copy, made on first use)
   bool gateup_epilogue = true;   // within the fused path: swiglu as the gate|up GEMV's epilogue, not the down GEMV's producer
   // within the fused path: blocks of the weight warm-up that runs beside each layer on a second
@@ -906,10 +907,14 @@ inline bool prefill_layers(model& M, int64_t T) {
       // o-proj and down leave their K-split parts; the residual norm adds them up as it reads
       int np = 0;
       ok &= gemm_parts(L.wo, P.at, P.parts, P.parts_bytes, T, &np);
-      ok = ok && hip::rmsnorm_res_parts(x, P.parts, np, L.fn, ro, P.h2, E, d.eps, T);
+      // (the norms are told which bf16 product reads their output: where that one runs over a
+      // prepared weight, the norm leaves the activation image it would otherwise make itself)
+      const auto cols = [&](const linear& W) { return W.fmt == wfmt::q4 || !M.norm_images ? int64_t(0) : W.N; };
+      ok = ok && hip::rmsnorm_res_parts(x, P.parts, np, L.fn, ro, P.h2, E, d.eps, T, cols(L.wgu));
       ok &= gemm_swiglu(L.wgu, P.h2, P.mb, T);   // the gate as the epilogue
       ok &= gemm_parts(L.wd, P.mb, P.parts, P.parts_bytes, T, &np);
-      ok = ok && hip::rmsnorm_res_parts(ro, P.parts, np, nextw, ro, P.h, E, d.eps, T);
+      ok = ok && hip::rmsnorm_res_parts(ro, P.parts, np, nextw, ro, P.h, E, d.eps, T,
+                                        l + 1 < d.n_layers ? cols(M.layers[(size_t)l + 1].wqkv) : int64_t(0));
     } else {
     ok &= gemm(L.wo, P.at, ro, T);
     ok &= hip::rmsnorm_res(ro, x, L.fn, ro, P.h2, E, d.eps, T);

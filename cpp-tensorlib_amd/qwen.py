@@ -63,6 +63,7 @@ def _load():
             "tlq_profile_steps": (cint, [P, i64, i64, i64, C.POINTER(C.c_double)]),
             "tlq_set_fused_attn": (None, [P, cint]),
             "tlq_set_merge_in_oproj": (None, [P, cint]),
+            "tlq_set_norm_images": (None, [P, cint]),
             "tlq_set_gateup_epilogue": (None, [P, cint]),
             "tlq_set_fused_prefill": (None, [P, cint]),
             "tlq_set_prompt_f16": (None, [P, cint]),
@@ -353,6 +354,11 @@ class QwenGPU:
     def set_fused_attn(self, on):
         """Within the fused path: run the q/k/v epilogue inside the attention launch (default) or alone."""
         self.L.tlq_set_fused_attn(self.h, 1 if on else 0)
+
+    def set_norm_images(self, on):
+        """Prompt chunks: let the residual norms leave the activation image of their output for the
+        prepared-weight product that reads it (default), or let every product cut its own."""
+        self.L.tlq_set_norm_images(self.h, 1 if on else 0)
 
     def set_merge_in_oproj(self, on):
         """Within the fused attention: let the o-projection's GEMV merge the attention's splits where

@@ -415,6 +415,26 @@ int tlhip_gemm_f16w_nt_parts(const void* A, const void* image, const void* exps,
                              int64_t parts_bytes, int64_t M, int64_t N, int64_t K, int* n_parts);
 int tlhip_gemm_f16w_nt_swiglu(const void* A, const void* image, const void* exps, void* act, int64_t M,
                               int64_t ff, int64_t K);
+/* The same three products over an ACTIVATION IMAGE made beforehand: the row exponents and the two
+ * f16 terms of A as slab images (tlhip_gemm_f16w_aimage_bytes(M, K) bytes, 16-byte aligned; 0: no
+ * image for this shape), which the products above make on every call and the producer of A can
+ * make while it still holds A's rows. One producer does: tlhip_rmsnorm_res_parts_aimage is
+ * tlhip_rmsnorm_res_parts (same arguments, same bits in xout and hout; n % 32 == 0, n <= 8192)
+ * that also leaves hout's image in `aimage`, saving the products' own pass over A (one launch and
+ * one read of A per product: the two norms of a layer feed q|k|v and gate|up). A must still be
+ * passed, and must be the rows the image was made from, unchanged: wide-range results are worked
+ * out from them (above). Same results bit for bit as the calls without an image. No counterpart
+ * in the reference (the products and the norm are separate ops, qwen_model.h:559-599). */
+int64_t tlhip_gemm_f16w_aimage_bytes(int64_t M, int64_t K);
+int tlhip_rmsnorm_res_parts_aimage(const void* x, const void* parts, int64_t S, const void* w, void* xout,
+                                   void* hout, int64_t n, float eps, int64_t rows, void* aimage);
+int tlhip_gemm_f16w_nt_aimage(const void* A, const void* aimage, const void* image, const void* exps, void* C,
+                              int64_t M, int64_t N, int64_t K);
+int tlhip_gemm_f16w_nt_parts_aimage(const void* A, const void* aimage, const void* image, const void* exps,
+                                    void* parts, int64_t parts_bytes, int64_t M, int64_t N, int64_t K,
+                                    int* n_parts);
+int tlhip_gemm_f16w_nt_swiglu_aimage(const void* A, const void* aimage, const void* image, const void* exps,
+                                     void* act, int64_t M, int64_t ff, int64_t K);
 /* The three prompt-chunk products over an int4 weight (qw = packed nibbles [N][K/2], scales
  * [N][K/32], group 32 - the operand of tlhip_gemv_q4): C = A . dequant(W)^T formed as
  * sum over groups of scale * (A . q) with exact products on the matrix pipe, fp32 sums - the decode

@@ -314,6 +314,48 @@ int main() {
     check("a weight element its f16 image cannot hold is taken from the weight itself where it shows", ok);
   }
 
+  {  // the residual norm of a prompt chunk leaves the activation image of its output with the
+     // output's buffer, and the product that follows uses it instead of cutting the rows itself:
+     // a host edit or a device write of the norm's output between the two must reach the product
+    const int64_t m = 512, n = 4096, k = 2048;      // m * n * k = 4.3e9: the product is prepared
+    buf x(m * k), parts(2 * m * k), nw(k), xo(m * k), h(m * k), w(n * k / 2), o(m * n), other(m * k);
+    fill(x); fill(parts, 0.25f); fill(other, 3.0f);
+    { float* p = nw.write(); for (int64_t i = 0; i < k; i++) p[i] = 1.0f + 0.1f * rnd(); }
+    uint16_t* pw = reinterpret_cast<uint16_t*>(w.write());
+    for (int64_t i = 0; i < n * k; i++) { const float v = 0.05f * rnd(); uint32_t u; std::memcpy(&u, &v, 4); pw[i] = (uint16_t)(u >> 16); }
+    auto rows_match = [&](const char* what) {        // o against h (read back) times w, in float64
+      std::vector<float> hh(h.read(), h.read() + m * k);
+      const float* got = o.read();
+      for (int64_t r : {int64_t(0), m / 2, m - 1})
+        for (int64_t c : {int64_t(0), int64_t(33), n - 1}) {
+          double want = 0;
+          for (int64_t i = 0; i < k; i++) {
+            const uint32_t u = (uint32_t)reinterpret_cast<const uint16_t*>(w.host)[c * k + i] << 16;
+            float f; std::memcpy(&f, &u, 4);
+            want += (double)hh[r * k + i] * (double)f;
+          }
+          if (!close(got[r * n + c], want)) {
+            std::printf("  %s at (%lld, %lld): got %.9g want %.9g\n", what, (long long)r, (long long)c, got[r * n + c], want);
+            return false;
+          }
+        }
+      return true;
+    };
+    auto norm = [&] { return hip::rmsnorm_res_parts(x.native, parts.native, 2, nw.native, xo.native, h.native, k, 1e-6f, m, n); };
+    bool ok = norm() && hip::gemm_bf16_nt(h.native, w.native, o.native, m, n, k) && rows_match("product after the norm");
+    ok = ok && norm();
+    h.write()[(m / 2) * k + 7] = 1000.0f;                                    // host edit of the norm's output
+    ok = ok && hip::gemm_bf16_nt(h.native, w.native, o.native, m, n, k) && rows_match("after a host edit of the rows");
+    ok = ok && norm();
+    other.read();
+    ok = ok && hip::copy_d2d(h.native, other.native, m * k * 4);             // device write of the norm's output
+    ok = ok && hip::gemm_bf16_nt(h.native, w.native, o.native, m, n, k) && rows_match("after a device copy into the rows");
+    hip::set_prompt_f16(false);
+    ok = ok && norm() && hip::gemm_bf16_nt(h.native, w.native, o.native, m, n, k) && rows_match("on the bf16 rows");
+    hip::set_prompt_f16(true);
+    check("the norm's activation image follows host edits and device writes of the norm's output", ok);
+  }
+
   {  // a product deeper than the prepared form goes (K > 32768) has no image and runs on the bf16 rows
     const int64_t m = 96, n = 1280, k = 32768 + 64;                          // m * n * k = 4.03e9: "large"
     buf a(m * k), w(n * k / 2), o(m * n);

@@ -385,3 +385,72 @@ def test_gemm_f16w_declines(lib):
     lib.last_error()
     for b in (a, w, c, img, ex):
         b.free()
+
+
+@pytest.mark.parametrize("rows,n,S", [(512, 3584, 4), (300, 896, 3), (77, 8192, 1), (512, 4096, 2), (1, 64, 1)])
+def test_norm_leaves_the_activation_image(lib, orc, rows, n, S):
+    """tlhip_rmsnorm_res_parts_aimage: the residual norm of a prompt chunk that writes the activation
+    image of its own output. xout and hout are the bits of tlhip_rmsnorm_res_parts, and the three
+    products over that image are the bits of the products that cut the activations themselves -
+    plain, K-split parts and gated - on ordinary rows and on rows with tiny elements under a large
+    one, a zero row and a row with an infinity (the image's small-element marks decide which
+    results the GEMM works out again)."""
+    print("case norm aimage", rows, n, S, flush=True)
+    x = orc.normal(rows * n, 201).reshape(rows, n)
+    parts = orc.normal(S * rows * n, 202, std=0.3).reshape(S, rows, n)
+    w = orc.normal(n, 203, 1.0, 0.1)
+    if rows > 8:
+        x[3, :] = 0.0
+        parts[:, 3, :] = 0.0                      # a zero row
+        x[5, ::7] *= 1e-9                         # elements far below their row's largest
+        x[5, 1] = 3e4
+        parts[:, 5, :] = 0.0
+        x[6, 2] = np.inf                          # a row that is not finite
+    dx, dp, dw = lib.to_device(x), lib.to_device(parts), lib.to_device(w)
+    xo1, h1, xo2, h2 = (lib.empty((rows, n)) for _ in range(4))
+    nb = lib.gemm_f16w_aimage_bytes(rows, n)
+    assert nb > 0
+    aimg = lib.empty_bytes(nb)
+    lib.rmsnorm_res_parts(dx, dp, S, dw, xo1, h1, n, 1e-6, rows)
+    lib.rmsnorm_res_parts_aimage(dx, dp, S, dw, xo2, h2, n, 1e-6, rows, aimg)
+    assert np.array_equal(xo1.numpy(), xo2.numpy(), equal_nan=True)
+    H1, H2 = h1.numpy(), h2.numpy()
+    assert np.array_equal(H1, H2, equal_nan=True)
+    # the products over the image against the products that make their own
+    N, ff = 384, 256
+    Wb = orc.to_bf16(orc.normal(N * n, 204, std=0.02)).reshape(N, n)
+    Wg = orc.to_bf16(orc.normal(2 * ff * n, 205, std=0.02)).reshape(2 * ff, n)
+    P, G = Prepared(lib, Wb), Prepared(lib, Wg, gated=True)
+    c1, c2 = lib.empty((rows, N)), lib.empty((rows, N))
+    lib.gemm_f16w_nt(h1, P.image, P.exps, c1, rows, N, n)
+    lib.gemm_f16w_nt_aimage(h2, aimg, P.image, P.exps, c2, rows, N, n)
+    assert np.array_equal(c1.numpy(), c2.numpy(), equal_nan=True)
+    a1, a2 = lib.empty((rows, ff)), lib.empty((rows, ff))
+    lib.gemm_f16w_nt_swiglu(h1, G.image, G.exps, a1, rows, ff, n)
+    lib.gemm_f16w_nt_swiglu_aimage(h2, aimg, G.image, G.exps, a2, rows, ff, n)
+    assert np.array_equal(a1.numpy(), a2.numpy(), equal_nan=True)
+    p1, p2 = lib.empty((8, rows, N)), lib.empty((8, rows, N))
+    s1 = lib.gemm_f16w_nt_parts(h1, P.image, P.exps, p1, rows, N, n)
+    s2 = lib.gemm_f16w_nt_parts_aimage(h2, aimg, P.image, P.exps, p2, rows, N, n)
+    assert s1 == s2 and np.array_equal(p1.numpy()[:s1], p2.numpy()[:s2], equal_nan=True)
+    # and against the oracle on the finite rows
+    fin = np.all(np.isfinite(H1), axis=1)
+    want = orc.gemm_bf16_nt(np.ascontiguousarray(H1[fin]), Wb)
+    got = c2.numpy()[fin]
+    ok, worst, _ = _same_as_fp32_chain(got, want, H1[fin], orc.bf16_widen(Wb).reshape(N, n))
+    assert ok, (worst, maxrel(got, want))
+    for b in (dx, dp, dw, xo1, h1, xo2, h2, aimg, c1, c2, a1, a2, p1, p2):
+        b.free()
+    P.free(); G.free()
+
+
+def test_norm_aimage_declines(lib):
+    """Shapes without an image: n not a multiple of 32, n beyond the register-resident norm."""
+    assert lib.gemm_f16w_aimage_bytes(512, 100) == 0
+    assert lib.gemm_f16w_aimage_bytes(512, 65536) == 0
+    x, p, w, o, h = (lib.empty((4, 16384)) for _ in range(5))
+    a = lib.empty_bytes(lib.gemm_f16w_aimage_bytes(4, 16384))
+    with pytest.raises(Exception):
+        lib.rmsnorm_res_parts_aimage(x, p, 1, w, o, h, 16384, 1e-6, 4, a)
+    for b in (x, p, w, o, h, a):
+        b.free()
