@@ -231,6 +231,17 @@ def decode_7b(lib, steps, eager=False, warm=None):
     # where the step's GPU time goes: events between the launches of five eager steps (the role
     # of the reference's StepProf, bench_qwen_decode.cpp:212-237); the events cost a little themselves
     layer_us = {k: round(v, 2) for k, v in g.profile_steps(11, pos, 5).items()}
+    # what an event costs: the same eager step without them, timed by two events around five steps
+    pe0, pe1 = lib.event(), lib.event()
+    lib.record(pe0)
+    for _ in range(5):
+        g.run_layers(11, pos)
+    lib.record(pe1)
+    g.flush()
+    plain_us = lib.elapsed_ms(pe0, pe1) * 1e3 / 5
+    n_events = 5 * g.d.n_layers + 2
+    layer_us["event_cost"] = round(max(0.0, (layer_us["step"] - plain_us) / n_events), 2)
+    layer_us["step_without_events"] = round(plain_us, 2)
     g.capture(11, pos)
     for _ in range(3):
         g.replay()
@@ -296,7 +307,7 @@ def decode_7b(lib, steps, eager=False, warm=None):
                  "tok_s_greedy_token_loop_on_device": round(1e3 / greedy_dev, 1)},
         "algorithmic_bytes": int(wbytes + kvbytes),
         "hbm_frac": round((wbytes + kvbytes) / (best * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "layer_us": dict(layer_us, what="eager step with an event between its regions: microseconds per layer "
+        "layer_us": dict(layer_us, what="eager step with an event between its regions: microseconds per layer, each region including one event's cost (event_cost, from the same step without events) "
                                         "(lm_head, step: per token); attention = q/k/v epilogue + attention + split combine"),
     }
 
